@@ -1,0 +1,217 @@
+/*
+ * saetta_hip.h -- C ABI of the MI355X (gfx950) attention hot path.
+ *
+ * The library replaces, for this one path, what the reference's Rust modules
+ * src/kv_quant.rs, src/attention.rs, src/rows.rs (verify attention) and
+ * src/attention_prefill.rs dispatch to Metal.  Every entry point is
+ * extern "C", takes plain device pointers, POD parameter blocks that are
+ * field-for-field the reference's #[repr(C)] structs, and an explicit HIP
+ * stream; it enqueues work on that stream and returns without synchronising.
+ *
+ * Return value: 0 on success; a negative SAETTA_E_* code for a rejected
+ * argument (the reference `assert!`s in these places, so a binding turns a
+ * non-zero return into a panic); a positive value is the hipError_t of a
+ * failed launch.  saetta_last_error() gives the text for the calling thread.
+ * Nothing is thrown across the boundary and nothing aborts.
+ *
+ * Device pointers must be valid on the current HIP device.  "d_tp" arguments
+ * point at a TokenParams record IN DEVICE MEMORY: launches read the position
+ * and length from it when they run, so a recorded sequence of launches (a
+ * plan, a HIP graph) serves every token position, as the reference's plans do
+ * (src/plan.rs:1-11).
+ */
+#ifndef SAETTA_HIP_H
+#define SAETTA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* hipStream_t, spelled without the HIP headers. */
+typedef void *saetta_stream_t;
+
+/* Fixed shape of the path (src/attention.rs:14-17, src/kv_quant.rs:9). */
+#define SAETTA_HEAD_DIM 256
+#define SAETTA_GQA_GROUP 8   /* q heads per kv head */
+#define SAETTA_QUANT_GROUP 64 /* values per scale/bias */
+#define SAETTA_CHUNK 128      /* tokens per split-K chunk */
+#define SAETTA_MAX_ROWS 8     /* src/rows.rs:9 */
+
+enum {
+    SAETTA_OK = 0,
+    SAETTA_E_BITS = -1,     /* bits not one the call accepts */
+    SAETTA_E_SHAPE = -2,    /* heads / kv_heads / head_dim / rows / capacity not supported */
+    SAETTA_E_NULL = -3,     /* a required pointer is NULL */
+    SAETTA_E_ALIGN = -4,    /* a pointer is not aligned as documented */
+    SAETTA_E_DEVICE = -5,   /* no gfx950 device / code object not loadable */
+    SAETTA_E_SCRATCH = -6   /* scratch too small for the request */
+};
+
+/* TokenParams (src/plan.rs:16-35; kernels/params.metal:7-15). */
+typedef struct saetta_token_params {
+    uint32_t token;
+    uint32_t position;
+    uint32_t kv_len; /* position + 1 */
+    uint32_t pad;
+} saetta_token_params;
+
+/* KvQuantParams (src/kv_quant.rs:147-153; kernels/kv_quant.metal:8-11). */
+typedef struct saetta_kv_quant_params {
+    uint32_t groups;    /* groups of 64 values to process, from x[0] */
+    uint32_t per_token; /* groups per token: kv_heads * 256 / 64 */
+} saetta_kv_quant_params;
+
+/* DecodeParams (src/attention.rs:19-26; kernels/attention.metal:18-23). */
+typedef struct saetta_decode_params {
+    uint32_t heads;
+    uint32_t kv_heads;
+    uint32_t capacity; /* tokens the cache has room for */
+    float scale;       /* 1/sqrt(256) */
+} saetta_decode_params;
+
+/* RowsAttentionParams (src/rows.rs:307-317; kernels/attention_rows.metal:58-65).
+ * `splits` is the number of partial results per (row, q head) the scratch
+ * has room for; the library uses min(splits, its own choice). */
+typedef struct saetta_rows_params {
+    uint32_t heads;
+    uint32_t kv_heads;
+    uint32_t capacity;
+    float scale;
+    uint32_t rows;   /* m, 1..8 */
+    uint32_t splits;
+} saetta_rows_params;
+
+/* FlashParams (src/attention_prefill.rs:4-14). */
+typedef struct saetta_flash_params {
+    uint32_t heads;
+    uint32_t kv_heads;
+    uint32_t pos;    /* position of the chunk's first token; token i sees keys 0..=pos+i */
+    uint32_t tokens;
+    float scale;
+} saetta_flash_params;
+
+/* The three arrays of one quantized cache, keys or values: QuantRows
+ * {data, scales, biases} (src/kv_quant.rs:156-180).  Token p's groups start
+ * at group p * per_token; group G's codes are words 2*bits*G onward, lowest
+ * bits first; scales and biases are IEEE halves. */
+typedef struct saetta_quant_rows {
+    uint32_t *data;
+    uint16_t *scales;
+    uint16_t *biases;
+} saetta_quant_rows;
+
+/* ---- set-up --------------------------------------------------------------- */
+
+/* Checks that the current device is gfx950 and that the kernels load.  Stands
+ * where Gpu::new() (src/gpu.rs:233-263) stands for this path.  Optional: every
+ * entry point does the same check on first use. */
+int saetta_init(void);
+
+/* Text of the last error on this thread ("" if none). */
+const char *saetta_last_error(void);
+
+/* ---- kv_quant (src/kv_quant.rs) -------------------------------------------- */
+
+/* QuantRows::record / record_at (src/kv_quant.rs:192-221) when d_tp != NULL:
+ * quantizes p.groups groups of x into the slots from token d_tp->position.
+ * QuantRows::encode (src/kv_quant.rs:256-282) when d_tp == NULL: the slots
+ * from token `pos`.  Kernel: kv_quantize_{8,4} (kernels/kv_quant.metal:15-59).
+ * Codes, scales and biases are bit-identical to the CPU quantize()
+ * (src/kv_quant.rs:54-87).  x must be 16-byte aligned. */
+int saetta_kv_quantize(saetta_stream_t stream, int bits, const float *x, saetta_quant_rows rows,
+                       saetta_kv_quant_params p, const saetta_token_params *d_tp, uint32_t pos);
+
+/* QuantRows::encode_dequantize (src/kv_quant.rs:225-252): groups 0..p.groups
+ * as halves, out[i] = half(f32(s) * q + f32(z)). */
+int saetta_kv_dequantize(saetta_stream_t stream, int bits, saetta_quant_rows rows, uint16_t *out_f16,
+                         saetta_kv_quant_params p);
+
+/* to_half (kernels/prefill.metal:1428-1432; src/prefill.rs:1658-1660,1690-1692):
+ * n floats to halves, round to nearest even. */
+int saetta_to_half(saetta_stream_t stream, const float *x, uint16_t *out_f16, size_t n);
+
+/* ---- decode and verify attention (src/attention.rs, src/rows.rs) ----------- */
+
+/* Bytes of part_o / part_ml scratch for a cache of `capacity` tokens and up
+ * to `rows` rows: never more than the reference allocates
+ * (rows * ceil(capacity/128) * heads * 256 * 4 and * 2 * 4,
+ * src/attention.rs:58-64, src/rows.rs:358-359). */
+size_t saetta_part_o_bytes(uint32_t heads, uint32_t capacity, uint32_t rows);
+size_t saetta_part_ml_bytes(uint32_t heads, uint32_t capacity, uint32_t rows);
+
+/* Stages of one attention call, for timing a kernel alone as the reference
+ * does with Plan::build_where (src/plan.rs:187-226, src/attention.rs:206). */
+#define SAETTA_STAGE_PARTIAL 1u
+#define SAETTA_STAGE_REDUCE 2u
+#define SAETTA_STAGE_ALL 3u
+
+/* DecodeAttention::record (src/attention.rs:73-92): one query token over a
+ * half cache.  q f32 [heads][256]; keys, values f16 [capacity][kv_heads][256];
+ * q_and_gate f32 [heads][512], the gate of head h at h*512+256; out f32
+ * [heads][256].  out = softmax(q K^T scale) V * sigmoid(gate) over the first
+ * min(d_tp->kv_len, capacity) tokens.  Kernels replaced: attention_partial,
+ * attention_partial_mma, attention_reduce (kernels/attention.metal:25-226,
+ * 367-409). */
+int saetta_attn_decode(saetta_stream_t stream, const float *q, const uint16_t *keys,
+                       const uint16_t *values, float *part_o, float *part_ml,
+                       const float *q_and_gate, float *out, saetta_decode_params p,
+                       const saetta_token_params *d_tp, uint32_t stages);
+
+/* DecodeAttention::record_quant (src/attention.rs:95-135): as above over an
+ * 8- or 4-bit cache.  Kernels replaced: attention_partial_mma_q{8,4}
+ * (kernels/attention.metal:242-360), attention_partial_q{8,4}
+ * (kernels/kv_quant.metal:101-204), attention_reduce. */
+int saetta_attn_decode_quant(saetta_stream_t stream, int bits, const float *q,
+                             saetta_quant_rows keys, saetta_quant_rows values, float *part_o,
+                             float *part_ml, const float *q_and_gate, float *out,
+                             saetta_decode_params p, const saetta_token_params *d_tp,
+                             uint32_t stages);
+
+/* AttentionRows::record (src/rows.rs:369-412): p.rows query tokens over a
+ * half cache; row r is at position d_tp->position + r and sees
+ * min(d_tp->position + r + 1, capacity) tokens.  q f32 [rows][heads][256],
+ * q_and_gate f32 [rows][heads][512], out f32 [rows][heads][256].  Kernels
+ * replaced: attention_partial_rows_chunks, attention_reduce_rows_chunks
+ * (kernels/attention_rows.metal:359-571). */
+int saetta_attn_rows(saetta_stream_t stream, const float *q, const uint16_t *keys,
+                     const uint16_t *values, float *part_o, float *part_ml,
+                     const float *q_and_gate, float *out, saetta_rows_params p,
+                     const saetta_token_params *d_tp, uint32_t stages);
+
+/* AttentionRows::record_quant (src/rows.rs:416-493).  Kernels replaced:
+ * attention_partial_rows<8|4>, attention_reduce_rows
+ * (kernels/attention_rows.metal:108-342). */
+int saetta_attn_rows_quant(saetta_stream_t stream, int bits, const float *q,
+                           saetta_quant_rows keys, saetta_quant_rows values, float *part_o,
+                           float *part_ml, const float *q_and_gate, float *out,
+                           saetta_rows_params p, const saetta_token_params *d_tp,
+                           uint32_t stages);
+
+/* ---- prefill attention (src/attention_prefill.rs, src/prefill.rs) ---------- */
+
+/* attention_prefill::encode (src/attention_prefill.rs:39-72): a causal chunk
+ * over a half cache that already holds the chunk's rows.  q f16
+ * [tokens][heads][256]; keys, values f16 [capacity][kv_heads][256] from
+ * position 0, capacity >= pos + tokens; q_and_gate f32 [tokens][heads][512];
+ * out f32 [tokens][heads][256].  Kernel replaced: attention_fa{4,8}
+ * (kernels/attention_prefill.metal:38-169). */
+int saetta_attn_prefill(saetta_stream_t stream, const uint16_t *q_f16, const uint16_t *keys,
+                        const uint16_t *values, const float *q_and_gate, float *out,
+                        saetta_flash_params p);
+
+/* The same chunk over an 8- or 4-bit cache read in place
+ * (src/prefill.rs:1674-1686,1735-1776); the cache is seen through half, as
+ * round_trip_as_half (src/kv_quant.rs:119-125) defines.  Kernels replaced:
+ * attention_rows_q{8,4}, attention_rows2_half_q{8,4}
+ * (kernels/attention_rows_q.metal:55-344). */
+int saetta_attn_prefill_quant(saetta_stream_t stream, int bits, const uint16_t *q_f16,
+                              saetta_quant_rows keys, saetta_quant_rows values,
+                              const float *q_and_gate, float *out, saetta_flash_params p);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SAETTA_HIP_H */

@@ -1,0 +1,32 @@
+// Shared by the kernel files of the gfx950 attention path: error plumbing for
+// the C ABI and a few device helpers.  HIP/CDNA4 only.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/saetta_hip.h"
+
+namespace saetta {
+
+// Per-thread text of the last failure, returned by saetta_last_error().
+char *error_buffer();
+int fail(int code, const char *fmt, ...);
+// Checks the device once per process; 0 or SAETTA_E_DEVICE.
+int ensure_device();
+// Turns the status of the launches since the last call into a return code.
+int launch_status(const char *what);
+
+inline hipStream_t as_stream(saetta_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+}  // namespace saetta
+
+#define SAETTA_REQUIRE(cond, code, ...)                       \
+    do {                                                      \
+        if (!(cond)) return saetta::fail((code), __VA_ARGS__); \
+    } while (0)

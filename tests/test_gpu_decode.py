@@ -1,0 +1,168 @@
+"""Decode and verify attention on the GPU against the oracle.
+
+Restates tests/attention.rs (half cache at lengths 1,2,127,128,129,1000,4096; quantized
+caches at 1,127,129,1000,1024; max abs error < 2e-5 against the f64 formula on the values
+the cache stands for) and src/rows.rs:666-743 (m rows == m single-row decodes, < 1e-4),
+plus the build's own bar: rel-RMS <= 1e-3 against the f32 CPU path (orc_attend).
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_common import D, H, KV, VALUES, cache_pair, dev, host, oracle, saetta
+
+pytestmark = pytest.mark.gpu
+KINDS = [saetta.KvBits.Half, saetta.KvBits.Eight, saetta.KvBits.Four]
+REL_RMS = 1e-3      # tolerance stated for the path, vs the f32 CPU reference
+MAX_ABS_F64 = 2e-5  # tests/attention.rs:91,198
+
+
+def run_decode(att, kind, q, kc, vc, qg, length):
+    out = torch.full((H, D), float("nan"), device="cuda")
+    plan = saetta.Plan()
+    if kind is saetta.KvBits.Half:
+        att.record(plan, q, kc, vc, qg, out)
+    else:
+        att.record_quant(plan, q, kc, vc, qg, out)
+    plan.set_params(saetta.TokenParams(0, length - 1))
+    plan.build().run()
+    return host(out)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_matches_cpu_at_several_lengths(kind):
+    capacity = 4096 if kind is saetta.KvBits.Half else 1024
+    lengths = [1, 2, 127, 128, 129, 1000, 4096] if kind is saetta.KvBits.Half else [1, 127, 129, 1000, 1024]
+    # Big keys make the softmax peaky, which tests the max handling.
+    k = (oracle.noise(capacity * VALUES, 1) * 4.0).reshape(capacity, VALUES)
+    v = oracle.noise(capacity * VALUES, 2).reshape(capacity, VALUES)
+    q = oracle.noise(H * D, 3)
+    qg = oracle.noise(H * 2 * D, 4)
+    kc, vc, kf, vf = cache_pair(k, v, kind, capacity, poison=False)
+    att = saetta.DecodeAttention(H, KV, D, capacity)
+    for length in lengths:
+        got = run_decode(att, kind, dev(q), kc, vc, dev(qg), length)
+        want64 = oracle.attention_f64(q, kf, vf, qg, length, threads=8)
+        worst = np.abs(got - want64).max()
+        assert worst < MAX_ABS_F64, f"{kind} len {length}: {worst}"
+        want32 = oracle.attend(q, kf, vf, length, q_and_gate=qg, threads=8)
+        assert oracle.rel_rms(got, want32) < REL_RMS
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_rows_past_the_context_never_reach_the_output(kind):
+    # hipMalloc'd caches are not zeroed: NaN scales, Inf biases and all-ones codes sit past kv_len.
+    capacity, length = 640, 333
+    rng = np.random.default_rng(4)
+    k = rng.standard_normal((length, VALUES)).astype(np.float32)
+    v = rng.standard_normal((length, VALUES)).astype(np.float32)
+    q = rng.standard_normal(H * D).astype(np.float32)
+    qg = rng.standard_normal(H * 2 * D).astype(np.float32)
+    kc, vc, kf, vf = cache_pair(k, v, kind, capacity, poison=True)
+    att = saetta.DecodeAttention(H, KV, D, capacity)
+    got = run_decode(att, kind, dev(q), kc, vc, dev(qg), length)
+    assert np.isfinite(got).all()
+    assert np.abs(got - oracle.attention_f64(q, kf, vf, qg, length, threads=8)).max() < MAX_ABS_F64
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8])
+def test_verify_rows_match_single_row_decodes(kind, m):
+    # src/rows.rs:666-743: contexts 40 and 1024 (+ one that is not a multiple of anything).
+    rng = np.random.default_rng(100 + m)
+    for ctx in (40, 1024, 1500):
+        capacity = -(-(ctx + saetta.MAX_ROWS) // 128) * 128
+        tokens = ctx - 1 + m
+        k = rng.standard_normal((tokens, VALUES)).astype(np.float32)
+        v = rng.standard_normal((tokens, VALUES)).astype(np.float32)
+        q = rng.standard_normal((m, H, D)).astype(np.float32)
+        qg = rng.standard_normal((m, H, 2 * D)).astype(np.float32)
+        kc, vc, kf, vf = cache_pair(k, v, kind, capacity)
+        rows = saetta.AttentionRows(H, KV, capacity, saetta.MAX_ROWS)
+        out = torch.full((m, H, D), float("nan"), device="cuda")
+        pos = ctx - 1
+        params = [saetta.TokenParams(0, pos + r).as_tensor("cuda") for r in range(m)]
+        plan = saetta.Plan()
+        if kind is saetta.KvBits.Half:
+            rows.record(plan, m, dev(q), kc, vc, dev(qg), out, params)
+        else:
+            rows.record_quant(plan, m, dev(q), kc, vc, dev(qg), out, params)
+        plan.build().run()
+        got = host(out)
+        want64 = oracle.rows(q, kf, vf, pos, m, q_and_gate=qg, threads=8, f64=True)
+        assert np.abs(got - want64).max() < MAX_ABS_F64, f"{kind} ctx {ctx} m {m}"
+        # ... and equal to m single-row decodes on the GPU (the reference's own check, < 1e-4).
+        att = saetta.DecodeAttention(H, KV, D, capacity)
+        for r in range(m):
+            one = run_decode(att, kind, dev(q[r]), kc, vc, dev(qg[r]), pos + r + 1)
+            assert np.abs(one - got[r]).max() < 1e-4
+
+
+@pytest.mark.parametrize("kind", [saetta.KvBits.Eight, saetta.KvBits.Four])
+def test_long_context_with_outlier_channels(kind):
+    # configs[1]/[3] in shape: 8-bit at 32768 + m rows, 4-bit with 1 % of channels x8; the new
+    # tokens are quantized on the device into the rows after the context.
+    rng = np.random.default_rng(8)
+    ctx, m = (32768, 4) if kind is saetta.KvBits.Eight else (20000, 1)
+    capacity = -(-(ctx + m) // 128) * 128
+    k = rng.standard_normal((ctx + m, VALUES)).astype(np.float32)
+    v = rng.standard_normal((ctx + m, VALUES)).astype(np.float32)
+    if kind is saetta.KvBits.Four:
+        ch = rng.choice(VALUES, 5, replace=False)
+        k[:, ch] *= 8
+        v[:, ch] *= 8
+    q = rng.standard_normal((m, H, D)).astype(np.float32)
+    qg = rng.standard_normal((m, H, 2 * D)).astype(np.float32)
+    kc, vc, kf, vf = cache_pair(k[:ctx], v[:ctx], kind, capacity)
+    kc.encode(dev(k[ctx:].reshape(-1)), ctx, m)
+    vc.encode(dev(v[ctx:].reshape(-1)), ctx, m)
+    bits = kind.value
+    kf = np.concatenate([kf, oracle.round_trip(k[ctx:], bits)])
+    vf = np.concatenate([vf, oracle.round_trip(v[ctx:], bits)])
+    rows = saetta.AttentionRows(H, KV, capacity, m)
+    out = torch.full((m, H, D), float("nan"), device="cuda")
+    plan = saetta.Plan()
+    rows.record_quant(plan, m, dev(q), kc, vc, dev(qg), out, [saetta.TokenParams(0, ctx).as_tensor("cuda")] * m)
+    plan.build().run()
+    got = host(out)
+    want = oracle.rows(q, kf, vf, ctx, m, q_and_gate=qg, threads=8)
+    assert oracle.rel_rms(got, want) < REL_RMS
+    want64 = oracle.rows(q, kf, vf, ctx, m, q_and_gate=qg, threads=8, f64=True)
+    # Outlier channels carry values 8x larger: the absolute bound scales with them.
+    assert np.abs(got - want64).max() < MAX_ABS_F64 * max(1.0, np.abs(want64).max())
+
+
+def test_one_plan_serves_every_position():
+    # Context length enters only through TokenParams (src/plan.rs:1-11).
+    capacity = 2048
+    rng = np.random.default_rng(5)
+    k = rng.standard_normal((capacity, VALUES)).astype(np.float32)
+    v = rng.standard_normal((capacity, VALUES)).astype(np.float32)
+    q, qg = rng.standard_normal(H * D).astype(np.float32), rng.standard_normal(H * 2 * D).astype(np.float32)
+    kc, vc, kf, vf = cache_pair(k, v, saetta.KvBits.Eight, capacity)
+    att = saetta.DecodeAttention(H, KV, D, capacity)
+    out = torch.zeros(H, D, device="cuda")
+    plan = saetta.Plan()
+    att.record_quant(plan, dev(q), kc, vc, dev(qg), out)
+    built = plan.build()
+    for length in (2048, 5, 700):
+        plan.set_params(saetta.TokenParams(0, length - 1))
+        built.run()
+        assert np.abs(host(out) - oracle.attention_f64(q, kf, vf, qg, length, threads=8)).max() < MAX_ABS_F64
+    # kv_len beyond the capacity is clamped (kernels/attention.metal:37).
+    plan.set_params(saetta.TokenParams(0, capacity + 50))
+    built.run()
+    assert np.abs(host(out) - oracle.attention_f64(q, kf, vf, qg, capacity, threads=8)).max() < MAX_ABS_F64
+    # Plan::build_where: the reduce alone reproduces the output from the partials.
+    out.zero_()
+    plan.build_where(lambda name: name == "attention_reduce").run()
+    assert np.abs(host(out) - oracle.attention_f64(q, kf, vf, qg, capacity, threads=8)).max() < MAX_ABS_F64
+
+
+def test_shape_checks():
+    with pytest.raises(ValueError):
+        saetta.DecodeAttention(16, 2, 128, 1024)
+    with pytest.raises(ValueError):
+        saetta.DecodeAttention(16, 4, 256, 1024)
+    with pytest.raises(ValueError):
+        saetta.AttentionRows(16, 2, 1024, 9)
