@@ -1,0 +1,308 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+Prints ONE JSON line.  The default workload is the one the headline metric is
+quoted on: decode attention for one query token over a 32768-token, 8-bit
+group-quantized KV cache (16 q heads / 2 kv heads, head dim 256).  A "step" is
+one decode token's attention over LAYERS independent layer caches back to
+back on one stream (split-K partial kernel + reduce kernel per layer), as the
+reference's own `bench-attention` does with `layers` distinct caches
+(src/attention.rs:173-231): one layer is only 35.65 MB, which would sit in the
+256 MB Infinity Cache if it were re-read.
+
+value      = LAYERS * (ctx + 1) * 1088 B / wall time of a step, in GB/s: the
+             algorithmic KV bytes (codes + scales + biases of keys and values,
+             each read once for all 8 q heads of a kv head).
+roofline   = the same bytes per launch of the partial kernel over that kernel's
+             average duration, measured with HIP events on the launch stream,
+             against 8 TB/s.
+cpu_baseline = the CPU oracle (a C restatement of the reference's
+             single-threaded f32 CPU attention) on one of the layers.
+
+Other workloads (--workload): decode4_150k (4-bit, 150000 tokens), verify2..4
+(2-4 query rows at 32k, 8-bit), prefill (4096-token chunk at position 4096).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+H, KV, D = 16, 2, 256
+VALUES = KV * D
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2]
+
+
+def make_decode_workload(s, torch, ctx, bits, rows, layers, seed=1234):
+    """LAYERS caches of ctx + rows tokens, quantized on the device from N(0,1)."""
+    kind = {8: s.KvBits.Eight, 4: s.KvBits.Four}[bits]
+    capacity = (ctx + rows + 127) // 128 * 128
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    caches = []
+    chunk = 8192
+    for _ in range(layers):
+        k, v = s.QuantRows(kind, VALUES, capacity), s.QuantRows(kind, VALUES, capacity)
+        for rows_q in (k, v):
+            for start in range(0, ctx + rows, chunk):
+                n = min(chunk, ctx + rows - start)
+                x = torch.randn(n, VALUES, generator=gen, device="cuda")
+                if bits == 4:
+                    # 1 % of the channels scaled x8, as outlier channels (same channels everywhere).
+                    x[:, [7, 101, 230, 333, 460]] *= 8.0
+                rows_q.encode(x.reshape(-1), start, n)
+        caches.append((k, v))
+    q = torch.randn(rows, H, D, generator=gen, device="cuda")
+    qg = torch.randn(rows, H, 2 * D, generator=gen, device="cuda")
+    out = torch.empty(rows, H, D, device="cuda")
+    return kind, capacity, caches, q, qg, out
+
+
+def bench_decode(s, torch, args, ctx, bits, rows, layers):
+    import oracle  # only for the CPU-baseline leg below
+
+    kind, capacity, caches, q, qg, out = make_decode_workload(s, torch, ctx, bits, rows, layers)
+    plan = s.Plan()
+    if rows == 1:
+        att = s.DecodeAttention(H, KV, D, capacity)
+        for k, v in caches:
+            att.record_quant(plan, q[0], k, v, qg[0], out[0])
+        plan.set_params(s.TokenParams(0, ctx))  # position ctx: sees ctx + 1 tokens
+    else:
+        att = s.AttentionRows(H, KV, capacity, rows)
+        tp = s.TokenParams(0, ctx).as_tensor("cuda")
+        for k, v in caches:
+            att.record_quant(plan, rows, q, k, v, qg, out, [tp] * rows)
+    graph = not args.no_graph
+    built = plan.build(graph)
+    partial_only = plan.build_where(lambda name: "partial" in name, graph)
+    reduce_only = plan.build_where(lambda name: "reduce" in name, graph)
+    bytes_per_token = {8: 1088, 4: 576}[bits]
+    layer_bytes = (ctx + rows) * bytes_per_token
+
+    for _ in range(args.warmup):
+        built.run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        built.run()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    value = layers * layer_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # Kernel durations with HIP events on the launch stream (torch's current stream is the
+    # one every launch above went to): all partial launches of a step between two events.
+    def kernel_us(b):
+        ts = []
+        for _ in range(max(5, args.steps)):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            b.run()
+            e1.record()
+            e1.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e3 / layers)
+        return median(ts), min(ts)
+
+    part_us, part_us_min = kernel_us(partial_only)
+    red_us, _ = kernel_us(reduce_only)
+    achieved = layer_bytes / (part_us * 1e-6) / 1e9
+
+    # CPU baseline: the oracle's f32 attention on layer 0 (what the reference's CPU path does,
+    # src/cpu/attention.rs:141-181), single thread and all threads the box gives us.
+    import numpy as np
+    k0, v0 = caches[0]
+    n_tok = ctx + 1
+    groups = n_tok * 8
+
+    def deq(rows_q):
+        return oracle.dequantize(rows_q.data[:groups * 2 * bits].cpu().numpy().view(np.uint32),
+                                 rows_q.scales[:groups].cpu().numpy().view(np.uint16),
+                                 rows_q.biases[:groups].cpu().numpy().view(np.uint16), bits)
+
+    kf, vf = deq(k0), deq(v0)
+    qh, qgh = q[0].cpu().numpy(), qg[0].cpu().numpy()
+    threads_all = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+
+    def cpu_time(threads, budget_s):
+        ts, spent = [], 0.0
+        while spent < budget_s or len(ts) < 2:
+            c0 = time.perf_counter()
+            ref = oracle.attend(qh, kf, vf, n_tok, q_and_gate=qgh, threads=threads)
+            ts.append(time.perf_counter() - c0)
+            spent += ts[-1]
+        return median(ts), ref
+
+    cpu1, ref = cpu_time(1, 8.0)
+    cpun, _ = cpu_time(threads_all, 4.0)
+    # The GPU's answer for the same layer, checked against the oracle while we are here.
+    check = s.Plan()
+    if rows == 1:
+        att.record_quant(check, q[0], k0, v0, qg[0], out[0])
+        check.set_params(s.TokenParams(0, ctx))
+    else:
+        att.record_quant(check, rows, q, k0, v0, qg, out, [s.TokenParams(0, ctx).as_tensor("cuda")] * rows)
+    check.build().run()
+    torch.cuda.synchronize()
+    rel_rms = oracle.rel_rms(out[0].cpu().numpy(), ref)
+
+    name = f"decode attention, {bits}-bit KV, ctx {ctx}, {rows} query row(s), {layers} layer caches per step"
+    return {
+        "metric": f"decode attn HBM GB/s @{ctx // 1024}k ctx {bits}-bit KV",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "ms_per_step": round(ms_per_step, 4),
+        "dtype": "u8 codes, f16 MFMA, f32 accumulate",
+        "config": {"workload": name, "heads": H, "kv_heads": KV, "head_dim": D, "ctx": ctx, "kv_bits": bits,
+                   "rows": rows, "layers_per_step": layers, "bytes_per_layer": layer_bytes},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "attention_partial_kernel", "avg_us": round(part_us, 3),
+                     "min_us": round(part_us_min, 3), "reduce_kernel_us": round(red_us, 3)},
+        "cpu_baseline": {"value": round(layer_bytes / cpu1 / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                         "sample": f"one of the {layers} layer caches, full shape, median of repeats; "
+                                   f"{cpu1 * 1e3:.1f} ms per layer",
+                         "all_cores": {"value": round(layer_bytes / cpun / 1e9, 4), "cores": threads_all,
+                                       "ms": round(cpun * 1e3, 2)}},
+        "parity_rel_rms_vs_oracle": float(f"{rel_rms:.3e}"),
+    }
+
+
+def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8):
+    import numpy as np
+    import oracle  # CPU-baseline leg only
+
+    kind = {8: s.KvBits.Eight, 4: s.KvBits.Four}[bits]
+    capacity = (pos + tokens + 127) // 128 * 128
+    gen = torch.Generator(device="cuda").manual_seed(99)
+    keys, values = s.QuantRows(kind, VALUES, capacity), s.QuantRows(kind, VALUES, capacity)
+    knew = torch.randn(pos + tokens, VALUES, generator=gen, device="cuda")
+    vnew = torch.randn(pos + tokens, VALUES, generator=gen, device="cuda")
+    keys.encode(knew[:pos].reshape(-1), 0, pos)
+    values.encode(vnew[:pos].reshape(-1), 0, pos)
+    q = torch.randn(tokens, H, D, generator=gen, device="cuda").to(torch.bfloat16).to(torch.float16)
+    qg = torch.randn(tokens, H, 2 * D, generator=gen, device="cuda")
+    out = torch.empty(tokens, H, D, device="cuda")
+    p = s.FlashParams(H, KV, pos, tokens, 1.0 / math.sqrt(D))
+    kx, vx = knew[pos:].reshape(-1).contiguous(), vnew[pos:].reshape(-1).contiguous()
+
+    def step():
+        # quantize-on-append of the chunk's K and V, then the attention over codes in place
+        keys.encode(kx, pos, tokens)
+        values.encode(vx, pos, tokens)
+        s.attention_prefill.encode_quant(q, keys, values, qg, out, p)
+
+    flops = 4.0 * H * D * (tokens * pos + tokens * (tokens + 1) / 2)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ts = []
+    for _ in range(max(3, args.steps)):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        s.attention_prefill.encode_quant(q, keys, values, qg, out, p)
+        e1.record()
+        e1.synchronize()
+        ts.append(e0.elapsed_time(e1) * 1e3)
+    kern_us = median(ts)
+    achieved = flops / (kern_us * 1e-6) / 1e12
+    # CPU baseline on a bounded sample: the last `sample` tokens of the chunk (the longest rows).
+    sample = 8
+    groups = (pos + tokens) * 8
+
+    def deq(rows_q):
+        x = oracle.dequantize(rows_q.data[:groups * 2 * bits].cpu().numpy().view(np.uint32),
+                              rows_q.scales[:groups].cpu().numpy().view(np.uint16),
+                              rows_q.biases[:groups].cpu().numpy().view(np.uint16), bits)
+        return x.astype(np.float16).astype(np.float32)  # read through half, as prefill does
+
+    kf, vf = deq(keys), deq(values)
+    qs = q[tokens - sample:].float().cpu().numpy()
+    qgs = qg[tokens - sample:].cpu().numpy()
+    c0 = time.perf_counter()
+    ref = oracle.prefill(qs, kf, vf, pos + tokens - sample, sample, q_and_gate=qgs, threads=1)
+    cpu_s = time.perf_counter() - c0
+    cpu_flops = 4.0 * H * D * sum(pos + tokens - sample + i + 1 for i in range(sample))
+    rel_rms = oracle.rel_rms(out[tokens - sample:].cpu().numpy(), ref)
+    return {
+        "metric": "prefill-chunk attn TFLOP/s",
+        "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s",
+        "ms_per_step": round(ms_per_step, 4),
+        "dtype": "f16 MFMA, f32 softmax state",
+        "config": {"workload": f"causal prefill chunk of {tokens} tokens at position {pos}, {bits}-bit KV cache "
+                               "read in place, chunk K/V quantized on append inside the step",
+                   "heads": H, "kv_heads": KV, "head_dim": D, "flops": flops},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "attention_prefill_kernel", "avg_us": round(kern_us, 2)},
+        "cpu_baseline": {"value": round(cpu_flops / cpu_s / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                         "sample": f"the last {sample} tokens of the chunk ({cpu_s:.2f} s)"},
+        "parity_rel_rms_vs_oracle": float(f"{rel_rms:.3e}"),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="decode8_32k",
+                    choices=["decode8_32k", "decode4_150k", "verify2", "verify3", "verify4", "prefill", "all"])
+    ap.add_argument("--no-graph", action="store_true", help="launch from Python instead of replaying a HIP graph")
+    ap.add_argument("--layers", type=int, default=0, help="layer caches per step (default 32; 12 at 150k)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    import __graft_entry__ as entry
+    s = entry.load_package()
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (there is no CPU fallback)", file=sys.stderr)
+        sys.exit(1)
+    s.ffi.check(s.ffi.lib().saetta_init(), "init")
+
+    def one(workload):
+        if workload == "decode8_32k":
+            return bench_decode(s, torch, args, 32768, 8, 1, args.layers or 32)
+        if workload == "decode4_150k":
+            return bench_decode(s, torch, args, 150000, 4, 1, args.layers or 12)
+        if workload.startswith("verify"):
+            return bench_decode(s, torch, args, 32768, 8, int(workload[-1]), args.layers or 32)
+        return bench_prefill(s, torch, args)
+
+    if args.workload == "all":
+        res = one("decode8_32k")
+        res["other_workloads"] = {}
+        for w in ["verify2", "verify3", "verify4", "decode4_150k", "prefill"]:
+            torch.cuda.empty_cache()
+            r = one(w)
+            res["other_workloads"][w] = {k: r[k] for k in ("metric", "value", "unit", "ms_per_step", "roofline",
+                                                            "parity_rel_rms_vs_oracle")}
+    else:
+        res = one(args.workload)
+    res.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
+                "scaling": "weak", "vs_baseline": None, "data": "synthetic"})
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -10,34 +10,40 @@
 // f16 scale and bias, x = s*q + z; layout in kv_quant.hip).
 //
 // Shape of the work: 2 kv heads only, so all parallelism comes from splitting
-// the context.  Workgroup (split, kv head) walks the 128-token chunks split,
-// split + nsplits, ... and keeps an online softmax per query row; it writes
-// one unnormalised partial (o, m, l) per (row, q head) and a second kernel
-// merges the partials and applies the gate.
+// the context.  The context actually in use (read from TokenParams in device
+// memory when the kernel runs) is cut into 16-token blocks and the blocks are
+// dealt evenly to the `nsplits` workgroups of each kv head, so every
+// workgroup streams the same number of bytes whatever the position is.  A
+// workgroup walks its range in iterations of up to 192 tokens, keeps an
+// online softmax per query row, and writes one unnormalised partial (o, m, l)
+// per (row, q head); a second kernel merges the partials and applies the gate.
 //
-// Inside a chunk the two contractions run on the matrix cores
+// Inside an iteration the two contractions run on the matrix cores
 // (v_mfma_f32_16x16x32_f16), because at 15-28 FLOP per cache byte a vector-ALU
 // dot product cannot keep up with HBM:
-//   phase A  S^T = K Q^T   wave w takes tokens 32w..32w+31 (two 16-token
-//            blocks); A operand = key codes of 16 tokens, B operand = the
-//            query rows.
-//   phase B  online softmax per row over the chunk's 128 scores (in LDS).
+//   phase A  S^T = K Q^T   wave w takes the 16-token blocks w, w+4, w+8;
+//            A operand = key codes of 16 tokens, B operand = the query rows.
+//   phase B  online softmax per row over the iteration's scores (in LDS).
 //   phase C  O += P V      wave w takes dims 64w..64w+63, which is exactly
-//            one quantization group, for all 128 tokens.
+//            one quantization group, for all tokens of the iteration.
 // Codes are never dequantized element by element.  A code byte c is placed in
 // the low mantissa bits of an f16 with a zero exponent, i.e. the subnormal
 // c * 2^-24, with one v_perm_b32 per two codes; the matrix cores take
-// subnormal inputs at full precision.  Scale and bias of a group are applied
-// to the 64-dim partial dot product (keys) or folded into the probability
-// operand (values):
-//   q.k   = sum_g  s_g * (q_g . c_g) + z_g * sum(q_g)
+// subnormal inputs.  Scale and bias of a group are applied to the 64-dim
+// partial dot product (keys) or folded into the probability operand (values):
+//   q.k   = sum_g  s_g * (q_g . c_g)  +  sum_g z_g * sum(q_g)
 //   P V_g = (P * s_g) C_g + (P . z_g)
+// and the key bias term sum_g z_g * sum(q_g) is itself one small MFMA.
 // The value operand needs (token, token+1) pairs per dim while memory holds
 // (dim, dim+1) pairs per token; the same v_perm_b32 that widens the bytes
 // picks them from two tokens' words, so the transposition costs nothing.
 // q and P are split into f16 hi + lo parts (two MFMAs into one accumulator,
 // or for a single row the hi and lo parts share one 16-row tile), which keeps
 // the result within ~1e-6 of an f32 evaluation.
+//
+// All cache reads are buffer loads with the cache's size as the bound: rows
+// past the capacity read as 0 instead of faulting, and the per-lane address is
+// one 32-bit offset plus scalar and immediate parts.
 #include "common.hpp"
 
 namespace saetta {
@@ -45,12 +51,17 @@ namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int DIM = SAETTA_HEAD_DIM;
-constexpr int CHUNK = SAETTA_CHUNK;
 constexpr int THREADS = 256;
-constexpr int SC_STRIDE = CHUNK + 4;  // floats; keeps rows on different LDS banks
-constexpr float NO_SCORE = -1e30f;    // finite "minus infinity" of the running max
+constexpr int BLOCK = 16;                     // tokens per MFMA block
+constexpr int IT_BLOCKS = 12;                 // blocks per iteration of a workgroup
+constexpr int IT_TOKENS = BLOCK * IT_BLOCKS;  // 192
+constexpr int SC_STRIDE = IT_TOKENS + 4;      // floats; keeps rows on different LDS banks
+constexpr float NO_SCORE = -1e30f;            // finite "minus infinity" of the running max
 
 // q is multiplied by scale * log2(e) * Q_UP before the hi/lo split so that
 // the lo part stays a normal f16; probabilities by P_UP for the same reason.
@@ -63,6 +74,11 @@ constexpr float P_UP = 256.0f;
 template <int BITS>
 constexpr float code_up() {
     return BITS == 8 ? 16777216.0f : BITS == 4 ? 1048576.0f : 1.0f;
+}
+// Bytes of one (token, kv head) of keys or values.
+template <int BITS>
+constexpr int row_bytes() {
+    return BITS == 16 ? 512 : BITS * 32;
 }
 
 struct PartialArgs {
@@ -84,66 +100,65 @@ __device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel)
 }
 
 __device__ __forceinline__ half8 as_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
-    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     u32x4 v = {a, b, c, d};
     return __builtin_bit_cast(half8, v);
 }
 
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, int(bytes), 0x00020000);
+}
+
 // ---- key codes: 16 dims of one token per lane and group ----------------------
 template <int BITS>
-struct KeyRegs;
-template <>
-struct KeyRegs<8> {
-    uint4 w;
-};
-template <>
-struct KeyRegs<4> {
-    uint2 w;
-};
-template <>
-struct KeyRegs<16> {
-    uint4 w[2];
+struct KeyRegs {
+    uint32_t w[BITS == 16 ? 8 : BITS / 2];  // 32 B (f16), 16 B (8-bit), 8 B (4-bit)
 };
 
-// Lane (t, j): dims 64g + 16j .. +15 of `token`, kv head kv.
+// Lane (t, j) reads dims 64g + 16j .. +15 of its token: `voff` is the lane's
+// byte offset of (token, kv head, j), `soff` the scalar part (block), g is an immediate.
 template <int BITS>
-__device__ __forceinline__ KeyRegs<BITS> load_key(const void *data, uint32_t token, uint32_t kv_heads,
-                                                  uint32_t kv, int g, int j) {
+__device__ __forceinline__ KeyRegs<BITS> load_key(__amdgpu_buffer_rsrc_t rsrc, int voff, int soff, int g) {
     KeyRegs<BITS> r;
     if constexpr (BITS == 8) {
-        const uint4 *p = reinterpret_cast<const uint4 *>(data);
-        r.w = p[(size_t(token) * kv_heads + kv) * 16 + g * 4 + j];
+        u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff + g * 64, soff, 0);
+        r.w[0] = v.x, r.w[1] = v.y, r.w[2] = v.z, r.w[3] = v.w;
     } else if constexpr (BITS == 4) {
-        const uint2 *p = reinterpret_cast<const uint2 *>(data);
-        r.w = p[(size_t(token) * kv_heads + kv) * 16 + g * 4 + j];
+        u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff + g * 32, soff, 0);
+        r.w[0] = v.x, r.w[1] = v.y;
     } else {
-        const uint4 *p = reinterpret_cast<const uint4 *>(data);
-        size_t i = (size_t(token) * kv_heads + kv) * 32 + g * 8 + j * 2;
-        r.w[0] = p[i];
-        r.w[1] = p[i + 1];
+        u32x4 v0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff + g * 128, soff, 0);
+        u32x4 v1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff + g * 128 + 16, soff, 0);
+        r.w[0] = v0.x, r.w[1] = v0.y, r.w[2] = v0.z, r.w[3] = v0.w;
+        r.w[4] = v1.x, r.w[5] = v1.y, r.w[6] = v1.z, r.w[7] = v1.w;
     }
     return r;
+}
+
+// Bytes of the lane's 16 dims inside a group.
+template <int BITS>
+constexpr int key_piece() {
+    return BITS == 16 ? 32 : BITS * 2;
 }
 
 // The A operand of k-step `ab` (0: the lane's first 8 dims, 1: the next 8).
 template <int BITS>
 __device__ __forceinline__ half8 key_operand(const KeyRegs<BITS> &r, int ab) {
     if constexpr (BITS == 8) {
-        uint32_t w0 = ab ? r.w.z : r.w.x, w1 = ab ? r.w.w : r.w.y;
+        const uint32_t w0 = r.w[2 * ab], w1 = r.w[2 * ab + 1];
         return as_half8(perm(0, w0, 0x0c010c00u), perm(0, w0, 0x0c030c02u), perm(0, w1, 0x0c010c00u),
                         perm(0, w1, 0x0c030c02u));
     } else if constexpr (BITS == 4) {
-        uint32_t w = ab ? r.w.y : r.w.x;
-        uint32_t x = (w << 4) & 0xf0f0f0f0u, y = w & 0xf0f0f0f0u;
+        const uint32_t w = r.w[ab];
+        const uint32_t x = (w << 4) & 0xf0f0f0f0u, y = w & 0xf0f0f0f0u;
         // slots: dims 0,2 | 4,6 | 1,3 | 5,7
         return as_half8(perm(0, x, 0x0c010c00u), perm(0, x, 0x0c030c02u), perm(0, y, 0x0c010c00u),
                         perm(0, y, 0x0c030c02u));
     } else {
-        const uint4 &v = r.w[ab];
-        return as_half8(v.x, v.y, v.z, v.w);
+        return as_half8(r.w[4 * ab], r.w[4 * ab + 1], r.w[4 * ab + 2], r.w[4 * ab + 3]);
     }
 }
 
+// Which of the lane's 8 dims of a k-step sits in MFMA slot e.
 template <int BITS>
 __device__ __forceinline__ constexpr int key_slot_dim(int e) {
     if (BITS == 4) {
@@ -162,17 +177,12 @@ struct ValRegs {
     uint32_t w[BITS == 16 ? 16 : 8];
 };
 
+// Byte offset of the lane's dword inside a (token, kv head) row.
 template <int BITS>
-__device__ __forceinline__ uint32_t load_val_word(const void *data, uint32_t token, uint32_t kv_heads,
-                                                  uint32_t kv, int wave, int n, int set) {
-    const uint32_t *p = reinterpret_cast<const uint32_t *>(data);
-    if constexpr (BITS == 8) {
-        return p[((size_t(token) * kv_heads + kv) * 4 + wave) * 16 + n];
-    } else if constexpr (BITS == 4) {
-        return p[((size_t(token) * kv_heads + kv) * 4 + wave) * 8 + (n >> 1)];
-    } else {
-        return p[(size_t(token) * kv_heads + kv) * 128 + wave * 32 + set * 16 + n];
-    }
+__device__ __forceinline__ int val_lane_offset(int wave, int n) {
+    if constexpr (BITS == 8) return wave * 64 + n * 4;
+    if constexpr (BITS == 4) return wave * 32 + (n >> 1) * 4;
+    return wave * 128 + n * 4;
 }
 
 // B operand of output tile `tile` (0..3) from the 8 tokens' words of a k-step.
@@ -190,7 +200,7 @@ __device__ __forceinline__ half8 val_operand(const ValRegs<BITS> &r, int tile, i
         const uint32_t sh = (n & 1) * 16, up = (tile & 1) ? 0 : 4;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            uint32_t a = ((r.w[2 * i] >> sh) << up) & 0xf0f0u, b = ((r.w[2 * i + 1] >> sh) << up) & 0xf0f0u;
+            const uint32_t a = ((r.w[2 * i] >> sh) << up) & 0xf0f0u, b = ((r.w[2 * i + 1] >> sh) << up) & 0xf0f0u;
             o[i] = perm(b, a, sel);
         }
     } else {
@@ -212,56 +222,72 @@ __device__ __forceinline__ void split_hi_lo(float x, _Float16 &hi, _Float16 &lo)
     lo = (_Float16)(x - h);
 }
 
+__device__ __forceinline__ float half_bits_to_float(uint32_t bits16) {
+    return (float)__builtin_bit_cast(_Float16, uint16_t(bits16));
+}
+
 // TILES: 16-row tiles of query rows (rows * 8 heads, rounded up).  PACKED: one
 // verify row; its 8 heads' hi parts are operand rows 0-7 and lo parts rows 8-15
 // of a single tile.  Otherwise hi and lo are two MFMAs into one accumulator.
 template <int BITS, int TILES, bool PACKED>
 struct Shape {
-    static constexpr int S_ROWS = 16 * TILES;               // rows of the score buffer
+    static constexpr bool QUANT = BITS != 16;
+    static constexpr int S_ROWS = 16 * TILES;                  // rows of the score buffer
     static constexpr int SOFT_ROWS = PACKED ? 8 : 16 * TILES;  // rows phase B walks
-    static constexpr int TPR = THREADS / SOFT_ROWS;          // threads per row in phase B
-    static constexpr int TPT = CHUNK / TPR;                  // tokens per thread in phase B
+    static constexpr int TPR = THREADS / SOFT_ROWS;            // threads per row in phase B
+    static constexpr int TPT = IT_TOKENS / TPR;                // tokens per thread in phase B
     static constexpr int PARTS = PACKED ? 1 : 2;
-    static constexpr int Q_BYTES = TILES * PARTS * 8 * 64 * 16;
-    static constexpr int S_BYTES = S_ROWS * SC_STRIDE * 4;
-    static constexpr int SCALE_BYTES = (BITS == 16) ? 0 : 4 * 4 * CHUNK * 4;
-    static constexpr int MISC_BYTES = (S_ROWS /*alpha*/ + TILES * 4 * 16 /*qsum*/ + 4 * S_ROWS /*zsum*/) * 4;
-    static constexpr int LDS_BYTES = Q_BYTES + S_BYTES + SCALE_BYTES + MISC_BYTES;
+    // LDS map, in bytes
+    static constexpr int Q_OFF = 0;
+    static constexpr int Q_BYTES = TILES * PARTS * 8 * 64 * 16;  // [tile][part][step][lane] half8
+    static constexpr int S_OFF = Q_OFF + Q_BYTES;
+    static constexpr int S_BYTES = S_ROWS * SC_STRIDE * 4;  // [row][token] f32
+    static constexpr int KS_OFF = S_OFF + S_BYTES;          // [token][4] f16
+    static constexpr int KZ_OFF = KS_OFF + (QUANT ? IT_TOKENS * 8 : 0);
+    static constexpr int VS_OFF = KZ_OFF + (QUANT ? IT_TOKENS * 8 : 0);  // [4][token] f16
+    static constexpr int VZ_OFF = VS_OFF + (QUANT ? IT_TOKENS * 8 : 0);
+    static constexpr int ALPHA_OFF = VZ_OFF + (QUANT ? IT_TOKENS * 8 : 0);  // [S_ROWS] f32
+    static constexpr int QSUM_OFF = ALPHA_OFF + S_ROWS * 4;                 // [tile][g][16] f32
+    static constexpr int QZ_OFF = QSUM_OFF + TILES * 64 * 4;                // [tile][16] half8
+    static constexpr int ZSUM_OFF = QZ_OFF + TILES * 16 * 16;               // [wave][S_ROWS] f32
+    static constexpr int LDS_BYTES = ZSUM_OFF + 4 * S_ROWS * 4;
 };
 
 template <int BITS, int TILES, bool PACKED>
-__global__ __launch_bounds__(THREADS) void attention_partial_kernel(PartialArgs a) {
+__device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     using Sh = Shape<BITS, TILES, PACKED>;
-    constexpr bool QUANT = BITS != 16;
+    constexpr bool QUANT = Sh::QUANT;
     constexpr int PARTS = Sh::PARTS;
+    constexpr int RB = row_bytes<BITS>();
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    half8 *q_lds = reinterpret_cast<half8 *>(lds_raw);                       // [tile][part][step][lane]
-    float *s_lds = reinterpret_cast<float *>(lds_raw + Sh::Q_BYTES);         // [S_ROWS][SC_STRIDE]
-    float *sc_lds = reinterpret_cast<float *>(lds_raw + Sh::Q_BYTES + Sh::S_BYTES);
-    float *ks_lds = sc_lds, *kz_lds = sc_lds + 4 * CHUNK, *vs_lds = sc_lds + 8 * CHUNK,
-          *vz_lds = sc_lds + 12 * CHUNK;                                      // [g][token]
-    float *misc = reinterpret_cast<float *>(lds_raw + Sh::Q_BYTES + Sh::S_BYTES + Sh::SCALE_BYTES);
-    float *alpha_lds = misc;                   // [S_ROWS]
-    float *qsum_lds = misc + Sh::S_ROWS;        // [tile][g][16]
-    float *zsum_lds = qsum_lds + TILES * 64;    // [wave][S_ROWS]
+    half8 *q_lds = reinterpret_cast<half8 *>(lds_raw + Sh::Q_OFF);
+    float *s_lds = reinterpret_cast<float *>(lds_raw + Sh::S_OFF);
+    uint16_t *ks_lds = reinterpret_cast<uint16_t *>(lds_raw + Sh::KS_OFF);
+    uint16_t *kz_lds = reinterpret_cast<uint16_t *>(lds_raw + Sh::KZ_OFF);
+    uint16_t *vs_lds = reinterpret_cast<uint16_t *>(lds_raw + Sh::VS_OFF);
+    uint16_t *vz_lds = reinterpret_cast<uint16_t *>(lds_raw + Sh::VZ_OFF);
+    float *alpha_lds = reinterpret_cast<float *>(lds_raw + Sh::ALPHA_OFF);
+    float *qsum_lds = reinterpret_cast<float *>(lds_raw + Sh::QSUM_OFF);
+    half8 *qz_lds = reinterpret_cast<half8 *>(lds_raw + Sh::QZ_OFF);
+    float *zsum_lds = reinterpret_cast<float *>(lds_raw + Sh::ZSUM_OFF);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, j = lane >> 4;
     const uint32_t split = blockIdx.x, kv = blockIdx.y;
     const uint32_t kvh = a.kv_heads;
-
-    const uint32_t position = a.tp->position;
-    // Tokens the last row sees; the longest context of the launch.
-    const uint32_t max_len =
-        min(a.decode_len ? a.tp->kv_len : position + a.rows, a.capacity);
-    if (split * CHUNK >= max_len) return;
     const uint32_t real_rows = a.rows * 8;  // (row, head) pairs of this kv head
 
-    // ---- prologue: query operands ------------------------------------------------
-    // Operand row `orow` of tile t: PACKED -> head orow & 7, part orow >> 3;
-    // else (row, head) pair 16t + orow, both parts.
+    // ---- prologue: query rows to f16 hi/lo operands in LDS ------------------------
+    // (before TokenParams is read, so that its latency hides behind these loads)
+    // Operand row `on` of tile t: PACKED -> head on & 7, part on >> 3;
+    // else (row, head) pair 16t + on, both parts.
+    if constexpr (QUANT) {
+        for (int i = tid; i < TILES * 64; i += THREADS) qsum_lds[i] = 0.0f;
+        __syncthreads();
+    }
     {
         const float qmul = a.scale * 1.4426950408889634f * Q_UP;
+#pragma unroll
         for (int item = tid; item < TILES * 8 * 64; item += THREADS) {
             const int t = item / 512, step = (item / 64) & 7, l = item & 63;
             const int on = l & 15, oj = l >> 4;
@@ -270,8 +296,8 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel(PartialArgs 
             float v[8];
             if (pair < int(real_rows)) {
                 const int row = pair >> 3, head = pair & 7;
-                const float *src = a.q + (size_t(row) * a.heads + kv * 8 + head) * DIM + 64 * g +
-                                   16 * oj + 8 * ab;
+                const float *src =
+                    a.q + (size_t(row) * a.heads + kv * 8 + head) * DIM + 64 * g + 16 * oj + 8 * ab;
                 const float4 f0 = *reinterpret_cast<const float4 *>(src);
                 const float4 f1 = *reinterpret_cast<const float4 *>(src + 4);
                 v[0] = f0.x, v[1] = f0.y, v[2] = f0.z, v[3] = f0.w;
@@ -281,52 +307,90 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel(PartialArgs 
                 for (int e = 0; e < 8; e++) v[e] = 0.0f;
             }
             half8 hi, lo;
+            float sum_hi = 0.0f, sum_lo = 0.0f;
 #pragma unroll
             for (int e = 0; e < 8; e++) {
                 _Float16 h, lw;
                 split_hi_lo(v[key_slot_dim<BITS>(e)] * qmul, h, lw);
                 hi[e] = h;
                 lo[e] = lw;
+                sum_hi += (float)h;
+                sum_lo += (float)lw;
             }
+            float sum;
             if constexpr (PACKED) {
                 q_lds[step * 64 + l] = (on < 8) ? hi : lo;
+                sum = (on < 8) ? sum_hi : sum_lo;
             } else {
                 q_lds[((t * 2 + 0) * 8 + step) * 64 + l] = hi;
                 q_lds[((t * 2 + 1) * 8 + step) * 64 + l] = lo;
+                sum = sum_hi + sum_lo;
+            }
+            // Sum of the operand row's values over the 64 dims of group g (for the key bias
+            // term): over the 4 lane groups here, over the two k-steps through LDS.
+            if constexpr (QUANT) {
+                sum += __shfl_xor(sum, 16);
+                sum += __shfl_xor(sum, 32);
+                if (oj == 0) atomicAdd(&qsum_lds[(t * 4 + g) * 16 + on], sum);
             }
         }
     }
     __syncthreads();
-    // Sum of each operand row's values per 64-dim group, for the key bias term.
+    // B operand of the key bias MFMA: lanes j == 0 hold hi(sum_g) in slots 0-3 and
+    // lo(sum_g) in slots 4-7, already divided by Q_UP; the A operand holds z_g twice.
     if constexpr (QUANT) {
-        for (int item = tid; item < TILES * 4 * 16; item += THREADS) {
-            const int t = item / 64, g = (item / 16) & 3, on = item & 15;
-            float sum = 0.0f;
-            for (int part = 0; part < PARTS; part++) {
-                for (int ab = 0; ab < 2; ab++) {
-                    for (int oj = 0; oj < 4; oj++) {
-                        half8 h = q_lds[((t * PARTS + part) * 8 + g * 2 + ab) * 64 + oj * 16 + on];
+        for (int i = tid; i < TILES * 16; i += THREADS) {
+            half8 qz;
 #pragma unroll
-                        for (int e = 0; e < 8; e++) sum += (float)h[e];
-                    }
-                }
+            for (int g = 0; g < 4; g++) {
+                _Float16 h, lw;
+                split_hi_lo(qsum_lds[((i >> 4) * 4 + g) * 16 + (i & 15)] * (1.0f / Q_UP), h, lw);
+                qz[g] = h;
+                qz[4 + g] = lw;
             }
-            qsum_lds[item] = sum;
+            qz_lds[i] = qz;
         }
+        __syncthreads();
     }
-    __syncthreads();
+
+    // ---- the context and this workgroup's share of it -----------------------------
+    const uint32_t position = a.tp->position;
+    const uint32_t kv_len = a.tp->kv_len;
+    // Tokens the last row sees; the longest context of the launch.
+    const uint32_t max_len = min(a.decode_len ? kv_len : position + a.rows, a.capacity);
+    const uint32_t nblocks = (max_len + BLOCK - 1) / BLOCK;
+    uint32_t blk_begin, blk_end;
+    if (nblocks <= a.nsplits) {
+        blk_begin = split;
+        blk_end = split + 1;
+        if (split >= nblocks) return;
+    } else {
+        blk_begin = uint32_t(uint64_t(split) * nblocks / a.nsplits);
+        blk_end = uint32_t(uint64_t(split + 1) * nblocks / a.nsplits);
+    }
+    const uint32_t range = blk_end - blk_begin;
+    const uint32_t n_it = (range + IT_BLOCKS - 1) / IT_BLOCKS;
+    const uint32_t per_it = (range + n_it - 1) / n_it;
 
     // Query operands of a single tile live in registers for the whole kernel.
     half8 q_reg[TILES == 1 ? PARTS * 8 : 1];
-    float qsum_reg[TILES == 1 ? 4 : 1];
+    half8 qz_reg = {0, 0, 0, 0, 0, 0, 0, 0};
     if constexpr (TILES == 1) {
 #pragma unroll
         for (int i = 0; i < PARTS * 8; i++) q_reg[i] = q_lds[i * 64 + lane];
         if constexpr (QUANT) {
-#pragma unroll
-            for (int g = 0; g < 4; g++) qsum_reg[g] = qsum_lds[g * 16 + n];
+            if (j == 0) qz_reg = qz_lds[n];
         }
     }
+
+    const uint32_t cap_rows = a.capacity * kvh;
+    const __amdgpu_buffer_rsrc_t k_rsrc = make_rsrc(a.kdata, cap_rows * RB);
+    const __amdgpu_buffer_rsrc_t v_rsrc = make_rsrc(a.vdata, cap_rows * RB);
+    const __amdgpu_buffer_rsrc_t ks_rsrc = make_rsrc(a.kscales, QUANT ? cap_rows * 8 : 0);
+    const __amdgpu_buffer_rsrc_t kz_rsrc = make_rsrc(a.kbiases, QUANT ? cap_rows * 8 : 0);
+    const __amdgpu_buffer_rsrc_t vs_rsrc = make_rsrc(a.vscales, QUANT ? cap_rows * 8 : 0);
+    const __amdgpu_buffer_rsrc_t vz_rsrc = make_rsrc(a.vbiases, QUANT ? cap_rows * 8 : 0);
+    const int tok_stride = int(kvh) * RB;  // bytes between tokens of one kv head
 
     // ---- running state -------------------------------------------------------------
     // Phase B: thread (row, part) of SOFT_ROWS x TPR.
@@ -335,7 +399,7 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel(PartialArgs 
     {
         const int vrow = PACKED ? 0 : b_row >> 3;
         const bool real = PACKED || b_row < int(real_rows);
-        const uint32_t len = a.decode_len ? a.tp->kv_len : position + vrow + 1;
+        const uint32_t len = a.decode_len ? kv_len : position + vrow + 1;
         b_len = real ? min(len, a.capacity) : 0;
     }
     float m_run = NO_SCORE, l_part = 0.0f;
@@ -349,97 +413,124 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel(PartialArgs 
         for (int e = 0; e < 4; e++) acc[t][e] = floatx4{0, 0, 0, 0};
     }
 
-    for (uint32_t chunk = split; chunk * CHUNK < max_len; chunk += a.nsplits) {
-        const uint32_t base = chunk * CHUNK;
-        const uint32_t last = a.capacity - 1;  // clamp for addresses past the cache
+    for (uint32_t it = 0; it < n_it; it++) {
+        const uint32_t blk0 = blk_begin + it * per_it;
+        const uint32_t nb = min(per_it, blk_end - blk0);  // blocks of this iteration, 1..12
+        const uint32_t base = blk0 * BLOCK;
+        const uint32_t it_tokens = nb * BLOCK;
+        const uint32_t ksteps = (nb + 1) / 2;
 
-        // ---- loads of the whole chunk, issued up front ---------------------------
-        KeyRegs<BITS> kreg[2][4];
+        // ---- loads of the whole iteration, issued up front -------------------------
+        KeyRegs<BITS> kreg[3][4];
+        {
+            const int voff = int((base + BLOCK * wave + n) * kvh + kv) * RB + j * key_piece<BITS>();
 #pragma unroll
-        for (int b = 0; b < 2; b++) {
-            const uint32_t token = min(base + 32 * wave + 16 * b + n, last);
+            for (int i = 0; i < 3; i++) {
+                if (uint32_t(wave + 4 * i) < nb) {
 #pragma unroll
-            for (int g = 0; g < 4; g++) kreg[b][g] = load_key<BITS>(a.kdata, token, kvh, kv, g, j);
-        }
-        ValRegs<BITS> vreg[4];
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const uint32_t tok = base + 32 * ks + 8 * j + e;
-                const uint32_t token = min(tok, last);
-                vreg[ks].w[e] = load_val_word<BITS>(a.vdata, token, kvh, kv, wave, n, 0);
-                if constexpr (BITS == 16) {
-                    vreg[ks].w[8 + e] = load_val_word<BITS>(a.vdata, token, kvh, kv, wave, n, 1);
-                    // Rows past the context may hold anything, NaN included: 0 * NaN must not reach O.
-                    if (tok >= max_len) vreg[ks].w[e] = 0, vreg[ks].w[8 + e] = 0;
+                    for (int g = 0; g < 4; g++) kreg[i][g] = load_key<BITS>(k_rsrc, voff, i * 64 * tok_stride, g);
                 }
             }
         }
-        // Scales and biases of the chunk: thread -> (array, token), 4 groups each.
-        if constexpr (QUANT) {
-            const int arr = tid >> 7, tok = tid & 127;  // 0: keys, 1: values
-            const uint32_t token = min(base + tok, last);
-            const bool live = base + tok < max_len;
-            const size_t gi = (size_t(token) * kvh + kv) * 4;
-            const uint2 sraw = *reinterpret_cast<const uint2 *>((arr ? a.vscales : a.kscales) + gi);
-            const uint2 zraw = *reinterpret_cast<const uint2 *>((arr ? a.vbiases : a.kbiases) + gi);
-            const float smul = arr ? P_UP : code_up<BITS>() / Q_UP;
-            const float zmul = arr ? 1.0f : 1.0f / Q_UP;
-            float *sdst = arr ? vs_lds : ks_lds, *zdst = arr ? vz_lds : kz_lds;
-            const uint32_t sw[2] = {sraw.x, sraw.y}, zw[2] = {zraw.x, zraw.y};
+        ValRegs<BITS> vreg[6];
+        {
+            const int voff = int((base + 8 * j) * kvh + kv) * RB + val_lane_offset<BITS>(wave, n);
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const __half s = __ushort_as_half(uint16_t(sw[g >> 1] >> (16 * (g & 1))));
-                const __half z = __ushort_as_half(uint16_t(zw[g >> 1] >> (16 * (g & 1))));
-                // Tokens past the context get 0 so that whatever their rows hold stays out.
-                sdst[g * CHUNK + tok] = live ? __half2float(s) * smul : 0.0f;
-                zdst[g * CHUNK + tok] = live ? __half2float(z) * zmul : 0.0f;
+            for (int ks = 0; ks < 6; ks++) {
+                if (uint32_t(ks) < ksteps) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        const int soff = (32 * ks + e) * tok_stride;
+                        vreg[ks].w[e] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, voff, soff, 0);
+                        if constexpr (BITS == 16) {
+                            vreg[ks].w[8 + e] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, voff + 64, soff, 0);
+                            // Rows past the context may hold anything, NaN included: 0 * NaN must not reach O.
+                            if (base + 32 * ks + 8 * j + e >= max_len) vreg[ks].w[e] = 0, vreg[ks].w[8 + e] = 0;
+                        }
+                    }
+                }
             }
         }
-        __syncthreads();  // scales visible; also orders the previous chunk's phase C before new S
+        // Scales and biases of the iteration's tokens: thread = token, 4 groups each.
+        if constexpr (QUANT) {
+            if (tid < IT_TOKENS) {
+                const int voff = int((base + tid) * kvh + kv) * 8;
+                const u32x2 ksr = __builtin_amdgcn_raw_buffer_load_b64(ks_rsrc, voff, 0, 0);
+                const u32x2 kzr = __builtin_amdgcn_raw_buffer_load_b64(kz_rsrc, voff, 0, 0);
+                u32x2 vsr = __builtin_amdgcn_raw_buffer_load_b64(vs_rsrc, voff, 0, 0);
+                u32x2 vzr = __builtin_amdgcn_raw_buffer_load_b64(vz_rsrc, voff, 0, 0);
+                // Tokens past the context or the iteration get value scale 0 and bias 0, so that
+                // whatever their rows hold stays out of O (their probabilities are 0 as well).
+                if (uint32_t(tid) >= it_tokens || base + tid >= max_len) vsr = u32x2{0, 0}, vzr = u32x2{0, 0};
+                *reinterpret_cast<u32x2 *>(ks_lds + 4 * tid) = ksr;
+                *reinterpret_cast<u32x2 *>(kz_lds + 4 * tid) = kzr;
+                vs_lds[0 * IT_TOKENS + tid] = uint16_t(vsr.x), vs_lds[1 * IT_TOKENS + tid] = uint16_t(vsr.x >> 16);
+                vs_lds[2 * IT_TOKENS + tid] = uint16_t(vsr.y), vs_lds[3 * IT_TOKENS + tid] = uint16_t(vsr.y >> 16);
+                vz_lds[0 * IT_TOKENS + tid] = uint16_t(vzr.x), vz_lds[1 * IT_TOKENS + tid] = uint16_t(vzr.x >> 16);
+                vz_lds[2 * IT_TOKENS + tid] = uint16_t(vzr.y), vz_lds[3 * IT_TOKENS + tid] = uint16_t(vzr.y >> 16);
+            }
+        }
+        __syncthreads();  // scales visible; the previous iteration's phase C is over
 
         // ---- phase A: scores -------------------------------------------------------
 #pragma unroll
         for (int t = 0; t < TILES; t++) {
             half8 qt[PARTS * 8];
-            float qs[4];
+            half8 qz = qz_reg;
             if constexpr (TILES == 1) {
 #pragma unroll
                 for (int i = 0; i < PARTS * 8; i++) qt[i] = q_reg[i];
-#pragma unroll
-                for (int g = 0; g < 4; g++) qs[g] = QUANT ? qsum_reg[g] : 0.0f;
             } else {
 #pragma unroll
                 for (int i = 0; i < PARTS * 8; i++) qt[i] = q_lds[(t * PARTS * 8 + i) * 64 + lane];
-#pragma unroll
-                for (int g = 0; g < 4; g++) qs[g] = QUANT ? qsum_lds[(t * 4 + g) * 16 + n] : 0.0f;
+                if constexpr (QUANT) {
+                    if (j == 0) qz = qz_lds[t * 16 + n];
+                }
             }
 #pragma unroll
-            for (int b = 0; b < 2; b++) {
+            for (int i = 0; i < 3; i++) {
+                const int blk = wave + 4 * i;
+                if (uint32_t(blk) >= nb) break;
+                const int tok0 = BLOCK * blk + 4 * j;  // this lane's 4 tokens in C layout
                 floatx4 s = {0, 0, 0, 0};
-                const int tok0 = 32 * wave + 16 * b + 4 * j;  // this lane's 4 tokens in C layout
+                if constexpr (QUANT) {
+                    // bias term: A = (z_0..z_3, z_0..z_3) of token n in lanes j == 0
+                    const u32x2 zr = *reinterpret_cast<const u32x2 *>(kz_lds + 4 * (BLOCK * blk + n));
+                    const half8 zop = (j == 0) ? as_half8(zr.x, zr.y, zr.x, zr.y) : as_half8(0, 0, 0, 0);
+                    s = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz, s, 0, 0, 0);
+                }
+                floatx4 r[4];
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
-                    floatx4 r = {0, 0, 0, 0};
+                    r[g] = floatx4{0, 0, 0, 0};
 #pragma unroll
                     for (int ab = 0; ab < 2; ab++) {
-                        const half8 kop = key_operand<BITS>(kreg[b][g], ab);
+                        const half8 kop = key_operand<BITS>(kreg[i][g], ab);
 #pragma unroll
                         for (int part = 0; part < PARTS; part++) {
-                            r = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop, qt[part * 8 + g * 2 + ab], r, 0,
-                                                                       0, 0);
+                            r[g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop, qt[part * 8 + g * 2 + ab], r[g], 0,
+                                                                          0, 0);
                         }
                     }
-                    if constexpr (QUANT) {
-                        const floatx4 sc = *reinterpret_cast<const floatx4 *>(ks_lds + g * CHUNK + tok0);
-                        const floatx4 zc = *reinterpret_cast<const floatx4 *>(kz_lds + g * CHUNK + tok0);
+                }
+                if constexpr (QUANT) {
+                    // scales of tokens tok0..tok0+3, 4 groups each: 32 contiguous bytes
+                    const u32x4 s01 = *reinterpret_cast<const u32x4 *>(ks_lds + 4 * tok0);
+                    const u32x4 s23 = *reinterpret_cast<const u32x4 *>(ks_lds + 4 * tok0 + 8);
+                    const uint32_t sw[8] = {s01.x, s01.y, s01.z, s01.w, s23.x, s23.y, s23.z, s23.w};
+                    constexpr float C1 = code_up<BITS>() / Q_UP;
 #pragma unroll
-                        for (int i = 0; i < 4; i++) s[i] += sc[i] * r[i] + zc[i] * qs[g];
-                    } else {
+                    for (int tk = 0; tk < 4; tk++) {
+                        float d = 0.0f;
 #pragma unroll
-                        for (int i = 0; i < 4; i++) s[i] += r[i] * (1.0f / Q_UP);
+                        for (int g = 0; g < 4; g++) {
+                            d += half_bits_to_float(sw[2 * tk + (g >> 1)] >> (16 * (g & 1))) * r[g][tk];
+                        }
+                        s[tk] += d * C1;
                     }
+                } else {
+#pragma unroll
+                    for (int tk = 0; tk < 4; tk++) s[tk] = (r[0][tk] + r[1][tk] + r[2][tk] + r[3][tk]) * (1.0f / Q_UP);
                 }
                 *reinterpret_cast<floatx4 *>(s_lds + (16 * t + n) * SC_STRIDE + tok0) = s;
             }
@@ -451,18 +542,19 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel(PartialArgs 
             float sv[Sh::TPT];
             float *row = s_lds + b_row * SC_STRIDE + b_part * Sh::TPT;
 #pragma unroll
-            for (int i = 0; i < Sh::TPT; i += 4) {
-                floatx4 v = *reinterpret_cast<const floatx4 *>(row + i);
+            for (int i = 0; i < Sh::TPT; i += 2) {
+                floatx2 v = *reinterpret_cast<const floatx2 *>(row + i);
                 if constexpr (PACKED) {
-                    const floatx4 w = *reinterpret_cast<const floatx4 *>(row + 8 * SC_STRIDE + i);
-                    v += w;
+                    v += *reinterpret_cast<const floatx2 *>(row + 8 * SC_STRIDE + i);
                 }
-                sv[i] = v[0], sv[i + 1] = v[1], sv[i + 2] = v[2], sv[i + 3] = v[3];
+                sv[i] = v[0], sv[i + 1] = v[1];
             }
-            const uint32_t tok0 = base + b_part * Sh::TPT;
+            const uint32_t tok0 = b_part * Sh::TPT;
+            // tokens of this row in this iteration: inside the iteration and inside the row's context
+            const uint32_t lim = b_len > base ? min(b_len - base, it_tokens) : 0;
             float cm = NO_SCORE;
 #pragma unroll
-            for (int i = 0; i < Sh::TPT; i++) cm = (tok0 + i < b_len) ? fmaxf(cm, sv[i]) : cm;
+            for (int i = 0; i < Sh::TPT; i++) cm = (tok0 + i < lim) ? fmaxf(cm, sv[i]) : cm;
 #pragma unroll
             for (int step = 1; step < Sh::TPR; step *= 2) cm = fmaxf(cm, __shfl_xor(cm, step));
             const float nm = fmaxf(m_run, cm);
@@ -470,14 +562,14 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel(PartialArgs 
             float sum = 0.0f;
 #pragma unroll
             for (int i = 0; i < Sh::TPT; i++) {
-                sv[i] = (tok0 + i < b_len) ? exp2f(sv[i] - nm) : 0.0f;
+                sv[i] = (tok0 + i < lim) ? exp2f(sv[i] - nm) : 0.0f;
                 sum += sv[i];
             }
             l_part = l_part * al + sum;
             m_run = nm;
 #pragma unroll
-            for (int i = 0; i < Sh::TPT; i += 4) {
-                *reinterpret_cast<floatx4 *>(row + i) = floatx4{sv[i], sv[i + 1], sv[i + 2], sv[i + 3]};
+            for (int i = 0; i < Sh::TPT; i += 2) {
+                *reinterpret_cast<floatx2 *>(row + i) = floatx2{sv[i], sv[i + 1]};
             }
             if (b_part == 0) alpha_lds[b_row] = al;
         }
@@ -487,7 +579,7 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel(PartialArgs 
 #pragma unroll
         for (int t = 0; t < TILES; t++) {
             // Rescale what was summed so far.  Accumulator rows (C layout) are 4j..4j+3.
-            {
+            if (it > 0) {
                 const int arow = PACKED ? ((4 * j) & 7) : 16 * t + 4 * j;
                 const floatx4 al = *reinterpret_cast<const floatx4 *>(alpha_lds + arow);
 #pragma unroll
@@ -495,38 +587,49 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel(PartialArgs 
                 zacc[t] *= alpha_lds[PACKED ? (n & 7) : 16 * t + n];
             }
             const float *prow = s_lds + (PACKED ? (n & 7) : 16 * t + n) * SC_STRIDE;
+            // hi lanes (PACKED: n < 8) keep x and let the conversion truncate it to its hi part;
+            // lo lanes subtract the hi part first.
+            const uint32_t lo_mask = (PACKED && n >= 8) ? 0xffffe000u : 0u;
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++) {
+            for (int ks = 0; ks < 6; ks++) {
+                if (uint32_t(ks) >= ksteps) break;
                 const int tk = 32 * ks + 8 * j;
                 const floatx4 p0 = *reinterpret_cast<const floatx4 *>(prow + tk);
                 const floatx4 p1 = *reinterpret_cast<const floatx4 *>(prow + tk + 4);
                 float pv[8] = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
                 if constexpr (QUANT) {
-                    const floatx4 s0 = *reinterpret_cast<const floatx4 *>(vs_lds + wave * CHUNK + tk);
-                    const floatx4 s1 = *reinterpret_cast<const floatx4 *>(vs_lds + wave * CHUNK + tk + 4);
-                    const floatx4 z0 = *reinterpret_cast<const floatx4 *>(vz_lds + wave * CHUNK + tk);
-                    const floatx4 z1 = *reinterpret_cast<const floatx4 *>(vz_lds + wave * CHUNK + tk + 4);
-                    const float sc[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
-                    const float zc[8] = {z0[0], z0[1], z0[2], z0[3], z1[0], z1[1], z1[2], z1[3]};
+                    const u32x4 sr = *reinterpret_cast<const u32x4 *>(vs_lds + wave * IT_TOKENS + tk);
+                    const u32x4 zr = *reinterpret_cast<const u32x4 *>(vz_lds + wave * IT_TOKENS + tk);
+                    const uint32_t sw[4] = {sr.x, sr.y, sr.z, sr.w}, zw[4] = {zr.x, zr.y, zr.z, zr.w};
 #pragma unroll
                     for (int e = 0; e < 8; e++) {
-                        zacc[t] += pv[e] * zc[e];
-                        pv[e] *= sc[e];
+                        zacc[t] += pv[e] * half_bits_to_float(zw[e >> 1] >> (16 * (e & 1)));
+                        pv[e] *= half_bits_to_float(sw[e >> 1] >> (16 * (e & 1))) * P_UP;
                     }
                 } else {
 #pragma unroll
                     for (int e = 0; e < 8; e++) pv[e] *= P_UP;
                 }
                 half8 phi, plo;
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    _Float16 h, lw;
-                    split_hi_lo(pv[e], h, lw);
-                    phi[e] = h;
-                    plo[e] = lw;
-                }
                 if constexpr (PACKED) {
-                    if (n >= 8) phi = plo;
+                    uint32_t o[4];
+#pragma unroll
+                    for (int e = 0; e < 8; e += 2) {
+                        const float x0 = pv[e] - __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, pv[e]) & lo_mask);
+                        const float x1 =
+                            pv[e + 1] - __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, pv[e + 1]) & lo_mask);
+                        // round toward zero: exact truncation to the hi part in hi lanes
+                        o[e / 2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x0, x1));
+                    }
+                    phi = as_half8(o[0], o[1], o[2], o[3]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        _Float16 h, lw;
+                        split_hi_lo(pv[e], h, lw);
+                        phi[e] = h;
+                        plo[e] = lw;
+                    }
                 }
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
@@ -538,21 +641,16 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel(PartialArgs 
                 }
             }
         }
-        // The next chunk's first barrier (after its loads) keeps its writes to the
-        // scale arrays behind this phase; S is rewritten only after that barrier too.
-        if (chunk + a.nsplits < (max_len + CHUNK - 1) / CHUNK) __syncthreads();
     }
 
     // ---- epilogue: one partial per (row, head) ------------------------------------
     // m and l from the phase B threads.
 #pragma unroll
     for (int step = 1; step < Sh::TPR; step *= 2) l_part += __shfl_xor(l_part, step);
-    const bool b_has = split * CHUNK < b_len;  // this row has tokens in this split
-    if (b_part == 0 && b_has) {
+    if (b_part == 0 && (PACKED || b_row < int(real_rows))) {
         const int vrow = PACKED ? 0 : b_row >> 3, head = b_row & 7;
         const size_t slot = (size_t(vrow) * a.nsplits + split) * a.heads + kv * 8 + head;
-        a.part_ml[2 * slot] = m_run;
-        a.part_ml[2 * slot + 1] = l_part;
+        *reinterpret_cast<floatx2 *>(a.part_ml + 2 * slot) = floatx2{m_run, l_part};
     }
     // Bias sums: reduce over the 4 lane groups, hand to the C-layout lanes through LDS.
     if constexpr (QUANT) {
@@ -566,7 +664,7 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel(PartialArgs 
         }
         __syncthreads();
     }
-    const float unscale = code_up<BITS>() / P_UP;
+    constexpr float unscale = code_up<BITS>() / P_UP;
 #pragma unroll
     for (int t = 0; t < TILES; t++) {
         floatx4 o[4];
@@ -585,17 +683,13 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel(PartialArgs 
             const int pair = 16 * t + 4 * j + i;  // (row, head) pair of this accumulator row
             if (pair >= int(real_rows)) continue;
             const int vrow = pair >> 3, head = pair & 7;
-            const uint32_t len = min(a.decode_len ? a.tp->kv_len : position + vrow + 1, a.capacity);
-            if (split * CHUNK >= len) continue;
             const float zb = QUANT ? zsum_lds[wave * Sh::S_ROWS + pair] : 0.0f;
             const size_t slot = (size_t(vrow) * a.nsplits + split) * a.heads + kv * 8 + head;
             float *dst = a.part_o + slot * DIM + 64 * wave;
             if constexpr (BITS == 16) {
                 // tile e: dims 32*(e/2) + 2n + e%2
-                *reinterpret_cast<float2 *>(dst + 2 * n) =
-                    make_float2(o[0][i] * unscale, o[1][i] * unscale);
-                *reinterpret_cast<float2 *>(dst + 32 + 2 * n) =
-                    make_float2(o[2][i] * unscale, o[3][i] * unscale);
+                *reinterpret_cast<float2 *>(dst + 2 * n) = make_float2(o[0][i] * unscale, o[1][i] * unscale);
+                *reinterpret_cast<float2 *>(dst + 32 + 2 * n) = make_float2(o[2][i] * unscale, o[3][i] * unscale);
             } else {
                 *reinterpret_cast<float4 *>(dst + 4 * n) =
                     make_float4(o[0][i] * unscale + zb, o[1][i] * unscale + zb, o[2][i] * unscale + zb,
@@ -605,8 +699,27 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel(PartialArgs 
     }
 }
 
-// Merges the splits of one (q head, row): weights 2^(m_c - M), then the gate.
-// 1024 threads = 4 slices x 256 dims, slice s takes splits s, s+4, ...
+// One 16-row tile of query rows fits two waves per SIMD (8 per CU, i.e. two
+// workgroups per CU, which is what the split count is sized for); more tiles
+// take the whole register file.
+template <int BITS, bool PACKED>
+__global__ __launch_bounds__(THREADS, 2) void attention_partial_kernel_1(PartialArgs a) {
+    attention_partial_body<BITS, 1, PACKED>(a);
+}
+
+template <int BITS, int TILES>
+__global__ __launch_bounds__(THREADS) void attention_partial_kernel_n(PartialArgs a) {
+    attention_partial_body<BITS, TILES, false>(a);
+}
+
+template <int BITS>
+__global__ __launch_bounds__(THREADS) void attention_partial_kernel_p(PartialArgs a) {
+    attention_partial_body<BITS, 1, true>(a);
+}
+
+// Merges the splits of one (q head, row) and a 64-dim quarter of the head:
+// weights 2^(m_c - M), then the gate.  256 threads: first one thread per split
+// for the weights, then (16 dim quads) x (16 slices of splits) for the sums.
 // (reference: attention_reduce / attention_reduce_rows,
 // kernels/attention.metal:367-409, kernels/attention_rows.metal:296-342).
 struct ReduceArgs {
@@ -614,50 +727,69 @@ struct ReduceArgs {
     const float *part_ml;
     const float *q_and_gate;
     float *out;
-    uint32_t heads, capacity, nsplits;
+    uint32_t heads, capacity, nsplits, rows;
     const saetta_token_params *tp;
     uint32_t decode_len;
 };
 
-__global__ __launch_bounds__(1024) void attention_reduce_kernel(ReduceArgs a) {
-    __shared__ float slice_m[4], slice_l[4];
-    __shared__ float slice_o[4][DIM];
-    const uint32_t h = blockIdx.x, row = blockIdx.y;
-    const uint32_t d = threadIdx.x & 255, s = threadIdx.x >> 8;
-    const uint32_t len = min(a.decode_len ? a.tp->kv_len : a.tp->position + row + 1, a.capacity);
-    const uint32_t parts = min(a.nsplits, (len + CHUNK - 1) / CHUNK);
+constexpr uint32_t MAX_SPLITS = 256;  // workgroups per kv head: 2 kv heads fill 512 slots of 256 CUs
+
+__global__ __launch_bounds__(256) void attention_reduce_kernel(ReduceArgs a) {
+    __shared__ float w_lds[MAX_SPLITS];
+    __shared__ float red[8];
+    __shared__ floatx4 o_lds[16][16];
+    const uint32_t h = blockIdx.x, row = blockIdx.y, quarter = blockIdx.z;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t max_len = min(a.decode_len ? a.tp->kv_len : a.tp->position + a.rows, a.capacity);
+    const uint32_t nblocks = (max_len + BLOCK - 1) / BLOCK;
+    const uint32_t parts = min(a.nsplits, nblocks);
     const float *ml = a.part_ml + size_t(2) * row * a.nsplits * a.heads;
     const float *po = a.part_o + size_t(row) * a.nsplits * a.heads * DIM;
-    float m = NO_SCORE;
-    for (uint32_t c = s; c < parts; c += 4) m = fmaxf(m, ml[2 * (size_t(c) * a.heads + h)]);
-    if (d == 0) slice_m[s] = m;
-    __syncthreads();
-    m = fmaxf(fmaxf(slice_m[0], slice_m[1]), fmaxf(slice_m[2], slice_m[3]));
-    float l = 0.0f, acc = 0.0f;
-    for (uint32_t c = s; c < parts; c += 4) {
-        const size_t i = size_t(c) * a.heads + h;
-        const float w = exp2f(ml[2 * i] - m);
-        l += w * ml[2 * i + 1];
-        acc += w * po[i * DIM + d];
+    // weights
+    float m = NO_SCORE, l = 0.0f;
+    if (tid < parts) {
+        const floatx2 v = *reinterpret_cast<const floatx2 *>(ml + 2 * (size_t(tid) * a.heads + h));
+        m = v[0], l = v[1];
     }
-    slice_o[s][d] = acc;
-    if (d == 0) slice_l[s] = l;
+    float mx = m;
+#pragma unroll
+    for (int step = 1; step < 64; step *= 2) mx = fmaxf(mx, __shfl_xor(mx, step));
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
     __syncthreads();
-    if (s == 0) {
-        const float o = slice_o[0][d] + slice_o[1][d] + slice_o[2][d] + slice_o[3][d];
-        const float total = slice_l[0] + slice_l[1] + slice_l[2] + slice_l[3];
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const float w = tid < parts ? exp2f(m - mx) : 0.0f;
+    w_lds[tid] = w;
+    float wl = w * l;
+#pragma unroll
+    for (int step = 1; step < 64; step *= 2) wl += __shfl_xor(wl, step);
+    if ((tid & 63) == 0) red[4 + (tid >> 6)] = wl;
+    __syncthreads();
+    const float total = red[4] + red[5] + red[6] + red[7];
+    // sums: thread (quad d4 of the quarter's 64 dims, slice s of the splits)
+    const uint32_t d4 = tid & 15, s = tid >> 4;
+    floatx4 acc = {0, 0, 0, 0};
+    for (uint32_t c = s; c < parts; c += 16) {
+        const floatx4 v =
+            *reinterpret_cast<const floatx4 *>(po + (size_t(c) * a.heads + h) * DIM + 64 * quarter + 4 * d4);
+        acc += v * w_lds[c];
+    }
+    o_lds[s][d4] = acc;
+    __syncthreads();
+    if (tid < 64) {
+        const uint32_t d = tid;  // dim inside the quarter
+        float o = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) o += o_lds[i][d >> 2][d & 3];
         const size_t qh = size_t(row) * a.heads + h;
-        const float g = a.q_and_gate[qh * 2 * DIM + DIM + d];
-        a.out[qh * DIM + d] = o / total * (1.0f / (1.0f + expf(-g)));
+        const float g = a.q_and_gate[qh * 2 * DIM + DIM + 64 * quarter + d];
+        a.out[qh * DIM + 64 * quarter + d] = o / total * (1.0f / (1.0f + expf(-g)));
     }
 }
 
-// Most workgroups per kv head.  A split costs one 8 KB partial per row and
-// kv head, so few is better; 512 keeps one chunk per workgroup up to 64k tokens.
-constexpr uint32_t MAX_SPLITS = 512;
-
 uint32_t splits_for(uint32_t capacity, uint32_t wanted) {
-    uint32_t chunks = (capacity + CHUNK - 1) / CHUNK;
+    // Never more than the 128-token chunks of the capacity, so that scratch sized as
+    // rows * ceil(capacity / 128) * heads partials is always enough.
+    const uint32_t chunks = (capacity + SAETTA_CHUNK - 1) / SAETTA_CHUNK;
     uint32_t s = chunks < MAX_SPLITS ? chunks : MAX_SPLITS;
     if (wanted && wanted < s) s = wanted;
     return s ? s : 1;
@@ -666,7 +798,14 @@ uint32_t splits_for(uint32_t capacity, uint32_t wanted) {
 template <int BITS, int TILES, bool PACKED>
 void launch_partial(hipStream_t stream, const PartialArgs &a) {
     using Sh = Shape<BITS, TILES, PACKED>;
-    auto kernel = attention_partial_kernel<BITS, TILES, PACKED>;
+    void (*kernel)(PartialArgs);
+    if constexpr (TILES == 1 && BITS != 16) {
+        kernel = attention_partial_kernel_1<BITS, PACKED>;
+    } else if constexpr (PACKED) {
+        kernel = attention_partial_kernel_p<BITS>;  // f16 cache: its registers do not fit two waves
+    } else {
+        kernel = attention_partial_kernel_n<BITS, TILES>;
+    }
     static bool attr_set = false;
     if (!attr_set && Sh::LDS_BYTES > 48 * 1024) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -698,20 +837,22 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
     SAETTA_REQUIRE(kv_heads > 0 && heads == kv_heads * SAETTA_GQA_GROUP, SAETTA_E_SHAPE,
                    "%s needs 8 q heads per kv head (heads %u, kv heads %u)", what, heads, kv_heads);
     SAETTA_REQUIRE(rows >= 1 && rows <= SAETTA_MAX_ROWS, SAETTA_E_SHAPE, "%s: %u rows (1..8)", what, rows);
-    SAETTA_REQUIRE(capacity > 0, SAETTA_E_SHAPE, "%s: capacity 0", what);
+    // Byte offsets into the cache are 32-bit: capacity * kv_heads * 512 B (the f16 row) must fit.
+    SAETTA_REQUIRE(capacity > 0 && uint64_t(capacity) * kv_heads * 512 < (uint64_t(1) << 31), SAETTA_E_SHAPE,
+                   "%s: capacity %u out of range", what, capacity);
     SAETTA_REQUIRE(q && kdata && vdata && part_o && part_ml && q_and_gate && out && d_tp, SAETTA_E_NULL,
                    "%s: null buffer", what);
     SAETTA_REQUIRE(bits == 16 || (ks && kz && vs && vz), SAETTA_E_NULL, "%s: null scales or biases", what);
     SAETTA_REQUIRE(aligned(q, 16) && aligned(kdata, 16) && aligned(vdata, 16) && aligned(part_o, 16) &&
-                       aligned(part_ml, 8),
+                       aligned(part_ml, 8) && aligned(q_and_gate, 4) && aligned(out, 4),
                    SAETTA_E_ALIGN, "%s: q, cache and scratch must be 16-byte aligned", what);
     SAETTA_REQUIRE(bits == 16 || (aligned(ks, 8) && aligned(kz, 8) && aligned(vs, 8) && aligned(vz, 8)),
                    SAETTA_E_ALIGN, "%s: scales and biases must be 8-byte aligned", what);
     if (int rc = ensure_device()) return rc;
     const uint32_t nsplits = splits_for(capacity, wanted_splits);
     if (stages & SAETTA_STAGE_PARTIAL) {
-        PartialArgs a{q,        kdata,  vdata, ks,    kz,      vs,   vz,   part_o, part_ml,
-                      heads,    kv_heads, capacity, scale, rows, nsplits, d_tp, decode_len ? 1u : 0u};
+        PartialArgs a{q,     kdata,    vdata,    ks,    kz,   vs,      vz,   part_o, part_ml,
+                      heads, kv_heads, capacity, scale, rows, nsplits, d_tp, decode_len ? 1u : 0u};
         if (bits == 8) {
             launch_partial_rows<8>(stream, a);
         } else if (bits == 4) {
@@ -721,8 +862,8 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
         }
     }
     if (stages & SAETTA_STAGE_REDUCE) {
-        ReduceArgs r{part_o, part_ml, q_and_gate, out, heads, capacity, nsplits, d_tp, decode_len ? 1u : 0u};
-        attention_reduce_kernel<<<dim3(heads, rows), 1024, 0, stream>>>(r);
+        ReduceArgs r{part_o, part_ml, q_and_gate, out, heads, capacity, nsplits, rows, d_tp, decode_len ? 1u : 0u};
+        attention_reduce_kernel<<<dim3(heads, rows, 4), 256, 0, stream>>>(r);
     }
     return launch_status(what);
 }

@@ -3,7 +3,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libsaetta_hip.so")
+LIB_PATH = os.environ.get("SAETTA_HIP_LIB") or os.path.join(_HERE, "lib", "libsaetta_hip.so")
 
 # Every symbol include/saetta_hip.h declares; tests check the library exports each.
 SYMBOLS = [

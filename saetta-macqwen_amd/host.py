@@ -90,19 +90,36 @@ class Plan:
         self.params.copy_(host, non_blocking=True)
         self._keep = host
 
-    def build(self):
-        return Built(list(self.ops))
+    def build(self, graph=False):
+        """Plan::build (src/plan.rs:229-235).  graph=True captures the launches into a HIP
+        graph, the counterpart of the reference's indirect command buffer: one submission
+        replays them all, and the position still comes from `params` at run time."""
+        return Built(list(self.ops), graph)
 
-    def build_where(self, keep):
+    def build_where(self, keep, graph=False):
         """Plan::build_where (src/plan.rs:187-226): only the ops whose kernel passes `keep`."""
-        return Built([(k, f) for k, f in self.ops if keep(k)])
+        return Built([(k, f) for k, f in self.ops if keep(k)], graph)
 
 
 class Built:
-    def __init__(self, ops):
+    def __init__(self, ops, graph=False):
         self.ops = ops
+        self.graph = None
+        if graph and ops:
+            # One eager run first: lazy one-time set-up must not happen under capture.
+            self.run()
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                s = _stream()
+                for _, launch in ops:
+                    launch(s)
+            self.graph = g
 
     def run(self, stream=None):
+        if self.graph is not None:
+            self.graph.replay()
+            return
         s = _stream(stream)
         for _, launch in self.ops:
             launch(s)
