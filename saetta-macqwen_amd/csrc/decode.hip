@@ -247,9 +247,8 @@ struct Shape {
     static constexpr int VS_OFF = KZ_OFF + (QUANT ? IT_TOKENS * 8 : 0);  // [4][token] f16
     static constexpr int VZ_OFF = VS_OFF + (QUANT ? IT_TOKENS * 8 : 0);
     static constexpr int ALPHA_OFF = VZ_OFF + (QUANT ? IT_TOKENS * 8 : 0);  // [S_ROWS] f32
-    static constexpr int QSUM_OFF = ALPHA_OFF + S_ROWS * 4;                 // [tile][g][16] f32
-    static constexpr int QZ_OFF = QSUM_OFF + TILES * 64 * 4;                // [tile][16] half8
-    static constexpr int ZSUM_OFF = QZ_OFF + TILES * 16 * 16;               // [wave][S_ROWS] f32
+    static constexpr int QZ_OFF = ALPHA_OFF + S_ROWS * 4;                   // [tile][hi, lo][lane] half8
+    static constexpr int ZSUM_OFF = QZ_OFF + TILES * 2 * 64 * 16;           // [wave][S_ROWS] f32
     static constexpr int LDS_BYTES = ZSUM_OFF + 4 * S_ROWS * 4;
 };
 
@@ -267,8 +266,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     uint16_t *vs_lds = reinterpret_cast<uint16_t *>(lds_raw + Sh::VS_OFF);
     uint16_t *vz_lds = reinterpret_cast<uint16_t *>(lds_raw + Sh::VZ_OFF);
     float *alpha_lds = reinterpret_cast<float *>(lds_raw + Sh::ALPHA_OFF);
-    float *qsum_lds = reinterpret_cast<float *>(lds_raw + Sh::QSUM_OFF);
-    half8 *qz_lds = reinterpret_cast<half8 *>(lds_raw + Sh::QZ_OFF);
+    _Float16 *qz_lds = reinterpret_cast<_Float16 *>(lds_raw + Sh::QZ_OFF);
     float *zsum_lds = reinterpret_cast<float *>(lds_raw + Sh::ZSUM_OFF);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -277,80 +275,31 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     const uint32_t kvh = a.kv_heads;
     const uint32_t real_rows = a.rows * 8;  // (row, head) pairs of this kv head
 
-    // ---- prologue: query rows to f16 hi/lo operands in LDS ------------------------
-    // (before TokenParams is read, so that its latency hides behind these loads)
-    // Operand row `on` of tile t: PACKED -> head on & 7, part on >> 3;
-    // else (row, head) pair 16t + on, both parts.
-    if constexpr (QUANT) {
-        for (int i = tid; i < TILES * 64; i += THREADS) qsum_lds[i] = 0.0f;
-        __syncthreads();
-    }
-    {
-        const float qmul = a.scale * 1.4426950408889634f * Q_UP;
+    // ---- query values: requested first, so that nothing they wait for is behind the cache ----
+    // Item (tile t, k-step, lane l) is the 8 values that lane l feeds to the MFMA k-step;
+    // operand row `on` of tile t: PACKED -> head on & 7, part on >> 3; else (row, head)
+    // pair 16t + on, both parts.
+    auto load_q_item = [&](int item, float (&v)[8]) {
+        const int t = item / 512, step = (item / 64) & 7, l = item & 63;
+        const int on = l & 15, oj = l >> 4;
+        const int g = step >> 1, ab = step & 1;
+        const int pair = PACKED ? (on & 7) : 16 * t + on;
+        if (pair < int(real_rows)) {
+            const int row = pair >> 3, head = pair & 7;
+            const float *src = a.q + (size_t(row) * a.heads + kv * 8 + head) * DIM + 64 * g + 16 * oj + 8 * ab;
+            const float4 f0 = *reinterpret_cast<const float4 *>(src);
+            const float4 f1 = *reinterpret_cast<const float4 *>(src + 4);
+            v[0] = f0.x, v[1] = f0.y, v[2] = f0.z, v[3] = f0.w;
+            v[4] = f1.x, v[5] = f1.y, v[6] = f1.z, v[7] = f1.w;
+        } else {
 #pragma unroll
-        for (int item = tid; item < TILES * 8 * 64; item += THREADS) {
-            const int t = item / 512, step = (item / 64) & 7, l = item & 63;
-            const int on = l & 15, oj = l >> 4;
-            const int g = step >> 1, ab = step & 1;
-            const int pair = PACKED ? (on & 7) : 16 * t + on;
-            float v[8];
-            if (pair < int(real_rows)) {
-                const int row = pair >> 3, head = pair & 7;
-                const float *src =
-                    a.q + (size_t(row) * a.heads + kv * 8 + head) * DIM + 64 * g + 16 * oj + 8 * ab;
-                const float4 f0 = *reinterpret_cast<const float4 *>(src);
-                const float4 f1 = *reinterpret_cast<const float4 *>(src + 4);
-                v[0] = f0.x, v[1] = f0.y, v[2] = f0.z, v[3] = f0.w;
-                v[4] = f1.x, v[5] = f1.y, v[6] = f1.z, v[7] = f1.w;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; e++) v[e] = 0.0f;
-            }
-            half8 hi, lo;
-            float sum_hi = 0.0f, sum_lo = 0.0f;
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                _Float16 h, lw;
-                split_hi_lo(v[key_slot_dim<BITS>(e)] * qmul, h, lw);
-                hi[e] = h;
-                lo[e] = lw;
-                sum_hi += (float)h;
-                sum_lo += (float)lw;
-            }
-            float sum;
-            if constexpr (PACKED) {
-                q_lds[step * 64 + l] = (on < 8) ? hi : lo;
-                sum = (on < 8) ? sum_hi : sum_lo;
-            } else {
-                q_lds[((t * 2 + 0) * 8 + step) * 64 + l] = hi;
-                q_lds[((t * 2 + 1) * 8 + step) * 64 + l] = lo;
-                sum = sum_hi + sum_lo;
-            }
-            // Sum of the operand row's values over the 64 dims of group g (for the key bias
-            // term): over the 4 lane groups here, over the two k-steps through LDS.
-            if constexpr (QUANT) {
-                sum += __shfl_xor(sum, 16);
-                sum += __shfl_xor(sum, 32);
-                if (oj == 0) atomicAdd(&qsum_lds[(t * 4 + g) * 16 + on], sum);
-            }
+            for (int e = 0; e < 8; e++) v[e] = 0.0f;
         }
-    }
-    __syncthreads();
-    // B operand of the key bias MFMA: lanes j == 0 hold hi(sum_g) in slots 0-3 and
-    // lo(sum_g) in slots 4-7, already divided by Q_UP; the A operand holds z_g twice.
-    if constexpr (QUANT) {
-        for (int i = tid; i < TILES * 16; i += THREADS) {
-            half8 qz;
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                _Float16 h, lw;
-                split_hi_lo(qsum_lds[((i >> 4) * 4 + g) * 16 + (i & 15)] * (1.0f / Q_UP), h, lw);
-                qz[g] = h;
-                qz[4 + g] = lw;
-            }
-            qz_lds[i] = qz;
-        }
-        __syncthreads();
+    };
+    float q_early[TILES == 1 ? 2 : 1][8];
+    if constexpr (TILES == 1) {
+        load_q_item(tid, q_early[0]);
+        load_q_item(tid + THREADS, q_early[1]);
     }
 
     // ---- the context and this workgroup's share of it -----------------------------
@@ -372,17 +321,6 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     const uint32_t n_it = (range + IT_BLOCKS - 1) / IT_BLOCKS;
     const uint32_t per_it = (range + n_it - 1) / n_it;
 
-    // Query operands of a single tile live in registers for the whole kernel.
-    half8 q_reg[TILES == 1 ? PARTS * 8 : 1];
-    half8 qz_reg = {0, 0, 0, 0, 0, 0, 0, 0};
-    if constexpr (TILES == 1) {
-#pragma unroll
-        for (int i = 0; i < PARTS * 8; i++) q_reg[i] = q_lds[i * 64 + lane];
-        if constexpr (QUANT) {
-            if (j == 0) qz_reg = qz_lds[n];
-        }
-    }
-
     const uint32_t cap_rows = a.capacity * kvh;
     const __amdgpu_buffer_rsrc_t k_rsrc = make_rsrc(a.kdata, cap_rows * RB);
     const __amdgpu_buffer_rsrc_t v_rsrc = make_rsrc(a.vdata, cap_rows * RB);
@@ -391,6 +329,120 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     const __amdgpu_buffer_rsrc_t vs_rsrc = make_rsrc(a.vscales, QUANT ? cap_rows * 8 : 0);
     const __amdgpu_buffer_rsrc_t vz_rsrc = make_rsrc(a.vbiases, QUANT ? cap_rows * 8 : 0);
     const int tok_stride = int(kvh) * RB;  // bytes between tokens of one kv head
+
+    // ---- the loads of one iteration ------------------------------------------------
+    // Everything an iteration reads is requested before anything is computed: keys first
+    // (phase A needs them first), then the small scale/bias rows, then the values.
+    KeyRegs<BITS> kreg[3][4];
+    ValRegs<BITS> vreg[6];
+    u32x2 ksr = {0, 0}, kzr = {0, 0}, vsr = {0, 0}, vzr = {0, 0};
+    auto blocks_of = [&](uint32_t it) { return min(per_it, blk_end - (blk_begin + it * per_it)); };
+    auto load_keys = [&](uint32_t it) {
+        const uint32_t base = (blk_begin + it * per_it) * BLOCK, nb = blocks_of(it);
+        const int voff = int((base + BLOCK * wave + n) * kvh + kv) * RB + j * key_piece<BITS>();
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            if (uint32_t(wave + 4 * i) < nb) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) kreg[i][g] = load_key<BITS>(k_rsrc, voff, i * 64 * tok_stride, g);
+            }
+        }
+    };
+    auto load_scales = [&](uint32_t it) {
+        if constexpr (QUANT) {
+            const uint32_t base = (blk_begin + it * per_it) * BLOCK;
+            if (tid < IT_TOKENS) {
+                const int voff = int((base + tid) * kvh + kv) * 8;
+                ksr = __builtin_amdgcn_raw_buffer_load_b64(ks_rsrc, voff, 0, 0);
+                kzr = __builtin_amdgcn_raw_buffer_load_b64(kz_rsrc, voff, 0, 0);
+                vsr = __builtin_amdgcn_raw_buffer_load_b64(vs_rsrc, voff, 0, 0);
+                vzr = __builtin_amdgcn_raw_buffer_load_b64(vz_rsrc, voff, 0, 0);
+            }
+        }
+    };
+    auto load_values = [&](uint32_t it) {
+        const uint32_t base = (blk_begin + it * per_it) * BLOCK, ksteps = (blocks_of(it) + 1) / 2;
+        const int voff = int((base + 8 * j) * kvh + kv) * RB + val_lane_offset<BITS>(wave, n);
+#pragma unroll
+        for (int ks = 0; ks < 6; ks++) {
+            if (uint32_t(ks) < ksteps) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int soff = (32 * ks + e) * tok_stride;
+                    vreg[ks].w[e] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, voff, soff, 0);
+                    if constexpr (BITS == 16) {
+                        vreg[ks].w[8 + e] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, voff + 64, soff, 0);
+                    }
+                }
+            }
+        }
+    };
+    load_keys(0);
+    load_scales(0);
+    if constexpr (TILES != 1) load_values(0);
+
+    // ---- prologue: query rows to f16 hi/lo operands in LDS ------------------------
+    // (while the first iteration's keys are in flight; the values are requested after it)
+    {
+        const float qmul = a.scale * 1.4426950408889634f * Q_UP;
+#pragma unroll
+        for (int k = 0; k < TILES * 2; k++) {
+            const int item = tid + k * THREADS;
+            const int t = item / 512, step = (item / 64) & 7, l = item & 63;
+            const int on = l & 15;
+            float v[8];
+            if constexpr (TILES == 1) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[e] = q_early[k][e];
+            } else {
+                load_q_item(item, v);
+            }
+            half8 hi, lo;
+            float sum_hi = 0.0f, sum_lo = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                _Float16 h, lw;
+                split_hi_lo(v[key_slot_dim<BITS>(e)] * qmul, h, lw);
+                hi[e] = h;
+                lo[e] = lw;
+                sum_hi += (float)h;
+                sum_lo += (float)lw;
+            }
+            float sum;
+            if constexpr (PACKED) {
+                q_lds[step * 64 + l] = (on < 8) ? hi : lo;
+                sum = (on < 8) ? sum_hi : sum_lo;
+            } else {
+                q_lds[((t * 2 + 0) * 8 + step) * 64 + l] = hi;
+                q_lds[((t * 2 + 1) * 8 + step) * 64 + l] = lo;
+                sum = sum_hi + sum_lo;
+            }
+            // The key bias term sum_g z_g * sum_{d in g} q_d is one more MFMA over the same 32
+            // (lane group, slot) pairs: its B operand holds, in lane l and slot `step`, the sum of
+            // the 8 operand values this item made (divided by Q_UP, as hi and lo halves), and its
+            // A operand holds z_g of the step's group.
+            if constexpr (QUANT) {
+                _Float16 h, lw;
+                split_hi_lo(sum * (1.0f / Q_UP), h, lw);
+                qz_lds[((t * 2 + 0) * 64 + l) * 8 + step] = h;
+                qz_lds[((t * 2 + 1) * 64 + l) * 8 + step] = lw;
+            }
+        }
+    }
+    __syncthreads();
+    if constexpr (TILES == 1) load_values(0);
+
+    // Query operands of a single tile live in registers for the whole kernel.
+    half8 q_reg[TILES == 1 ? PARTS * 8 : 1];
+    half8 qz_reg[2] = {{0, 0, 0, 0, 0, 0, 0, 0}, {0, 0, 0, 0, 0, 0, 0, 0}};
+    if constexpr (TILES == 1) {
+#pragma unroll
+        for (int i = 0; i < PARTS * 8; i++) q_reg[i] = q_lds[i * 64 + lane];
+        if constexpr (QUANT) {
+            qz_reg[0] = *reinterpret_cast<const half8 *>(qz_lds + lane * 8);
+            qz_reg[1] = *reinterpret_cast<const half8 *>(qz_lds + (64 + lane) * 8);
+        }
+    }
 
     // ---- running state -------------------------------------------------------------
     // Phase B: thread (row, part) of SOFT_ROWS x TPR.
@@ -420,45 +472,9 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
         const uint32_t it_tokens = nb * BLOCK;
         const uint32_t ksteps = (nb + 1) / 2;
 
-        // ---- loads of the whole iteration, issued up front -------------------------
-        KeyRegs<BITS> kreg[3][4];
-        {
-            const int voff = int((base + BLOCK * wave + n) * kvh + kv) * RB + j * key_piece<BITS>();
-#pragma unroll
-            for (int i = 0; i < 3; i++) {
-                if (uint32_t(wave + 4 * i) < nb) {
-#pragma unroll
-                    for (int g = 0; g < 4; g++) kreg[i][g] = load_key<BITS>(k_rsrc, voff, i * 64 * tok_stride, g);
-                }
-            }
-        }
-        ValRegs<BITS> vreg[6];
-        {
-            const int voff = int((base + 8 * j) * kvh + kv) * RB + val_lane_offset<BITS>(wave, n);
-#pragma unroll
-            for (int ks = 0; ks < 6; ks++) {
-                if (uint32_t(ks) < ksteps) {
-#pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        const int soff = (32 * ks + e) * tok_stride;
-                        vreg[ks].w[e] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, voff, soff, 0);
-                        if constexpr (BITS == 16) {
-                            vreg[ks].w[8 + e] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, voff + 64, soff, 0);
-                            // Rows past the context may hold anything, NaN included: 0 * NaN must not reach O.
-                            if (base + 32 * ks + 8 * j + e >= max_len) vreg[ks].w[e] = 0, vreg[ks].w[8 + e] = 0;
-                        }
-                    }
-                }
-            }
-        }
-        // Scales and biases of the iteration's tokens: thread = token, 4 groups each.
+        // Scales and biases of the iteration's tokens to LDS: thread = token, 4 groups each.
         if constexpr (QUANT) {
             if (tid < IT_TOKENS) {
-                const int voff = int((base + tid) * kvh + kv) * 8;
-                const u32x2 ksr = __builtin_amdgcn_raw_buffer_load_b64(ks_rsrc, voff, 0, 0);
-                const u32x2 kzr = __builtin_amdgcn_raw_buffer_load_b64(kz_rsrc, voff, 0, 0);
-                u32x2 vsr = __builtin_amdgcn_raw_buffer_load_b64(vs_rsrc, voff, 0, 0);
-                u32x2 vzr = __builtin_amdgcn_raw_buffer_load_b64(vz_rsrc, voff, 0, 0);
                 // Tokens past the context or the iteration get value scale 0 and bias 0, so that
                 // whatever their rows hold stays out of O (their probabilities are 0 as well).
                 if (uint32_t(tid) >= it_tokens || base + tid >= max_len) vsr = u32x2{0, 0}, vzr = u32x2{0, 0};
@@ -476,7 +492,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
 #pragma unroll
         for (int t = 0; t < TILES; t++) {
             half8 qt[PARTS * 8];
-            half8 qz = qz_reg;
+            half8 qz[2] = {qz_reg[0], qz_reg[1]};
             if constexpr (TILES == 1) {
 #pragma unroll
                 for (int i = 0; i < PARTS * 8; i++) qt[i] = q_reg[i];
@@ -484,7 +500,8 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
 #pragma unroll
                 for (int i = 0; i < PARTS * 8; i++) qt[i] = q_lds[(t * PARTS * 8 + i) * 64 + lane];
                 if constexpr (QUANT) {
-                    if (j == 0) qz = qz_lds[t * 16 + n];
+                    qz[0] = *reinterpret_cast<const half8 *>(qz_lds + ((t * 2 + 0) * 64 + lane) * 8);
+                    qz[1] = *reinterpret_cast<const half8 *>(qz_lds + ((t * 2 + 1) * 64 + lane) * 8);
                 }
             }
 #pragma unroll
@@ -494,10 +511,12 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
                 const int tok0 = BLOCK * blk + 4 * j;  // this lane's 4 tokens in C layout
                 floatx4 s = {0, 0, 0, 0};
                 if constexpr (QUANT) {
-                    // bias term: A = (z_0..z_3, z_0..z_3) of token n in lanes j == 0
+                    // bias term: slot e of every lane group belongs to group e / 2 of token n
                     const u32x2 zr = *reinterpret_cast<const u32x2 *>(kz_lds + 4 * (BLOCK * blk + n));
-                    const half8 zop = (j == 0) ? as_half8(zr.x, zr.y, zr.x, zr.y) : as_half8(0, 0, 0, 0);
-                    s = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz, s, 0, 0, 0);
+                    const half8 zop = as_half8(perm(0, zr.x, 0x01000100u), perm(0, zr.x, 0x03020302u),
+                                               perm(0, zr.y, 0x01000100u), perm(0, zr.y, 0x03020302u));
+                    s = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz[0], s, 0, 0, 0);
+                    s = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz[1], s, 0, 0, 0);
                 }
                 floatx4 r[4];
 #pragma unroll
@@ -535,9 +554,15 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
                 *reinterpret_cast<floatx4 *>(s_lds + (16 * t + n) * SC_STRIDE + tok0) = s;
             }
         }
+        // The key registers and the scale registers are free: request the next iteration's.
+        if (it + 1 < n_it) {
+            load_keys(it + 1);
+            load_scales(it + 1);
+        }
         __syncthreads();
 
         // ---- phase B: online softmax per row ---------------------------------------
+        // Writes P * P_UP over the scores; l sums the plain P.
         {
             float sv[Sh::TPT];
             float *row = s_lds + b_row * SC_STRIDE + b_part * Sh::TPT;
@@ -558,24 +583,67 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
 #pragma unroll
             for (int step = 1; step < Sh::TPR; step *= 2) cm = fmaxf(cm, __shfl_xor(cm, step));
             const float nm = fmaxf(m_run, cm);
-            const float al = exp2f(m_run - nm);
+            const float al = __builtin_amdgcn_exp2f(m_run - nm);
             float sum = 0.0f;
 #pragma unroll
             for (int i = 0; i < Sh::TPT; i++) {
-                sv[i] = (tok0 + i < lim) ? exp2f(sv[i] - nm) : 0.0f;
+                sv[i] = (tok0 + i < lim) ? __builtin_amdgcn_exp2f(sv[i] - nm) : 0.0f;
                 sum += sv[i];
             }
             l_part = l_part * al + sum;
             m_run = nm;
 #pragma unroll
             for (int i = 0; i < Sh::TPT; i += 2) {
-                *reinterpret_cast<floatx2 *>(row + i) = floatx2{sv[i], sv[i + 1]};
+                *reinterpret_cast<floatx2 *>(row + i) = floatx2{sv[i] * P_UP, sv[i + 1] * P_UP};
             }
             if (b_part == 0) alpha_lds[b_row] = al;
         }
         __syncthreads();
 
         // ---- phase C: O += P V for this wave's group -------------------------------
+        // The probability operands need only P and the value scales, so they are all built
+        // before the first value code is touched: what is left to do once the (large,
+        // last-requested) value loads land is the byte permutes and the MFMAs.
+        auto build_p = [&](int t, int ks, half8 &phi, half8 &plo) {
+            const float *prow = s_lds + (PACKED ? (n & 7) : 16 * t + n) * SC_STRIDE;
+            const int tk = 32 * ks + 8 * j;
+            const floatx4 p0 = *reinterpret_cast<const floatx4 *>(prow + tk);
+            const floatx4 p1 = *reinterpret_cast<const floatx4 *>(prow + tk + 4);
+            float pv[8] = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
+            if constexpr (QUANT) {
+                const u32x4 sr = *reinterpret_cast<const u32x4 *>(vs_lds + wave * IT_TOKENS + tk);
+                const u32x4 zr = *reinterpret_cast<const u32x4 *>(vz_lds + wave * IT_TOKENS + tk);
+                const uint32_t sw[4] = {sr.x, sr.y, sr.z, sr.w}, zw[4] = {zr.x, zr.y, zr.z, zr.w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    zacc[t] += pv[e] * half_bits_to_float(zw[e >> 1] >> (16 * (e & 1)));
+                    pv[e] *= half_bits_to_float(sw[e >> 1] >> (16 * (e & 1)));
+                }
+            }
+            if constexpr (PACKED) {
+                // hi lanes (n < 8) keep x and let the conversion truncate it to its hi part;
+                // lo lanes subtract the hi part first.
+                const uint32_t lo_mask = (n >= 8) ? 0xffffe000u : 0u;
+                uint32_t o[4];
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                    const float x0 = pv[e] - __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, pv[e]) & lo_mask);
+                    const float x1 =
+                        pv[e + 1] - __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, pv[e + 1]) & lo_mask);
+                    // round toward zero: exact truncation to the hi part in hi lanes
+                    o[e / 2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x0, x1));
+                }
+                phi = as_half8(o[0], o[1], o[2], o[3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    _Float16 h, lw;
+                    split_hi_lo(pv[e], h, lw);
+                    phi[e] = h;
+                    plo[e] = lw;
+                }
+            }
+        };
 #pragma unroll
         for (int t = 0; t < TILES; t++) {
             // Rescale what was summed so far.  Accumulator rows (C layout) are 4j..4j+3.
@@ -586,61 +654,55 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
                 for (int e = 0; e < 4; e++) acc[t][e] *= al;
                 zacc[t] *= alpha_lds[PACKED ? (n & 7) : 16 * t + n];
             }
-            const float *prow = s_lds + (PACKED ? (n & 7) : 16 * t + n) * SC_STRIDE;
-            // hi lanes (PACKED: n < 8) keep x and let the conversion truncate it to its hi part;
-            // lo lanes subtract the hi part first.
-            const uint32_t lo_mask = (PACKED && n >= 8) ? 0xffffe000u : 0u;
+            if constexpr (PACKED) {
+                half8 phi[6], plo[6];
 #pragma unroll
-            for (int ks = 0; ks < 6; ks++) {
-                if (uint32_t(ks) >= ksteps) break;
-                const int tk = 32 * ks + 8 * j;
-                const floatx4 p0 = *reinterpret_cast<const floatx4 *>(prow + tk);
-                const floatx4 p1 = *reinterpret_cast<const floatx4 *>(prow + tk + 4);
-                float pv[8] = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
-                if constexpr (QUANT) {
-                    const u32x4 sr = *reinterpret_cast<const u32x4 *>(vs_lds + wave * IT_TOKENS + tk);
-                    const u32x4 zr = *reinterpret_cast<const u32x4 *>(vz_lds + wave * IT_TOKENS + tk);
-                    const uint32_t sw[4] = {sr.x, sr.y, sr.z, sr.w}, zw[4] = {zr.x, zr.y, zr.z, zr.w};
-#pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        zacc[t] += pv[e] * half_bits_to_float(zw[e >> 1] >> (16 * (e & 1)));
-                        pv[e] *= half_bits_to_float(sw[e >> 1] >> (16 * (e & 1))) * P_UP;
-                    }
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; e++) pv[e] *= P_UP;
-                }
-                half8 phi, plo;
-                if constexpr (PACKED) {
-                    uint32_t o[4];
-#pragma unroll
-                    for (int e = 0; e < 8; e += 2) {
-                        const float x0 = pv[e] - __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, pv[e]) & lo_mask);
-                        const float x1 =
-                            pv[e + 1] - __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, pv[e + 1]) & lo_mask);
-                        // round toward zero: exact truncation to the hi part in hi lanes
-                        o[e / 2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x0, x1));
-                    }
-                    phi = as_half8(o[0], o[1], o[2], o[3]);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        _Float16 h, lw;
-                        split_hi_lo(pv[e], h, lw);
-                        phi[e] = h;
-                        plo[e] = lw;
-                    }
+                for (int ks = 0; ks < 6; ks++) {
+                    if (uint32_t(ks) < ksteps) build_p(t, ks, phi[ks], plo[ks]);
                 }
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const half8 vop = val_operand<BITS>(vreg[ks], e, n);
-                    acc[t][e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(phi, vop, acc[t][e], 0, 0, 0);
-                    if constexpr (!PACKED) {
+                for (int ks = 0; ks < 6; ks++) {
+                    if (uint32_t(ks) >= ksteps) break;
+                    if constexpr (BITS == 16) {
+                        // Rows past the context may hold anything, NaN included: 0 * NaN must not reach O.
+#pragma unroll
+                        for (int e = 0; e < 8; e++) {
+                            if (base + 32 * ks + 8 * j + e >= max_len) vreg[ks].w[e] = 0, vreg[ks].w[8 + e] = 0;
+                        }
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const half8 vop = val_operand<BITS>(vreg[ks], e, n);
+                        acc[t][e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(phi[ks], vop, acc[t][e], 0, 0, 0);
+                        if constexpr (!PACKED) {
+                            acc[t][e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(plo[ks], vop, acc[t][e], 0, 0, 0);
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int ks = 0; ks < 6; ks++) {
+                    if (uint32_t(ks) >= ksteps) break;
+                    half8 phi, plo;
+                    build_p(t, ks, phi, plo);
+                    if constexpr (BITS == 16) {
+                        if (t == 0) {
+#pragma unroll
+                            for (int e = 0; e < 8; e++) {
+                                if (base + 32 * ks + 8 * j + e >= max_len) vreg[ks].w[e] = 0, vreg[ks].w[8 + e] = 0;
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const half8 vop = val_operand<BITS>(vreg[ks], e, n);
+                        acc[t][e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(phi, vop, acc[t][e], 0, 0, 0);
                         acc[t][e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(plo, vop, acc[t][e], 0, 0, 0);
                     }
                 }
             }
         }
+        if (it + 1 < n_it) load_values(it + 1);
     }
 
     // ---- epilogue: one partial per (row, head) ------------------------------------
@@ -683,7 +745,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
             const int pair = 16 * t + 4 * j + i;  // (row, head) pair of this accumulator row
             if (pair >= int(real_rows)) continue;
             const int vrow = pair >> 3, head = pair & 7;
-            const float zb = QUANT ? zsum_lds[wave * Sh::S_ROWS + pair] : 0.0f;
+            const float zb = QUANT ? zsum_lds[wave * Sh::S_ROWS + pair] * (1.0f / P_UP) : 0.0f;
             const size_t slot = (size_t(vrow) * a.nsplits + split) * a.heads + kv * 8 + head;
             float *dst = a.part_o + slot * DIM + 64 * wave;
             if constexpr (BITS == 16) {
