@@ -1,0 +1,368 @@
+// Host side of the attention hot path in C++, above the C ABI of include/saetta_hip.h.
+//
+// The reference's host code for this path is Rust calling Metal; this header mirrors its public
+// items one for one (same names, argument meaning, ownership and error behaviour) so that a
+// caller of src/kv_quant.rs, src/attention.rs, src/rows.rs and src/attention_prefill.rs finds
+// the same surface:
+//
+//   gpu::Gpu, gpu::Buffer, View        src/gpu.rs:233-290, src/qmv.rs:18-23
+//   plan::TokenParams, Plan, Built     src/plan.rs:16-35, 63-146, 187-273
+//   kv_quant::KvBits, GROUP, QuantRows src/kv_quant.rs:8-50, 156-283
+//   attention::DecodeAttention         src/attention.rs:28-171
+//   rows::MAX_ROWS, AttentionRows      src/rows.rs:8-9, 344-494
+//   attention_prefill::FlashParams, KERNELS, DEFAULT, KEY_BLOCK, encode
+//                                      src/attention_prefill.rs:4-72
+//
+// Where the reference asserts or panics, these throw std::runtime_error.  Buffers are
+// reference-counted and zero-filled like Metal's (src/gpu.rs:287-290); a Plan keeps every
+// buffer it binds alive (src/plan.rs:113-123).  Single-threaded use, like the reference's Gpu.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <functional>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "../../include/saetta_hip.h"
+
+namespace saetta {
+
+inline void check(int rc, const char *what) {
+    if (rc != 0) throw std::runtime_error(std::string(what) + ": " + saetta_last_error() + " (code " + std::to_string(rc) + ")");
+}
+inline void hip_check(hipError_t e, const char *what) {
+    if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+namespace gpu {
+
+// A device allocation, zero-filled, freed when the last handle goes.
+class Buffer {
+  public:
+    Buffer() = default;
+    explicit Buffer(size_t bytes) : bytes_(bytes) {
+        void *p = nullptr;
+        hip_check(hipMalloc(&p, bytes ? bytes : 1), "hipMalloc");
+        hip_check(hipMemset(p, 0, bytes ? bytes : 1), "hipMemset");
+        ptr_ = std::shared_ptr<void>(p, [](void *q) { (void)hipFree(q); });
+    }
+    void *get() const { return ptr_.get(); }
+    size_t length() const { return bytes_; }
+
+  private:
+    std::shared_ptr<void> ptr_;
+    size_t bytes_ = 0;
+};
+
+// Device + stream (Gpu::new, src/gpu.rs:233-263).
+class Gpu {
+  public:
+    Gpu() {
+        check(saetta_init(), "Gpu::new");
+        hip_check(hipStreamCreate(&stream_), "hipStreamCreate");
+    }
+    ~Gpu() { (void)hipStreamDestroy(stream_); }
+    Gpu(const Gpu &) = delete;
+    Gpu &operator=(const Gpu &) = delete;
+    Buffer buffer(size_t bytes) const { return Buffer(bytes); }
+    template <typename T>
+    Buffer buffer_from(const std::vector<T> &data) const {
+        Buffer b(data.size() * sizeof(T));
+        hip_check(hipMemcpy(b.get(), data.data(), data.size() * sizeof(T), hipMemcpyHostToDevice), "hipMemcpy");
+        return b;
+    }
+    hipStream_t stream() const { return stream_; }
+    void sync() const { hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize"); }
+
+  private:
+    hipStream_t stream_ = nullptr;
+};
+
+// contents::<T>(buffer, n) of src/gpu.rs: a host copy of the first n elements.
+template <typename T>
+std::vector<T> contents(const Buffer &b, size_t n, size_t byte_offset = 0) {
+    std::vector<T> out(n);
+    hip_check(hipMemcpy(out.data(), static_cast<char *>(b.get()) + byte_offset, n * sizeof(T), hipMemcpyDeviceToHost),
+              "hipMemcpy");
+    return out;
+}
+
+}  // namespace gpu
+
+// A buffer and a byte offset into it (src/qmv.rs:18-23).
+struct View {
+    gpu::Buffer buffer;
+    uint64_t offset = 0;
+    View() = default;
+    explicit View(gpu::Buffer b, uint64_t off = 0) : buffer(std::move(b)), offset(off) {}
+    template <typename T>
+    T *ptr() const { return reinterpret_cast<T *>(static_cast<char *>(buffer.get()) + offset); }
+    View at(uint64_t bytes) const { return View(buffer, offset + bytes); }
+};
+
+namespace plan {
+
+using TokenParams = saetta_token_params;
+inline TokenParams token_params(uint32_t token, uint32_t position) {  // TokenParams::new
+    return TokenParams{token, position, position + 1, 0};
+}
+
+class Built {
+  public:
+    explicit Built(std::vector<std::pair<std::string, std::function<void(hipStream_t)>>> ops) : ops_(std::move(ops)) {}
+    void run(const gpu::Gpu &gpu) const {
+        for (auto &op : ops_) op.second(gpu.stream());
+        gpu.sync();
+    }
+    // Replays without waiting, for timing many runs back to back.
+    void enqueue(const gpu::Gpu &gpu) const {
+        for (auto &op : ops_) op.second(gpu.stream());
+    }
+
+  private:
+    std::vector<std::pair<std::string, std::function<void(hipStream_t)>>> ops_;
+};
+
+// A list of launches recorded once and run for every token; what changes per token is in the
+// TokenParams buffer, which the kernels read when they run.
+class Plan {
+  public:
+    explicit Plan(const gpu::Gpu &gpu) : params(gpu.buffer(sizeof(TokenParams))), gpu_(gpu) {}
+    View params;
+    void op(std::string kernel, std::function<void(hipStream_t)> launch) { ops_.emplace_back(std::move(kernel), std::move(launch)); }
+    void set_params(TokenParams tp) {
+        hip_check(hipMemcpyAsync(params.ptr<void>(), &tp, sizeof tp, hipMemcpyHostToDevice, gpu_.stream()), "set_params");
+        gpu_.sync();
+    }
+    Built build() const { return Built(ops_); }
+    Built build_where(const std::function<bool(const std::string &)> &keep) const {
+        std::vector<std::pair<std::string, std::function<void(hipStream_t)>>> kept;
+        for (auto &op : ops_) {
+            if (keep(op.first)) kept.push_back(op);
+        }
+        return Built(std::move(kept));
+    }
+
+  private:
+    std::vector<std::pair<std::string, std::function<void(hipStream_t)>>> ops_;
+    const gpu::Gpu &gpu_;
+};
+
+}  // namespace plan
+
+namespace kv_quant {
+
+constexpr size_t GROUP = 64;
+
+enum class KvBits { Half, Eight, Four };
+
+inline bool parse(const std::string &s, KvBits &out) {
+    if (s == "16") return out = KvBits::Half, true;
+    if (s == "8") return out = KvBits::Eight, true;
+    if (s == "4") return out = KvBits::Four, true;
+    return false;
+}
+inline uint32_t bits(KvBits b) { return b == KvBits::Half ? 16 : b == KvBits::Eight ? 8 : 4; }
+inline size_t words_per_group(KvBits b) { return 2 * bits(b); }
+inline double bytes_per_value(KvBits b) { return b == KvBits::Half ? 2.0 : bits(b) / 8.0 + 4.0 / GROUP; }
+
+// The codes, scales and biases of one cache (keys or values).
+struct QuantRows {
+    gpu::Buffer data, scales, biases;
+    KvBits bits;
+    size_t per_token;
+
+    QuantRows(const gpu::Gpu &gpu, KvBits b, size_t values, size_t capacity) : bits(b), per_token(values / GROUP) {
+        if (b == KvBits::Half || values % GROUP != 0) throw std::runtime_error("QuantRows::new: bits must be 8 or 4, values a multiple of 64");
+        const size_t groups = per_token * capacity;
+        data = gpu.buffer(groups * words_per_group(b) * 4);
+        scales = gpu.buffer(groups * 2);
+        biases = gpu.buffer(groups * 2);
+    }
+    saetta_quant_rows c() const {
+        return saetta_quant_rows{static_cast<uint32_t *>(data.get()), static_cast<uint16_t *>(scales.get()),
+                                 static_cast<uint16_t *>(biases.get())};
+    }
+    // One token's values x into its slot, at the plan's position.
+    void record(plan::Plan &plan, const View &x) const { record_at(plan, x, plan.params, false); }
+    void record_at(plan::Plan &plan, const View &x, const View &params, bool /*parallel*/) const {
+        const saetta_kv_quant_params p{uint32_t(per_token), uint32_t(per_token)};
+        const QuantRows self = *this;
+        const int nbits = int(kv_quant::bits(bits));
+        plan.op(nbits == 8 ? "kv_quantize_8" : "kv_quantize_4", [=](hipStream_t s) {
+            check(saetta_kv_quantize(s, nbits, x.ptr<float>(), self.c(), p, params.ptr<saetta_token_params>(), 0), "kv_quantize");
+        });
+    }
+    // `tokens` tokens of x into the slots from pos.
+    void encode(const gpu::Gpu &gpu, const View &x, size_t pos, size_t tokens) const {
+        const saetta_kv_quant_params p{uint32_t(per_token * tokens), uint32_t(per_token)};
+        check(saetta_kv_quantize(gpu.stream(), int(kv_quant::bits(bits)), x.ptr<float>(), c(), p, nullptr, uint32_t(pos)), "kv_quantize");
+    }
+    // Tokens 0..tokens as half into out.
+    void encode_dequantize(const gpu::Gpu &gpu, const View &out, size_t tokens) const {
+        const saetta_kv_quant_params p{uint32_t(per_token * tokens), uint32_t(per_token)};
+        check(saetta_kv_dequantize(gpu.stream(), int(kv_quant::bits(bits)), c(), out.ptr<uint16_t>(), p), "kv_dequantize");
+    }
+};
+
+}  // namespace kv_quant
+
+namespace attention {
+
+constexpr size_t DIM = 256;
+
+class DecodeAttention {
+  public:
+    DecodeAttention(const gpu::Gpu &gpu, size_t heads, size_t kv_heads, size_t head_dim, size_t capacity)
+        : heads_(heads), kv_heads_(kv_heads), capacity_(capacity) {
+        if (head_dim != DIM) throw std::runtime_error("decode attention is written for head dim 256");
+        if (heads != kv_heads * 8) throw std::runtime_error("decode attention needs 8 q heads per kv head");
+        part_o_ = gpu.buffer(saetta_part_o_bytes(uint32_t(heads), uint32_t(capacity), 1));
+        part_ml_ = gpu.buffer(saetta_part_ml_bytes(uint32_t(heads), uint32_t(capacity), 1));
+    }
+    std::string kernel = "attention_partial_mma";
+
+    void record(plan::Plan &plan, const View &q, const View &keys, const View &values, const View &q_and_gate, const View &out) const {
+        const auto p = params();
+        const View tp = plan.params;
+        const gpu::Buffer po = part_o_, pml = part_ml_;
+        auto launch = [=](uint32_t stage) {
+            return [=](hipStream_t s) {
+                check(saetta_attn_decode(s, q.ptr<float>(), keys.ptr<uint16_t>(), values.ptr<uint16_t>(), static_cast<float *>(po.get()),
+                                         static_cast<float *>(pml.get()), q_and_gate.ptr<float>(), out.ptr<float>(), p,
+                                         tp.ptr<saetta_token_params>(), stage),
+                      "attn_decode");
+            };
+        };
+        plan.op(kernel, launch(SAETTA_STAGE_PARTIAL));
+        plan.op("attention_reduce", launch(SAETTA_STAGE_REDUCE));
+    }
+    void record_quant(plan::Plan &plan, const View &q, const kv_quant::QuantRows &keys, const kv_quant::QuantRows &values,
+                      const View &q_and_gate, const View &out) const {
+        if (keys.bits == kv_quant::KvBits::Half) throw std::runtime_error("a half cache goes through record");
+        const auto p = params();
+        const View tp = plan.params;
+        const gpu::Buffer po = part_o_, pml = part_ml_;
+        const kv_quant::QuantRows k = keys, v = values;
+        const int nbits = int(kv_quant::bits(keys.bits));
+        auto launch = [=](uint32_t stage) {
+            return [=](hipStream_t s) {
+                check(saetta_attn_decode_quant(s, nbits, q.ptr<float>(), k.c(), v.c(), static_cast<float *>(po.get()),
+                                               static_cast<float *>(pml.get()), q_and_gate.ptr<float>(), out.ptr<float>(), p,
+                                               tp.ptr<saetta_token_params>(), stage),
+                      "attn_decode_quant");
+            };
+        };
+        plan.op(kernel + (nbits == 8 ? "_q8" : "_q4"), launch(SAETTA_STAGE_PARTIAL));
+        plan.op("attention_reduce", launch(SAETTA_STAGE_REDUCE));
+    }
+
+  private:
+    saetta_decode_params params() const {
+        return saetta_decode_params{uint32_t(heads_), uint32_t(kv_heads_), uint32_t(capacity_), 1.0f / std::sqrt(float(DIM))};
+    }
+    size_t heads_, kv_heads_, capacity_;
+    gpu::Buffer part_o_, part_ml_;
+};
+
+}  // namespace attention
+
+namespace rows {
+
+constexpr size_t MAX_ROWS = 8;
+
+class AttentionRows {
+  public:
+    AttentionRows(const gpu::Gpu &gpu, size_t heads, size_t kv_heads, size_t capacity, size_t rows)
+        : heads_(heads), kv_heads_(kv_heads), capacity_(capacity), rows_(rows) {
+        if (heads != kv_heads * 8) throw std::runtime_error("rows attention needs 8 q heads per kv head");
+        if (rows < 1 || rows > MAX_ROWS) throw std::runtime_error(std::to_string(rows) + " rows");
+        splits_ = saetta_part_ml_bytes(uint32_t(heads), uint32_t(capacity), 1) / (heads * 8);
+        part_o_ = gpu.buffer(saetta_part_o_bytes(uint32_t(heads), uint32_t(capacity), uint32_t(rows)));
+        part_ml_ = gpu.buffer(saetta_part_ml_bytes(uint32_t(heads), uint32_t(capacity), uint32_t(rows)));
+    }
+    // Row r takes its position from params[0] + r, as the reference's kernels do.
+    void record(plan::Plan &plan, size_t m, const View &q, const View &keys, const View &values, const View &q_and_gate,
+                const View &out, const std::vector<View> &params) const {
+        if (m > rows_ || params.size() < m) throw std::runtime_error("AttentionRows::record: too many rows");
+        const auto p = rows_params(m);
+        const View tp = params[0];
+        const gpu::Buffer po = part_o_, pml = part_ml_;
+        auto launch = [=](uint32_t stage) {
+            return [=](hipStream_t s) {
+                check(saetta_attn_rows(s, q.ptr<float>(), keys.ptr<uint16_t>(), values.ptr<uint16_t>(), static_cast<float *>(po.get()),
+                                       static_cast<float *>(pml.get()), q_and_gate.ptr<float>(), out.ptr<float>(), p,
+                                       tp.ptr<saetta_token_params>(), stage),
+                      "attn_rows");
+            };
+        };
+        plan.op("attention_partial_rows_chunks", launch(SAETTA_STAGE_PARTIAL));
+        plan.op("attention_reduce_rows_chunks", launch(SAETTA_STAGE_REDUCE));
+    }
+    void record_quant(plan::Plan &plan, size_t m, const View &q, const kv_quant::QuantRows &keys, const kv_quant::QuantRows &values,
+                      const View &q_and_gate, const View &out, const std::vector<View> &params) const {
+        if (m > rows_ || params.size() < m) throw std::runtime_error("AttentionRows::record_quant: too many rows");
+        if (keys.bits == kv_quant::KvBits::Half) throw std::runtime_error("a half cache goes through record");
+        const auto p = rows_params(m);
+        const View tp = params[0];
+        const gpu::Buffer po = part_o_, pml = part_ml_;
+        const kv_quant::QuantRows k = keys, v = values;
+        const int nbits = int(kv_quant::bits(keys.bits));
+        auto launch = [=](uint32_t stage) {
+            return [=](hipStream_t s) {
+                check(saetta_attn_rows_quant(s, nbits, q.ptr<float>(), k.c(), v.c(), static_cast<float *>(po.get()),
+                                             static_cast<float *>(pml.get()), q_and_gate.ptr<float>(), out.ptr<float>(), p,
+                                             tp.ptr<saetta_token_params>(), stage),
+                      "attn_rows_quant");
+            };
+        };
+        plan.op(nbits == 8 ? "attention_partial_rows_q8" : "attention_partial_rows_q4", launch(SAETTA_STAGE_PARTIAL));
+        plan.op("attention_reduce_rows", launch(SAETTA_STAGE_REDUCE));
+    }
+
+  private:
+    saetta_rows_params rows_params(size_t m) const {
+        return saetta_rows_params{uint32_t(heads_), uint32_t(kv_heads_), uint32_t(capacity_), 1.0f / 16.0f, uint32_t(m), uint32_t(splits_)};
+    }
+    size_t heads_, kv_heads_, capacity_, rows_, splits_ = 0;
+    gpu::Buffer part_o_, part_ml_;
+};
+
+}  // namespace rows
+
+namespace attention_prefill {
+
+using FlashParams = saetta_flash_params;
+inline const char *const KERNELS[2] = {"attention_fa8", "attention_fa4"};
+inline const char *const DEFAULT = "attention_fa8";
+constexpr size_t KEY_BLOCK = 16;
+
+// out[t, h] = softmax(q[t, h] K^T * scale) V * sigmoid(gate[t, h]) over a half cache that holds
+// the chunk's rows.  `kernel` picks a tile size in the reference; one gfx950 kernel serves both.
+inline void encode(const gpu::Gpu &gpu, const std::string &kernel, const View &q, const View &keys, const View &values,
+                   const View &q_and_gate, const View &out, FlashParams p) {
+    if (kernel != KERNELS[0] && kernel != KERNELS[1]) throw std::runtime_error("no prefill attention kernel " + kernel);
+    if (p.heads != p.kv_heads * 8) throw std::runtime_error(kernel + " needs 8 q heads per kv head");
+    check(saetta_attn_prefill(gpu.stream(), q.ptr<uint16_t>(), keys.ptr<uint16_t>(), values.ptr<uint16_t>(), q_and_gate.ptr<float>(),
+                              out.ptr<float>(), p),
+          "attn_prefill");
+}
+
+// The same chunk over a quantized cache read in place (src/prefill.rs:1735-1776).
+inline void encode_quant(const gpu::Gpu &gpu, const View &q, const kv_quant::QuantRows &keys, const kv_quant::QuantRows &values,
+                         const View &q_and_gate, const View &out, FlashParams p) {
+    if (p.heads != p.kv_heads * 8) throw std::runtime_error("prefill attention needs 8 q heads per kv head");
+    check(saetta_attn_prefill_quant(gpu.stream(), int(kv_quant::bits(keys.bits)), q.ptr<uint16_t>(), keys.c(), values.c(),
+                                    q_and_gate.ptr<float>(), out.ptr<float>(), p),
+          "attn_prefill_quant");
+}
+
+}  // namespace attention_prefill
+
+}  // namespace saetta

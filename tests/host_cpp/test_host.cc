@@ -1,0 +1,151 @@
+// The reference's own GPU tests for this path, restated in C++ against the host mirror
+// (saetta-macqwen_amd/host/saetta.hpp) with the CPU oracle as the other side:
+//   tests/kv_quant.rs   prefill_rows_match_cpu, decode_row_matches_cpu, dequantize_matches_cpu
+//   tests/attention.rs  quantized_matches_cpu
+// Exit code 0 = all passed.  Run by tests/test_gpu_host_cpp.py on a GPU box.
+#include <cstdio>
+#include <cstdlib>
+
+#include "../../saetta-macqwen_amd/host/saetta.hpp"
+
+extern "C" {  // oracle/saetta_oracle.c (the checker)
+int orc_quantize(const float *x, size_t n, int bits, uint32_t *data, uint16_t *scales, uint16_t *biases);
+int orc_dequantize(const uint32_t *data, const uint16_t *scales, const uint16_t *biases, size_t groups, int bits, float *out);
+uint16_t orc_f32_to_f16(float f);
+void orc_noise(float *out, size_t n, uint64_t seed);
+void orc_quant_rows(float *out, size_t tokens, size_t values);
+int orc_attention_f64(const float *q, const float *k, const float *v, const float *q_and_gate, size_t len, size_t heads,
+                      size_t kv_heads, size_t dim, double *out, int threads);
+}
+
+using namespace saetta;
+using kv_quant::KvBits;
+using kv_quant::QuantRows;
+
+static int failures = 0;
+#define EXPECT(cond, ...)                 \
+    do {                                  \
+        if (!(cond)) {                    \
+            failures++;                   \
+            std::printf("FAIL: " __VA_ARGS__); \
+            std::printf("\n");            \
+        }                                 \
+    } while (0)
+
+constexpr size_t VALUES = 2 * 256, HEADS = 16, KV = 2, DIM = 256;
+
+static void compare(const QuantRows &rows, const std::vector<float> &x, size_t from_token, KvBits bits) {
+    const int b = int(kv_quant::bits(bits));
+    const size_t groups = x.size() / 64, first = from_token * rows.per_token, words = kv_quant::words_per_group(bits);
+    auto data = gpu::contents<uint32_t>(rows.data, groups * words, first * words * 4);
+    auto scales = gpu::contents<uint16_t>(rows.scales, groups, first * 2);
+    auto biases = gpu::contents<uint16_t>(rows.biases, groups, first * 2);
+    std::vector<uint32_t> wd(groups * words);
+    std::vector<uint16_t> ws(groups), wz(groups);
+    orc_quantize(x.data(), x.size(), b, wd.data(), ws.data(), wz.data());
+    EXPECT(scales == ws, "%d-bit scales", b);
+    EXPECT(biases == wz, "%d-bit biases", b);
+    size_t off = 0;
+    for (size_t i = 0; i < wd.size(); i++) off += data[i] != wd[i];
+    EXPECT(off == 0, "%d-bit: %zu code words differ", b, off);
+}
+
+int main() {
+    gpu::Gpu gpu;
+    for (KvBits bits : {KvBits::Eight, KvBits::Four}) {
+        {  // prefill_rows_match_cpu
+            const size_t tokens = 37;
+            QuantRows cache(gpu, bits, VALUES, 64);
+            std::vector<float> x(tokens * VALUES);
+            orc_quant_rows(x.data(), tokens, VALUES);
+            View xb(gpu.buffer_from(x));
+            cache.encode(gpu, xb, 5, tokens);
+            gpu.sync();
+            compare(cache, x, 5, bits);
+        }
+        {  // decode_row_matches_cpu
+            QuantRows cache(gpu, bits, VALUES, 64);
+            std::vector<float> x(VALUES);
+            orc_quant_rows(x.data(), 1, VALUES);
+            View xb(gpu.buffer_from(x));
+            plan::Plan plan(gpu);
+            cache.record(plan, xb);
+            auto built = plan.build();
+            plan.set_params(plan::token_params(0, 41));
+            built.run(gpu);
+            compare(cache, x, 41, bits);
+        }
+        {  // dequantize_matches_cpu
+            const size_t tokens = 9;
+            QuantRows cache(gpu, bits, VALUES, 64);
+            std::vector<float> x(tokens * VALUES);
+            orc_quant_rows(x.data(), tokens, VALUES);
+            View xb(gpu.buffer_from(x)), out(gpu.buffer(tokens * VALUES * 2));
+            cache.encode(gpu, xb, 0, tokens);
+            cache.encode_dequantize(gpu, out, tokens);
+            gpu.sync();
+            const size_t groups = tokens * cache.per_token;
+            auto data = gpu::contents<uint32_t>(cache.data, groups * kv_quant::words_per_group(bits));
+            auto scales = gpu::contents<uint16_t>(cache.scales, groups);
+            auto biases = gpu::contents<uint16_t>(cache.biases, groups);
+            std::vector<float> want(tokens * VALUES);
+            orc_dequantize(data.data(), scales.data(), biases.data(), groups, int(kv_quant::bits(bits)), want.data());
+            auto got = gpu::contents<uint16_t>(out.buffer, tokens * VALUES);
+            size_t bad = 0;
+            for (size_t i = 0; i < got.size(); i++) bad += got[i] != orc_f32_to_f16(want[i]);
+            EXPECT(bad == 0, "dequantize: %zu halves differ", bad);
+        }
+        {  // quantized_matches_cpu (tests/attention.rs:98-201)
+            const size_t capacity = 1024;
+            std::vector<float> q(HEADS * DIM), qg(HEADS * 2 * DIM), keys(capacity * KV * DIM), values(capacity * KV * DIM);
+            orc_noise(q.data(), q.size(), 3);
+            orc_noise(qg.data(), qg.size(), 4);
+            orc_noise(keys.data(), keys.size(), 1);
+            for (auto &k : keys) k *= 4.0f;
+            orc_noise(values.data(), values.size(), 2);
+            QuantRows kc(gpu, bits, VALUES, capacity), vc(gpu, bits, VALUES, capacity);
+            View kx(gpu.buffer_from(keys)), vx(gpu.buffer_from(values));
+            kc.encode(gpu, kx, 0, capacity);
+            vc.encode(gpu, vx, 0, capacity);
+            gpu.sync();
+            const size_t groups = capacity * 8, words = kv_quant::words_per_group(bits);
+            std::vector<float> kf(keys.size()), vf(values.size());
+            {
+                auto d = gpu::contents<uint32_t>(kc.data, groups * words);
+                auto s = gpu::contents<uint16_t>(kc.scales, groups);
+                auto z = gpu::contents<uint16_t>(kc.biases, groups);
+                orc_dequantize(d.data(), s.data(), z.data(), groups, int(kv_quant::bits(bits)), kf.data());
+                d = gpu::contents<uint32_t>(vc.data, groups * words);
+                s = gpu::contents<uint16_t>(vc.scales, groups);
+                z = gpu::contents<uint16_t>(vc.biases, groups);
+                orc_dequantize(d.data(), s.data(), z.data(), groups, int(kv_quant::bits(bits)), vf.data());
+            }
+            View qb(gpu.buffer_from(q)), gb(gpu.buffer_from(qg)), out(gpu.buffer(HEADS * DIM * 4));
+            attention::DecodeAttention att(gpu, HEADS, KV, DIM, capacity);
+            plan::Plan plan(gpu);
+            att.record_quant(plan, qb, kc, vc, gb, out);
+            auto built = plan.build();
+            for (size_t len : {1, 127, 129, 1000, 1024}) {
+                plan.set_params(plan::token_params(0, uint32_t(len - 1)));
+                built.run(gpu);
+                auto got = gpu::contents<float>(out.buffer, HEADS * DIM);
+                std::vector<double> want(HEADS * DIM);
+                orc_attention_f64(q.data(), kf.data(), vf.data(), qg.data(), len, HEADS, KV, DIM, want.data(), 4);
+                double worst = 0;
+                for (size_t i = 0; i < got.size(); i++) worst = std::fmax(worst, std::fabs(double(got[i]) - want[i]));
+                std::printf("%d-bit len %zu: worst error %.2e\n", int(kv_quant::bits(bits)), len, worst);
+                EXPECT(worst < 2e-5, "%d-bit len %zu: %g", int(kv_quant::bits(bits)), len, worst);
+            }
+        }
+    }
+    // shape checks panic (throw) as the reference asserts
+    bool threw = false;
+    try {
+        attention::DecodeAttention bad(gpu, 16, 2, 128, 1024);
+    } catch (const std::runtime_error &) {
+        threw = true;
+    }
+    EXPECT(threw, "DecodeAttention accepted head dim 128");
+    std::printf(failures ? "%d FAILURES\n" : "all host tests passed\n", failures);
+    return failures ? 1 : 0;
+}
