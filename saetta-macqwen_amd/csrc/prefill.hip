@@ -11,7 +11,7 @@
 // cache is seen "through half": every value is f16(f32(s)*code + f32(z)),
 // exactly what round_trip_as_half (src/kv_quant.rs:119-125) gives the CPU path.
 //
-// Work split: workgroup (token tile of 16, kv head), 4 waves; wave w owns 4
+// Work split: workgroup (token tile of 32, kv head), 8 waves; wave w owns 4
 // tokens x 8 heads = 32 query rows, one 32-row MFMA tile.  Keys are walked
 // in blocks of 32.  Per block the workgroup stages K[32][256] and the
 // transposed V^T[256][32] as f16 in LDS (dequantizing on the way), then every
@@ -22,9 +22,9 @@
 // the 32x32 accumulator layout a lane holds column l % 32, so the row's
 // running max and sum, the rescale of O and the final 1/l and gate are plain
 // per-lane values and the softmax needs one cross-lane exchange per block.
-// The accumulators (128 floats per lane) live in AGPRs and two workgroups
-// share a CU, so one's staging overlaps the other's MFMAs; tiles are issued
-// heaviest first, which evens out the causal imbalance.
+// The accumulators (128 floats per lane) live in AGPRs; two waves share a
+// SIMD, so one's staging and softmax overlap the other's MFMAs; the tiles are
+// double-buffered (one barrier per block) and issued heaviest first.
 // The running max is only raised when a block exceeds it by more than 2^8
 // (the usual lazy rescale), so O is rarely rescaled.
 // The next block's codes are fetched into registers while the current block
@@ -42,9 +42,10 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int DIM = SAETTA_HEAD_DIM;
-constexpr int THREADS = 256;
+constexpr int THREADS = 512;
 constexpr int NT = 1;                   // 32-row MFMA tiles per wave (4 tokens x 8 heads each)
-constexpr int TQ = 16 * NT;             // tokens per workgroup
+constexpr int WAVES = THREADS / 64;
+constexpr int TQ = 4 * NT * WAVES;      // tokens per workgroup
 constexpr int BK = 32;                  // keys per block
 constexpr int K_STRIDE = DIM * 2 + 16;  // bytes per key row of the K tile (padded against bank conflicts)
 constexpr int V_STRIDE = BK * 2 + 16;   // bytes per dim row of the V^T tile
@@ -90,14 +91,14 @@ __device__ __forceinline__ uint32_t code_of(uint32_t w, int i) {
 }
 
 // ---- staging registers: what one thread fetches for one key block ----------------
-// K: thread (key = t / 8, piece = t % 8) takes 32 dims of one key.
-// V: thread (dq = t % 32, kq = t / 32) takes 8 dims of 4 keys.
+// K: thread (key = t / 16, piece = t % 16) takes 16 dims of one key.
+// V: thread (dq = t % 64, kq = t / 64) takes 4 dims of 4 keys.
 template <int BITS>
 struct Stage {
-    uint32_t k[BITS == 16 ? 16 : BITS];  // 32 dims: 64 B (f16), 32 B (8-bit), 16 B (4-bit)
-    uint32_t v[4][BITS == 16 ? 4 : BITS / 4];  // per key 8 dims: 16 B (f16), 8 B, 4 B
-    uint32_t ks, kz;                     // f16 scale and bias of (key, group of the piece)
-    uint32_t vs[4], vz[4];               // per key, group of dq
+    uint32_t k[BITS == 16 ? 8 : BITS / 2];  // 16 dims: 32 B (f16), 16 B (8-bit), 8 B (4-bit)
+    uint32_t v[4][BITS == 16 ? 2 : 1];      // per key 4 dims: 8 B (f16), 4 B (8-bit), 2 B (4-bit)
+    uint32_t ks, kz;                        // f16 scale and bias of (key, group of the piece)
+    uint32_t vs[4], vz[4];                  // per key, group of dq
 };
 
 template <int BITS>
@@ -108,47 +109,44 @@ __device__ __forceinline__ void stage_load(Stage<BITS> &st, const PrefillArgs &a
     constexpr int RB = row_bytes<BITS>();
     const uint32_t kvh = a.kv_heads;
     {
-        const int key = tid >> 3, piece = tid & 7;
+        const int key = tid >> 4, piece = tid & 15;
         const int row = int((key0 + key) * kvh + kv);
-        const int off = row * RB + piece * (RB / 8);
+        const int off = row * RB + piece * (RB / 16);
         if constexpr (BITS == 8) {
             const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, off, 0, 0);
-            const u32x4 y = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, off + 16, 0, 0);
             st.k[0] = x.x, st.k[1] = x.y, st.k[2] = x.z, st.k[3] = x.w;
-            st.k[4] = y.x, st.k[5] = y.y, st.k[6] = y.z, st.k[7] = y.w;
         } else if constexpr (BITS == 4) {
-            const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, off, 0, 0);
-            st.k[0] = x.x, st.k[1] = x.y, st.k[2] = x.z, st.k[3] = x.w;
+            const u32x2 x = __builtin_amdgcn_raw_buffer_load_b64(k_rsrc, off, 0, 0);
+            st.k[0] = x.x, st.k[1] = x.y;
         } else {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
+            for (int i = 0; i < 2; i++) {
                 const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, off + 16 * i, 0, 0);
                 st.k[4 * i] = x.x, st.k[4 * i + 1] = x.y, st.k[4 * i + 2] = x.z, st.k[4 * i + 3] = x.w;
             }
         }
         if constexpr (BITS != 16) {
-            const int soff = (row * 4 + (piece >> 1)) * 2;
+            const int soff = (row * 4 + (piece >> 2)) * 2;
             st.ks = __builtin_amdgcn_raw_buffer_load_b16(ks_rsrc, soff, 0, 0);
             st.kz = __builtin_amdgcn_raw_buffer_load_b16(kz_rsrc, soff, 0, 0);
         }
     }
     {
-        const int dq = tid & 31, kq = tid >> 5;
+        const int dq = tid & 63, kq = tid >> 6;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int row = int((key0 + 4 * kq + i) * kvh + kv);
-            const int off = row * RB + dq * (RB / 32);
+            const int off = row * RB + dq * (RB / 64);
             if constexpr (BITS == 8) {
+                st.v[i][0] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, off, 0, 0);
+            } else if constexpr (BITS == 4) {
+                st.v[i][0] = uint16_t(__builtin_amdgcn_raw_buffer_load_b16(v_rsrc, off, 0, 0));
+            } else {
                 const u32x2 x = __builtin_amdgcn_raw_buffer_load_b64(v_rsrc, off, 0, 0);
                 st.v[i][0] = x.x, st.v[i][1] = x.y;
-            } else if constexpr (BITS == 4) {
-                st.v[i][0] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, off, 0, 0);
-            } else {
-                const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, off, 0, 0);
-                st.v[i][0] = x.x, st.v[i][1] = x.y, st.v[i][2] = x.z, st.v[i][3] = x.w;
             }
             if constexpr (BITS != 16) {
-                const int soff = (row * 4 + (dq >> 3)) * 2;
+                const int soff = (row * 4 + (dq >> 4)) * 2;
                 st.vs[i] = __builtin_amdgcn_raw_buffer_load_b16(vs_rsrc, soff, 0, 0);
                 st.vz[i] = __builtin_amdgcn_raw_buffer_load_b16(vz_rsrc, soff, 0, 0);
             }
@@ -174,16 +172,16 @@ template <int BITS>
 __device__ __forceinline__ void stage_store(const Stage<BITS> &st, unsigned char *k_lds, unsigned char *v_lds,
                                             uint32_t key0, uint32_t key_limit, int tid) {
     {
-        const int key = tid >> 3, piece = tid & 7;
-        uint32_t o[16];
+        const int key = tid >> 4, piece = tid & 15;
+        uint32_t o[8];
         if constexpr (BITS == 16) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) o[i] = st.k[i];
+            for (int i = 0; i < 8; i++) o[i] = st.k[i];
         } else {
             const float s = h2f(st.ks), z = h2f(st.kz);
             constexpr int PER = 32 / BITS;
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
+            for (int i = 0; i < 8; i++) {
                 const uint32_t w = st.k[(2 * i) / PER];
                 o[i] = pack_half2(dequant(s, z, code_of<BITS>(w, (2 * i) % PER)),
                                   dequant(s, z, code_of<BITS>(w, (2 * i + 1) % PER)));
@@ -191,36 +189,33 @@ __device__ __forceinline__ void stage_store(const Stage<BITS> &st, unsigned char
         }
         if (key0 + key >= key_limit) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) o[i] = 0;
+            for (int i = 0; i < 8; i++) o[i] = 0;
         }
-        u32x4 *dst = reinterpret_cast<u32x4 *>(k_lds + key * K_STRIDE + piece * 64);
-#pragma unroll
-        for (int i = 0; i < 4; i++) dst[i] = u32x4{o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+        u32x4 *dst = reinterpret_cast<u32x4 *>(k_lds + key * K_STRIDE + piece * 32);
+        dst[0] = u32x4{o[0], o[1], o[2], o[3]};
+        dst[1] = u32x4{o[4], o[5], o[6], o[7]};
     }
     {
-        const int dq = tid & 31, kq = tid >> 5;
-        float x[4][8];
+        const int dq = tid & 63, kq = tid >> 6;
+        float x[4][4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const bool live = key0 + 4 * kq + i < key_limit;
             if constexpr (BITS == 16) {
 #pragma unroll
-                for (int d = 0; d < 8; d++) x[i][d] = live ? h2f(st.v[i][d >> 1] >> (16 * (d & 1))) : 0.0f;
+                for (int d = 0; d < 4; d++) x[i][d] = live ? h2f(st.v[i][d >> 1] >> (16 * (d & 1))) : 0.0f;
             } else {
                 const float s = h2f(st.vs[i]), z = h2f(st.vz[i]);
-                constexpr int PER = 32 / BITS;
 #pragma unroll
-                for (int d = 0; d < 8; d++) {
-                    x[i][d] = live ? dequant(s, z, code_of<BITS>(st.v[i][d / PER], d % PER)) : 0.0f;
-                }
+                for (int d = 0; d < 4; d++) x[i][d] = live ? dequant(s, z, code_of<BITS>(st.v[i][0], d)) : 0.0f;
             }
         }
         // keys 4kq..4kq+3 are neighbours in the row's key order
         const int p0 = vt_pos(4 * kq);
 #pragma unroll
-        for (int d = 0; d < 8; d++) {
+        for (int d = 0; d < 4; d++) {
             u32x2 w = {pack_half2(x[0][d], x[1][d]), pack_half2(x[2][d], x[3][d])};
-            *reinterpret_cast<u32x2 *>(v_lds + (8 * dq + d) * V_STRIDE + 2 * p0) = w;
+            *reinterpret_cast<u32x2 *>(v_lds + (4 * dq + d) * V_STRIDE + 2 * p0) = w;
         }
     }
 }
@@ -228,8 +223,8 @@ __device__ __forceinline__ void stage_store(const Stage<BITS> &st, unsigned char
 template <int BITS>
 __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(PrefillArgs a) {
     constexpr int RB = row_bytes<BITS>();
-    __shared__ __attribute__((aligned(16))) unsigned char k_lds[K_BYTES];
-    __shared__ __attribute__((aligned(16))) unsigned char v_lds[V_BYTES];
+    // two buffers of (K tile, V^T tile): block kb lives in buffer kb & 1
+    extern __shared__ __attribute__((aligned(16))) unsigned char tiles[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, hf = lane >> 5;
@@ -285,16 +280,28 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(PrefillArgs 
 
     Stage<BITS> st;
     stage_load<BITS>(st, a, k_rsrc, v_rsrc, ks_rsrc, kz_rsrc, vs_rsrc, vz_rsrc, 0, kv, tid);
+    stage_store<BITS>(st, tiles, tiles + K_BYTES, 0, key_limit, tid);
+    if (nblocks > 1) stage_load<BITS>(st, a, k_rsrc, v_rsrc, ks_rsrc, kz_rsrc, vs_rsrc, vz_rsrc, BK, kv, tid);
+    __syncthreads();
 
     for (uint32_t kb = 0; kb < nblocks; kb++) {
         const uint32_t key0 = kb * BK;
-        __syncthreads();  // every wave is done reading the previous block's tiles
-        stage_store<BITS>(st, k_lds, v_lds, key0, key_limit, tid);
-        __syncthreads();
+        const unsigned char *k_lds = tiles + (kb & 1) * (K_BYTES + V_BYTES);
+        const unsigned char *v_lds = k_lds + K_BYTES;
+        // Block kb + 1 goes into the other buffer (every wave left it at the barrier below),
+        // block kb + 2 into the registers.
         if (kb + 1 < nblocks) {
-            stage_load<BITS>(st, a, k_rsrc, v_rsrc, ks_rsrc, kz_rsrc, vs_rsrc, vz_rsrc, key0 + BK, kv, tid);
+            unsigned char *nk = tiles + ((kb + 1) & 1) * (K_BYTES + V_BYTES);
+            stage_store<BITS>(st, nk, nk + K_BYTES, key0 + BK, key_limit, tid);
+            if (kb + 2 < nblocks) {
+                stage_load<BITS>(st, a, k_rsrc, v_rsrc, ks_rsrc, kz_rsrc, vs_rsrc, vz_rsrc, key0 + 2 * BK, kv, tid);
+            }
         }
-        if (key0 >= wave_keys) continue;  // nothing in this block is visible to this wave (uniform)
+        if (key0 >= wave_keys) {  // nothing in this block is visible to this wave (uniform)
+            __syncthreads();
+            continue;
+        }
+  // nothing in this block is visible to this wave (uniform)
 
         // ---- S^T = K Q^T: rows = the block's 32 keys, columns = query rows ----------
         floatx16 s[NT];
@@ -374,6 +381,7 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(PrefillArgs 
                 }
             }
         }
+        __syncthreads();
     }
 
     // ---- out = O / l * sigmoid(gate) ---------------------------------------------------
@@ -422,12 +430,23 @@ int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kda
     PrefillArgs a{q, kdata, vdata, ks, kz, vs, vz, q_and_gate, out, p.heads, p.kv_heads, p.pos, p.tokens, p.scale,
                   uint32_t(rows)};
     const dim3 grid((p.tokens + TQ - 1) / TQ, p.kv_heads);
+    constexpr int LDS = 2 * (K_BYTES + V_BYTES);
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(attention_prefill_kernel<8>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(attention_prefill_kernel<4>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(attention_prefill_kernel<16>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        attr_set = true;
+    }
     if (bits == 8) {
-        attention_prefill_kernel<8><<<grid, THREADS, 0, stream>>>(a);
+        attention_prefill_kernel<8><<<grid, THREADS, LDS, stream>>>(a);
     } else if (bits == 4) {
-        attention_prefill_kernel<4><<<grid, THREADS, 0, stream>>>(a);
+        attention_prefill_kernel<4><<<grid, THREADS, LDS, stream>>>(a);
     } else {
-        attention_prefill_kernel<16><<<grid, THREADS, 0, stream>>>(a);
+        attention_prefill_kernel<16><<<grid, THREADS, LDS, stream>>>(a);
     }
     return launch_status(what);
 }
