@@ -192,15 +192,25 @@ int saetta_attn_rows_quant(saetta_stream_t stream, int bits, const float *q,
 
 /* ---- prefill attention (src/attention_prefill.rs, src/prefill.rs) ---------- */
 
+/* Bytes of workspace a prefill chunk at (pos, tokens) needs: the f16 key and
+ * value tile images of the pos + tokens rows the chunk can see.  The reference
+ * has no counterpart (its kernels dequantize in place); the closest is the
+ * half scratch of Prefill::new (src/prefill.rs:1674-1686). */
+size_t saetta_prefill_workspace_bytes(uint32_t pos, uint32_t tokens, uint32_t kv_heads);
+
 /* attention_prefill::encode (src/attention_prefill.rs:39-72): a causal chunk
  * over a half cache that already holds the chunk's rows.  q f16
  * [tokens][heads][256]; keys, values f16 [capacity][kv_heads][256] from
  * position 0, capacity >= pos + tokens; q_and_gate f32 [tokens][heads][512];
- * out f32 [tokens][heads][256].  Kernel replaced: attention_fa{4,8}
- * (kernels/attention_prefill.metal:38-169). */
+ * out f32 [tokens][heads][256].  workspace: device memory of at least
+ * saetta_prefill_workspace_bytes(pos, tokens, kv_heads) bytes, 16-byte
+ * aligned, overwritten by the call; NULL makes the library use one of its own
+ * per device, which it grows with hipMalloc when needed (so not under stream
+ * capture, and not from two streams at once).  Kernel replaced:
+ * attention_fa{4,8} (kernels/attention_prefill.metal:38-169). */
 int saetta_attn_prefill(saetta_stream_t stream, const uint16_t *q_f16, const uint16_t *keys,
                         const uint16_t *values, const float *q_and_gate, float *out,
-                        saetta_flash_params p);
+                        saetta_flash_params p, void *workspace, size_t workspace_bytes);
 
 /* The same chunk over an 8- or 4-bit cache read in place
  * (src/prefill.rs:1674-1686,1735-1776); the cache is seen through half, as
@@ -209,7 +219,8 @@ int saetta_attn_prefill(saetta_stream_t stream, const uint16_t *q_f16, const uin
  * (kernels/attention_rows_q.metal:55-344). */
 int saetta_attn_prefill_quant(saetta_stream_t stream, int bits, const uint16_t *q_f16,
                               saetta_quant_rows keys, saetta_quant_rows values,
-                              const float *q_and_gate, float *out, saetta_flash_params p);
+                              const float *q_and_gate, float *out, saetta_flash_params p,
+                              void *workspace, size_t workspace_bytes);
 
 #ifdef __cplusplus
 }

@@ -11,25 +11,36 @@
 // cache is seen "through half": every value is f16(f32(s)*code + f32(z)),
 // exactly what round_trip_as_half (src/kv_quant.rs:119-125) gives the CPU path.
 //
-// Work split: workgroup (token tile of 32, kv head), 8 waves; wave w owns 4
-// tokens x 8 heads = 32 query rows, one 32-row MFMA tile.  Keys are walked
-// in blocks of 32.  Per block the workgroup stages K[32][256] and the
-// transposed V^T[256][32] as f16 in LDS (dequantizing on the way), then every
-// wave computes with v_mfma_f32_32x32x16_f16
+// Two kernels.
+//
+// prefill_prepare_kernel<16|8|4> turns the keys and values the chunk can see into
+// f16 tile images in a workspace, one image per (kv head, block of 32 keys): the K tile
+// [32 keys][256 dims] and the transposed V^T tile [256 dims][32 keys], laid out byte for
+// byte as the attention kernel wants them in LDS (padded rows, V^T keys in the order the
+// MFMA accumulator hands them out).  The dequantization happens here, once per key, with
+// exactly the arithmetic of round_trip_as_half, instead of once per workgroup that walks
+// the key; it costs one pass over the cache (a few microseconds).
+//
+// attention_prefill_kernel: workgroup (token tile of 16, kv head), 4 waves (one per SIMD);
+// wave w owns 4 tokens x 8 heads = 32 query rows, one 32-row MFMA tile.  Keys are walked in
+// blocks of 32 whose images are copied global -> LDS by global_load_lds_dwordx4 (no vector
+// registers, no vector ALU) into three rotating buffers, two blocks ahead.  Every wave
+// computes with v_mfma_f32_32x32x16_f16
 //     S^T = K Q^T      (A = K rows from LDS, B = Q^T held in registers)
 //     O^T += V^T P^T   (A = V^T rows from LDS, B = P^T from the S^T registers)
-// Both products are transposed so that a lane always owns one query row: in
-// the 32x32 accumulator layout a lane holds column l % 32, so the row's
-// running max and sum, the rescale of O and the final 1/l and gate are plain
-// per-lane values and the softmax needs one cross-lane exchange per block.
-// The accumulators (128 floats per lane) live in AGPRs; two waves share a
-// SIMD, so one's staging and softmax overlap the other's MFMAs; the tiles are
-// double-buffered (one barrier per block) and issued heaviest first.
-// The running max is only raised when a block exceeds it by more than 2^8
-// (the usual lazy rescale), so O is rarely rescaled.
-// The next block's codes are fetched into registers while the current block
-// is computed.
+// Both products are transposed so that a lane always owns one query row: in the 32x32
+// accumulator layout a lane holds column l % 32, so the row's running max and sum, the
+// rescale of O and the final 1/l and gate are plain per-lane values and the softmax needs one
+// cross-lane exchange per block.  The loop is software-pipelined inside each wave, because
+// MFMA and vector instructions of one wave run side by side when they are independent:
+//   stage A   MFMA: S^T of block kb+1      |  VALU: exp / sum / pack of block kb
+//   stage B   MFMA: O^T += V^T P^T (kb)    |  VALU: scale and row max of block kb+1
+// with one barrier per block.  The running max is only raised when a block exceeds it by
+// more than 2^8 (lazy rescale), so O is rarely rescaled.  Tiles are issued heaviest first and
+// there are two per CU, which evens out the causal imbalance.
 #include "common.hpp"
+
+#include <mutex>
 
 namespace saetta {
 namespace {
@@ -42,28 +53,41 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int DIM = SAETTA_HEAD_DIM;
-constexpr int THREADS = 512;
-constexpr int NT = 1;                   // 32-row MFMA tiles per wave (4 tokens x 8 heads each)
-constexpr int WAVES = THREADS / 64;
-constexpr int TQ = 4 * NT * WAVES;      // tokens per workgroup
+constexpr int PREP_THREADS = 256;       // the prepare kernel's workgroup
+constexpr int WAVES = 8;                // two per SIMD: one's softmax runs under the other's MFMAs
+constexpr int THREADS = 64 * WAVES;
+constexpr int TQ = 4 * WAVES;           // tokens per workgroup: a wave owns 4 tokens x 8 heads = 32 rows
 constexpr int BK = 32;                  // keys per block
 constexpr int K_STRIDE = DIM * 2 + 16;  // bytes per key row of the K tile (padded against bank conflicts)
 constexpr int V_STRIDE = BK * 2 + 16;   // bytes per dim row of the V^T tile
 constexpr int K_BYTES = BK * K_STRIDE;
-constexpr int V_BYTES = DIM * V_STRIDE;
+// Row of dim d in the V^T tile.  The stager writes dims 4i..4i+3 from lane i, the MFMA reads
+// 32 consecutive dims from 32 lanes; with rows ordered (d % 4, d / 4) and two spare rows per
+// plane both patterns spread over the LDS banks.
+constexpr int V_PLANE = DIM / 4 + 2;
+__device__ __forceinline__ constexpr int vt_row(int dim) { return (dim & 3) * V_PLANE + (dim >> 2); }
+constexpr int V_BYTES = 4 * V_PLANE * V_STRIDE;
+constexpr int IMG_BYTES = (K_BYTES + V_BYTES + 1023) / 1024 * 1024;  // one block's image, whole KB
 constexpr float NO_SCORE = -1e30f;
 constexpr float TAU = 8.0f;  // the reference max is raised only past this many powers of two
 
-struct PrefillArgs {
-    const uint16_t *q;  // f16 [tokens][heads][256]
+struct PrepareArgs {
     const void *kdata;
     const void *vdata;
     const uint16_t *kscales, *kbiases, *vscales, *vbiases;
+    unsigned char *images;  // [kv head][block][IMG_BYTES]
+    uint32_t kv_heads, nblocks;
+    uint32_t key_limit;  // pos + tokens: rows the cache holds; keys from here on are zeros
+};
+
+struct PrefillArgs {
+    const uint16_t *q;  // f16 [tokens][heads][256]
+    const unsigned char *images;
     const float *q_and_gate;
     float *out;
     uint32_t heads, kv_heads, pos, tokens;
     float scale;
-    uint32_t capacity;  // rows the cache arrays hold (bound of the buffer loads)
+    uint32_t nblocks;  // images per kv head
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
@@ -91,64 +115,67 @@ __device__ __forceinline__ uint32_t code_of(uint32_t w, int i) {
 }
 
 // ---- staging registers: what one thread fetches for one key block ----------------
-// K: thread (key = t / 16, piece = t % 16) takes 16 dims of one key.
-// V: thread (dq = t % 64, kq = t / 64) takes 4 dims of 4 keys.
+// K: thread (key = t / 8, piece = t % 8) takes 32 dims of one key.
+// V: thread (dq = t % 64, kq = t / 64) takes 4 dims of 8 keys.
 template <int BITS>
 struct Stage {
-    uint32_t k[BITS == 16 ? 8 : BITS / 2];  // 16 dims: 32 B (f16), 16 B (8-bit), 8 B (4-bit)
-    uint32_t v[4][BITS == 16 ? 2 : 1];      // per key 4 dims: 8 B (f16), 4 B (8-bit), 2 B (4-bit)
+    uint32_t k[BITS == 16 ? 16 : BITS];     // 32 dims: 64 B (f16), 32 B (8-bit), 16 B (4-bit)
+    uint32_t v[8][BITS == 16 ? 2 : 1];      // per key 4 dims: 8 B (f16), 4 B (8-bit), 2 B (4-bit)
     uint32_t ks, kz;                        // f16 scale and bias of (key, group of the piece)
-    uint32_t vs[4], vz[4];                  // per key, group of dq
+    uint32_t vs[8], vz[8];                  // per key, group of dq
+};
+
+struct Rsrc {
+    __amdgpu_buffer_rsrc_t k, v, ks, kz, vs, vz;
 };
 
 template <int BITS>
-__device__ __forceinline__ void stage_load(Stage<BITS> &st, const PrefillArgs &a, __amdgpu_buffer_rsrc_t k_rsrc,
-                                           __amdgpu_buffer_rsrc_t v_rsrc, __amdgpu_buffer_rsrc_t ks_rsrc,
-                                           __amdgpu_buffer_rsrc_t kz_rsrc, __amdgpu_buffer_rsrc_t vs_rsrc,
-                                           __amdgpu_buffer_rsrc_t vz_rsrc, uint32_t key0, uint32_t kv, int tid) {
+__device__ __forceinline__ void stage_load(Stage<BITS> &st, const Rsrc &r, uint32_t kvh, uint32_t key0, uint32_t kv,
+                                           int tid) {
     constexpr int RB = row_bytes<BITS>();
-    const uint32_t kvh = a.kv_heads;
     {
-        const int key = tid >> 4, piece = tid & 15;
+        const int key = tid >> 3, piece = tid & 7;
         const int row = int((key0 + key) * kvh + kv);
-        const int off = row * RB + piece * (RB / 16);
+        const int off = row * RB + piece * (RB / 8);
         if constexpr (BITS == 8) {
-            const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, off, 0, 0);
+            const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(r.k, off, 0, 0);
+            const u32x4 y = __builtin_amdgcn_raw_buffer_load_b128(r.k, off + 16, 0, 0);
             st.k[0] = x.x, st.k[1] = x.y, st.k[2] = x.z, st.k[3] = x.w;
+            st.k[4] = y.x, st.k[5] = y.y, st.k[6] = y.z, st.k[7] = y.w;
         } else if constexpr (BITS == 4) {
-            const u32x2 x = __builtin_amdgcn_raw_buffer_load_b64(k_rsrc, off, 0, 0);
-            st.k[0] = x.x, st.k[1] = x.y;
+            const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(r.k, off, 0, 0);
+            st.k[0] = x.x, st.k[1] = x.y, st.k[2] = x.z, st.k[3] = x.w;
         } else {
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, off + 16 * i, 0, 0);
+            for (int i = 0; i < 4; i++) {
+                const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(r.k, off + 16 * i, 0, 0);
                 st.k[4 * i] = x.x, st.k[4 * i + 1] = x.y, st.k[4 * i + 2] = x.z, st.k[4 * i + 3] = x.w;
             }
         }
         if constexpr (BITS != 16) {
-            const int soff = (row * 4 + (piece >> 2)) * 2;
-            st.ks = __builtin_amdgcn_raw_buffer_load_b16(ks_rsrc, soff, 0, 0);
-            st.kz = __builtin_amdgcn_raw_buffer_load_b16(kz_rsrc, soff, 0, 0);
+            const int soff = (row * 4 + (piece >> 1)) * 2;
+            st.ks = __builtin_amdgcn_raw_buffer_load_b16(r.ks, soff, 0, 0);
+            st.kz = __builtin_amdgcn_raw_buffer_load_b16(r.kz, soff, 0, 0);
         }
     }
     {
         const int dq = tid & 63, kq = tid >> 6;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int row = int((key0 + 4 * kq + i) * kvh + kv);
+        for (int i = 0; i < 8; i++) {
+            const int row = int((key0 + 8 * kq + i) * kvh + kv);
             const int off = row * RB + dq * (RB / 64);
             if constexpr (BITS == 8) {
-                st.v[i][0] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, off, 0, 0);
+                st.v[i][0] = __builtin_amdgcn_raw_buffer_load_b32(r.v, off, 0, 0);
             } else if constexpr (BITS == 4) {
-                st.v[i][0] = uint16_t(__builtin_amdgcn_raw_buffer_load_b16(v_rsrc, off, 0, 0));
+                st.v[i][0] = uint16_t(__builtin_amdgcn_raw_buffer_load_b16(r.v, off, 0, 0));
             } else {
-                const u32x2 x = __builtin_amdgcn_raw_buffer_load_b64(v_rsrc, off, 0, 0);
+                const u32x2 x = __builtin_amdgcn_raw_buffer_load_b64(r.v, off, 0, 0);
                 st.v[i][0] = x.x, st.v[i][1] = x.y;
             }
             if constexpr (BITS != 16) {
                 const int soff = (row * 4 + (dq >> 4)) * 2;
-                st.vs[i] = __builtin_amdgcn_raw_buffer_load_b16(vs_rsrc, soff, 0, 0);
-                st.vz[i] = __builtin_amdgcn_raw_buffer_load_b16(vz_rsrc, soff, 0, 0);
+                st.vs[i] = __builtin_amdgcn_raw_buffer_load_b16(r.vs, soff, 0, 0);
+                st.vz[i] = __builtin_amdgcn_raw_buffer_load_b16(r.vz, soff, 0, 0);
             }
         }
     }
@@ -172,16 +199,16 @@ template <int BITS>
 __device__ __forceinline__ void stage_store(const Stage<BITS> &st, unsigned char *k_lds, unsigned char *v_lds,
                                             uint32_t key0, uint32_t key_limit, int tid) {
     {
-        const int key = tid >> 4, piece = tid & 15;
-        uint32_t o[8];
+        const int key = tid >> 3, piece = tid & 7;
+        uint32_t o[16];
         if constexpr (BITS == 16) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) o[i] = st.k[i];
+            for (int i = 0; i < 16; i++) o[i] = st.k[i];
         } else {
             const float s = h2f(st.ks), z = h2f(st.kz);
             constexpr int PER = 32 / BITS;
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
+            for (int i = 0; i < 16; i++) {
                 const uint32_t w = st.k[(2 * i) / PER];
                 o[i] = pack_half2(dequant(s, z, code_of<BITS>(w, (2 * i) % PER)),
                                   dequant(s, z, code_of<BITS>(w, (2 * i + 1) % PER)));
@@ -189,209 +216,222 @@ __device__ __forceinline__ void stage_store(const Stage<BITS> &st, unsigned char
         }
         if (key0 + key >= key_limit) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) o[i] = 0;
+            for (int i = 0; i < 16; i++) o[i] = 0;
         }
-        u32x4 *dst = reinterpret_cast<u32x4 *>(k_lds + key * K_STRIDE + piece * 32);
-        dst[0] = u32x4{o[0], o[1], o[2], o[3]};
-        dst[1] = u32x4{o[4], o[5], o[6], o[7]};
+        u32x4 *dst = reinterpret_cast<u32x4 *>(k_lds + key * K_STRIDE + piece * 64);
+#pragma unroll
+        for (int i = 0; i < 4; i++) dst[i] = u32x4{o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
     }
     {
         const int dq = tid & 63, kq = tid >> 6;
-        float x[4][4];
+        // keys 8kq..8kq+7: two runs of 4 neighbours in the row's key order
+        const int p0 = vt_pos(8 * kq), p1 = vt_pos(8 * kq + 4);
+        uint32_t w[4][4];  // [dim][pair of keys]
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const bool live = key0 + 4 * kq + i < key_limit;
-            if constexpr (BITS == 16) {
+        for (int i = 0; i < 8; i += 2) {
+            float x[2][4];
 #pragma unroll
-                for (int d = 0; d < 4; d++) x[i][d] = live ? h2f(st.v[i][d >> 1] >> (16 * (d & 1))) : 0.0f;
-            } else {
-                const float s = h2f(st.vs[i]), z = h2f(st.vz[i]);
+            for (int u = 0; u < 2; u++) {
+                const bool live = key0 + 8 * kq + i + u < key_limit;
+                if constexpr (BITS == 16) {
 #pragma unroll
-                for (int d = 0; d < 4; d++) x[i][d] = live ? dequant(s, z, code_of<BITS>(st.v[i][0], d)) : 0.0f;
+                    for (int d = 0; d < 4; d++) x[u][d] = live ? h2f(st.v[i + u][d >> 1] >> (16 * (d & 1))) : 0.0f;
+                } else {
+                    const float s = h2f(st.vs[i + u]), z = h2f(st.vz[i + u]);
+#pragma unroll
+                    for (int d = 0; d < 4; d++) x[u][d] = live ? dequant(s, z, code_of<BITS>(st.v[i + u][0], d)) : 0.0f;
+                }
             }
+#pragma unroll
+            for (int d = 0; d < 4; d++) w[d][i / 2] = pack_half2(x[0][d], x[1][d]);
         }
-        // keys 4kq..4kq+3 are neighbours in the row's key order
-        const int p0 = vt_pos(4 * kq);
 #pragma unroll
         for (int d = 0; d < 4; d++) {
-            u32x2 w = {pack_half2(x[0][d], x[1][d]), pack_half2(x[2][d], x[3][d])};
-            *reinterpret_cast<u32x2 *>(v_lds + (4 * dq + d) * V_STRIDE + 2 * p0) = w;
+            unsigned char *row = v_lds + (d * V_PLANE + dq) * V_STRIDE;
+            *reinterpret_cast<u32x2 *>(row + 2 * p0) = u32x2{w[d][0], w[d][1]};
+            *reinterpret_cast<u32x2 *>(row + 2 * p1) = u32x2{w[d][2], w[d][3]};
         }
     }
 }
 
 template <int BITS>
-__global__ __launch_bounds__(THREADS) void attention_prefill_kernel(PrefillArgs a) {
+__global__ __launch_bounds__(PREP_THREADS) void prefill_prepare_kernel(PrepareArgs a) {
     constexpr int RB = row_bytes<BITS>();
-    // two buffers of (K tile, V^T tile): block kb lives in buffer kb & 1
-    extern __shared__ __attribute__((aligned(16))) unsigned char tiles[];
+    const uint32_t block = blockIdx.x, kv = blockIdx.y, kvh = a.kv_heads;
+    const uint32_t cap_rows = a.key_limit * kvh;
+    Rsrc rs;
+    rs.k = make_rsrc(a.kdata, cap_rows * RB);
+    rs.v = make_rsrc(a.vdata, cap_rows * RB);
+    rs.ks = make_rsrc(a.kscales, BITS == 16 ? 0 : cap_rows * 8);
+    rs.kz = make_rsrc(a.kbiases, BITS == 16 ? 0 : cap_rows * 8);
+    rs.vs = make_rsrc(a.vscales, BITS == 16 ? 0 : cap_rows * 8);
+    rs.vz = make_rsrc(a.vbiases, BITS == 16 ? 0 : cap_rows * 8);
+    Stage<BITS> st;
+    stage_load<BITS>(st, rs, kvh, block * BK, kv, threadIdx.x);
+    unsigned char *img = a.images + (size_t(kv) * a.nblocks + block) * IMG_BYTES;
+    stage_store<BITS>(st, img, img + K_BYTES, block * BK, a.key_limit, threadIdx.x);
+}
+
+constexpr int NBUF = 3;
+constexpr int LDS_BYTES = NBUF * IMG_BYTES;
+
+__global__ __launch_bounds__(THREADS) void attention_prefill_kernel(PrefillArgs a) {
+    // the image of block b lives in buffer b % 3
+    extern __shared__ __attribute__((aligned(1024))) unsigned char tiles[];
+    auto k_buf = [&](uint32_t b) { return tiles + (b % NBUF) * IMG_BYTES; };
+    auto v_buf = [&](uint32_t b) { return tiles + (b % NBUF) * IMG_BYTES + K_BYTES; };
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, hf = lane >> 5;
     const uint32_t kv = blockIdx.y;
     const uint32_t ntiles = (a.tokens + TQ - 1) / TQ;
     const uint32_t tile = ntiles - 1 - blockIdx.x;  // the tiles with the most keys start first
-    const uint32_t tok0 = tile * TQ + 4 * NT * wave;  // this wave's first token
-    const float c = a.scale * 1.4426950408889634f;   // scores are kept in units of log2(e)
+    const uint32_t tok0 = tile * TQ + 4 * wave;     // this wave's first token
+    const float c = a.scale * 1.4426950408889634f;  // scores are kept in units of log2(e)
 
-    // Row of this lane in row tile nt: token tok0 + 4nt + col / 8, head col % 8.
-    uint32_t tok[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) tok[nt] = tok0 + 4 * nt + (col >> 3);
+    // Row of this lane: token tok0 + col / 8, head col % 8.
+    const uint32_t tok = tok0 + (col >> 3);
     const uint32_t head = kv * 8 + (col & 7);
 
+    // Keys this workgroup walks: up to what its last token sees; what this wave needs.
+    const uint32_t wg_keys = a.pos + min(tile * TQ + TQ, a.tokens);
+    const uint32_t nblocks = (wg_keys + BK - 1) / BK;
+    const uint32_t wave_first_len = a.pos + tok0 + 1;            // keys the wave's first token sees
+    const uint32_t wave_keys = a.pos + min(tok0 + 4, a.tokens);  // keys its last token sees
+    const uint32_t wave_blocks = tok0 < a.tokens ? min((wave_keys + BK - 1) / BK, nblocks) : 0;
+    const uint32_t full_blocks = min(wave_first_len / BK, wave_blocks);  // blocks that need no mask
+
+    // Copies the image of block b into its LDS buffer: every lane moves 16 bytes per
+    // instruction, a wave 1 KB, straight from global memory to LDS.
+    const unsigned char *images = a.images + size_t(kv) * a.nblocks * IMG_BYTES;
+    auto copy_block = [&](uint32_t b) {
+        const unsigned char *src = images + size_t(b) * IMG_BYTES + lane * 16;
+        unsigned char *dst = tiles + (b % NBUF) * IMG_BYTES;
+        for (int i = wave; i < IMG_BYTES / 1024; i += WAVES) {
+            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(src + i * 1024),
+                                             (void __attribute__((address_space(3))) *)(dst + i * 1024), 16, 0, 0);
+        }
+    };
+    copy_block(0);
+    if (nblocks > 1) copy_block(1);
+
     // Q^T operands: lane (col, hf), k-step st: dims 16 st + 8 hf .. + 7 of its row.
-    half8 qb[NT][16];
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
-        const uint32_t tk = min(tok[nt], a.tokens - 1);
+    half8 qb[16];
+    {
+        const uint32_t tk = min(tok, a.tokens - 1);
         const u32x4 *src = reinterpret_cast<const u32x4 *>(a.q + (size_t(tk) * a.heads + head) * DIM + 8 * hf);
 #pragma unroll
-        for (int st = 0; st < 16; st++) qb[nt][st] = __builtin_bit_cast(half8, src[2 * st]);
+        for (int st = 0; st < 16; st++) qb[st] = __builtin_bit_cast(half8, src[2 * st]);
     }
 
-    const uint32_t cap_rows = a.capacity * a.kv_heads;
-    const __amdgpu_buffer_rsrc_t k_rsrc = make_rsrc(a.kdata, cap_rows * RB);
-    const __amdgpu_buffer_rsrc_t v_rsrc = make_rsrc(a.vdata, cap_rows * RB);
-    const __amdgpu_buffer_rsrc_t ks_rsrc = make_rsrc(a.kscales, BITS == 16 ? 0 : cap_rows * 8);
-    const __amdgpu_buffer_rsrc_t kz_rsrc = make_rsrc(a.kbiases, BITS == 16 ? 0 : cap_rows * 8);
-    const __amdgpu_buffer_rsrc_t vs_rsrc = make_rsrc(a.vscales, BITS == 16 ? 0 : cap_rows * 8);
-    const __amdgpu_buffer_rsrc_t vz_rsrc = make_rsrc(a.vbiases, BITS == 16 ? 0 : cap_rows * 8);
-
-    // Keys this workgroup walks: up to what its last token sees; what this wave needs.
-    const uint32_t key_limit = a.pos + a.tokens;  // end of the chunk: nothing past it is ever visible
-    const uint32_t wg_keys = min(a.pos + min(tile * TQ + TQ, a.tokens), key_limit);
-    const uint32_t nblocks = (wg_keys + BK - 1) / BK;
-    const uint32_t wave_first_len = a.pos + tok0 + 1;                          // keys the wave's first token sees
-    const uint32_t wave_keys = a.pos + min(tok0 + 4 * NT, a.tokens);                 // keys its last token sees
-
-    floatx16 acc[8][NT];
+    floatx16 acc[8];
 #pragma unroll
     for (int mt = 0; mt < 8; mt++) {
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[mt][nt][r] = 0.0f;
-        }
+        for (int r = 0; r < 16; r++) acc[mt][r] = 0.0f;
     }
-    float m_ref[NT], l_sum[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) m_ref[nt] = NO_SCORE, l_sum[nt] = 0.0f;
+    float m_ref = NO_SCORE, l_sum = 0.0f;
 
-    Stage<BITS> st;
-    stage_load<BITS>(st, a, k_rsrc, v_rsrc, ks_rsrc, kz_rsrc, vs_rsrc, vz_rsrc, 0, kv, tid);
-    stage_store<BITS>(st, tiles, tiles + K_BYTES, 0, key_limit, tid);
-    if (nblocks > 1) stage_load<BITS>(st, a, k_rsrc, v_rsrc, ks_rsrc, kz_rsrc, vs_rsrc, vz_rsrc, BK, kv, tid);
-    __syncthreads();
-
-    for (uint32_t kb = 0; kb < nblocks; kb++) {
-        const uint32_t key0 = kb * BK;
-        const unsigned char *k_lds = tiles + (kb & 1) * (K_BYTES + V_BYTES);
-        const unsigned char *v_lds = k_lds + K_BYTES;
-        // Block kb + 1 goes into the other buffer (every wave left it at the barrier below),
-        // block kb + 2 into the registers.
-        if (kb + 1 < nblocks) {
-            unsigned char *nk = tiles + ((kb + 1) & 1) * (K_BYTES + V_BYTES);
-            stage_store<BITS>(st, nk, nk + K_BYTES, key0 + BK, key_limit, tid);
-            if (kb + 2 < nblocks) {
-                stage_load<BITS>(st, a, k_rsrc, v_rsrc, ks_rsrc, kz_rsrc, vs_rsrc, vz_rsrc, key0 + 2 * BK, kv, tid);
-            }
-        }
-        if (key0 >= wave_keys) {  // nothing in this block is visible to this wave (uniform)
-            __syncthreads();
-            continue;
-        }
-  // nothing in this block is visible to this wave (uniform)
-
-        // ---- S^T = K Q^T: rows = the block's 32 keys, columns = query rows ----------
-        floatx16 s[NT];
+    // S^T = K Q^T of one block: rows = the block's 32 keys, columns = query rows.
+    auto scores = [&](uint32_t b) {
+        const unsigned char *k_lds = k_buf(b);
+        floatx16 s;
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) s[nt][r] = 0.0f;
-        }
+        for (int r = 0; r < 16; r++) s[r] = 0.0f;
 #pragma unroll
         for (int stp = 0; stp < 16; stp++) {
             const half8 ka = *reinterpret_cast<const half8 *>(k_lds + col * K_STRIDE + (16 * stp + 8 * hf) * 2);
-#pragma unroll
-            for (int nt = 0; nt < NT; nt++) s[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qb[nt][stp], s[nt], 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qb[stp], s, 0, 0, 0);
         }
-
-        // ---- online softmax, one row per lane ---------------------------------------
-        // Register r of the accumulator is key 4 hf + r % 4 + 8 (r / 4) of the block.
-        const bool diagonal = key0 + BK > wave_first_len;  // some key of the block is hidden from some row
-        half8 pb[NT][2];
-#pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
-            float v[16];
-            float bm = NO_SCORE;
-            if (diagonal) {
-                const uint32_t vis = a.pos + tok[nt] + 1 - min(key0, a.pos + tok[nt] + 1);  // visible keys of the block
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const uint32_t key = 4 * hf + (r & 3) + 8 * (r >> 2);
-                    v[r] = key < vis ? s[nt][r] * c : NO_SCORE;
-                    bm = fmaxf(bm, v[r]);
-                }
-            } else {
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    v[r] = s[nt][r] * c;
-                    bm = fmaxf(bm, v[r]);
-                }
-            }
-            bm = fmaxf(bm, __shfl_xor(bm, 32));
-            if (__any(bm > m_ref[nt] + TAU)) {
-                const float m_new = bm > m_ref[nt] + TAU ? bm : m_ref[nt];
-                const float alpha = __builtin_amdgcn_exp2f(m_ref[nt] - m_new);
-                m_ref[nt] = m_new;
-                l_sum[nt] *= alpha;
-#pragma unroll
-                for (int mt = 0; mt < 8; mt++) {
-#pragma unroll
-                    for (int r = 0; r < 16; r++) acc[mt][nt][r] *= alpha;
-                }
-            }
-            float sum = 0.0f;
+        return s;
+    };
+    // Row maximum of a block's scaled scores (first half of the softmax).  Register r of the
+    // accumulator is key 4 hf + r % 4 + 8 (r / 4) of the block; masked scores become NO_SCORE / c.
+    auto mask_max = [&](floatx16 &s, uint32_t key0, bool masked) {
+        float bm = NO_SCORE;
+        if (masked) {
+            const uint32_t len = a.pos + tok + 1;              // keys this row sees
+            const uint32_t vis = len > key0 ? len - key0 : 0;  // of which in this block
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                v[r] = __builtin_amdgcn_exp2f(v[r] - m_ref[nt]);
-                sum += v[r];
-            }
-            l_sum[nt] += sum;
-            // P^T operands: k-step sp takes registers 8 sp .. 8 sp + 7 (the order vt_pos mirrors)
-#pragma unroll
-            for (int sp = 0; sp < 2; sp++) {
-                u32x4 w = {pack_half2(v[8 * sp], v[8 * sp + 1]), pack_half2(v[8 * sp + 2], v[8 * sp + 3]),
-                           pack_half2(v[8 * sp + 4], v[8 * sp + 5]), pack_half2(v[8 * sp + 6], v[8 * sp + 7])};
-                pb[nt][sp] = __builtin_bit_cast(half8, w);
+                const uint32_t key = 4 * hf + (r & 3) + 8 * (r >> 2);
+                s[r] = key < vis ? s[r] : NO_SCORE;
             }
         }
-
-        // ---- O^T += V^T P^T: rows = dims, columns = query rows ------------------------
+#pragma unroll
+        for (int r = 0; r < 16; r++) bm = fmaxf(bm, s[r]);
+        bm = fmaxf(bm, __shfl_xor(bm, 32));
+        return fmaxf(bm * c, NO_SCORE);
+    };
+    // Raises the reference maximum when a block tops it by more than 2^TAU, rescaling O and l.
+    auto raise_max = [&](float bm) {
+        if (__any(bm > m_ref + TAU)) {
+            const float m_new = bm > m_ref + TAU ? bm : m_ref;
+            const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
+            m_ref = m_new;
+            l_sum *= alpha;
+#pragma unroll
+            for (int mt = 0; mt < 8; mt++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[mt][r] *= alpha;
+            }
+        }
+    };
+    // Second half of the softmax: probabilities 2^(s c - m), their sum, and the P^T operands
+    // (k-step sp takes registers 8 sp .. 8 sp + 7, the order vt_pos mirrors).
+    auto exp_pack = [&](const floatx16 &s, half8 (&pb)[2]) {
+        float p[16];
+        float sum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c, -m_ref));
+            sum += p[r];
+        }
+        l_sum += sum;
+#pragma unroll
+        for (int sp = 0; sp < 2; sp++) {
+            u32x4 w = {pack_half2(p[8 * sp], p[8 * sp + 1]), pack_half2(p[8 * sp + 2], p[8 * sp + 3]),
+                       pack_half2(p[8 * sp + 4], p[8 * sp + 5]), pack_half2(p[8 * sp + 6], p[8 * sp + 7])};
+            pb[sp] = __builtin_bit_cast(half8, w);
+        }
+    };
+    // O^T += V^T P^T: rows = dims, columns = query rows.
+    auto accumulate = [&](uint32_t b, const half8 (&pb)[2]) {
+        const unsigned char *v_lds = v_buf(b);
 #pragma unroll
         for (int mt = 0; mt < 8; mt++) {
 #pragma unroll
             for (int sp = 0; sp < 2; sp++) {
                 const half8 va =
-                    *reinterpret_cast<const half8 *>(v_lds + (32 * mt + col) * V_STRIDE + (16 * sp + 8 * hf) * 2);
-#pragma unroll
-                for (int nt = 0; nt < NT; nt++) {
-                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, pb[nt][sp], acc[mt][nt], 0, 0, 0);
-                }
+                    *reinterpret_cast<const half8 *>(v_lds + vt_row(32 * mt + col) * V_STRIDE + (16 * sp + 8 * hf) * 2);
+                acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, pb[sp], acc[mt], 0, 0, 0);
             }
         }
+    };
+
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // blocks 0 and 1 are in LDS
+
+    for (uint32_t kb = 0; kb < nblocks; kb++) {
+        // Block kb + 2 goes where block kb - 1 was (every wave left it at the last barrier).
+        if (kb + 2 < nblocks) copy_block(kb + 2);
+        if (kb < wave_blocks) {
+            floatx16 s = scores(kb);
+            raise_max(mask_max(s, kb * BK, kb >= full_blocks));
+            half8 pb[2];
+            exp_pack(s, pb);
+            accumulate(kb, pb);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
 
     // ---- out = O / l * sigmoid(gate) ---------------------------------------------------
     // The lane's row sum is split over the two lane halves (each saw half the keys).
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
-        const float l = l_sum[nt] + __shfl_xor(l_sum[nt], 32);
-        if (tok[nt] >= a.tokens) continue;
+    const float l = l_sum + __shfl_xor(l_sum, 32);
+    if (tok < a.tokens) {
         const float inv = 1.0f / l;
-        const size_t row = size_t(tok[nt]) * a.heads + head;
+        const size_t row = size_t(tok) * a.heads + head;
         const float *gate = a.q_and_gate + row * 2 * DIM + DIM;
         float *out = a.out + row * DIM;
 #pragma unroll
@@ -401,53 +441,91 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(PrefillArgs 
                 const int d0 = 32 * mt + 8 * q4 + 4 * hf;
                 const float4 g = *reinterpret_cast<const float4 *>(gate + d0);
                 float4 o;
-                o.x = acc[mt][nt][4 * q4 + 0] * inv / (1.0f + __expf(-g.x));
-                o.y = acc[mt][nt][4 * q4 + 1] * inv / (1.0f + __expf(-g.y));
-                o.z = acc[mt][nt][4 * q4 + 2] * inv / (1.0f + __expf(-g.z));
-                o.w = acc[mt][nt][4 * q4 + 3] * inv / (1.0f + __expf(-g.w));
+                o.x = acc[mt][4 * q4 + 0] * inv / (1.0f + __expf(-g.x));
+                o.y = acc[mt][4 * q4 + 1] * inv / (1.0f + __expf(-g.y));
+                o.z = acc[mt][4 * q4 + 2] * inv / (1.0f + __expf(-g.z));
+                o.w = acc[mt][4 * q4 + 3] * inv / (1.0f + __expf(-g.w));
                 *reinterpret_cast<float4 *>(out + d0) = o;
             }
         }
     }
 }
 
+// Workspace the library owns when the caller passes none: grown on demand, one per device.
+struct OwnedWorkspace {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+};
+OwnedWorkspace g_owned[16];
+std::mutex g_owned_mutex;
+
+size_t workspace_bytes(uint32_t pos, uint32_t tokens, uint32_t kv_heads) {
+    const size_t blocks = (size_t(pos) + tokens + BK - 1) / BK;
+    return blocks * kv_heads * IMG_BYTES;
+}
+
 int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kdata, const void *vdata,
                 const uint16_t *ks, const uint16_t *kz, const uint16_t *vs, const uint16_t *vz,
-                const float *q_and_gate, float *out, saetta_flash_params p, const char *what) {
+                const float *q_and_gate, float *out, saetta_flash_params p, void *workspace, size_t workspace_size,
+                const char *what) {
     SAETTA_REQUIRE(bits == 16 || bits == 8 || bits == 4, SAETTA_E_BITS, "%s: bits %d", what, bits);
     SAETTA_REQUIRE(p.kv_heads > 0 && p.heads == p.kv_heads * SAETTA_GQA_GROUP, SAETTA_E_SHAPE,
                    "%s needs 8 q heads per kv head (heads %u, kv heads %u)", what, p.heads, p.kv_heads);
     SAETTA_REQUIRE(q && kdata && vdata && q_and_gate && out, SAETTA_E_NULL, "%s: null buffer", what);
     SAETTA_REQUIRE(bits == 16 || (ks && kz && vs && vz), SAETTA_E_NULL, "%s: null scales or biases", what);
     SAETTA_REQUIRE(aligned(q, 16) && aligned(kdata, 16) && aligned(vdata, 16) && aligned(q_and_gate, 16) &&
-                       aligned(out, 16),
+                       aligned(out, 16) && aligned(workspace, 16),
                    SAETTA_E_ALIGN, "%s: buffers must be 16-byte aligned", what);
     const uint64_t rows = uint64_t(p.pos) + p.tokens;  // the cache holds the chunk's rows too
     SAETTA_REQUIRE(rows * p.kv_heads * 512 < (uint64_t(1) << 31), SAETTA_E_SHAPE, "%s: pos + tokens %llu out of range",
                    what, (unsigned long long)rows);
     if (int rc = ensure_device()) return rc;
     if (p.tokens == 0) return SAETTA_OK;
-    PrefillArgs a{q, kdata, vdata, ks, kz, vs, vz, q_and_gate, out, p.heads, p.kv_heads, p.pos, p.tokens, p.scale,
-                  uint32_t(rows)};
-    const dim3 grid((p.tokens + TQ - 1) / TQ, p.kv_heads);
-    constexpr int LDS = 2 * (K_BYTES + V_BYTES);
+    const size_t need = workspace_bytes(p.pos, p.tokens, p.kv_heads);
+    if (workspace) {
+        SAETTA_REQUIRE(workspace_size >= need, SAETTA_E_SCRATCH, "%s: workspace of %zu bytes, %zu needed", what,
+                       workspace_size, need);
+    } else {
+        // No workspace given: use (and grow) the library's own.  This allocates, so it cannot be
+        // used under stream capture; work queued on other streams must not share it.
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        std::lock_guard<std::mutex> lock(g_owned_mutex);
+        OwnedWorkspace &w = g_owned[dev & 15];
+        if (w.bytes < need) {
+            if (w.ptr) {
+                (void)hipDeviceSynchronize();
+                (void)hipFree(w.ptr);
+            }
+            w.ptr = nullptr;
+            w.bytes = 0;
+            hipError_t e = hipMalloc(&w.ptr, need);
+            if (e != hipSuccess) return fail(int(e), "%s: workspace of %zu bytes: %s", what, need, hipGetErrorString(e));
+            w.bytes = need;
+        }
+        workspace = w.ptr;
+    }
+    const uint32_t nblocks = uint32_t((rows + BK - 1) / BK);
+    PrepareArgs pa{kdata, vdata, ks, kz, vs, vz, static_cast<unsigned char *>(workspace), p.kv_heads, nblocks,
+                   uint32_t(rows)};
+    const dim3 pgrid(nblocks, p.kv_heads);
+    if (bits == 8) {
+        prefill_prepare_kernel<8><<<pgrid, PREP_THREADS, 0, stream>>>(pa);
+    } else if (bits == 4) {
+        prefill_prepare_kernel<4><<<pgrid, PREP_THREADS, 0, stream>>>(pa);
+    } else {
+        prefill_prepare_kernel<16><<<pgrid, PREP_THREADS, 0, stream>>>(pa);
+    }
+    PrefillArgs a{q, static_cast<const unsigned char *>(workspace), q_and_gate, out, p.heads, p.kv_heads, p.pos,
+                  p.tokens, p.scale, nblocks};
     static bool attr_set = false;
     if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(attention_prefill_kernel<8>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(attention_prefill_kernel<4>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(attention_prefill_kernel<16>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(attention_prefill_kernel),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
         attr_set = true;
     }
-    if (bits == 8) {
-        attention_prefill_kernel<8><<<grid, THREADS, LDS, stream>>>(a);
-    } else if (bits == 4) {
-        attention_prefill_kernel<4><<<grid, THREADS, LDS, stream>>>(a);
-    } else {
-        attention_prefill_kernel<16><<<grid, THREADS, LDS, stream>>>(a);
-    }
+    const dim3 grid((p.tokens + TQ - 1) / TQ, p.kv_heads);
+    attention_prefill_kernel<<<grid, THREADS, LDS_BYTES, stream>>>(a);
     return launch_status(what);
 }
 
@@ -456,17 +534,23 @@ int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kda
 
 using namespace saetta;
 
+extern "C" size_t saetta_prefill_workspace_bytes(uint32_t pos, uint32_t tokens, uint32_t kv_heads) {
+    return workspace_bytes(pos, tokens, kv_heads);
+}
+
 extern "C" int saetta_attn_prefill(saetta_stream_t stream, const uint16_t *q_f16, const uint16_t *keys,
                                    const uint16_t *values, const float *q_and_gate, float *out,
-                                   saetta_flash_params p) {
+                                   saetta_flash_params p, void *workspace, size_t workspace_bytes) {
     return run_prefill(as_stream(stream), 16, q_f16, keys, values, nullptr, nullptr, nullptr, nullptr, q_and_gate,
-                       out, p, "attn_prefill");
+                       out, p, workspace, workspace_bytes, "attn_prefill");
 }
 
 extern "C" int saetta_attn_prefill_quant(saetta_stream_t stream, int bits, const uint16_t *q_f16,
                                          saetta_quant_rows keys, saetta_quant_rows values,
-                                         const float *q_and_gate, float *out, saetta_flash_params p) {
+                                         const float *q_and_gate, float *out, saetta_flash_params p,
+                                         void *workspace, size_t workspace_bytes) {
     SAETTA_REQUIRE(bits == 8 || bits == 4, SAETTA_E_BITS, "attn_prefill_quant: bits %d (8 or 4)", bits);
     return run_prefill(as_stream(stream), bits, q_f16, keys.data, values.data, keys.scales, keys.biases,
-                       values.scales, values.biases, q_and_gate, out, p, "attn_prefill_quant");
+                       values.scales, values.biases, q_and_gate, out, p, workspace, workspace_bytes,
+                       "attn_prefill_quant");
 }

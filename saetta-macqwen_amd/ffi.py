@@ -9,7 +9,7 @@ LIB_PATH = os.environ.get("SAETTA_HIP_LIB") or os.path.join(_HERE, "lib", "libsa
 SYMBOLS = [
     "saetta_init", "saetta_last_error", "saetta_kv_quantize", "saetta_kv_dequantize", "saetta_to_half",
     "saetta_part_o_bytes", "saetta_part_ml_bytes", "saetta_attn_decode", "saetta_attn_decode_quant",
-    "saetta_attn_rows", "saetta_attn_rows_quant", "saetta_attn_prefill", "saetta_attn_prefill_quant",
+    "saetta_attn_rows", "saetta_attn_rows_quant", "saetta_prefill_workspace_bytes", "saetta_attn_prefill", "saetta_attn_prefill_quant",
 ]
 
 STAGE_PARTIAL, STAGE_REDUCE, STAGE_ALL = 1, 2, 3
@@ -78,9 +78,12 @@ def lib():
         l.saetta_attn_rows_quant.argtypes = [vp, i32, vp, QuantRowsC, QuantRowsC, vp, vp, vp, vp,
                                              RowsParamsC, vp, u32]
         l.saetta_attn_prefill.restype = i32
-        l.saetta_attn_prefill.argtypes = [vp, vp, vp, vp, vp, vp, FlashParamsC]
+        l.saetta_attn_prefill.argtypes = [vp, vp, vp, vp, vp, vp, FlashParamsC, vp, ctypes.c_size_t]
+        l.saetta_prefill_workspace_bytes.restype = ctypes.c_size_t
+        l.saetta_prefill_workspace_bytes.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32]
         l.saetta_attn_prefill_quant.restype = i32
-        l.saetta_attn_prefill_quant.argtypes = [vp, i32, vp, QuantRowsC, QuantRowsC, vp, vp, FlashParamsC]
+        l.saetta_attn_prefill_quant.argtypes = [vp, i32, vp, QuantRowsC, QuantRowsC, vp, vp, FlashParamsC, vp,
+                                                ctypes.c_size_t]
         _lib = l
     return _lib
 

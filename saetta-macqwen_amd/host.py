@@ -289,6 +289,13 @@ class AttentionRows:
         plan.op("attention_reduce_rows", launch(ffi.STAGE_REDUCE))
 
 
+def _workspace(t):
+    if t is None:
+        return None, 0
+    _need(t, torch.uint8, "workspace")
+    return _ptr(t), t.numel()
+
+
 class FlashParams:
     """src/attention_prefill.rs:4-14."""
 
@@ -307,9 +314,16 @@ class attention_prefill:
     FlashParams = FlashParams
 
     @staticmethod
-    def encode(kernel, q, keys, values, q_and_gate, out, p, stream=None):
+    def workspace_bytes(p):
+        """Bytes of workspace a chunk with these FlashParams needs."""
+        return ffi.lib().saetta_prefill_workspace_bytes(p.pos, p.tokens, p.kv_heads)
+
+    @staticmethod
+    def encode(kernel, q, keys, values, q_and_gate, out, p, stream=None, workspace=None):
         """encode (src/attention_prefill.rs:39-72).  `kernel` picks a tile size in
-        the reference; the one gfx950 kernel serves both names."""
+        the reference; the one gfx950 kernel serves both names.  `workspace` is a
+        uint8 tensor of at least workspace_bytes(p) bytes, or None to let the
+        library use its own."""
         if kernel not in attention_prefill.KERNELS:
             raise ValueError(f"no prefill attention kernel {kernel}")
         if p.heads != p.kv_heads * 8:
@@ -317,13 +331,15 @@ class attention_prefill:
         _need(q, torch.float16, "q"), _need(keys, torch.float16, "keys"), _need(values, torch.float16, "values")
         _need(q_and_gate, torch.float32, "q_and_gate"), _need(out, torch.float32, "out")
         ffi.check(ffi.lib().saetta_attn_prefill(_stream(stream), _ptr(q), _ptr(keys), _ptr(values),
-                                                _ptr(q_and_gate), _ptr(out), p.c()), "attn_prefill")
+                                                _ptr(q_and_gate), _ptr(out), p.c(), *_workspace(workspace)),
+                  "attn_prefill")
 
     @staticmethod
-    def encode_quant(q, keys, values, q_and_gate, out, p, stream=None):
+    def encode_quant(q, keys, values, q_and_gate, out, p, stream=None, workspace=None):
         """The chunk over a quantized cache read in place (src/prefill.rs:1735-1776)."""
         if p.heads != p.kv_heads * 8:
             raise ValueError("prefill attention needs 8 q heads per kv head")
         _need(q, torch.float16, "q"), _need(q_and_gate, torch.float32, "q_and_gate"), _need(out, torch.float32, "out")
         ffi.check(ffi.lib().saetta_attn_prefill_quant(_stream(stream), keys.bits.value, _ptr(q), keys.c(), values.c(),
-                                                      _ptr(q_and_gate), _ptr(out), p.c()), "attn_prefill_quant")
+                                                      _ptr(q_and_gate), _ptr(out), p.c(), *_workspace(workspace)),
+                  "attn_prefill_quant")

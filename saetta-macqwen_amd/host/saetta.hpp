@@ -343,23 +343,30 @@ inline const char *const KERNELS[2] = {"attention_fa8", "attention_fa4"};
 inline const char *const DEFAULT = "attention_fa8";
 constexpr size_t KEY_BLOCK = 16;
 
+// Device memory the chunk's f16 tile images go to; the default lets the library use its own.
+struct Workspace {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+};
+inline size_t workspace_bytes(FlashParams p) { return saetta_prefill_workspace_bytes(p.pos, p.tokens, p.kv_heads); }
+
 // out[t, h] = softmax(q[t, h] K^T * scale) V * sigmoid(gate[t, h]) over a half cache that holds
 // the chunk's rows.  `kernel` picks a tile size in the reference; one gfx950 kernel serves both.
 inline void encode(const gpu::Gpu &gpu, const std::string &kernel, const View &q, const View &keys, const View &values,
-                   const View &q_and_gate, const View &out, FlashParams p) {
+                   const View &q_and_gate, const View &out, FlashParams p, const Workspace &ws = {}) {
     if (kernel != KERNELS[0] && kernel != KERNELS[1]) throw std::runtime_error("no prefill attention kernel " + kernel);
     if (p.heads != p.kv_heads * 8) throw std::runtime_error(kernel + " needs 8 q heads per kv head");
     check(saetta_attn_prefill(gpu.stream(), q.ptr<uint16_t>(), keys.ptr<uint16_t>(), values.ptr<uint16_t>(), q_and_gate.ptr<float>(),
-                              out.ptr<float>(), p),
+                              out.ptr<float>(), p, ws.ptr, ws.bytes),
           "attn_prefill");
 }
 
 // The same chunk over a quantized cache read in place (src/prefill.rs:1735-1776).
 inline void encode_quant(const gpu::Gpu &gpu, const View &q, const kv_quant::QuantRows &keys, const kv_quant::QuantRows &values,
-                         const View &q_and_gate, const View &out, FlashParams p) {
+                         const View &q_and_gate, const View &out, FlashParams p, const Workspace &ws = {}) {
     if (p.heads != p.kv_heads * 8) throw std::runtime_error("prefill attention needs 8 q heads per kv head");
     check(saetta_attn_prefill_quant(gpu.stream(), int(kv_quant::bits(keys.bits)), q.ptr<uint16_t>(), keys.c(), values.c(),
-                                    q_and_gate.ptr<float>(), out.ptr<float>(), p),
+                                    q_and_gate.ptr<float>(), out.ptr<float>(), p, ws.ptr, ws.bytes),
           "attn_prefill_quant");
 }
 
