@@ -61,12 +61,7 @@ constexpr int BK = 32;                  // keys per block
 constexpr int K_STRIDE = DIM * 2 + 16;  // bytes per key row of the K tile (padded against bank conflicts)
 constexpr int V_STRIDE = BK * 2 + 16;   // bytes per dim row of the V^T tile
 constexpr int K_BYTES = BK * K_STRIDE;
-// Row of dim d in the V^T tile.  The stager writes dims 4i..4i+3 from lane i, the MFMA reads
-// 32 consecutive dims from 32 lanes; with rows ordered (d % 4, d / 4) and two spare rows per
-// plane both patterns spread over the LDS banks.
-constexpr int V_PLANE = DIM / 4 + 2;
-__device__ __forceinline__ constexpr int vt_row(int dim) { return (dim & 3) * V_PLANE + (dim >> 2); }
-constexpr int V_BYTES = 4 * V_PLANE * V_STRIDE;
+constexpr int V_BYTES = DIM * V_STRIDE;  // V^T tile: row = dim, 32 keys in vt_pos order (+ padding)
 constexpr int IMG_BYTES = (K_BYTES + V_BYTES + 1023) / 1024 * 1024;  // one block's image, whole KB
 constexpr float NO_SCORE = -1e30f;
 constexpr float TAU = 8.0f;  // the reference max is raised only past this many powers of two
@@ -247,7 +242,7 @@ __device__ __forceinline__ void stage_store(const Stage<BITS> &st, unsigned char
         }
 #pragma unroll
         for (int d = 0; d < 4; d++) {
-            unsigned char *row = v_lds + (d * V_PLANE + dq) * V_STRIDE;
+            unsigned char *row = v_lds + (4 * dq + d) * V_STRIDE;
             *reinterpret_cast<u32x2 *>(row + 2 * p0) = u32x2{w[d][0], w[d][1]};
             *reinterpret_cast<u32x2 *>(row + 2 * p1) = u32x2{w[d][2], w[d][3]};
         }
@@ -272,14 +267,88 @@ __global__ __launch_bounds__(PREP_THREADS) void prefill_prepare_kernel(PrepareAr
     stage_store<BITS>(st, img, img + K_BYTES, block * BK, a.key_limit, threadIdx.x);
 }
 
+// S^T = K Q^T of one block as one instruction stream: 16 LDS reads of K rows kept four ahead of
+// the 16 MFMAs that use them.  kaddr: LDS byte address of the lane's key row (col) plus 16 hf.
+// Ends with the wait states an MFMA result needs before vector ALU instructions may read it.
+__device__ __forceinline__ void scores_block(floatx16 &s, const half8 (&q)[16], uint32_t kaddr) {
+    half8 a0, a1, a2, a3;
+#define SAETTA_S_STEP(A, Q, OFF, CNT)                                  \
+    "s_waitcnt lgkmcnt(" #CNT ")\n"                                    \
+    "v_mfma_f32_32x32x16_f16 %[s], %[" #A "], %[" #Q "], %[s]\n"       \
+    "ds_read_b128 %[" #A "], %[addr] offset:" #OFF "\n"
+#define SAETTA_S_LAST(A, Q, CNT)                                       \
+    "s_waitcnt lgkmcnt(" #CNT ")\n"                                    \
+    "v_mfma_f32_32x32x16_f16 %[s], %[" #A "], %[" #Q "], %[s]\n"
+    asm volatile(
+        "s_waitcnt lgkmcnt(0)\n"
+        "ds_read_b128 %[a0], %[addr]\n"
+        "ds_read_b128 %[a1], %[addr] offset:32\n"
+        "ds_read_b128 %[a2], %[addr] offset:64\n"
+        "ds_read_b128 %[a3], %[addr] offset:96\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a0], %[q0], 0\n"
+        "ds_read_b128 %[a0], %[addr] offset:128\n"
+        SAETTA_S_STEP(a1, q1, 160, 3) SAETTA_S_STEP(a2, q2, 192, 3) SAETTA_S_STEP(a3, q3, 224, 3)
+        SAETTA_S_STEP(a0, q4, 256, 3) SAETTA_S_STEP(a1, q5, 288, 3) SAETTA_S_STEP(a2, q6, 320, 3)
+        SAETTA_S_STEP(a3, q7, 352, 3) SAETTA_S_STEP(a0, q8, 384, 3) SAETTA_S_STEP(a1, q9, 416, 3)
+        SAETTA_S_STEP(a2, q10, 448, 3) SAETTA_S_STEP(a3, q11, 480, 3)
+        SAETTA_S_LAST(a0, q12, 3) SAETTA_S_LAST(a1, q13, 2) SAETTA_S_LAST(a2, q14, 1) SAETTA_S_LAST(a3, q15, 0)
+        "s_nop 15\n"
+        "s_nop 3\n"
+        : [s] "=&v"(s), [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2), [a3] "=&v"(a3)
+        : [addr] "v"(kaddr), [q0] "v"(q[0]), [q1] "v"(q[1]), [q2] "v"(q[2]), [q3] "v"(q[3]), [q4] "v"(q[4]),
+          [q5] "v"(q[5]), [q6] "v"(q[6]), [q7] "v"(q[7]), [q8] "v"(q[8]), [q9] "v"(q[9]), [q10] "v"(q[10]),
+          [q11] "v"(q[11]), [q12] "v"(q[12]), [q13] "v"(q[13]), [q14] "v"(q[14]), [q15] "v"(q[15])
+        : "memory");
+#undef SAETTA_S_STEP
+#undef SAETTA_S_LAST
+}
+
+// O^T += V^T P^T of one block, the same way: 16 reads of V^T rows four ahead of 16 MFMAs.
+// vaddr: LDS byte address of the lane's dim row (col) of the V^T tile plus 16 hf; the tile of
+// dims 32 mt .. 32 mt + 31 is 32 rows further, k-step sp 32 bytes further.
+__device__ __forceinline__ void accumulate_block(floatx16 (&o)[8], const half8 (&p)[2], uint32_t vaddr) {
+    half8 a0, a1, a2, a3;
+#define SAETTA_O_STEP(A, ACC, P, OFF, CNT)                                   \
+    "s_waitcnt lgkmcnt(" #CNT ")\n"                                          \
+    "v_mfma_f32_32x32x16_f16 %[" #ACC "], %[" #A "], %[" #P "], %[" #ACC "]\n" \
+    "ds_read_b128 %[" #A "], %[addr] offset:" #OFF "\n"
+#define SAETTA_O_LAST(A, ACC, P, CNT)                                        \
+    "s_waitcnt lgkmcnt(" #CNT ")\n"                                          \
+    "v_mfma_f32_32x32x16_f16 %[" #ACC "], %[" #A "], %[" #P "], %[" #ACC "]\n"
+    // read i serves MFMA i: i < 8 is (sp 0, mt i) at offset 2560 i, i >= 8 is (sp 1, mt i - 8) at 2560 (i - 8) + 32
+    asm volatile(
+        "s_waitcnt lgkmcnt(0)\n"
+        "ds_read_b128 %[a0], %[addr]\n"
+        "ds_read_b128 %[a1], %[addr] offset:2560\n"
+        "ds_read_b128 %[a2], %[addr] offset:5120\n"
+        "ds_read_b128 %[a3], %[addr] offset:7680\n"
+        SAETTA_O_STEP(a0, o0, p0, 10240, 3) SAETTA_O_STEP(a1, o1, p0, 12800, 3) SAETTA_O_STEP(a2, o2, p0, 15360, 3)
+        SAETTA_O_STEP(a3, o3, p0, 17920, 3) SAETTA_O_STEP(a0, o4, p0, 32, 3) SAETTA_O_STEP(a1, o5, p0, 2592, 3)
+        SAETTA_O_STEP(a2, o6, p0, 5152, 3) SAETTA_O_STEP(a3, o7, p0, 7712, 3) SAETTA_O_STEP(a0, o0, p1, 10272, 3)
+        SAETTA_O_STEP(a1, o1, p1, 12832, 3) SAETTA_O_STEP(a2, o2, p1, 15392, 3) SAETTA_O_STEP(a3, o3, p1, 17952, 3)
+        SAETTA_O_LAST(a0, o4, p1, 3) SAETTA_O_LAST(a1, o5, p1, 2) SAETTA_O_LAST(a2, o6, p1, 1)
+        SAETTA_O_LAST(a3, o7, p1, 0)
+        : [o0] "+v"(o[0]), [o1] "+v"(o[1]), [o2] "+v"(o[2]), [o3] "+v"(o[3]), [o4] "+v"(o[4]), [o5] "+v"(o[5]),
+          [o6] "+v"(o[6]), [o7] "+v"(o[7]), [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2), [a3] "=&v"(a3)
+        : [addr] "v"(vaddr), [p0] "v"(p[0]), [p1] "v"(p[1])
+        : "memory");
+#undef SAETTA_O_STEP
+#undef SAETTA_O_LAST
+}
+
+// The wait states after which vector ALU instructions may read what the last MFMAs wrote.
+__device__ __forceinline__ void settle(floatx16 (&o)[8]) {
+    asm volatile("s_nop 15\ns_nop 3\n"
+                 : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]), "+v"(o[4]), "+v"(o[5]), "+v"(o[6]), "+v"(o[7]));
+}
+
 constexpr int NBUF = 3;
 constexpr int LDS_BYTES = NBUF * IMG_BYTES;
 
 __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(PrefillArgs a) {
     // the image of block b lives in buffer b % 3
     extern __shared__ __attribute__((aligned(1024))) unsigned char tiles[];
-    auto k_buf = [&](uint32_t b) { return tiles + (b % NBUF) * IMG_BYTES; };
-    auto v_buf = [&](uint32_t b) { return tiles + (b % NBUF) * IMG_BYTES + K_BYTES; };
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, hf = lane >> 5;
@@ -332,19 +401,6 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(PrefillArgs 
     }
     float m_ref = NO_SCORE, l_sum = 0.0f;
 
-    // S^T = K Q^T of one block: rows = the block's 32 keys, columns = query rows.
-    auto scores = [&](uint32_t b) {
-        const unsigned char *k_lds = k_buf(b);
-        floatx16 s;
-#pragma unroll
-        for (int r = 0; r < 16; r++) s[r] = 0.0f;
-#pragma unroll
-        for (int stp = 0; stp < 16; stp++) {
-            const half8 ka = *reinterpret_cast<const half8 *>(k_lds + col * K_STRIDE + (16 * stp + 8 * hf) * 2);
-            s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qb[stp], s, 0, 0, 0);
-        }
-        return s;
-    };
     // Row maximum of a block's scaled scores (first half of the softmax).  Register r of the
     // accumulator is key 4 hf + r % 4 + 8 (r / 4) of the block; masked scores become NO_SCORE / c.
     auto mask_max = [&](floatx16 &s, uint32_t key0, bool masked) {
@@ -395,19 +451,10 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(PrefillArgs 
             pb[sp] = __builtin_bit_cast(half8, w);
         }
     };
-    // O^T += V^T P^T: rows = dims, columns = query rows.
-    auto accumulate = [&](uint32_t b, const half8 (&pb)[2]) {
-        const unsigned char *v_lds = v_buf(b);
-#pragma unroll
-        for (int mt = 0; mt < 8; mt++) {
-#pragma unroll
-            for (int sp = 0; sp < 2; sp++) {
-                const half8 va =
-                    *reinterpret_cast<const half8 *>(v_lds + vt_row(32 * mt + col) * V_STRIDE + (16 * sp + 8 * hf) * 2);
-                acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, pb[sp], acc[mt], 0, 0, 0);
-            }
-        }
-    };
+    // LDS addresses (bytes) of the lane's rows in buffer 0
+    const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(tiles));
+    const uint32_t k_lane = lds0 + col * K_STRIDE + 16 * hf;
+    const uint32_t v_lane = lds0 + K_BYTES + col * V_STRIDE + 16 * hf;
 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();  // blocks 0 and 1 are in LDS
@@ -416,15 +463,19 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(PrefillArgs 
         // Block kb + 2 goes where block kb - 1 was (every wave left it at the last barrier).
         if (kb + 2 < nblocks) copy_block(kb + 2);
         if (kb < wave_blocks) {
-            floatx16 s = scores(kb);
+            const uint32_t buf = (kb % NBUF) * IMG_BYTES;
+            floatx16 s;
+            scores_block(s, qb, k_lane + buf);
             raise_max(mask_max(s, kb * BK, kb >= full_blocks));
             half8 pb[2];
             exp_pack(s, pb);
-            accumulate(kb, pb);
+            accumulate_block(acc, pb, v_lane + buf);
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
+
+    settle(acc);
 
     // ---- out = O / l * sigmoid(gate) ---------------------------------------------------
     // The lane's row sum is split over the two lane halves (each saw half the keys).
