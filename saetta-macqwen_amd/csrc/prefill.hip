@@ -54,15 +54,17 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int DIM = SAETTA_HEAD_DIM;
 constexpr int PREP_THREADS = 256;       // the prepare kernel's workgroup
-constexpr int WAVES = 8;                // two per SIMD: one's softmax runs under the other's MFMAs
+constexpr int WAVES = 8;                // 4 row groups x 2 waves that take alternate key blocks
 constexpr int THREADS = 64 * WAVES;
-constexpr int TQ = 4 * WAVES;           // tokens per workgroup: a wave owns 4 tokens x 8 heads = 32 rows
+constexpr int TQ = 16;                  // tokens per workgroup: a row group is 4 tokens x 8 heads = 32 rows
 constexpr int BK = 32;                  // keys per block
-constexpr int K_STRIDE = DIM * 2 + 16;  // bytes per key row of the K tile (padded against bank conflicts)
-constexpr int V_STRIDE = BK * 2 + 16;   // bytes per dim row of the V^T tile
-constexpr int K_BYTES = BK * K_STRIDE;
-constexpr int V_BYTES = DIM * V_STRIDE;  // V^T tile: row = dim, 32 keys in vt_pos order (+ padding)
-constexpr int IMG_BYTES = (K_BYTES + V_BYTES + 1023) / 1024 * 1024;  // one block's image, whole KB
+// One key block's image: the K tile and the V^T tile in MFMA fragment order, 16 KB each.  A
+// fragment is what one ds_read_b128 of a wave fetches: 64 lanes x 16 bytes, lane (col, hf) at
+// byte 512 hf + 16 col, so every fragment read is one contiguous kilobyte.
+//   K fragment stp (0..15):           lane holds dims 16 stp + 8 hf .. + 7 of key col
+//   V^T fragment 2 mt + sp (0..15):   lane holds key positions 16 sp + 8 hf .. + 7 of dim 32 mt + col
+constexpr int PART_BYTES = BK * DIM * 2;
+constexpr int IMG_BYTES = 2 * PART_BYTES;
 constexpr float NO_SCORE = -1e30f;
 constexpr float TAU = 8.0f;  // the reference max is raised only past this many powers of two
 
@@ -187,11 +189,11 @@ __device__ __forceinline__ constexpr int vt_pos(int key) {
     return 16 * s + 8 * ((u & 7) >> 2) + 4 * (u >> 3) + (u & 3);
 }
 
-// Dequantizes the staged registers into the LDS tiles.  Keys at or past key_limit
+// Dequantizes the staged registers into the two parts of the block's image.  Keys at or past key_limit
 // (the end of the chunk) are written as zeros: their probabilities are 0, and 0 * 0
 // stays 0 whatever the cache rows hold.
 template <int BITS>
-__device__ __forceinline__ void stage_store(const Stage<BITS> &st, unsigned char *k_lds, unsigned char *v_lds,
+__device__ __forceinline__ void stage_store(const Stage<BITS> &st, unsigned char *k_img, unsigned char *v_img,
                                             uint32_t key0, uint32_t key_limit, int tid) {
     {
         const int key = tid >> 3, piece = tid & 7;
@@ -213,9 +215,12 @@ __device__ __forceinline__ void stage_store(const Stage<BITS> &st, unsigned char
 #pragma unroll
             for (int i = 0; i < 16; i++) o[i] = 0;
         }
-        u32x4 *dst = reinterpret_cast<u32x4 *>(k_lds + key * K_STRIDE + piece * 64);
+        // dims 32 piece + 8 j .. + 7 are the (hf = j % 2) half of fragment 2 piece + j / 2
 #pragma unroll
-        for (int i = 0; i < 4; i++) dst[i] = u32x4{o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+        for (int j = 0; j < 4; j++) {
+            *reinterpret_cast<u32x4 *>(k_img + (4 * piece + j) * 512 + key * 16) =
+                u32x4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
+        }
     }
     {
         const int dq = tid & 63, kq = tid >> 6;
@@ -242,9 +247,10 @@ __device__ __forceinline__ void stage_store(const Stage<BITS> &st, unsigned char
         }
 #pragma unroll
         for (int d = 0; d < 4; d++) {
-            unsigned char *row = v_lds + (4 * dq + d) * V_STRIDE;
-            *reinterpret_cast<u32x2 *>(row + 2 * p0) = u32x2{w[d][0], w[d][1]};
-            *reinterpret_cast<u32x2 *>(row + 2 * p1) = u32x2{w[d][2], w[d][3]};
+            const int dim = 4 * dq + d;
+            unsigned char *frag = v_img + (dim >> 5) * 2048 + (dim & 31) * 16;  // position 0 of the dim
+            *reinterpret_cast<u32x2 *>(frag + (p0 >> 3) * 512 + (p0 & 7) * 2) = u32x2{w[d][0], w[d][1]};
+            *reinterpret_cast<u32x2 *>(frag + (p1 >> 3) * 512 + (p1 & 7) * 2) = u32x2{w[d][2], w[d][3]};
         }
     }
 }
@@ -264,13 +270,38 @@ __global__ __launch_bounds__(PREP_THREADS) void prefill_prepare_kernel(PrepareAr
     Stage<BITS> st;
     stage_load<BITS>(st, rs, kvh, block * BK, kv, threadIdx.x);
     unsigned char *img = a.images + (size_t(kv) * a.nblocks + block) * IMG_BYTES;
-    stage_store<BITS>(st, img, img + K_BYTES, block * BK, a.key_limit, threadIdx.x);
+    stage_store<BITS>(st, img, img + PART_BYTES, block * BK, a.key_limit, threadIdx.x);
 }
 
-// S^T = K Q^T of one block as one instruction stream: 16 LDS reads of K rows kept four ahead of
-// the 16 MFMAs that use them.  kaddr: LDS byte address of the lane's key row (col) plus 16 hf.
-// Ends with the wait states an MFMA result needs before vector ALU instructions may read it.
-__device__ __forceinline__ void scores_block(floatx16 &s, const half8 (&q)[16], uint32_t kaddr) {
+// What a wave copies global -> LDS while one of its MFMA streams runs: 4 KB as four
+// global_load_lds_dwordx4 (64 lanes x 16 bytes each) spread between the MFMAs, so that the
+// texture path drains between them and the issue never stalls the wave.
+struct Copy {
+    uint64_t src;  // global address of the 4 KB (wave-uniform)
+    uint32_t dst;  // LDS byte address they go to (wave-uniform)
+};
+
+__device__ __forceinline__ void copy_plain(const Copy &c, uint32_t lane16) {
+    asm volatile(
+        "s_mov_b32 m0, %[dst]\n"
+        "s_nop 0\n"
+        "global_load_lds_dwordx4 %[off], %[src]\n"
+        "global_load_lds_dwordx4 %[off], %[src] offset:1024\n"
+        "global_load_lds_dwordx4 %[off], %[src] offset:2048\n"
+        "global_load_lds_dwordx4 %[off], %[src] offset:3072\n"
+        :
+        : [off] "v"(lane16), [src] "s"(c.src), [dst] "s"(c.dst)
+        : "memory", "m0");
+}
+
+#define SAETTA_COPY(OFF) "global_load_lds_dwordx4 %[off], %[src] offset:" #OFF "\n"
+
+// S^T = K Q^T of one block as one instruction stream: 16 LDS reads of K fragments kept four
+// ahead of the 16 MFMAs that use them, and the wave's copy.  kaddr: LDS byte address of the K
+// part plus 16 lane.  Ends with the wait states an MFMA result needs before vector ALU
+// instructions may read it.
+__device__ __forceinline__ void scores_block(floatx16 &s, const half8 (&q)[16], uint32_t kaddr, const Copy &c,
+                                             uint32_t lane16) {
     half8 a0, a1, a2, a3;
 #define SAETTA_S_STEP(A, Q, OFF, CNT)                                  \
     "s_waitcnt lgkmcnt(" #CNT ")\n"                                    \
@@ -281,33 +312,38 @@ __device__ __forceinline__ void scores_block(floatx16 &s, const half8 (&q)[16], 
     "v_mfma_f32_32x32x16_f16 %[s], %[" #A "], %[" #Q "], %[s]\n"
     asm volatile(
         "s_waitcnt lgkmcnt(0)\n"
+        "s_mov_b32 m0, %[dst]\n"
         "ds_read_b128 %[a0], %[addr]\n"
-        "ds_read_b128 %[a1], %[addr] offset:32\n"
-        "ds_read_b128 %[a2], %[addr] offset:64\n"
-        "ds_read_b128 %[a3], %[addr] offset:96\n"
+        "ds_read_b128 %[a1], %[addr] offset:1024\n"
+        "ds_read_b128 %[a2], %[addr] offset:2048\n"
+        "ds_read_b128 %[a3], %[addr] offset:3072\n"
         "s_waitcnt lgkmcnt(3)\n"
         "v_mfma_f32_32x32x16_f16 %[s], %[a0], %[q0], 0\n"
-        "ds_read_b128 %[a0], %[addr] offset:128\n"
-        SAETTA_S_STEP(a1, q1, 160, 3) SAETTA_S_STEP(a2, q2, 192, 3) SAETTA_S_STEP(a3, q3, 224, 3)
-        SAETTA_S_STEP(a0, q4, 256, 3) SAETTA_S_STEP(a1, q5, 288, 3) SAETTA_S_STEP(a2, q6, 320, 3)
-        SAETTA_S_STEP(a3, q7, 352, 3) SAETTA_S_STEP(a0, q8, 384, 3) SAETTA_S_STEP(a1, q9, 416, 3)
-        SAETTA_S_STEP(a2, q10, 448, 3) SAETTA_S_STEP(a3, q11, 480, 3)
-        SAETTA_S_LAST(a0, q12, 3) SAETTA_S_LAST(a1, q13, 2) SAETTA_S_LAST(a2, q14, 1) SAETTA_S_LAST(a3, q15, 0)
+        "ds_read_b128 %[a0], %[addr] offset:4096\n"
+        SAETTA_S_STEP(a1, q1, 5120, 3) SAETTA_COPY(0) SAETTA_S_STEP(a2, q2, 6144, 3)
+        SAETTA_S_STEP(a3, q3, 7168, 3) SAETTA_S_STEP(a0, q4, 8192, 3) SAETTA_S_STEP(a1, q5, 9216, 3) SAETTA_COPY(1024)
+        SAETTA_S_STEP(a2, q6, 10240, 3) SAETTA_S_STEP(a3, q7, 11264, 3) SAETTA_S_STEP(a0, q8, 12288, 3)
+        SAETTA_S_STEP(a1, q9, 13312, 3) SAETTA_COPY(2048) SAETTA_S_STEP(a2, q10, 14336, 3)
+        SAETTA_S_STEP(a3, q11, 15360, 3)
+        SAETTA_S_LAST(a0, q12, 3) SAETTA_S_LAST(a1, q13, 2) SAETTA_COPY(3072) SAETTA_S_LAST(a2, q14, 1)
+        SAETTA_S_LAST(a3, q15, 0)
         "s_nop 15\n"
         "s_nop 3\n"
         : [s] "=&v"(s), [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2), [a3] "=&v"(a3)
         : [addr] "v"(kaddr), [q0] "v"(q[0]), [q1] "v"(q[1]), [q2] "v"(q[2]), [q3] "v"(q[3]), [q4] "v"(q[4]),
           [q5] "v"(q[5]), [q6] "v"(q[6]), [q7] "v"(q[7]), [q8] "v"(q[8]), [q9] "v"(q[9]), [q10] "v"(q[10]),
-          [q11] "v"(q[11]), [q12] "v"(q[12]), [q13] "v"(q[13]), [q14] "v"(q[14]), [q15] "v"(q[15])
-        : "memory");
+          [q11] "v"(q[11]), [q12] "v"(q[12]), [q13] "v"(q[13]), [q14] "v"(q[14]), [q15] "v"(q[15]),
+          [off] "v"(lane16), [src] "s"(c.src), [dst] "s"(c.dst)
+        : "memory", "m0");
 #undef SAETTA_S_STEP
 #undef SAETTA_S_LAST
 }
 
-// O^T += V^T P^T of one block, the same way: 16 reads of V^T rows four ahead of 16 MFMAs.
-// vaddr: LDS byte address of the lane's dim row (col) of the V^T tile plus 16 hf; the tile of
-// dims 32 mt .. 32 mt + 31 is 32 rows further, k-step sp 32 bytes further.
-__device__ __forceinline__ void accumulate_block(floatx16 (&o)[8], const half8 (&p)[2], uint32_t vaddr) {
+// O^T += V^T P^T of one block, the same way: 16 reads of V^T fragments four ahead of 16
+// MFMAs, and the wave's copy.  vaddr: LDS byte address of the V^T part plus 16 lane; fragment
+// 2 mt + sp serves accumulator mt with k-step sp.
+__device__ __forceinline__ void accumulate_block(floatx16 (&o)[8], const half8 (&p)[2], uint32_t vaddr,
+                                                 const Copy &c, uint32_t lane16) {
     half8 a0, a1, a2, a3;
 #define SAETTA_O_STEP(A, ACC, P, OFF, CNT)                                   \
     "s_waitcnt lgkmcnt(" #CNT ")\n"                                          \
@@ -316,26 +352,29 @@ __device__ __forceinline__ void accumulate_block(floatx16 (&o)[8], const half8 (
 #define SAETTA_O_LAST(A, ACC, P, CNT)                                        \
     "s_waitcnt lgkmcnt(" #CNT ")\n"                                          \
     "v_mfma_f32_32x32x16_f16 %[" #ACC "], %[" #A "], %[" #P "], %[" #ACC "]\n"
-    // read i serves MFMA i: i < 8 is (sp 0, mt i) at offset 2560 i, i >= 8 is (sp 1, mt i - 8) at 2560 (i - 8) + 32
+    // read i serves MFMA i: i < 8 is (sp 0, mt i), fragment 2 i; i >= 8 is (sp 1, mt i - 8), fragment 2 (i - 8) + 1
     asm volatile(
         "s_waitcnt lgkmcnt(0)\n"
+        "s_mov_b32 m0, %[dst]\n"
         "ds_read_b128 %[a0], %[addr]\n"
-        "ds_read_b128 %[a1], %[addr] offset:2560\n"
-        "ds_read_b128 %[a2], %[addr] offset:5120\n"
-        "ds_read_b128 %[a3], %[addr] offset:7680\n"
-        SAETTA_O_STEP(a0, o0, p0, 10240, 3) SAETTA_O_STEP(a1, o1, p0, 12800, 3) SAETTA_O_STEP(a2, o2, p0, 15360, 3)
-        SAETTA_O_STEP(a3, o3, p0, 17920, 3) SAETTA_O_STEP(a0, o4, p0, 32, 3) SAETTA_O_STEP(a1, o5, p0, 2592, 3)
-        SAETTA_O_STEP(a2, o6, p0, 5152, 3) SAETTA_O_STEP(a3, o7, p0, 7712, 3) SAETTA_O_STEP(a0, o0, p1, 10272, 3)
-        SAETTA_O_STEP(a1, o1, p1, 12832, 3) SAETTA_O_STEP(a2, o2, p1, 15392, 3) SAETTA_O_STEP(a3, o3, p1, 17952, 3)
-        SAETTA_O_LAST(a0, o4, p1, 3) SAETTA_O_LAST(a1, o5, p1, 2) SAETTA_O_LAST(a2, o6, p1, 1)
+        "ds_read_b128 %[a1], %[addr] offset:2048\n"
+        "ds_read_b128 %[a2], %[addr] offset:4096\n"
+        "ds_read_b128 %[a3], %[addr] offset:6144\n"
+        SAETTA_O_STEP(a0, o0, p0, 8192, 3) SAETTA_O_STEP(a1, o1, p0, 10240, 3) SAETTA_COPY(0)
+        SAETTA_O_STEP(a2, o2, p0, 12288, 3) SAETTA_O_STEP(a3, o3, p0, 14336, 3) SAETTA_O_STEP(a0, o4, p0, 1024, 3)
+        SAETTA_O_STEP(a1, o5, p0, 3072, 3) SAETTA_COPY(1024) SAETTA_O_STEP(a2, o6, p0, 5120, 3)
+        SAETTA_O_STEP(a3, o7, p0, 7168, 3) SAETTA_O_STEP(a0, o0, p1, 9216, 3) SAETTA_O_STEP(a1, o1, p1, 11264, 3)
+        SAETTA_COPY(2048) SAETTA_O_STEP(a2, o2, p1, 13312, 3) SAETTA_O_STEP(a3, o3, p1, 15360, 3)
+        SAETTA_O_LAST(a0, o4, p1, 3) SAETTA_O_LAST(a1, o5, p1, 2) SAETTA_COPY(3072) SAETTA_O_LAST(a2, o6, p1, 1)
         SAETTA_O_LAST(a3, o7, p1, 0)
         : [o0] "+v"(o[0]), [o1] "+v"(o[1]), [o2] "+v"(o[2]), [o3] "+v"(o[3]), [o4] "+v"(o[4]), [o5] "+v"(o[5]),
           [o6] "+v"(o[6]), [o7] "+v"(o[7]), [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2), [a3] "=&v"(a3)
-        : [addr] "v"(vaddr), [p0] "v"(p[0]), [p1] "v"(p[1])
-        : "memory");
+        : [addr] "v"(vaddr), [p0] "v"(p[0]), [p1] "v"(p[1]), [off] "v"(lane16), [src] "s"(c.src), [dst] "s"(c.dst)
+        : "memory", "m0");
 #undef SAETTA_O_STEP
 #undef SAETTA_O_LAST
 }
+#undef SAETTA_COPY
 
 // The wait states after which vector ALU instructions may read what the last MFMAs wrote.
 __device__ __forceinline__ void settle(floatx16 (&o)[8]) {
@@ -343,19 +382,33 @@ __device__ __forceinline__ void settle(floatx16 (&o)[8]) {
                  : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]), "+v"(o[4]), "+v"(o[5]), "+v"(o[6]), "+v"(o[7]));
 }
 
-constexpr int NBUF = 3;
-constexpr int LDS_BYTES = NBUF * IMG_BYTES;
+// max over the two lanes l and l ^ 32, without a trip through LDS
+__device__ __forceinline__ float max_across_halves(float x) {
+    uint32_t u = __builtin_bit_cast(uint32_t, x), v = u;
+    // Swaps the upper half of u with the lower half of v: u = (lo, lo), v = (hi, hi).  The
+    // instruction may not read a register a vector instruction wrote in the two cycles before.
+    asm volatile("s_nop 1\nv_permlane32_swap_b32 %0, %1\n" : "+v"(u), "+v"(v));
+    return fmaxf(__builtin_bit_cast(float, u), __builtin_bit_cast(float, v));
+}
 
-__global__ __launch_bounds__(THREADS) void attention_prefill_kernel(PrefillArgs a) {
-    // the image of block b lives in buffer b % 3
+// LDS: four K slots, then four V^T slots.  Even blocks alternate between K slots 0 and 1, odd
+// blocks between 2 and 3 (an odd block's K is needed one step before its V^T, see the kernel).
+constexpr int MERGE_WAVE_BYTES = (8 * 16 + 2) * 64 * 4;  // one wave's O, m, l on their way to its partner
+constexpr int LDS_BYTES = 4 * MERGE_WAVE_BYTES > 8 * PART_BYTES ? 4 * MERGE_WAVE_BYTES : 8 * PART_BYTES;
+__device__ __forceinline__ uint32_t k_slot(uint32_t b) { return (((b & 1) << 1) | ((b >> 1) & 1)) * PART_BYTES; }
+__device__ __forceinline__ uint32_t v_slot(uint32_t b) { return (4 + (b & 3)) * PART_BYTES; }
+
+__global__ __launch_bounds__(THREADS, 2) void attention_prefill_kernel(PrefillArgs a) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char tiles[];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, hf = lane >> 5;
+    const int group = wave & 3, parity = wave >> 2;  // the wave's rows; which key blocks it takes
     const uint32_t kv = blockIdx.y;
     const uint32_t ntiles = (a.tokens + TQ - 1) / TQ;
     const uint32_t tile = ntiles - 1 - blockIdx.x;  // the tiles with the most keys start first
-    const uint32_t tok0 = tile * TQ + 4 * wave;     // this wave's first token
+    const uint32_t tok0 = tile * TQ + 4 * group;    // this wave's first token
     const float c = a.scale * 1.4426950408889634f;  // scores are kept in units of log2(e)
 
     // Row of this lane: token tok0 + col / 8, head col % 8.
@@ -370,19 +423,40 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(PrefillArgs 
     const uint32_t wave_blocks = tok0 < a.tokens ? min((wave_keys + BK - 1) / BK, nblocks) : 0;
     const uint32_t full_blocks = min(wave_first_len / BK, wave_blocks);  // blocks that need no mask
 
-    // Copies the image of block b into its LDS buffer: every lane moves 16 bytes per
-    // instruction, a wave 1 KB, straight from global memory to LDS.
+    const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(tiles));
+    const uint32_t lane16 = lane * 16;
     const unsigned char *images = a.images + size_t(kv) * a.nblocks * IMG_BYTES;
-    auto copy_block = [&](uint32_t b) {
-        const unsigned char *src = images + size_t(b) * IMG_BYTES + lane * 16;
-        unsigned char *dst = tiles + (b % NBUF) * IMG_BYTES;
-        for (int i = wave; i < IMG_BYTES / 1024; i += WAVES) {
-            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(src + i * 1024),
-                                             (void __attribute__((address_space(3))) *)(dst + i * 1024), 16, 0, 0);
-        }
+    // The wave's 4 KB number `quarter` (0..3) of part `v` (0 = K, 1 = V^T) of block b.  Blocks
+    // past the cache's end are read from the last image instead; nobody looks at their slots.
+    auto piece = [&](uint32_t b, int v, int quarter) {
+        const uint32_t bb = min(b, a.nblocks - 1);
+        Copy cp;
+        cp.src = reinterpret_cast<uint64_t>(images) + uint64_t(bb) * IMG_BYTES + v * PART_BYTES + quarter * 4096;
+        cp.dst = lds0 + (v ? v_slot(b) : k_slot(b)) + quarter * 4096;
+        return cp;
     };
-    copy_block(0);
-    if (nblocks > 1) copy_block(1);
+
+    // Step s works on blocks 2s (even waves: parity 0) and 2s + 1 (parity 1).  The two waves of a
+    // SIMD are kept half a step apart, so that one's softmax runs under the other's MFMAs:
+    //   parity 0:  S(2s)       softmax(2s)     O(2s)
+    //   parity 1:  softmax(2s+1)   O(2s+1)     S(2s+3)
+    // so an odd block's K must be in LDS one step before its V^T.  During step s the workgroup
+    // copies K(2s+2), K(2s+5), V(2s+2), V(2s+3): wave w takes half (w % 2) of part w / 2 of that list.
+    // Before the loop: K(0), K(1), K(3), V(0), V(1), ten pieces per wave.
+    for (int i = wave; i < 40; i += WAVES) {
+        const int part = i >> 3, quarter = (i >> 1) & 3, v = part >= 3;
+        const uint32_t b = part == 0 ? 0 : part == 1 ? 1 : part == 2 ? 3 : part == 3 ? 0 : 1;
+        Copy cp = piece(b, v, quarter);
+        cp.src += (i & 1) * 2048, cp.dst += (i & 1) * 2048;
+        asm volatile(
+            "s_mov_b32 m0, %[dst]\n"
+            "s_nop 0\n"
+            "global_load_lds_dwordx4 %[off], %[src]\n"
+            "global_load_lds_dwordx4 %[off], %[src] offset:1024\n"
+            :
+            : [off] "v"(lane16), [src] "s"(cp.src), [dst] "s"(cp.dst)
+            : "memory", "m0");
+    }
 
     // Q^T operands: lane (col, hf), k-step st: dims 16 st + 8 hf .. + 7 of its row.
     half8 qb[16];
@@ -416,7 +490,7 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(PrefillArgs 
         }
 #pragma unroll
         for (int r = 0; r < 16; r++) bm = fmaxf(bm, s[r]);
-        bm = fmaxf(bm, __shfl_xor(bm, 32));
+        bm = max_across_halves(bm);
         return fmaxf(bm * c, NO_SCORE);
     };
     // Raises the reference maximum when a block tops it by more than 2^TAU, rescaling O and l.
@@ -451,31 +525,98 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(PrefillArgs 
             pb[sp] = __builtin_bit_cast(half8, w);
         }
     };
-    // LDS addresses (bytes) of the lane's rows in buffer 0
-    const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(tiles));
-    const uint32_t k_lane = lds0 + col * K_STRIDE + 16 * hf;
-    const uint32_t v_lane = lds0 + K_BYTES + col * V_STRIDE + 16 * hf;
 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();  // blocks 0 and 1 are in LDS
+    __syncthreads();  // K(0), K(1), K(3), V(0), V(1) are in LDS
 
-    for (uint32_t kb = 0; kb < nblocks; kb++) {
-        // Block kb + 2 goes where block kb - 1 was (every wave left it at the last barrier).
-        if (kb + 2 < nblocks) copy_block(kb + 2);
-        if (kb < wave_blocks) {
-            const uint32_t buf = (kb % NBUF) * IMG_BYTES;
-            floatx16 s;
-            scores_block(s, qb, k_lane + buf);
-            raise_max(mask_max(s, kb * BK, kb >= full_blocks));
-            half8 pb[2];
-            exp_pack(s, pb);
-            accumulate_block(acc, pb, v_lane + buf);
+    const uint32_t nsteps = (nblocks + 1) / 2;
+    const int part = wave >> 1, half = wave & 1;  // what the wave copies in every step
+    auto copies_of = [&](uint32_t step, Copy &first, Copy &second) {
+        const uint32_t cb = part == 0 ? 2 * step + 2 : part == 1 ? 2 * step + 5 : part == 2 ? 2 * step + 2 : 2 * step + 3;
+        first = piece(cb, part >= 2, 2 * half), second = piece(cb, part >= 2, 2 * half + 1);
+    };
+    if (parity == 0) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();  // the odd waves compute S(1) here
+        for (uint32_t step = 0; step < nsteps; step++) {
+            Copy first, second;
+            copies_of(step, first, second);
+            const uint32_t kb = 2 * step;
+            if (kb < wave_blocks) {
+                floatx16 s;
+                scores_block(s, qb, lds0 + k_slot(kb) + lane16, first, lane16);
+                raise_max(mask_max(s, kb * BK, kb >= full_blocks));
+                half8 pb[2];
+                exp_pack(s, pb);
+                accumulate_block(acc, pb, lds0 + v_slot(kb) + lane16, second, lane16);
+            } else {
+                copy_plain(first, lane16);
+                copy_plain(second, lane16);
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+    } else {
+        // The odd waves enter the loop with the scores of block 1 in hand.
+        floatx16 s;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = 0.0f;
+        if (1 < wave_blocks) {
+            // (the copy it carries rewrites 4 KB of K(0) with themselves; nobody reads K(0) yet)
+            scores_block(s, qb, lds0 + k_slot(1) + lane16, piece(0, 0, 0), lane16);
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+        for (uint32_t step = 0; step < nsteps; step++) {
+            Copy first, second;
+            copies_of(step, first, second);
+            const uint32_t kb = 2 * step + 1;
+            if (kb < wave_blocks) {
+                raise_max(mask_max(s, kb * BK, kb >= full_blocks));
+                half8 pb[2];
+                exp_pack(s, pb);
+                accumulate_block(acc, pb, lds0 + v_slot(kb) + lane16, first, lane16);
+            } else {
+                copy_plain(first, lane16);
+            }
+            if (kb + 2 < wave_blocks) {
+                scores_block(s, qb, lds0 + k_slot(kb + 2) + lane16, second, lane16);
+            } else {
+                copy_plain(second, lane16);
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
     }
 
     settle(acc);
+
+    // ---- the two waves of a row group merge their halves of the keys ----------------------
+    // The odd-block wave hands O, m and l over through LDS (the tiles are done with: the loop
+    // ended on a barrier); element e of lane L sits at word e * 64 + L.
+    {
+        float *xchg = reinterpret_cast<float *>(tiles + group * MERGE_WAVE_BYTES) + lane;
+        if (parity == 1) {
+#pragma unroll
+            for (int mt = 0; mt < 8; mt++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) xchg[(16 * mt + r) * 64] = acc[mt][r];
+            }
+            xchg[128 * 64] = m_ref;
+            xchg[129 * 64] = l_sum;
+        }
+        __syncthreads();
+        if (parity == 1) return;
+        const float m_other = xchg[128 * 64], l_other = xchg[129 * 64];
+        const float m_new = fmaxf(m_ref, m_other);
+        const float mine = __builtin_amdgcn_exp2f(m_ref - m_new), theirs = __builtin_amdgcn_exp2f(m_other - m_new);
+        l_sum = l_sum * mine + l_other * theirs;
+#pragma unroll
+        for (int mt = 0; mt < 8; mt++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[mt][r] = acc[mt][r] * mine + xchg[(16 * mt + r) * 64] * theirs;
+        }
+    }
 
     // ---- out = O / l * sigmoid(gate) ---------------------------------------------------
     // The lane's row sum is split over the two lane halves (each saw half the keys).
