@@ -273,11 +273,11 @@ __global__ __launch_bounds__(PREP_THREADS) void prefill_prepare_kernel(PrepareAr
     stage_store<BITS>(st, img, img + PART_BYTES, block * BK, a.key_limit, threadIdx.x);
 }
 
-// What a wave copies global -> LDS while one of its MFMA streams runs: 4 KB as four
-// global_load_lds_dwordx4 (64 lanes x 16 bytes each) spread between the MFMAs, so that the
-// texture path drains between them and the issue never stalls the wave.
+// What a wave copies global -> LDS per step: 8 KB as eight global_load_lds_dwordx4 (64 lanes x
+// 16 bytes each).  Inside the MFMA stream they are spread between the MFMAs, so that the
+// texture path drains between them and their issue never stalls the wave.
 struct Copy {
-    uint64_t src;  // global address of the 4 KB (wave-uniform)
+    uint64_t src;  // global address of the 8 KB (wave-uniform)
     uint32_t dst;  // LDS byte address they go to (wave-uniform)
 };
 
@@ -289,19 +289,22 @@ __device__ __forceinline__ void copy_plain(const Copy &c, uint32_t lane16) {
         "global_load_lds_dwordx4 %[off], %[src] offset:1024\n"
         "global_load_lds_dwordx4 %[off], %[src] offset:2048\n"
         "global_load_lds_dwordx4 %[off], %[src] offset:3072\n"
+        "s_add_u32 m0, m0, 0x1000\n"
+        "s_nop 0\n"
+        "global_load_lds_dwordx4 %[off], %[src2]\n"
+        "global_load_lds_dwordx4 %[off], %[src2] offset:1024\n"
+        "global_load_lds_dwordx4 %[off], %[src2] offset:2048\n"
+        "global_load_lds_dwordx4 %[off], %[src2] offset:3072\n"
         :
-        : [off] "v"(lane16), [src] "s"(c.src), [dst] "s"(c.dst)
+        : [off] "v"(lane16), [src] "s"(c.src), [src2] "s"(c.src + 4096), [dst] "s"(c.dst)
         : "memory", "m0");
 }
 
-#define SAETTA_COPY(OFF) "global_load_lds_dwordx4 %[off], %[src] offset:" #OFF "\n"
-
 // S^T = K Q^T of one block as one instruction stream: 16 LDS reads of K fragments kept four
-// ahead of the 16 MFMAs that use them, and the wave's copy.  kaddr: LDS byte address of the K
-// part plus 16 lane.  Ends with the wait states an MFMA result needs before vector ALU
-// instructions may read it.
-__device__ __forceinline__ void scores_block(floatx16 &s, const half8 (&q)[16], uint32_t kaddr, const Copy &c,
-                                             uint32_t lane16) {
+// ahead of the 16 MFMAs that use them.  kaddr: LDS byte address of the K part plus 16 lane.
+// Ends with the wait states an MFMA result needs before vector ALU instructions may read it.
+// (Used before the loop only; in the loop the scores are part of stream_block.)
+__device__ __forceinline__ void scores_block(floatx16 &s, const half8 (&q)[16], uint32_t kaddr) {
     half8 a0, a1, a2, a3;
 #define SAETTA_S_STEP(A, Q, OFF, CNT)                                  \
     "s_waitcnt lgkmcnt(" #CNT ")\n"                                    \
@@ -312,7 +315,6 @@ __device__ __forceinline__ void scores_block(floatx16 &s, const half8 (&q)[16], 
     "v_mfma_f32_32x32x16_f16 %[s], %[" #A "], %[" #Q "], %[s]\n"
     asm volatile(
         "s_waitcnt lgkmcnt(0)\n"
-        "s_mov_b32 m0, %[dst]\n"
         "ds_read_b128 %[a0], %[addr]\n"
         "ds_read_b128 %[a1], %[addr] offset:1024\n"
         "ds_read_b128 %[a2], %[addr] offset:2048\n"
@@ -320,61 +322,152 @@ __device__ __forceinline__ void scores_block(floatx16 &s, const half8 (&q)[16], 
         "s_waitcnt lgkmcnt(3)\n"
         "v_mfma_f32_32x32x16_f16 %[s], %[a0], %[q0], 0\n"
         "ds_read_b128 %[a0], %[addr] offset:4096\n"
-        SAETTA_S_STEP(a1, q1, 5120, 3) SAETTA_COPY(0) SAETTA_S_STEP(a2, q2, 6144, 3)
-        SAETTA_S_STEP(a3, q3, 7168, 3) SAETTA_S_STEP(a0, q4, 8192, 3) SAETTA_S_STEP(a1, q5, 9216, 3) SAETTA_COPY(1024)
-        SAETTA_S_STEP(a2, q6, 10240, 3) SAETTA_S_STEP(a3, q7, 11264, 3) SAETTA_S_STEP(a0, q8, 12288, 3)
-        SAETTA_S_STEP(a1, q9, 13312, 3) SAETTA_COPY(2048) SAETTA_S_STEP(a2, q10, 14336, 3)
-        SAETTA_S_STEP(a3, q11, 15360, 3)
-        SAETTA_S_LAST(a0, q12, 3) SAETTA_S_LAST(a1, q13, 2) SAETTA_COPY(3072) SAETTA_S_LAST(a2, q14, 1)
-        SAETTA_S_LAST(a3, q15, 0)
+        SAETTA_S_STEP(a1, q1, 5120, 3) SAETTA_S_STEP(a2, q2, 6144, 3) SAETTA_S_STEP(a3, q3, 7168, 3)
+        SAETTA_S_STEP(a0, q4, 8192, 3) SAETTA_S_STEP(a1, q5, 9216, 3) SAETTA_S_STEP(a2, q6, 10240, 3)
+        SAETTA_S_STEP(a3, q7, 11264, 3) SAETTA_S_STEP(a0, q8, 12288, 3) SAETTA_S_STEP(a1, q9, 13312, 3)
+        SAETTA_S_STEP(a2, q10, 14336, 3) SAETTA_S_STEP(a3, q11, 15360, 3)
+        SAETTA_S_LAST(a0, q12, 3) SAETTA_S_LAST(a1, q13, 2) SAETTA_S_LAST(a2, q14, 1) SAETTA_S_LAST(a3, q15, 0)
         "s_nop 15\n"
         "s_nop 3\n"
         : [s] "=&v"(s), [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2), [a3] "=&v"(a3)
         : [addr] "v"(kaddr), [q0] "v"(q[0]), [q1] "v"(q[1]), [q2] "v"(q[2]), [q3] "v"(q[3]), [q4] "v"(q[4]),
           [q5] "v"(q[5]), [q6] "v"(q[6]), [q7] "v"(q[7]), [q8] "v"(q[8]), [q9] "v"(q[9]), [q10] "v"(q[10]),
-          [q11] "v"(q[11]), [q12] "v"(q[12]), [q13] "v"(q[13]), [q14] "v"(q[14]), [q15] "v"(q[15]),
-          [off] "v"(lane16), [src] "s"(c.src), [dst] "s"(c.dst)
-        : "memory", "m0");
+          [q11] "v"(q[11]), [q12] "v"(q[12]), [q13] "v"(q[13]), [q14] "v"(q[14]), [q15] "v"(q[15])
+        : "memory");
 #undef SAETTA_S_STEP
 #undef SAETTA_S_LAST
 }
 
-// O^T += V^T P^T of one block, the same way: 16 reads of V^T fragments four ahead of 16
-// MFMAs, and the wave's copy.  vaddr: LDS byte address of the V^T part plus 16 lane; fragment
-// 2 mt + sp serves accumulator mt with k-step sp.
-__device__ __forceinline__ void accumulate_block(floatx16 (&o)[8], const half8 (&p)[2], uint32_t vaddr,
-                                                 const Copy &c, uint32_t lane16) {
+// One step of a wave as one instruction stream: O^T += V^T P^T of the block whose
+// probabilities are in p, interleaved MFMA by MFMA with S^T = K Q^T of the wave's next block
+// (the scores chain through one accumulator, so alone they would wait on each other), 32 LDS
+// fragment reads kept four ahead of the MFMAs, and the wave's copy.  kaddr / vaddr: LDS byte
+// addresses of the next block's K part / this block's V^T part, plus 16 lane.  V^T fragment
+// 2 mt + sp serves accumulator mt with k-step sp.  Ends with the wait states an MFMA result
+// needs before vector ALU instructions may read it.
+__device__ __forceinline__ void stream_block(floatx16 &s, floatx16 (&o)[8], const half8 (&q)[16], const half8 (&p)[2],
+                                             uint32_t kaddr, uint32_t vaddr, const Copy &c, uint32_t lane16) {
     half8 a0, a1, a2, a3;
-#define SAETTA_O_STEP(A, ACC, P, OFF, CNT)                                   \
-    "s_waitcnt lgkmcnt(" #CNT ")\n"                                          \
-    "v_mfma_f32_32x32x16_f16 %[" #ACC "], %[" #A "], %[" #P "], %[" #ACC "]\n" \
-    "ds_read_b128 %[" #A "], %[addr] offset:" #OFF "\n"
-#define SAETTA_O_LAST(A, ACC, P, CNT)                                        \
-    "s_waitcnt lgkmcnt(" #CNT ")\n"                                          \
-    "v_mfma_f32_32x32x16_f16 %[" #ACC "], %[" #A "], %[" #P "], %[" #ACC "]\n"
-    // read i serves MFMA i: i < 8 is (sp 0, mt i), fragment 2 i; i >= 8 is (sp 1, mt i - 8), fragment 2 (i - 8) + 1
     asm volatile(
         "s_waitcnt lgkmcnt(0)\n"
         "s_mov_b32 m0, %[dst]\n"
-        "ds_read_b128 %[a0], %[addr]\n"
-        "ds_read_b128 %[a1], %[addr] offset:2048\n"
-        "ds_read_b128 %[a2], %[addr] offset:4096\n"
-        "ds_read_b128 %[a3], %[addr] offset:6144\n"
-        SAETTA_O_STEP(a0, o0, p0, 8192, 3) SAETTA_O_STEP(a1, o1, p0, 10240, 3) SAETTA_COPY(0)
-        SAETTA_O_STEP(a2, o2, p0, 12288, 3) SAETTA_O_STEP(a3, o3, p0, 14336, 3) SAETTA_O_STEP(a0, o4, p0, 1024, 3)
-        SAETTA_O_STEP(a1, o5, p0, 3072, 3) SAETTA_COPY(1024) SAETTA_O_STEP(a2, o6, p0, 5120, 3)
-        SAETTA_O_STEP(a3, o7, p0, 7168, 3) SAETTA_O_STEP(a0, o0, p1, 9216, 3) SAETTA_O_STEP(a1, o1, p1, 11264, 3)
-        SAETTA_COPY(2048) SAETTA_O_STEP(a2, o2, p1, 13312, 3) SAETTA_O_STEP(a3, o3, p1, 15360, 3)
-        SAETTA_O_LAST(a0, o4, p1, 3) SAETTA_O_LAST(a1, o5, p1, 2) SAETTA_COPY(3072) SAETTA_O_LAST(a2, o6, p1, 1)
-        SAETTA_O_LAST(a3, o7, p1, 0)
-        : [o0] "+v"(o[0]), [o1] "+v"(o[1]), [o2] "+v"(o[2]), [o3] "+v"(o[3]), [o4] "+v"(o[4]), [o5] "+v"(o[5]),
-          [o6] "+v"(o[6]), [o7] "+v"(o[7]), [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2), [a3] "=&v"(a3)
-        : [addr] "v"(vaddr), [p0] "v"(p[0]), [p1] "v"(p[1]), [off] "v"(lane16), [src] "s"(c.src), [dst] "s"(c.dst)
+        "ds_read_b128 %[a0], %[kaddr] offset:0\n"
+        "ds_read_b128 %[a1], %[vaddr] offset:0\n"
+        "ds_read_b128 %[a2], %[kaddr] offset:1024\n"
+        "ds_read_b128 %[a3], %[vaddr] offset:2048\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a0], %[q0], 0\n"
+        "ds_read_b128 %[a0], %[kaddr] offset:2048\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[o0], %[a1], %[p0], %[o0]\n"
+        "ds_read_b128 %[a1], %[vaddr] offset:4096\n"
+        "global_load_lds_dwordx4 %[off], %[src] offset:0\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a2], %[q1], %[s]\n"
+        "ds_read_b128 %[a2], %[kaddr] offset:3072\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[o1], %[a3], %[p0], %[o1]\n"
+        "ds_read_b128 %[a3], %[vaddr] offset:6144\n"
+        "global_load_lds_dwordx4 %[off], %[src] offset:1024\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a0], %[q2], %[s]\n"
+        "ds_read_b128 %[a0], %[kaddr] offset:4096\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[o2], %[a1], %[p0], %[o2]\n"
+        "ds_read_b128 %[a1], %[vaddr] offset:8192\n"
+        "global_load_lds_dwordx4 %[off], %[src] offset:2048\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a2], %[q3], %[s]\n"
+        "ds_read_b128 %[a2], %[kaddr] offset:5120\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[o3], %[a3], %[p0], %[o3]\n"
+        "ds_read_b128 %[a3], %[vaddr] offset:10240\n"
+        "global_load_lds_dwordx4 %[off], %[src] offset:3072\n"
+        "s_add_u32 m0, m0, 0x1000\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a0], %[q4], %[s]\n"
+        "ds_read_b128 %[a0], %[kaddr] offset:6144\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[o4], %[a1], %[p0], %[o4]\n"
+        "ds_read_b128 %[a1], %[vaddr] offset:12288\n"
+        "global_load_lds_dwordx4 %[off], %[src2] offset:0\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a2], %[q5], %[s]\n"
+        "ds_read_b128 %[a2], %[kaddr] offset:7168\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[o5], %[a3], %[p0], %[o5]\n"
+        "ds_read_b128 %[a3], %[vaddr] offset:14336\n"
+        "global_load_lds_dwordx4 %[off], %[src2] offset:1024\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a0], %[q6], %[s]\n"
+        "ds_read_b128 %[a0], %[kaddr] offset:8192\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[o6], %[a1], %[p0], %[o6]\n"
+        "ds_read_b128 %[a1], %[vaddr] offset:1024\n"
+        "global_load_lds_dwordx4 %[off], %[src2] offset:2048\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a2], %[q7], %[s]\n"
+        "ds_read_b128 %[a2], %[kaddr] offset:9216\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[o7], %[a3], %[p0], %[o7]\n"
+        "ds_read_b128 %[a3], %[vaddr] offset:3072\n"
+        "global_load_lds_dwordx4 %[off], %[src2] offset:3072\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a0], %[q8], %[s]\n"
+        "ds_read_b128 %[a0], %[kaddr] offset:10240\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[o0], %[a1], %[p1], %[o0]\n"
+        "ds_read_b128 %[a1], %[vaddr] offset:5120\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a2], %[q9], %[s]\n"
+        "ds_read_b128 %[a2], %[kaddr] offset:11264\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[o1], %[a3], %[p1], %[o1]\n"
+        "ds_read_b128 %[a3], %[vaddr] offset:7168\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a0], %[q10], %[s]\n"
+        "ds_read_b128 %[a0], %[kaddr] offset:12288\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[o2], %[a1], %[p1], %[o2]\n"
+        "ds_read_b128 %[a1], %[vaddr] offset:9216\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a2], %[q11], %[s]\n"
+        "ds_read_b128 %[a2], %[kaddr] offset:13312\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[o3], %[a3], %[p1], %[o3]\n"
+        "ds_read_b128 %[a3], %[vaddr] offset:11264\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a0], %[q12], %[s]\n"
+        "ds_read_b128 %[a0], %[kaddr] offset:14336\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[o4], %[a1], %[p1], %[o4]\n"
+        "ds_read_b128 %[a1], %[vaddr] offset:13312\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a2], %[q13], %[s]\n"
+        "ds_read_b128 %[a2], %[kaddr] offset:15360\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[o5], %[a3], %[p1], %[o5]\n"
+        "ds_read_b128 %[a3], %[vaddr] offset:15360\n"
+        "s_waitcnt lgkmcnt(3)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a0], %[q14], %[s]\n"
+        "s_waitcnt lgkmcnt(2)\n"
+        "v_mfma_f32_32x32x16_f16 %[o6], %[a1], %[p1], %[o6]\n"
+        "s_waitcnt lgkmcnt(1)\n"
+        "v_mfma_f32_32x32x16_f16 %[s], %[a2], %[q15], %[s]\n"
+        "s_waitcnt lgkmcnt(0)\n"
+        "v_mfma_f32_32x32x16_f16 %[o7], %[a3], %[p1], %[o7]\n"
+        "s_nop 15\n"
+        "s_nop 3\n"
+        : [s] "=&v"(s), [o0] "+v"(o[0]), [o1] "+v"(o[1]), [o2] "+v"(o[2]), [o3] "+v"(o[3]), [o4] "+v"(o[4]),
+          [o5] "+v"(o[5]), [o6] "+v"(o[6]), [o7] "+v"(o[7]), [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2),
+          [a3] "=&v"(a3)
+        : [kaddr] "v"(kaddr), [vaddr] "v"(vaddr), [q0] "v"(q[0]), [q1] "v"(q[1]), [q2] "v"(q[2]), [q3] "v"(q[3]),
+          [q4] "v"(q[4]), [q5] "v"(q[5]), [q6] "v"(q[6]), [q7] "v"(q[7]), [q8] "v"(q[8]), [q9] "v"(q[9]),
+          [q10] "v"(q[10]), [q11] "v"(q[11]), [q12] "v"(q[12]), [q13] "v"(q[13]), [q14] "v"(q[14]), [q15] "v"(q[15]),
+          [p0] "v"(p[0]), [p1] "v"(p[1]), [off] "v"(lane16), [src] "s"(c.src), [src2] "s"(c.src + 4096),
+          [dst] "s"(c.dst)
         : "memory", "m0");
-#undef SAETTA_O_STEP
-#undef SAETTA_O_LAST
 }
-#undef SAETTA_COPY
 
 // The wait states after which vector ALU instructions may read what the last MFMAs wrote.
 __device__ __forceinline__ void settle(floatx16 (&o)[8]) {
@@ -391,11 +484,10 @@ __device__ __forceinline__ float max_across_halves(float x) {
     return fmaxf(__builtin_bit_cast(float, u), __builtin_bit_cast(float, v));
 }
 
-// LDS: four K slots, then four V^T slots.  Even blocks alternate between K slots 0 and 1, odd
-// blocks between 2 and 3 (an odd block's K is needed one step before its V^T, see the kernel).
+// LDS: four K slots, then four V^T slots; block b uses slot b % 4 of each.
 constexpr int MERGE_WAVE_BYTES = (8 * 16 + 2) * 64 * 4;  // one wave's O, m, l on their way to its partner
 constexpr int LDS_BYTES = 4 * MERGE_WAVE_BYTES > 8 * PART_BYTES ? 4 * MERGE_WAVE_BYTES : 8 * PART_BYTES;
-__device__ __forceinline__ uint32_t k_slot(uint32_t b) { return (((b & 1) << 1) | ((b >> 1) & 1)) * PART_BYTES; }
+__device__ __forceinline__ uint32_t k_slot(uint32_t b) { return (b & 3) * PART_BYTES; }
 __device__ __forceinline__ uint32_t v_slot(uint32_t b) { return (4 + (b & 3)) * PART_BYTES; }
 
 __global__ __launch_bounds__(THREADS, 2) void attention_prefill_kernel(PrefillArgs a) {
@@ -426,28 +518,30 @@ __global__ __launch_bounds__(THREADS, 2) void attention_prefill_kernel(PrefillAr
     const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(tiles));
     const uint32_t lane16 = lane * 16;
     const unsigned char *images = a.images + size_t(kv) * a.nblocks * IMG_BYTES;
-    // The wave's 4 KB number `quarter` (0..3) of part `v` (0 = K, 1 = V^T) of block b.  Blocks
-    // past the cache's end are read from the last image instead; nobody looks at their slots.
-    auto piece = [&](uint32_t b, int v, int quarter) {
+    // Half `half` (8 KB) of part `v` (0 = K, 1 = V^T) of block b.  Blocks past the cache's end
+    // are read from the last image instead; nobody looks at their slots.
+    auto piece = [&](uint32_t b, int v, int half) {
         const uint32_t bb = min(b, a.nblocks - 1);
         Copy cp;
-        cp.src = reinterpret_cast<uint64_t>(images) + uint64_t(bb) * IMG_BYTES + v * PART_BYTES + quarter * 4096;
-        cp.dst = lds0 + (v ? v_slot(b) : k_slot(b)) + quarter * 4096;
+        cp.src = reinterpret_cast<uint64_t>(images) + uint64_t(bb) * IMG_BYTES + v * PART_BYTES + half * 8192;
+        cp.dst = lds0 + (v ? v_slot(b) : k_slot(b)) + half * 8192;
         return cp;
     };
 
-    // Step s works on blocks 2s (even waves: parity 0) and 2s + 1 (parity 1).  The two waves of a
-    // SIMD are kept half a step apart, so that one's softmax runs under the other's MFMAs:
-    //   parity 0:  S(2s)       softmax(2s)     O(2s)
-    //   parity 1:  softmax(2s+1)   O(2s+1)     S(2s+3)
-    // so an odd block's K must be in LDS one step before its V^T.  During step s the workgroup
-    // copies K(2s+2), K(2s+5), V(2s+2), V(2s+3): wave w takes half (w % 2) of part w / 2 of that list.
-    // Before the loop: K(0), K(1), K(3), V(0), V(1), ten pieces per wave.
-    for (int i = wave; i < 40; i += WAVES) {
-        const int part = i >> 3, quarter = (i >> 1) & 3, v = part >= 3;
-        const uint32_t b = part == 0 ? 0 : part == 1 ? 1 : part == 2 ? 3 : part == 3 ? 0 : 1;
-        Copy cp = piece(b, v, quarter);
-        cp.src += (i & 1) * 2048, cp.dst += (i & 1) * 2048;
+    // Step s works on blocks 2s (waves 0..3: parity 0) and 2s + 1 (waves 4..7: parity 1).  A
+    // wave's step is a softmax (vector ALU) and an MFMA stream that adds the block to O and
+    // computes the scores of the wave's next block; the two waves of a SIMD run them in opposite
+    // order, so that one's softmax runs under the other's MFMAs:
+    //   parity 0:  softmax(2s)               | O(2s) + S(2s+2)
+    //   parity 1:  O(2s+1) + S(2s+3)         | softmax(2s+3)
+    // During step s the workgroup copies what step s + 1 reads: K(2s+4), K(2s+5), V(2s+2),
+    // V(2s+3); wave w takes half (w % 2) of part w / 2 of that list.  Before the loop: K(0..3),
+    // V(0), V(1), twelve kilobytes per wave.
+    for (int i = wave; i < 48; i += WAVES) {
+        const int part = i >> 3, v = part >= 4;
+        const uint32_t b = v ? part - 4 : part;
+        Copy cp = piece(b, v, 0);
+        cp.src += (i & 7) * 2048, cp.dst += (i & 7) * 2048;
         asm volatile(
             "s_mov_b32 m0, %[dst]\n"
             "s_nop 0\n"
@@ -527,62 +621,56 @@ __global__ __launch_bounds__(THREADS, 2) void attention_prefill_kernel(PrefillAr
     };
 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();  // K(0), K(1), K(3), V(0), V(1) are in LDS
+    __syncthreads();  // K(0..3), V(0), V(1) are in LDS
 
     const uint32_t nsteps = (nblocks + 1) / 2;
     const int part = wave >> 1, half = wave & 1;  // what the wave copies in every step
-    auto copies_of = [&](uint32_t step, Copy &first, Copy &second) {
-        const uint32_t cb = part == 0 ? 2 * step + 2 : part == 1 ? 2 * step + 5 : part == 2 ? 2 * step + 2 : 2 * step + 3;
-        first = piece(cb, part >= 2, 2 * half), second = piece(cb, part >= 2, 2 * half + 1);
+    auto copy_of = [&](uint32_t step) {
+        const uint32_t cb = part == 0 ? 2 * step + 4 : part == 1 ? 2 * step + 5 : part == 2 ? 2 * step + 2 : 2 * step + 3;
+        return piece(cb, part >= 2, half);
     };
     if (parity == 0) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();  // the odd waves compute S(1) here
+        floatx16 s;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = 0.0f;
+        if (0 < wave_blocks) scores_block(s, qb, lds0 + k_slot(0) + lane16);
+        __syncthreads();  // the first step's copies overwrite K(0) and K(1)
         for (uint32_t step = 0; step < nsteps; step++) {
-            Copy first, second;
-            copies_of(step, first, second);
+            const Copy cp = copy_of(step);
             const uint32_t kb = 2 * step;
             if (kb < wave_blocks) {
-                floatx16 s;
-                scores_block(s, qb, lds0 + k_slot(kb) + lane16, first, lane16);
                 raise_max(mask_max(s, kb * BK, kb >= full_blocks));
                 half8 pb[2];
                 exp_pack(s, pb);
-                accumulate_block(acc, pb, lds0 + v_slot(kb) + lane16, second, lane16);
+                // (past the wave's last block the scores are of stale keys and never looked at)
+                stream_block(s, acc, qb, pb, lds0 + k_slot(kb + 2) + lane16, lds0 + v_slot(kb) + lane16, cp, lane16);
             } else {
-                copy_plain(first, lane16);
-                copy_plain(second, lane16);
+                copy_plain(cp, lane16);
             }
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
         }
     } else {
-        // The odd waves enter the loop with the scores of block 1 in hand.
-        floatx16 s;
-#pragma unroll
-        for (int r = 0; r < 16; r++) s[r] = 0.0f;
+        half8 pb[2] = {};
         if (1 < wave_blocks) {
-            // (the copy it carries rewrites 4 KB of K(0) with themselves; nobody reads K(0) yet)
-            scores_block(s, qb, lds0 + k_slot(1) + lane16, piece(0, 0, 0), lane16);
+            floatx16 s;
+            scores_block(s, qb, lds0 + k_slot(1) + lane16);
+            raise_max(mask_max(s, BK, 1 >= full_blocks));
+            exp_pack(s, pb);
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         for (uint32_t step = 0; step < nsteps; step++) {
-            Copy first, second;
-            copies_of(step, first, second);
+            const Copy cp = copy_of(step);
             const uint32_t kb = 2 * step + 1;
             if (kb < wave_blocks) {
-                raise_max(mask_max(s, kb * BK, kb >= full_blocks));
-                half8 pb[2];
-                exp_pack(s, pb);
-                accumulate_block(acc, pb, lds0 + v_slot(kb) + lane16, first, lane16);
+                floatx16 s;
+                stream_block(s, acc, qb, pb, lds0 + k_slot(kb + 2) + lane16, lds0 + v_slot(kb) + lane16, cp, lane16);
+                if (kb + 2 < wave_blocks) {
+                    raise_max(mask_max(s, (kb + 2) * BK, kb + 2 >= full_blocks));
+                    exp_pack(s, pb);
+                }
             } else {
-                copy_plain(first, lane16);
-            }
-            if (kb + 2 < wave_blocks) {
-                scores_block(s, qb, lds0 + k_slot(kb + 2) + lane16, second, lane16);
-            } else {
-                copy_plain(second, lane16);
+                copy_plain(cp, lane16);
             }
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
