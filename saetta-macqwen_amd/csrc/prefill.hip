@@ -485,8 +485,8 @@ __device__ __forceinline__ float max_across_halves(float x) {
 }
 
 // LDS: four K slots, then four V^T slots; block b uses slot b % 4 of each.
-constexpr int MERGE_WAVE_BYTES = (8 * 16 + 2) * 64 * 4;  // one wave's O, m, l on their way to its partner
-constexpr int LDS_BYTES = 4 * MERGE_WAVE_BYTES > 8 * PART_BYTES ? 4 * MERGE_WAVE_BYTES : 8 * PART_BYTES;
+constexpr int MERGE_WAVE_BYTES = (4 * 16 + 2) * 64 * 4;  // half of a wave's O, its m and l, on their way to its partner
+constexpr int LDS_BYTES = 8 * MERGE_WAVE_BYTES > 8 * PART_BYTES ? 8 * MERGE_WAVE_BYTES : 8 * PART_BYTES;
 __device__ __forceinline__ uint32_t k_slot(uint32_t b) { return (b & 3) * PART_BYTES; }
 __device__ __forceinline__ uint32_t v_slot(uint32_t b) { return (4 + (b & 3)) * PART_BYTES; }
 
@@ -663,8 +663,12 @@ __global__ __launch_bounds__(THREADS, 2) void attention_prefill_kernel(PrefillAr
             const Copy cp = copy_of(step);
             const uint32_t kb = 2 * step + 1;
             if (kb < wave_blocks) {
+                // This wave's stream comes before its softmax, the other wave's of the SIMD after: let
+                // this one's MFMAs go first, so that its softmax still finds the other's to run under.
                 floatx16 s;
+                __builtin_amdgcn_s_setprio(2);
                 stream_block(s, acc, qb, pb, lds0 + k_slot(kb + 2) + lane16, lds0 + v_slot(kb) + lane16, cp, lane16);
+                __builtin_amdgcn_s_setprio(0);
                 if (kb + 2 < wave_blocks) {
                     raise_max(mask_max(s, (kb + 2) * BK, kb + 2 >= full_blocks));
                     exp_pack(s, pb);
@@ -680,31 +684,34 @@ __global__ __launch_bounds__(THREADS, 2) void attention_prefill_kernel(PrefillAr
     settle(acc);
 
     // ---- the two waves of a row group merge their halves of the keys ----------------------
-    // The odd-block wave hands O, m and l over through LDS (the tiles are done with: the loop
-    // ended on a barrier); element e of lane L sits at word e * 64 + L.
-    {
-        float *xchg = reinterpret_cast<float *>(tiles + group * MERGE_WAVE_BYTES) + lane;
-        if (parity == 1) {
+    // Each wave finishes half of the dims: parity 0 the accumulators 0..3 (dims 0..127), parity 1
+    // the rest.  It hands the other half, m and l to its partner through LDS (the tiles are done
+    // with: the loop ended on a barrier); element e of lane L sits at word e * 64 + L.
+    float *mine_out = reinterpret_cast<float *>(tiles + wave * MERGE_WAVE_BYTES) + lane;
+    const float *theirs_in = reinterpret_cast<const float *>(tiles + (wave ^ 4) * MERGE_WAVE_BYTES) + lane;
+    floatx16 fin[4];
+    if (parity == 0) {
 #pragma unroll
-            for (int mt = 0; mt < 8; mt++) {
+        for (int i = 0; i < 4; i++) {
+            fin[i] = acc[i];
 #pragma unroll
-                for (int r = 0; r < 16; r++) xchg[(16 * mt + r) * 64] = acc[mt][r];
-            }
-            xchg[128 * 64] = m_ref;
-            xchg[129 * 64] = l_sum;
+            for (int r = 0; r < 16; r++) mine_out[(16 * i + r) * 64] = acc[4 + i][r];
         }
-        __syncthreads();
-        if (parity == 1) return;
-        const float m_other = xchg[128 * 64], l_other = xchg[129 * 64];
-        const float m_new = fmaxf(m_ref, m_other);
-        const float mine = __builtin_amdgcn_exp2f(m_ref - m_new), theirs = __builtin_amdgcn_exp2f(m_other - m_new);
-        l_sum = l_sum * mine + l_other * theirs;
+    } else {
 #pragma unroll
-        for (int mt = 0; mt < 8; mt++) {
+        for (int i = 0; i < 4; i++) {
+            fin[i] = acc[4 + i];
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[mt][r] = acc[mt][r] * mine + xchg[(16 * mt + r) * 64] * theirs;
+            for (int r = 0; r < 16; r++) mine_out[(16 * i + r) * 64] = acc[i][r];
         }
     }
+    mine_out[64 * 64] = m_ref;
+    mine_out[65 * 64] = l_sum;
+    __syncthreads();
+    const float m_other = theirs_in[64 * 64], l_other = theirs_in[65 * 64];
+    const float m_new = fmaxf(m_ref, m_other);
+    const float mine = __builtin_amdgcn_exp2f(m_ref - m_new), theirs = __builtin_amdgcn_exp2f(m_other - m_new);
+    l_sum = l_sum * mine + l_other * theirs;
 
     // ---- out = O / l * sigmoid(gate) ---------------------------------------------------
     // The lane's row sum is split over the two lane halves (each saw half the keys).
@@ -712,21 +719,27 @@ __global__ __launch_bounds__(THREADS, 2) void attention_prefill_kernel(PrefillAr
     if (tok < a.tokens) {
         const float inv = 1.0f / l;
         const size_t row = size_t(tok) * a.heads + head;
-        const float *gate = a.q_and_gate + row * 2 * DIM + DIM;
-        float *out = a.out + row * DIM;
+        const float *gate = a.q_and_gate + row * 2 * DIM + DIM + 128 * parity;
+        float *out = a.out + row * DIM + 128 * parity;
+        // all the gate loads first: they are scattered 16-byte pieces, one round trip for the lot
+        float4 g[16];
 #pragma unroll
-        for (int mt = 0; mt < 8; mt++) {
+        for (int i = 0; i < 16; i++) g[i] = *reinterpret_cast<const float4 *>(gate + 32 * (i >> 2) + 8 * (i & 3) + 4 * hf);
 #pragma unroll
-            for (int q4 = 0; q4 < 4; q4++) {
-                const int d0 = 32 * mt + 8 * q4 + 4 * hf;
-                const float4 g = *reinterpret_cast<const float4 *>(gate + d0);
-                float4 o;
-                o.x = acc[mt][4 * q4 + 0] * inv / (1.0f + __expf(-g.x));
-                o.y = acc[mt][4 * q4 + 1] * inv / (1.0f + __expf(-g.y));
-                o.z = acc[mt][4 * q4 + 2] * inv / (1.0f + __expf(-g.z));
-                o.w = acc[mt][4 * q4 + 3] * inv / (1.0f + __expf(-g.w));
-                *reinterpret_cast<float4 *>(out + d0) = o;
+        for (int i = 0; i < 16; i++) {
+            const int mt = i >> 2, q4 = i & 3;
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int r = 4 * q4 + e;
+                o[e] = (fin[mt][r] * mine + theirs_in[(16 * mt + r) * 64] * theirs) * inv;
             }
+            float4 w;
+            w.x = o[0] * __builtin_amdgcn_rcpf(1.0f + __expf(-g[i].x));
+            w.y = o[1] * __builtin_amdgcn_rcpf(1.0f + __expf(-g[i].y));
+            w.z = o[2] * __builtin_amdgcn_rcpf(1.0f + __expf(-g[i].z));
+            w.w = o[3] * __builtin_amdgcn_rcpf(1.0f + __expf(-g[i].w));
+            *reinterpret_cast<float4 *>(out + 32 * mt + 8 * q4 + 4 * hf) = w;
         }
     }
 }
