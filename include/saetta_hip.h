@@ -129,6 +129,12 @@ int saetta_kv_quantize(saetta_stream_t stream, int bits, const float *x, saetta_
 int saetta_kv_dequantize(saetta_stream_t stream, int bits, saetta_quant_rows rows, uint16_t *out_f16,
                          saetta_kv_quant_params p);
 
+/* dequantize (src/kv_quant.rs:90-105), the CPU function: out f32
+ * [groups][64] = f32(scale) * code + f32(bias), not rounded to half.  With
+ * saetta_kv_quantize before it this is round_trip (src/kv_quant.rs:107-117). */
+int saetta_kv_dequantize_f32(saetta_stream_t stream, int bits, saetta_quant_rows rows, float *out,
+                             saetta_kv_quant_params p);
+
 /* to_half (kernels/prefill.metal:1428-1432; src/prefill.rs:1658-1660,1690-1692):
  * n floats to halves, round to nearest even. */
 int saetta_to_half(saetta_stream_t stream, const float *x, uint16_t *out_f16, size_t n);

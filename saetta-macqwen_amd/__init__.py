@@ -10,7 +10,9 @@ be checked), every call needs the library and a gfx950 device.
 """
 from . import ffi
 from .host import (GROUP, MAX_ROWS, AttentionRows, Built, DecodeAttention, FlashParams, KvBits, Plan,
-                   QuantRows, TokenParams, attention_prefill, to_half)
+                   QuantRows, TokenParams, attention_prefill, bench, dequantize, quantize, round_trip,
+                   round_trip_as_half, test_slack, to_half)
 
 __all__ = ["ffi", "GROUP", "MAX_ROWS", "AttentionRows", "Built", "DecodeAttention", "FlashParams", "KvBits",
-           "Plan", "QuantRows", "TokenParams", "attention_prefill", "to_half"]
+           "Plan", "QuantRows", "TokenParams", "attention_prefill", "bench", "dequantize", "quantize",
+           "round_trip", "round_trip_as_half", "test_slack", "to_half"]

@@ -123,6 +123,33 @@ __global__ __launch_bounds__(256) void kv_dequantize_kernel(const uint32_t *__re
     }
 }
 
+// s * q + z in f32 (one rounding in the multiply, which is exact, and one in the add): what
+// dequantize() returns on the CPU (src/kv_quant.rs:90-105), i.e. round_trip of the input.
+template <int BITS>
+__global__ __launch_bounds__(256) void kv_dequantize_f32_kernel(const uint32_t *__restrict__ data,
+                                                                const uint16_t *__restrict__ scales,
+                                                                const uint16_t *__restrict__ biases,
+                                                                float *__restrict__ out, saetta_kv_quant_params p) {
+    constexpr int VPL = 32 / BITS;
+    constexpr int LANES = SAETTA_QUANT_GROUP / VPL;
+    const uint32_t word = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t g = word / LANES;
+    if (g >= p.groups) return;
+    const uint32_t w = data[word];
+    const float s = __half2float(__ushort_as_half(scales[g]));
+    const float z = __half2float(__ushort_as_half(biases[g]));
+    float4 *dst = reinterpret_cast<float4 *>(out) + size_t(word) * (VPL / 4);
+#pragma unroll
+    for (int i = 0; i < VPL; i += 4) {
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            o[e] = __fadd_rn(__fmul_rn(s, float((w >> ((i + e) * BITS)) & ((1u << BITS) - 1))), z);
+        }
+        dst[i / 4] = make_float4(o[0], o[1], o[2], o[3]);
+    }
+}
+
 // f32 -> f16, four values per lane.
 __global__ __launch_bounds__(256) void to_half_kernel(const float *__restrict__ x,
                                                       uint16_t *__restrict__ out, size_t n) {
@@ -184,6 +211,23 @@ extern "C" int saetta_kv_dequantize(saetta_stream_t stream, int bits, saetta_qua
                                                                        rows.biases, out_f16, p);
     }
     return launch_status("kv_dequantize");
+}
+
+extern "C" int saetta_kv_dequantize_f32(saetta_stream_t stream, int bits, saetta_quant_rows rows, float *out,
+                                        saetta_kv_quant_params p) {
+    SAETTA_REQUIRE(bits == 8 || bits == 4, SAETTA_E_BITS, "kv_dequantize_f32: bits %d (8 or 4)", bits);
+    SAETTA_REQUIRE(out && rows.data && rows.scales && rows.biases, SAETTA_E_NULL, "kv_dequantize_f32: null buffer");
+    SAETTA_REQUIRE(aligned(out, 16), SAETTA_E_ALIGN, "kv_dequantize_f32: out must be 16-byte aligned");
+    if (int rc = ensure_device()) return rc;
+    if (p.groups == 0) return SAETTA_OK;
+    const uint32_t lanes = bits == 8 ? 16 : 8;
+    const uint32_t blocks = (p.groups * lanes + 255) / 256;
+    if (bits == 8) {
+        kv_dequantize_f32_kernel<8><<<blocks, 256, 0, as_stream(stream)>>>(rows.data, rows.scales, rows.biases, out, p);
+    } else {
+        kv_dequantize_f32_kernel<4><<<blocks, 256, 0, as_stream(stream)>>>(rows.data, rows.scales, rows.biases, out, p);
+    }
+    return launch_status("kv_dequantize_f32");
 }
 
 extern "C" int saetta_to_half(saetta_stream_t stream, const float *x, uint16_t *out_f16, size_t n) {

@@ -7,7 +7,7 @@ LIB_PATH = os.environ.get("SAETTA_HIP_LIB") or os.path.join(_HERE, "lib", "libsa
 
 # Every symbol include/saetta_hip.h declares; tests check the library exports each.
 SYMBOLS = [
-    "saetta_init", "saetta_last_error", "saetta_kv_quantize", "saetta_kv_dequantize", "saetta_to_half",
+    "saetta_init", "saetta_last_error", "saetta_kv_quantize", "saetta_kv_dequantize", "saetta_kv_dequantize_f32", "saetta_to_half",
     "saetta_part_o_bytes", "saetta_part_ml_bytes", "saetta_attn_decode", "saetta_attn_decode_quant",
     "saetta_attn_rows", "saetta_attn_rows_quant", "saetta_prefill_workspace_bytes", "saetta_attn_prefill", "saetta_attn_prefill_quant",
 ]
@@ -64,6 +64,8 @@ def lib():
         l.saetta_kv_quantize.argtypes = [vp, i32, vp, QuantRowsC, KvQuantParamsC, vp, u32]
         l.saetta_kv_dequantize.restype = i32
         l.saetta_kv_dequantize.argtypes = [vp, i32, QuantRowsC, vp, KvQuantParamsC]
+        l.saetta_kv_dequantize_f32.restype = i32
+        l.saetta_kv_dequantize_f32.argtypes = [vp, i32, QuantRowsC, vp, KvQuantParamsC]
         l.saetta_to_half.restype, l.saetta_to_half.argtypes = i32, [vp, vp, vp, sz]
         l.saetta_part_o_bytes.restype, l.saetta_part_o_bytes.argtypes = sz, [u32, u32, u32]
         l.saetta_part_ml_bytes.restype, l.saetta_part_ml_bytes.argtypes = sz, [u32, u32, u32]

@@ -172,6 +172,54 @@ class QuantRows:
                   "kv_dequantize")
 
 
+def quantize(x, bits, stream=None):
+    """quantize (src/kv_quant.rs:54-87) of a device f32 tensor whose length is a multiple of
+    64: (codes int32 [groups * 2 * bits], scales f16 [groups], biases f16 [groups])."""
+    _need(x, torch.float32, "quantize x")
+    if bits is KvBits.Half or x.numel() % GROUP:
+        raise ValueError("quantize: bits must be Eight or Four and the length a multiple of 64")
+    rows = QuantRows(bits, GROUP, x.numel() // GROUP, device=x.device)
+    rows.encode(x, 0, x.numel() // GROUP, stream)
+    return rows.data, rows.scales, rows.biases
+
+
+def dequantize(data, scales, biases, bits, stream=None):
+    """dequantize (src/kv_quant.rs:90-105): f32 [groups * 64] = f32(s) * code + f32(z)."""
+    _need(data, torch.int32, "dequantize data"), _need(scales, torch.float16, "dequantize scales")
+    _need(biases, torch.float16, "dequantize biases")
+    groups = scales.numel()
+    if bits is KvBits.Half or data.numel() != groups * bits.words_per_group() or biases.numel() != groups:
+        raise ValueError("dequantize: sizes do not match the bit width")
+    out = torch.empty(groups * GROUP, dtype=torch.float32, device=data.device)
+    rows = ffi.QuantRowsC(data.data_ptr(), scales.data_ptr(), biases.data_ptr())
+    ffi.check(ffi.lib().saetta_kv_dequantize_f32(_stream(stream), bits.value, rows, _ptr(out),
+                                                 ffi.KvQuantParamsC(groups, groups)), "kv_dequantize_f32")
+    return out
+
+
+def round_trip(x, bits, stream=None):
+    """round_trip (src/kv_quant.rs:107-117): what a decode cache holds of x."""
+    if bits is KvBits.Half:
+        return x.to(torch.float16).to(torch.float32)
+    return dequantize(*quantize(x, bits, stream), bits, stream)
+
+
+def round_trip_as_half(x, bits, stream=None):
+    """round_trip_as_half (src/kv_quant.rs:119-125): what prefill sees of x, f16."""
+    if bits is KvBits.Half:
+        return x.to(torch.float16)
+    rows = QuantRows(bits, GROUP, x.numel() // GROUP, device=x.device)
+    rows.encode(x, 0, x.numel() // GROUP, stream)
+    out = torch.empty(x.numel(), dtype=torch.float16, device=x.device)
+    rows.encode_dequantize(out, x.numel() // GROUP, stream)
+    return out
+
+
+def test_slack(bits):
+    """test_slack (src/kv_quant.rs:127-135): how much looser a test bound is per cache kind."""
+    return {KvBits.Half: 1.0, KvBits.Eight: 4.0, KvBits.Four: 16.0}[bits]
+
+
 def to_half(x, out, stream=None):
     """to_half (kernels/prefill.metal:1428-1432)."""
     _need(x, torch.float32, "to_half x")
@@ -235,6 +283,56 @@ class DecodeAttention:
 
         plan.op(f"{self.kernel}_q{bits}", launch(ffi.STAGE_PARTIAL))
         plan.op("attention_reduce", launch(ffi.STAGE_REDUCE))
+
+
+def _median_ms(run, runs):
+    """One warm-up, then the median of `runs` event-timed calls, in milliseconds."""
+    ts = []
+    for i in range(runs + 1):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        run()
+        e1.record()
+        e1.synchronize()
+        if i:
+            ts.append(e0.elapsed_time(e1))
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+def bench(lengths, layers, runs, bits=KvBits.Half, device="cuda"):
+    """attention::bench (src/attention.rs:173-231): one token's attention over `layers` caches of
+    their own, at each context length; same fill values, median of `runs` after a warm-up,
+    bytes = layers * len * token * 2 (K, V) * bytes per value.  Returns one dict per length."""
+    heads, kv = 16, 2
+    capacity = -(-max(lengths) // CHUNK) * CHUNK
+    token = kv * DIM
+    i = torch.arange(capacity * token, device=device, dtype=torch.int64)
+    fill = (((i * 7919) % 2000).to(torch.float32) / 1000.0 - 1.0)
+    caches = []
+    for _ in range(layers):
+        if bits is KvBits.Half:
+            caches.append((fill.to(torch.float16), fill.to(torch.float16)))
+        else:
+            k, v = QuantRows(bits, token, capacity, device), QuantRows(bits, token, capacity, device)
+            k.encode(fill, 0, capacity), v.encode(fill, 0, capacity)
+            caches.append((k, v))
+    q = torch.full((heads * DIM,), 0.01, device=device)
+    qg = torch.full((heads * 2 * DIM,), 0.5, device=device)
+    out = torch.empty(heads * DIM, device=device)
+    att = DecodeAttention(heads, kv, DIM, capacity, device)
+    plan = Plan(device)
+    for k, v in caches:
+        (att.record if bits is KvBits.Half else att.record_quant)(plan, q, k, v, qg, out)
+    built = plan.build(graph=True)
+    reduce = plan.build_where(lambda name: name == "attention_reduce", graph=True)
+    rows = []
+    for n in lengths:
+        plan.set_params(TokenParams(0, n - 1))
+        ms, reduce_ms = _median_ms(built.run, runs), _median_ms(reduce.run, runs)
+        nbytes = layers * n * token * 2 * bits.bytes_per_value()
+        rows.append({"tokens": n, "ms": ms, "GB/s": nbytes / ms / 1e6, "reduce_ms": reduce_ms})
+    return rows
 
 
 class AttentionRows:
@@ -333,6 +431,66 @@ class attention_prefill:
         ffi.check(ffi.lib().saetta_attn_prefill(_stream(stream), _ptr(q), _ptr(keys), _ptr(values),
                                                 _ptr(q_and_gate), _ptr(out), p.c(), *_workspace(workspace)),
                   "attn_prefill")
+
+    @staticmethod
+    def encode_rows2(q, keys, values, q_and_gate, out, p, stream=None, workspace=None):
+        """encode_rows2 (src/attention_prefill.rs:74-100): the reference's attention_rows2_half on
+        the same buffers, its baseline in `bench`; here the same kernel as `encode`."""
+        attention_prefill.encode(attention_prefill.DEFAULT, q, keys, values, q_and_gate, out, p, stream, workspace)
+
+    @staticmethod
+    def spread(n, seed, device="cuda"):
+        """spread (src/attention_prefill.rs:102-108): half values in about -2 .. 2.  Test data,
+        made on the host in IEEE f32 (one division, one subtraction, one rounding to half) and
+        copied to the device."""
+        import numpy as np
+        i = np.arange(n, dtype=np.int64)
+        x = ((i * 7919 + seed * 104729) % 1999).astype(np.float32) / np.float32(500.0) - np.float32(2.0)
+        return torch.from_numpy(x.astype(np.float16)).to(device)
+
+    @staticmethod
+    def bench(contexts, chunk, layers, device="cuda"):
+        """bench (src/attention_prefill.rs:110-176): a chunk of `chunk` tokens at the middle and at
+        the end of a prefill of each context, best of 3 after a warm-up; TFLOP/s by the causal
+        count 4 * heads * dim * (chunk * pos + chunk * (chunk + 1) / 2).  One dict per context."""
+        heads, kv, dim = 16, 2, DIM
+        rows = []
+        for n in contexts:
+            n = -(-n // chunk) * chunk
+            capacity = -(-n // 64) * 64 + 64
+            q = attention_prefill.spread(chunk * heads * dim, 1, device)
+            k = attention_prefill.spread(capacity * kv * dim, 2, device)
+            v = attention_prefill.spread(capacity * kv * dim, 3, device)
+            g = ((torch.arange(chunk * heads * 2 * dim, device=device) % 7) - 3).to(torch.float32)
+            out = torch.empty(chunk * heads * dim, dtype=torch.float32, device=device)
+            chunks = n // chunk
+            mid, last = (chunks // 2) * chunk, n - chunk
+
+            def flops(pos):
+                return 4.0 * heads * dim * (chunk * pos + chunk * (chunk + 1) / 2)
+
+            def best_ms(pos):
+                p = FlashParams(heads, kv, pos, chunk, 1.0 / math.sqrt(dim))
+                ws = torch.empty(attention_prefill.workspace_bytes(p), dtype=torch.uint8, device=device)
+
+                def run():
+                    attention_prefill.encode(attention_prefill.DEFAULT, q, k, v, g, out, p, workspace=ws)
+
+                run()
+                best = float("inf")
+                for _ in range(3):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    run()
+                    e1.record()
+                    e1.synchronize()
+                    best = min(best, e0.elapsed_time(e1))
+                return best
+
+            tm, tl = best_ms(mid), best_ms(last)
+            rows.append({"context": n, "chunk": chunk, "last_ms": tl, "last_TFLOP/s": flops(last) / tl / 1e9,
+                         "mid_TFLOP/s": flops(mid) / tm / 1e9, "prefill_attention_s": tm * 1e-3 * chunks * layers})
+        return rows
 
     @staticmethod
     def encode_quant(q, keys, values, q_and_gate, out, p, stream=None, workspace=None):

@@ -211,6 +211,61 @@ struct QuantRows {
     }
 };
 
+// The CPU-side functions of src/kv_quant.rs:54-135 with host vectors in and out; the arithmetic
+// runs on the device (the same kernels the cache uses), so the results are the cache's own.
+struct Quantized {
+    std::vector<uint32_t> data;
+    std::vector<uint16_t> scales, biases;  // f16 bits
+};
+
+template <typename T>
+inline std::vector<T> download(const gpu::Gpu &gpu, const gpu::Buffer &b, size_t n) {
+    gpu.sync();
+    return gpu::contents<T>(b, n);
+}
+
+inline Quantized quantize(const gpu::Gpu &gpu, const std::vector<float> &x, KvBits b) {
+    if (x.size() % GROUP != 0) throw std::runtime_error("quantize: length must be a multiple of 64");
+    const size_t groups = x.size() / GROUP;
+    QuantRows rows(gpu, b, GROUP, groups);
+    rows.encode(gpu, View(gpu.buffer_from(x)), 0, groups);
+    return Quantized{download<uint32_t>(gpu, rows.data, groups * words_per_group(b)), download<uint16_t>(gpu, rows.scales, groups),
+                     download<uint16_t>(gpu, rows.biases, groups)};
+}
+
+inline std::vector<float> dequantize(const gpu::Gpu &gpu, const Quantized &q, KvBits b) {
+    const size_t groups = q.scales.size();
+    if (b == KvBits::Half || q.data.size() != groups * words_per_group(b) || q.biases.size() != groups)
+        throw std::runtime_error("dequantize: sizes do not match the bit width");
+    const gpu::Buffer data = gpu.buffer_from(q.data), scales = gpu.buffer_from(q.scales), biases = gpu.buffer_from(q.biases);
+    const gpu::Buffer out = gpu.buffer(groups * GROUP * 4);
+    const saetta_quant_rows rows{static_cast<uint32_t *>(data.get()), static_cast<uint16_t *>(scales.get()),
+                                 static_cast<uint16_t *>(biases.get())};
+    check(saetta_kv_dequantize_f32(gpu.stream(), int(bits(b)), rows, static_cast<float *>(out.get()),
+                                   saetta_kv_quant_params{uint32_t(groups), uint32_t(groups)}),
+          "kv_dequantize_f32");
+    return download<float>(gpu, out, groups * GROUP);
+}
+
+// x after a round trip through the cache, as a decode cache holds it.  (A half cache rounds to
+// half; that case is left to the caller's own half type.)
+inline std::vector<float> round_trip(const gpu::Gpu &gpu, const std::vector<float> &x, KvBits b) {
+    if (b == KvBits::Half) throw std::runtime_error("round_trip: a half cache is a plain conversion to half");
+    return dequantize(gpu, quantize(gpu, x, b), b);
+}
+
+// ... and through the half copy prefill attention reads (f16 bits).
+inline std::vector<uint16_t> round_trip_as_half(const gpu::Gpu &gpu, const std::vector<float> &x, KvBits b) {
+    const size_t groups = x.size() / GROUP;
+    QuantRows rows(gpu, b, GROUP, groups);
+    rows.encode(gpu, View(gpu.buffer_from(x)), 0, groups);
+    const gpu::Buffer out = gpu.buffer(x.size() * 2);
+    rows.encode_dequantize(gpu, View(out), groups);
+    return download<uint16_t>(gpu, out, x.size());
+}
+
+inline float test_slack(KvBits b) { return b == KvBits::Half ? 1.0f : b == KvBits::Eight ? 4.0f : 16.0f; }
+
 }  // namespace kv_quant
 
 namespace attention {
@@ -359,6 +414,24 @@ inline void encode(const gpu::Gpu &gpu, const std::string &kernel, const View &q
     check(saetta_attn_prefill(gpu.stream(), q.ptr<uint16_t>(), keys.ptr<uint16_t>(), values.ptr<uint16_t>(), q_and_gate.ptr<float>(),
                               out.ptr<float>(), p, ws.ptr, ws.bytes),
           "attn_prefill");
+}
+
+// encode_rows2 (src/attention_prefill.rs:74-100): the reference's attention_rows2_half on the same
+// buffers, its baseline in `bench`; here the same kernel as `encode`.
+inline void encode_rows2(const gpu::Gpu &gpu, const View &q, const View &keys, const View &values, const View &q_and_gate,
+                         const View &out, FlashParams p, const Workspace &ws = {}) {
+    encode(gpu, DEFAULT, q, keys, values, q_and_gate, out, p, ws);
+}
+
+// spread (src/attention_prefill.rs:102-108): half values in about -2 .. 2, as f16 bits.
+inline std::vector<uint16_t> spread(size_t n, size_t seed) {
+    std::vector<uint16_t> out(n);
+    for (size_t i = 0; i < n; i++) {
+        const float x = float((i * 7919 + seed * 104729) % 1999) / 500.0f - 2.0f;
+        const _Float16 h = static_cast<_Float16>(x);
+        std::memcpy(&out[i], &h, 2);
+    }
+    return out;
 }
 
 // The same chunk over a quantized cache read in place (src/prefill.rs:1735-1776).

@@ -138,6 +138,36 @@ int main() {
             }
         }
     }
+    // The module functions of src/kv_quant.rs (quantize, dequantize, round_trip, round_trip_as_half,
+    // test_slack) and attention_prefill::spread, against the oracle.
+    for (KvBits bits : {KvBits::Eight, KvBits::Four}) {
+        const int b = int(kv_quant::bits(bits));
+        std::vector<float> x(9 * VALUES);
+        orc_quant_rows(x.data(), 9, VALUES);
+        const size_t groups = x.size() / 64, words = kv_quant::words_per_group(bits);
+        std::vector<uint32_t> wd(groups * words);
+        std::vector<uint16_t> ws(groups), wz(groups);
+        orc_quantize(x.data(), x.size(), b, wd.data(), ws.data(), wz.data());
+        const auto q = kv_quant::quantize(gpu, x, bits);
+        EXPECT(q.data == wd && q.scales == ws && q.biases == wz, "%d-bit quantize() differs from the CPU", b);
+        std::vector<float> want(x.size());
+        orc_dequantize(wd.data(), ws.data(), wz.data(), groups, b, want.data());
+        const auto back = kv_quant::round_trip(gpu, x, bits);
+        EXPECT(std::memcmp(back.data(), want.data(), want.size() * 4) == 0, "%d-bit round_trip differs", b);
+        const auto half = kv_quant::round_trip_as_half(gpu, x, bits);
+        size_t off = 0;
+        for (size_t i = 0; i < want.size(); i++) off += half[i] != orc_f32_to_f16(want[i]);
+        EXPECT(off == 0, "%d-bit round_trip_as_half: %zu values differ", b, off);
+        EXPECT(kv_quant::test_slack(bits) == (b == 8 ? 4.0f : 16.0f), "test_slack");
+    }
+    {
+        const auto s = attention_prefill::spread(4000, 2);
+        size_t off = 0;
+        for (size_t i = 0; i < s.size(); i++) {
+            off += s[i] != orc_f32_to_f16(float((i * 7919 + 2 * 104729) % 1999) / 500.0f - 2.0f);
+        }
+        EXPECT(off == 0 && s.size() == 4000, "spread: %zu values differ", off);
+    }
     // shape checks panic (throw) as the reference asserts
     bool threw = false;
     try {

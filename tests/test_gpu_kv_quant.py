@@ -133,3 +133,26 @@ def test_to_half_rounds_to_nearest_even():
     out = torch.zeros(x.size, dtype=torch.float16, device="cuda")
     saetta.to_half(dev(x), out)
     assert np.array_equal(host(out).view(np.uint16), oracle.f32_to_f16_bits(x))
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_module_functions_match_cpu(kind):
+    # quantize / dequantize / round_trip / round_trip_as_half of src/kv_quant.rs:54-125 as device functions.
+    bits = kind.value
+    x = oracle.quant_rows(11)
+    data, scales, biases = saetta.quantize(dev(x), kind)
+    wd, ws, wz = oracle.quantize(x, bits)
+    assert np.array_equal(host(data).view(np.uint32), wd)
+    assert np.array_equal(host(scales).view(np.uint16), ws) and np.array_equal(host(biases).view(np.uint16), wz)
+    back = host(saetta.dequantize(data, scales, biases, kind))
+    assert np.array_equal(back.view(np.uint32), oracle.dequantize(wd, ws, wz, bits).view(np.uint32))
+    assert np.array_equal(host(saetta.round_trip(dev(x), kind)).view(np.uint32),
+                          oracle.round_trip(x, bits).reshape(-1).view(np.uint32))
+    as_half = host(saetta.round_trip_as_half(dev(x), kind)).astype(np.float32)
+    assert np.array_equal(as_half, oracle.round_trip_as_half(x, bits).reshape(-1))
+    # the half step bound of src/kv_quant.rs:302-317, on the device result
+    step = host(scales).astype(np.float32).repeat(64)
+    assert (np.abs(back - x.reshape(-1)) <= 0.5 * step + 2e-3 * np.abs(x.reshape(-1)).max()).all()
+    assert saetta.test_slack(kind) == {8: 4.0, 4: 16.0}[bits] and saetta.test_slack(saetta.KvBits.Half) == 1.0
+    half = host(saetta.round_trip(dev(x), saetta.KvBits.Half))
+    assert np.array_equal(half, x.reshape(-1).astype(np.float16).astype(np.float32))

@@ -154,3 +154,28 @@ def test_shape_and_argument_checks():
         saetta.attention_prefill.encode("attention_fa8", q, kc, kc, qg, out, saetta.FlashParams(H, 4, 0, 1, 0.0625))
     # zero tokens: nothing to do
     saetta.attention_prefill.encode("attention_fa8", q, kc, kc, qg, out, saetta.FlashParams(H, KV, 0, 0, 0.0625))
+
+
+def test_spread_rows2_and_bench_mirror_the_reference():
+    # spread (src/attention_prefill.rs:102-108) against the oracle's restatement
+    got = host(saetta.attention_prefill.spread(5000, 3)).astype(np.float32)
+    assert np.array_equal(got, oracle.spread(5000, 3).astype(np.float32))
+    # encode_rows2 is the same computation as encode
+    pos, tokens = 40, 24
+    n = pos + tokens
+    q16 = oracle.spread(tokens * H * D, 1).reshape(tokens, H, D)
+    k = torch.from_numpy(oracle.spread(n * VALUES, 2)).cuda()
+    v = torch.from_numpy(oracle.spread(n * VALUES, 3)).cuda()
+    qg = dev(((np.arange(tokens * H * 2 * D) % 7) - 3).astype(np.float32))
+    q = torch.from_numpy(q16).cuda()
+    a, b = torch.empty(tokens, H, D, device="cuda"), torch.empty(tokens, H, D, device="cuda")
+    p = saetta.FlashParams(H, KV, pos, tokens, 1 / 16)
+    saetta.attention_prefill.encode("attention_fa4", q, k, v, qg, a, p)
+    saetta.attention_prefill.encode_rows2(q, k, v, qg, b, p)
+    assert torch.equal(a, b)
+    # bench of both modules on toy sizes: shapes and sanity of what they report
+    rows = saetta.attention_prefill.bench([100], 64, 2)
+    assert rows[0]["context"] == 128 and rows[0]["last_TFLOP/s"] > 0 and rows[0]["mid_TFLOP/s"] > 0
+    for bits in (saetta.KvBits.Half, saetta.KvBits.Eight):
+        rows = saetta.bench([256, 1000], 2, 3, bits)
+        assert [r["tokens"] for r in rows] == [256, 1000] and all(r["GB/s"] > 0 and r["reduce_ms"] > 0 for r in rows)
