@@ -40,6 +40,13 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
+# HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE and WRITE_SIZE of
+# rocprofv3 --pmc, each scaled by what the same counter reads for a 256 MiB copy in the same run;
+# the runs are summarised in profiles/*_hbm_traffic.txt).  Counters cannot be read inside this
+# script, so the figures are carried here for the workloads they were measured on.
+MEASURED_TRAFFIC = {"decode8_32k": 46.4e6, "prefill": 376.4e6}
+
+
 def median(xs):
     xs = sorted(xs)
     return xs[len(xs) // 2]
@@ -167,7 +174,7 @@ def bench_decode(s, torch, args, ctx, bits, rows, layers):
         "config": {"workload": name, "heads": H, "kv_heads": KV, "head_dim": D, "ctx": ctx, "kv_bits": bits,
                    "rows": rows, "layers_per_step": layers, "bytes_per_layer": layer_bytes},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("decode8_32k") if (ctx, bits, rows) == (32768, 8, 1) else None,
                      "kernel": "attention_partial_kernel", "avg_us": round(part_us, 3),
                      "min_us": round(part_us_min, 3), "reduce_kernel_us": round(red_us, 3)},
         "cpu_baseline": {"value": round(layer_bytes / cpu1 / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
@@ -250,7 +257,8 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8):
                                "read in place, chunk K/V quantized on append inside the step",
                    "heads": H, "kv_heads": KV, "head_dim": D, "flops": flops},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC.get("prefill") if (tokens, pos, bits) == (4096, 4096, 8) else None,
                      "kernel": "attention_prefill_kernel", "avg_us": round(kern_us, 2)},
         "cpu_baseline": {"value": round(cpu_flops / cpu_s / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
                          "sample": f"the last {sample} tokens of the chunk ({cpu_s:.2f} s)"},
@@ -267,6 +275,9 @@ def main():
                     choices=["decode8_32k", "decode4_150k", "verify2", "verify3", "verify4", "prefill", "all"])
     ap.add_argument("--no-graph", action="store_true", help="launch from Python instead of replaying a HIP graph")
     ap.add_argument("--layers", type=int, default=0, help="layer caches per step (default 32; 12 at 150k)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first run a plain device copy of 256 MiB (three times): a kernel of known traffic for a "
+                         "hardware-counter run of the same command to be scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -279,6 +290,13 @@ def main():
         print("bench.py needs a GPU (there is no CPU fallback)", file=sys.stderr)
         sys.exit(1)
     s.ffi.check(s.ffi.lib().saetta_init(), "init")
+    if args.calibrate_copy:
+        src = torch.ones(64 << 20, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     def one(workload):
         if workload == "decode8_32k":
