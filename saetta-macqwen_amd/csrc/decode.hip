@@ -858,11 +858,15 @@ uint32_t splits_for(uint32_t capacity, uint32_t wanted) {
 }
 
 template <int BITS, int TILES, bool PACKED>
-void launch_partial(hipStream_t stream, const PartialArgs &a) {
+void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu) {
     using Sh = Shape<BITS, TILES, PACKED>;
     void (*kernel)(PartialArgs);
-    if constexpr (TILES == 1 && BITS != 16) {
-        kernel = attention_partial_kernel_1<BITS, PACKED>;
+    if constexpr (TILES == 1 && BITS != 16 && PACKED) {
+        if (one_per_cu) {
+            kernel = attention_partial_kernel_p<BITS>;
+        } else {
+            kernel = attention_partial_kernel_1<BITS, PACKED>;
+        }
     } else if constexpr (PACKED) {
         kernel = attention_partial_kernel_p<BITS>;  // f16 cache: its registers do not fit two waves
     } else {
@@ -878,15 +882,15 @@ void launch_partial(hipStream_t stream, const PartialArgs &a) {
 }
 
 template <int BITS>
-void launch_partial_rows(hipStream_t stream, const PartialArgs &a) {
+void launch_partial_rows(hipStream_t stream, const PartialArgs &a, bool one_per_cu) {
     if (a.rows == 1) {
-        launch_partial<BITS, 1, true>(stream, a);
+        launch_partial<BITS, 1, true>(stream, a, one_per_cu);
     } else if (a.rows == 2) {
-        launch_partial<BITS, 1, false>(stream, a);
+        launch_partial<BITS, 1, false>(stream, a, one_per_cu);
     } else if (a.rows <= 4) {
-        launch_partial<BITS, 2, false>(stream, a);
+        launch_partial<BITS, 2, false>(stream, a, one_per_cu);
     } else {
-        launch_partial<BITS, 4, false>(stream, a);
+        launch_partial<BITS, 4, false>(stream, a, one_per_cu);
     }
 }
 
@@ -911,16 +915,23 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
     SAETTA_REQUIRE(bits == 16 || (aligned(ks, 8) && aligned(kz, 8) && aligned(vs, 8) && aligned(vz, 8)),
                    SAETTA_E_ALIGN, "%s: scales and biases must be 8-byte aligned", what);
     if (int rc = ensure_device()) return rc;
-    const uint32_t nsplits = splits_for(capacity, wanted_splits);
+    uint32_t nsplits = splits_for(capacity, wanted_splits);
+    // One workgroup per CU (half as many splits, each twice as long) or two.  Two rows and more and a
+    // half cache need the whole register file anyway; one row over codes fits two workgroups per CU,
+    // which pays only for long contexts: up to 64k tokens the shorter merge of half as many partials
+    // is worth more (measured: 19.4 against 20.6 us per layer at 32k, 28.3 against 29.7 at 64k,
+    // but 44 against 35 at 146k, 4-bit).  Both stages derive the same number from the same arguments.
+    const bool one_per_cu = rows >= 2 || bits == 16 || capacity <= 80 * 1024;
+    if (one_per_cu && nsplits > MAX_SPLITS / 2) nsplits = MAX_SPLITS / 2;
     if (stages & SAETTA_STAGE_PARTIAL) {
         PartialArgs a{q,     kdata,    vdata,    ks,    kz,   vs,      vz,   part_o, part_ml,
                       heads, kv_heads, capacity, scale, rows, nsplits, d_tp, decode_len ? 1u : 0u};
         if (bits == 8) {
-            launch_partial_rows<8>(stream, a);
+            launch_partial_rows<8>(stream, a, one_per_cu);
         } else if (bits == 4) {
-            launch_partial_rows<4>(stream, a);
+            launch_partial_rows<4>(stream, a, one_per_cu);
         } else {
-            launch_partial_rows<16>(stream, a);
+            launch_partial_rows<16>(stream, a, one_per_cu);
         }
     }
     if (stages & SAETTA_STAGE_REDUCE) {
