@@ -802,17 +802,31 @@ __global__ __launch_bounds__(256) void attention_reduce_kernel(ReduceArgs a) {
     __shared__ floatx4 o_lds[16][16];
     const uint32_t h = blockIdx.x, row = blockIdx.y, quarter = blockIdx.z;
     const uint32_t tid = threadIdx.x;
+    const float *ml = a.part_ml + size_t(2) * row * a.nsplits * a.heads;
+    const float *po = a.part_o + size_t(row) * a.nsplits * a.heads * DIM;
+    // Everything the kernel reads is requested before anything is waited for: (m, l) of every split
+    // slot, the partial sums (thread = quad d4 of the quarter's 64 dims, slice s of the splits) and
+    // the gate do not need TokenParams for their addresses, only for which of them count.  Slots
+    // past the splits at work hold old values: they are dropped by select, never multiplied.
+    floatx2 mlv = {NO_SCORE, 0.0f};
+    if (tid < a.nsplits) mlv = *reinterpret_cast<const floatx2 *>(ml + 2 * (size_t(tid) * a.heads + h));
+    const uint32_t d4 = tid & 15, s = tid >> 4;
+    floatx4 pv[MAX_SPLITS / 16];
+#pragma unroll
+    for (uint32_t i = 0; i < MAX_SPLITS / 16; i++) {
+        const uint32_t c = s + 16 * i;
+        pv[i] = floatx4{0, 0, 0, 0};
+        if (c < a.nsplits) {
+            pv[i] = *reinterpret_cast<const floatx4 *>(po + (size_t(c) * a.heads + h) * DIM + 64 * quarter + 4 * d4);
+        }
+    }
+    const size_t qh = size_t(row) * a.heads + h;
+    const float g = tid < 64 ? a.q_and_gate[qh * 2 * DIM + DIM + 64 * quarter + tid] : 0.0f;
     const uint32_t max_len = min(a.decode_len ? a.tp->kv_len : a.tp->position + a.rows, a.capacity);
     const uint32_t nblocks = (max_len + BLOCK - 1) / BLOCK;
     const uint32_t parts = min(a.nsplits, nblocks);
-    const float *ml = a.part_ml + size_t(2) * row * a.nsplits * a.heads;
-    const float *po = a.part_o + size_t(row) * a.nsplits * a.heads * DIM;
     // weights
-    float m = NO_SCORE, l = 0.0f;
-    if (tid < parts) {
-        const floatx2 v = *reinterpret_cast<const floatx2 *>(ml + 2 * (size_t(tid) * a.heads + h));
-        m = v[0], l = v[1];
-    }
+    const float m = tid < parts ? mlv[0] : NO_SCORE, l = tid < parts ? mlv[1] : 0.0f;
     float mx = m;
 #pragma unroll
     for (int step = 1; step < 64; step *= 2) mx = fmaxf(mx, __shfl_xor(mx, step));
@@ -827,13 +841,11 @@ __global__ __launch_bounds__(256) void attention_reduce_kernel(ReduceArgs a) {
     if ((tid & 63) == 0) red[4 + (tid >> 6)] = wl;
     __syncthreads();
     const float total = red[4] + red[5] + red[6] + red[7];
-    // sums: thread (quad d4 of the quarter's 64 dims, slice s of the splits)
-    const uint32_t d4 = tid & 15, s = tid >> 4;
     floatx4 acc = {0, 0, 0, 0};
-    for (uint32_t c = s; c < parts; c += 16) {
-        const floatx4 v =
-            *reinterpret_cast<const floatx4 *>(po + (size_t(c) * a.heads + h) * DIM + 64 * quarter + 4 * d4);
-        acc += v * w_lds[c];
+#pragma unroll
+    for (uint32_t i = 0; i < MAX_SPLITS / 16; i++) {
+        const uint32_t c = s + 16 * i;
+        if (c < parts) acc += pv[i] * w_lds[c];
     }
     o_lds[s][d4] = acc;
     __syncthreads();
@@ -842,8 +854,6 @@ __global__ __launch_bounds__(256) void attention_reduce_kernel(ReduceArgs a) {
         float o = 0.0f;
 #pragma unroll
         for (int i = 0; i < 16; i++) o += o_lds[i][d >> 2][d & 3];
-        const size_t qh = size_t(row) * a.heads + h;
-        const float g = a.q_and_gate[qh * 2 * DIM + DIM + 64 * quarter + d];
         a.out[qh * DIM + 64 * quarter + d] = o / total * (1.0f / (1.0f + expf(-g)));
     }
 }
