@@ -314,8 +314,9 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
         blk_end = split + 1;
         if (split >= nblocks) return;
     } else {
-        blk_begin = uint32_t(uint64_t(split) * nblocks / a.nsplits);
-        blk_end = uint32_t(uint64_t(split + 1) * nblocks / a.nsplits);
+        // (split + 1) * nblocks < 2^32: at most 256 splits and 2^27 blocks (32-bit cache offsets)
+        blk_begin = split * nblocks / a.nsplits;
+        blk_end = (split + 1) * nblocks / a.nsplits;
     }
     const uint32_t range = blk_end - blk_begin;
     const uint32_t n_it = (range + IT_BLOCKS - 1) / IT_BLOCKS;
