@@ -115,18 +115,41 @@ inline TokenParams token_params(uint32_t token, uint32_t position) {  // TokenPa
 
 class Built {
   public:
-    explicit Built(std::vector<std::pair<std::string, std::function<void(hipStream_t)>>> ops) : ops_(std::move(ops)) {}
-    void run(const gpu::Gpu &gpu) const {
+    using Ops = std::vector<std::pair<std::string, std::function<void(hipStream_t)>>>;
+    // graph: the launches are captured once into a HIP graph (the counterpart of the reference's
+    // indirect command buffer, src/plan.rs:229-235) and every run is one graph launch.  Every
+    // entry point of the library only enqueues kernels, so a plan can always be captured, with
+    // one exception: prefill without a caller's workspace allocates.
+    Built(Ops ops, const gpu::Gpu &gpu, bool graph) : ops_(std::move(ops)) {
+        if (!graph || ops_.empty()) return;
+        for (auto &op : ops_) op.second(gpu.stream());  // once outside the capture: first-call set-up
+        gpu.sync();
+        hipGraph_t g = nullptr;
+        hip_check(hipStreamBeginCapture(gpu.stream(), hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
         for (auto &op : ops_) op.second(gpu.stream());
+        hip_check(hipStreamEndCapture(gpu.stream(), &g), "hipStreamEndCapture");
+        hipGraphExec_t e = nullptr;
+        hip_check(hipGraphInstantiate(&e, g, nullptr, nullptr, 0), "hipGraphInstantiate");
+        hip_check(hipGraphDestroy(g), "hipGraphDestroy");
+        exec_ = std::shared_ptr<hipGraphExec>(e, [](hipGraphExec_t x) { (void)hipGraphExecDestroy(x); });
+    }
+    void run(const gpu::Gpu &gpu) const {
+        enqueue(gpu);
         gpu.sync();
     }
     // Replays without waiting, for timing many runs back to back.
     void enqueue(const gpu::Gpu &gpu) const {
-        for (auto &op : ops_) op.second(gpu.stream());
+        if (exec_) {
+            hip_check(hipGraphLaunch(exec_.get(), gpu.stream()), "hipGraphLaunch");
+        } else {
+            for (auto &op : ops_) op.second(gpu.stream());
+        }
     }
+    bool is_graph() const { return bool(exec_); }
 
   private:
-    std::vector<std::pair<std::string, std::function<void(hipStream_t)>>> ops_;
+    Ops ops_;
+    std::shared_ptr<hipGraphExec> exec_;
 };
 
 // A list of launches recorded once and run for every token; what changes per token is in the
@@ -140,13 +163,14 @@ class Plan {
         hip_check(hipMemcpyAsync(params.ptr<void>(), &tp, sizeof tp, hipMemcpyHostToDevice, gpu_.stream()), "set_params");
         gpu_.sync();
     }
-    Built build() const { return Built(ops_); }
-    Built build_where(const std::function<bool(const std::string &)> &keep) const {
-        std::vector<std::pair<std::string, std::function<void(hipStream_t)>>> kept;
+    Built build(bool graph = false) const { return Built(ops_, gpu_, graph); }
+    // Only the launches whose kernel name `keep` accepts (Plan::build_where, src/plan.rs:237-273).
+    Built build_where(const std::function<bool(const std::string &)> &keep, bool graph = false) const {
+        Built::Ops kept;
         for (auto &op : ops_) {
             if (keep(op.first)) kept.push_back(op);
         }
-        return Built(std::move(kept));
+        return Built(std::move(kept), gpu_, graph);
     }
 
   private:

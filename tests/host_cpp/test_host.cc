@@ -125,9 +125,17 @@ int main() {
             plan::Plan plan(gpu);
             att.record_quant(plan, qb, kc, vc, gb, out);
             auto built = plan.build();
+            auto replay = plan.build(true);  // the same launches as one HIP graph
+            EXPECT(replay.is_graph(), "plan was not captured");
             for (size_t len : {1, 127, 129, 1000, 1024}) {
                 plan.set_params(plan::token_params(0, uint32_t(len - 1)));
+                // serial == replay, exactly (tests/plan.rs:27-45)
+                replay.run(gpu);
+                const auto from_graph = gpu::contents<float>(out.buffer, HEADS * DIM);
+                hip_check(hipMemset(out.buffer.get(), 0xff, HEADS * DIM * 4), "hipMemset");
                 built.run(gpu);
+                EXPECT(std::memcmp(from_graph.data(), gpu::contents<float>(out.buffer, HEADS * DIM).data(), HEADS * DIM * 4) == 0,
+                       "%d-bit len %zu: graph replay differs from the serial run", int(kv_quant::bits(bits)), len);
                 auto got = gpu::contents<float>(out.buffer, HEADS * DIM);
                 std::vector<double> want(HEADS * DIM);
                 orc_attention_f64(q.data(), kf.data(), vf.data(), qg.data(), len, HEADS, KV, DIM, want.data(), 4);
