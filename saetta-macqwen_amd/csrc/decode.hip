@@ -226,6 +226,52 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t bits16) {
     return (float)__builtin_bit_cast(_Float16, uint16_t(bits16));
 }
 
+// ---- reductions over aligned groups of lanes without LDS -------------------------------------
+// Steps inside a 16-lane row are DPP moves (quad permutes, then the two mirrors: once the quads
+// agree, mirroring the half row and the row brings in the other quads).  Rows are joined by
+// v_permlane16_swap / v_permlane32_swap, which exchange 16- and 32-lane rows of two registers;
+// they may not read a register a vector instruction wrote in the two cycles before.
+template <int CTRL>
+__device__ __forceinline__ float dpp(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ void swap_rows16(uint32_t &u, uint32_t &v) {
+    asm volatile("s_nop 1\nv_permlane16_swap_b32 %0, %1\n" : "+v"(u), "+v"(v));
+}
+__device__ __forceinline__ void swap_rows32(uint32_t &u, uint32_t &v) {
+    asm volatile("s_nop 1\nv_permlane32_swap_b32 %0, %1\n" : "+v"(u), "+v"(v));
+}
+struct MaxOp {
+    __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+};
+struct SumOp {
+    __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+// x combined over the lanes l ^ 16 (FROM <= 16 < WIDTH) and l ^ 32 (FROM <= 32 < WIDTH)
+template <int FROM, int WIDTH, typename Op>
+__device__ __forceinline__ float across_rows(float x, Op op) {
+    if constexpr (FROM <= 16 && WIDTH > 16) {
+        uint32_t u = __builtin_bit_cast(uint32_t, x), v = u;
+        swap_rows16(u, v);  // u = rows (0, 0, 2, 2), v = rows (1, 1, 3, 3)
+        x = op(__builtin_bit_cast(float, u), __builtin_bit_cast(float, v));
+    }
+    if constexpr (FROM <= 32 && WIDTH > 32) {
+        uint32_t u = __builtin_bit_cast(uint32_t, x), v = u;
+        swap_rows32(u, v);  // u = (lower half, lower half), v = (upper, upper)
+        x = op(__builtin_bit_cast(float, u), __builtin_bit_cast(float, v));
+    }
+    return x;
+}
+// x combined over aligned groups of WIDTH lanes (1, 2, 4, ... 64); every lane gets the result
+template <int WIDTH, typename Op>
+__device__ __forceinline__ float group_reduce(float x, Op op) {
+    if constexpr (WIDTH > 1) x = op(x, dpp<0xb1>(x));   // quad_perm [1, 0, 3, 2]
+    if constexpr (WIDTH > 2) x = op(x, dpp<0x4e>(x));   // quad_perm [2, 3, 0, 1]
+    if constexpr (WIDTH > 4) x = op(x, dpp<0x141>(x));  // row_half_mirror
+    if constexpr (WIDTH > 8) x = op(x, dpp<0x140>(x));  // row_mirror
+    return across_rows<16, WIDTH>(x, op);
+}
+
 // TILES: 16-row tiles of query rows (rows * 8 heads, rounded up).  PACKED: one
 // verify row; its 8 heads' hi parts are operand rows 0-7 and lo parts rows 8-15
 // of a single tile.  Otherwise hi and lo are two MFMAs into one accumulator.
@@ -581,8 +627,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
             float cm = NO_SCORE;
 #pragma unroll
             for (int i = 0; i < Sh::TPT; i++) cm = (tok0 + i < lim) ? fmaxf(cm, sv[i]) : cm;
-#pragma unroll
-            for (int step = 1; step < Sh::TPR; step *= 2) cm = fmaxf(cm, __shfl_xor(cm, step));
+            cm = group_reduce<Sh::TPR>(cm, MaxOp());
             const float nm = fmaxf(m_run, cm);
             const float al = __builtin_amdgcn_exp2f(m_run - nm);
             float sum = 0.0f;
@@ -708,8 +753,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
 
     // ---- epilogue: one partial per (row, head) ------------------------------------
     // m and l from the phase B threads.
-#pragma unroll
-    for (int step = 1; step < Sh::TPR; step *= 2) l_part += __shfl_xor(l_part, step);
+    l_part = group_reduce<Sh::TPR>(l_part, SumOp());
     if (b_part == 0 && (PACKED || b_row < int(real_rows))) {
         const int vrow = PACKED ? 0 : b_row >> 3, head = b_row & 7;
         const size_t slot = (size_t(vrow) * a.nsplits + split) * a.heads + kv * 8 + head;
@@ -720,8 +764,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
 #pragma unroll
         for (int t = 0; t < TILES; t++) {
             float z = zacc[t];
-            z += __shfl_xor(z, 16);
-            z += __shfl_xor(z, 32);
+            z = across_rows<16, 64>(z, SumOp());
             // One copy per wave: the sum of wave w's group lives at [w][row].
             if (j == 0 && (!PACKED || n < 8)) zsum_lds[wave * Sh::S_ROWS + 16 * t + n] = z;
         }
@@ -737,7 +780,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
             if constexpr (PACKED) {
                 // rows 8-15 hold the lo part of rows 0-7: lanes j and j + 2.
 #pragma unroll
-                for (int i = 0; i < 4; i++) o[e][i] += __shfl_xor(o[e][i], 32);
+                for (int i = 0; i < 4; i++) o[e][i] = across_rows<32, 64>(o[e][i], SumOp());
             }
         }
         if (PACKED && j >= 2) continue;
@@ -829,16 +872,14 @@ __global__ __launch_bounds__(256) void attention_reduce_kernel(ReduceArgs a) {
     // weights
     const float m = tid < parts ? mlv[0] : NO_SCORE, l = tid < parts ? mlv[1] : 0.0f;
     float mx = m;
-#pragma unroll
-    for (int step = 1; step < 64; step *= 2) mx = fmaxf(mx, __shfl_xor(mx, step));
+    mx = group_reduce<64>(mx, MaxOp());
     if ((tid & 63) == 0) red[tid >> 6] = mx;
     __syncthreads();
     mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     const float w = tid < parts ? exp2f(m - mx) : 0.0f;
     w_lds[tid] = w;
     float wl = w * l;
-#pragma unroll
-    for (int step = 1; step < 64; step *= 2) wl += __shfl_xor(wl, step);
+    wl = group_reduce<64>(wl, SumOp());
     if ((tid & 63) == 0) red[4 + (tid >> 6)] = wl;
     __syncthreads();
     const float total = red[4] + red[5] + red[6] + red[7];
