@@ -768,7 +768,9 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
             // One copy per wave: the sum of wave w's group lives at [w][row].
             if (j == 0 && (!PACKED || n < 8)) zsum_lds[wave * Sh::S_ROWS + 16 * t + n] = z;
         }
-        __syncthreads();
+        // written and read by lanes of the same wave: no workgroup barrier
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
     }
     constexpr float unscale = code_up<BITS>() / P_UP;
 #pragma unroll
