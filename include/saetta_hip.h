@@ -93,6 +93,16 @@ typedef struct saetta_flash_params {
     float scale;
 } saetta_flash_params;
 
+/* PrepParams (src/gpu_layers.rs:387-394; kernels/layers.metal:639-646). */
+typedef struct saetta_prep_params {
+    uint32_t heads;
+    uint32_t kv_heads;
+    uint32_t dim;        /* head dim: 256 */
+    uint32_t half_dims;  /* rotary dims / 2 */
+    float log2_theta;
+    float eps;
+} saetta_prep_params;
+
 /* The three arrays of one quantized cache, keys or values: QuantRows
  * {data, scales, biases} (src/kv_quant.rs:156-180).  Token p's groups start
  * at group p * per_token; group G's codes are words 2*bits*G onward, lowest
@@ -195,6 +205,26 @@ int saetta_attn_rows_quant(saetta_stream_t stream, int bits, const float *q,
                            float *part_ml, const float *q_and_gate, float *out,
                            saetta_rows_params p, const saetta_token_params *d_tp,
                            uint32_t stages);
+
+/* ---- the step before the scores (src/gpu_layers.rs) -------------------------- */
+
+/* GpuAttention::record_store (src/gpu_layers.rs:370-411): q norm and RoPE into
+ * q_out, k norm and RoPE, then the token's key and value into their cache
+ * slot, in ONE launch.  Replaces attention_prep / attention_prep_float
+ * (kernels/layers.metal:637-702) and, for a quantized cache, the two
+ * kv_quantize dispatches that follow it (src/kv_quant.rs:192-221).
+ * q_and_gate f32 [rows][heads][512], k, v f32 [rows][kv_heads][256], q_norm,
+ * k_norm f32 [256], q_out f32 [rows][heads][256].  bits 16: keys_half,
+ * values_half are the half cache [capacity][kv_heads][256] and the quantized
+ * rows are ignored; bits 8 or 4: the other way round.  Row r is the token at
+ * TokenParams.position + r; a row at or past `capacity` is not stored.
+ * k_back (or NULL): f32 [rows][kv_heads][256] gets the normed, rotated key,
+ * which is what attention_prep_float leaves in k. */
+int saetta_attn_prep_store(saetta_stream_t stream, int bits, const float *q_and_gate, const float *k,
+                           const float *v, const float *q_norm, const float *k_norm, float *q_out,
+                           uint16_t *keys_half, uint16_t *values_half, saetta_quant_rows keys,
+                           saetta_quant_rows values, float *k_back, saetta_prep_params p, uint32_t rows,
+                           uint32_t capacity, const saetta_token_params *d_tp);
 
 /* ---- prefill attention (src/attention_prefill.rs, src/prefill.rs) ---------- */
 

@@ -162,6 +162,17 @@ def rope(head, dims, pos, theta):
     return y
 
 
+def attention_prep(q_and_gate, k, v, q_norm, k_norm, heads, kv_heads, dim, rope_dims, pos, theta, eps):
+    """What attention_at does to one token before the scores (src/cpu/attention.rs:110-138):
+    q and k through rms_norm and rope per head, v as it is.  Returns (q, k, v) as f32
+    [heads * dim], [kv_heads * dim], [kv_heads * dim]."""
+    qg = _c32(q_and_gate).reshape(heads, 2 * dim)
+    q = np.stack([rope(rms_norm(qg[h, :dim], q_norm, eps), rope_dims, pos, theta) for h in range(heads)])
+    kk = _c32(k).reshape(kv_heads, dim)
+    kk = np.stack([rope(rms_norm(kk[h], k_norm, eps), rope_dims, pos, theta) for h in range(kv_heads)])
+    return q.reshape(-1), kk.reshape(-1), _c32(v).reshape(-1).copy()
+
+
 # ------------------------------------------------------------ attention ----
 
 def _shape(keys, heads, kv_heads, dim):

@@ -15,16 +15,12 @@
 // float4 per lane, contiguous across the wavefront; every lane stores one
 // dword of codes, contiguous as well.
 #include "common.hpp"
+#include "kv_quant_device.hpp"
 
 namespace saetta {
 namespace {
 
-// Every float operation that decides a bit is spelled with a rounding
-// intrinsic, so the compiler can neither fuse nor reassociate:
-//   s   = half_rn((hi - lo) / levels)      IEEE divide
-//   z   = half_rn(lo)
-//   inv = s > 0 ? 1 / f32(s) : 0           IEEE divide
-//   q   = clamp(rint((v - f32(z)) * inv), 0, levels), NaN -> 0
+// The arithmetic of a group is quantize_lane (kv_quant_device.hpp).
 template <int BITS>
 __global__ __launch_bounds__(256) void kv_quantize_kernel(const float *__restrict__ x,
                                                           uint32_t *__restrict__ data,
@@ -35,7 +31,6 @@ __global__ __launch_bounds__(256) void kv_quantize_kernel(const float *__restric
                                                           uint32_t pos_arg) {
     constexpr int VPL = 32 / BITS;               // values per lane = codes per word
     constexpr int LANES = SAETTA_QUANT_GROUP / VPL;  // lanes per group
-    constexpr float LEVELS = float((1u << BITS) - 1);
     const uint32_t word = blockIdx.x * 256u + threadIdx.x;  // word index from x[0]
     const uint32_t g = word / LANES;
     const bool live = g < p.groups;
@@ -55,30 +50,8 @@ __global__ __launch_bounds__(256) void kv_quantize_kernel(const float *__restric
 #pragma unroll
         for (int i = 0; i < VPL; i++) v[i] = 0.0f;
     }
-    // fminf/fmaxf return the other operand when one is NaN, as f32::min/max do.
-    float lo = INFINITY, hi = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < VPL; i++) {
-        lo = fminf(lo, v[i]);
-        hi = fmaxf(hi, v[i]);
-    }
-#pragma unroll
-    for (int step = 1; step < LANES; step *= 2) {
-        lo = fminf(lo, __shfl_xor(lo, step));
-        hi = fmaxf(hi, __shfl_xor(hi, step));
-    }
-    const __half s = __float2half_rn(__fdiv_rn(__fsub_rn(hi, lo), LEVELS));
-    const __half z = __float2half_rn(lo);
-    const float sf = __half2float(s), zf = __half2float(z);
-    const float inv = sf > 0.0f ? __fdiv_rn(1.0f, sf) : 0.0f;
-    uint32_t packed = 0;
-#pragma unroll
-    for (int i = 0; i < VPL; i++) {
-        float r = rintf(__fmul_rn(__fsub_rn(v[i], zf), inv));
-        // NaN fails both comparisons of the clamp in Rust and casts to 0.
-        uint32_t q = (r != r) ? 0u : uint32_t(fminf(fmaxf(r, 0.0f), LEVELS));
-        packed |= q << (i * BITS);
-    }
+    __half s, z;
+    const uint32_t packed = quantize_lane<BITS>(v, s, z);
     if (!live) return;
     const uint32_t pos = d_tp ? d_tp->position : pos_arg;
     const size_t first = size_t(pos) * p.per_token;  // destination group of g = 0

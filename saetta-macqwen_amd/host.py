@@ -285,6 +285,45 @@ class DecodeAttention:
         plan.op("attention_reduce", launch(ffi.STAGE_REDUCE))
 
 
+class PrepParams:
+    """PrepParams (src/gpu_layers.rs:387-394)."""
+
+    def __init__(self, heads, kv_heads, dim, rope_dims, rope_theta, eps):
+        self.heads, self.kv_heads, self.dim, self.half_dims = heads, kv_heads, dim, rope_dims // 2
+        self.log2_theta, self.eps = math.log2(rope_theta), eps
+
+    def c(self):
+        return ffi.PrepParamsC(self.heads, self.kv_heads, self.dim, self.half_dims, self.log2_theta, self.eps)
+
+
+def record_store(plan, q_and_gate, k, v, q_norm, k_norm, q, keys, values, p, capacity, rows=1, k_back=None):
+    """GpuAttention::record_store (src/gpu_layers.rs:370-411): q norm and RoPE into q, k norm and
+    RoPE, then the token's key and value into the cache slot at the plan's position: as half
+    (`keys`, `values` f16 tensors) or as codes (`keys`, `values` QuantRows), in one launch where the
+    reference records attention_prep{,_float} and two kv_quantize dispatches.  k_back: an f32
+    tensor that gets the normed, rotated key (what attention_prep_float leaves in k), or None."""
+    for t, what in ((q_and_gate, "q_and_gate"), (k, "k"), (v, "v"), (q_norm, "q_norm"), (k_norm, "k_norm"), (q, "q")):
+        _need(t, torch.float32, what)
+    quant = isinstance(keys, QuantRows)
+    if quant != isinstance(values, QuantRows):
+        raise ValueError("record_store: keys and values must be the same kind of cache")
+    none = ffi.QuantRowsC(None, None, None)
+    if quant:
+        bits, kh, vh, kq, vq = keys.bits.value, None, None, keys.c(), values.c()
+    else:
+        _need(keys, torch.float16, "keys"), _need(values, torch.float16, "values")
+        bits, kh, vh, kq, vq = 16, _ptr(keys), _ptr(values), none, none
+    pc, tp = p.c(), plan.params
+    kb = None if k_back is None else _ptr(k_back)
+
+    def launch(s):
+        ffi.check(ffi.lib().saetta_attn_prep_store(s, bits, _ptr(q_and_gate), _ptr(k), _ptr(v), _ptr(q_norm),
+                                                   _ptr(k_norm), _ptr(q), kh, vh, kq, vq, kb, pc, rows, capacity,
+                                                   _ptr(tp)), "attn_prep_store")
+
+    plan.op("attention_prep_store", launch)
+
+
 def _median_ms(run, runs):
     """One warm-up, then the median of `runs` event-timed calls, in milliseconds."""
     ts = []

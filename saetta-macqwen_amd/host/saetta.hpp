@@ -292,6 +292,48 @@ inline float test_slack(KvBits b) { return b == KvBits::Half ? 1.0f : b == KvBit
 
 }  // namespace kv_quant
 
+namespace gpu_layers {
+
+using PrepParams = saetta_prep_params;
+inline PrepParams prep_params(size_t heads, size_t kv_heads, size_t dim, size_t rope_dims, float rope_theta, float eps) {
+    return PrepParams{uint32_t(heads), uint32_t(kv_heads), uint32_t(dim), uint32_t(rope_dims / 2), std::log2(rope_theta), eps};
+}
+
+// GpuAttention::record_store (src/gpu_layers.rs:370-411): q norm and RoPE into q, k norm and RoPE,
+// then the token's key and value into the cache slot at the plan's position, in one launch where the
+// reference records attention_prep{,_float} and two kv_quantize dispatches.  Half cache:
+inline void record_store(plan::Plan &plan, const View &q_and_gate, const View &k, const View &v, const View &q_norm,
+                         const View &k_norm, const View &q, const View &keys, const View &values, PrepParams p,
+                         size_t capacity, size_t rows = 1) {
+    const View tp = plan.params;
+    plan.op("attention_prep_store", [=](hipStream_t s) {
+        check(saetta_attn_prep_store(s, 16, q_and_gate.ptr<float>(), k.ptr<float>(), v.ptr<float>(), q_norm.ptr<float>(),
+                                     k_norm.ptr<float>(), q.ptr<float>(), keys.ptr<uint16_t>(), values.ptr<uint16_t>(),
+                                     saetta_quant_rows{}, saetta_quant_rows{}, nullptr, p, uint32_t(rows), uint32_t(capacity),
+                                     tp.ptr<saetta_token_params>()),
+              "attn_prep_store");
+    });
+}
+// ... and a quantized cache; k_back (optional) gets the normed, rotated key in f32.
+inline void record_store(plan::Plan &plan, const View &q_and_gate, const View &k, const View &v, const View &q_norm,
+                         const View &k_norm, const View &q, const kv_quant::QuantRows &keys, const kv_quant::QuantRows &values,
+                         PrepParams p, size_t capacity, size_t rows = 1, const View *k_back = nullptr) {
+    const View tp = plan.params;
+    const kv_quant::QuantRows kq = keys, vq = values;
+    const int nbits = int(kv_quant::bits(keys.bits));
+    const View kb = k_back ? *k_back : View();
+    const bool has_kb = k_back != nullptr;
+    plan.op("attention_prep_store", [=](hipStream_t s) {
+        check(saetta_attn_prep_store(s, nbits, q_and_gate.ptr<float>(), k.ptr<float>(), v.ptr<float>(), q_norm.ptr<float>(),
+                                     k_norm.ptr<float>(), q.ptr<float>(), nullptr, nullptr, kq.c(), vq.c(),
+                                     has_kb ? kb.ptr<float>() : nullptr, p, uint32_t(rows), uint32_t(capacity),
+                                     tp.ptr<saetta_token_params>()),
+              "attn_prep_store");
+    });
+}
+
+}  // namespace gpu_layers
+
 namespace attention {
 
 constexpr size_t DIM = 256;

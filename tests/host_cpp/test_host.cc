@@ -176,6 +176,23 @@ int main() {
         }
         EXPECT(off == 0 && s.size() == 4000, "spread: %zu values differ", off);
     }
+    {   // record_store: the codes it writes are the quantizer's codes of the key it reports
+        const size_t pos = 41, capacity = 64;
+        std::vector<float> qg(HEADS * 2 * DIM), k(KV * DIM), v(KV * DIM), ones(DIM, 1.0f);
+        orc_noise(qg.data(), qg.size(), 21);
+        orc_noise(k.data(), k.size(), 22);
+        orc_noise(v.data(), v.size(), 23);
+        QuantRows kc(gpu, KvBits::Eight, VALUES, capacity), vc(gpu, KvBits::Eight, VALUES, capacity);
+        View q(gpu.buffer(HEADS * DIM * 4)), kb(gpu.buffer(KV * DIM * 4));
+        plan::Plan plan(gpu);
+        gpu_layers::record_store(plan, View(gpu.buffer_from(qg)), View(gpu.buffer_from(k)), View(gpu.buffer_from(v)),
+                                 View(gpu.buffer_from(ones)), View(gpu.buffer_from(ones)), q, kc, vc,
+                                 gpu_layers::prep_params(HEADS, KV, DIM, 64, 1e7f, 1e-6f), capacity, 1, &kb);
+        plan.set_params(plan::token_params(0, uint32_t(pos)));
+        plan.build(true).run(gpu);
+        compare(kc, gpu::contents<float>(kb.buffer, KV * DIM), pos, KvBits::Eight);
+        compare(vc, v, pos, KvBits::Eight);
+    }
     // shape checks panic (throw) as the reference asserts
     bool threw = false;
     try {
