@@ -103,6 +103,18 @@ typedef struct saetta_prep_params {
     float eps;
 } saetta_prep_params;
 
+/* ConvParams (kernels/layers.metal:198-201) and StepParams (kernels/layers.metal:290-295). */
+typedef struct saetta_conv_params {
+    uint32_t channels;
+    uint32_t kernel_size;
+} saetta_conv_params;
+typedef struct saetta_step_params {
+    uint32_t k_heads;
+    uint32_t v_heads;
+    uint32_t v_dim;
+    float eps;
+} saetta_step_params;
+
 /* The three arrays of one quantized cache, keys or values: QuantRows
  * {data, scales, biases} (src/kv_quant.rs:156-180).  Token p's groups start
  * at group p * per_token; group G's codes are words 2*bits*G onward, lowest
@@ -225,6 +237,27 @@ int saetta_attn_prep_store(saetta_stream_t stream, int bits, const float *q_and_
                            uint16_t *keys_half, uint16_t *values_half, saetta_quant_rows keys,
                            saetta_quant_rows values, float *k_back, saetta_prep_params p, uint32_t rows,
                            uint32_t capacity, const saetta_token_params *d_tp);
+
+/* ---- Gated DeltaNet, one token (src/cpu/deltanet.rs, src/gpu_layers.rs) ------ */
+
+/* conv_step (src/cpu/deltanet.rs:117-131); kernel deltanet_conv
+ * (kernels/layers.metal:203-226): depthwise causal conv1d over the stored
+ * inputs and x, then SiLU; x shifts into the state.  x, out f32 [channels];
+ * w f32 [channels][kernel_size], last column = newest token; state f32
+ * [kernel_size - 1][channels], oldest first, updated in place. */
+int saetta_deltanet_conv(saetta_stream_t stream, const float *x, const float *w, float *state, float *out,
+                         saetta_conv_params p);
+
+/* Everything between the conv and out_proj (src/cpu/deltanet.rs:86-112,133-155);
+ * kernel deltanet_step (kernels/layers.metal:297-357): L2 norm of q and k, the
+ * gates, the delta rule on every value head's state and the gated RMSNorm.
+ * q, k f32 [k_heads][128]; v, z, y f32 [v_heads][v_dim]; a, b, a_log, dt_bias
+ * f32 [v_heads]; state f32 [v_heads][v_dim][128], updated in place; norm_w
+ * f32 [v_dim].  Key dim 128, v_dim up to 256. */
+int saetta_deltanet_step(saetta_stream_t stream, const float *q, const float *k, const float *v,
+                         const float *a, const float *b, const float *a_log, const float *dt_bias,
+                         float *state, const float *z, const float *norm_w, float *y,
+                         saetta_step_params p);
 
 /* ---- prefill attention (src/attention_prefill.rs, src/prefill.rs) ---------- */
 

@@ -65,6 +65,11 @@ _prefill = _sig("orc_prefill", _int, _f32p, _f32p, _f32p, _sz, _sz, _sz, _sz, _s
 _layer = _sig(
     "orc_attention_layer", _int, _f32p, _sz, _sz, _sz, _sz, _sz, ctypes.c_float, ctypes.c_float,
     _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _sz, _sz, _int, _f32p)
+_dn_conv = _sig("orc_deltanet_conv", None, _f32p, _f32p, _f32p, _sz, _sz, _f32p)
+_dn_step = _sig("orc_deltanet_step", None, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p,
+                _sz, _sz, _sz, _sz, ctypes.c_float, _f32p)
+_dn_layer = _sig("orc_deltanet_layer", None, _f32p, _sz, _sz, _sz, _sz, _sz, _sz, ctypes.c_float, _f32p, _f32p, _f32p,
+                 _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p)
 _noise = _sig("orc_noise", None, _f32p, _sz, ctypes.c_uint64)
 _spread = _sig("orc_spread", None, _u16p, _sz, _sz)
 _quant_rows = _sig("orc_quant_rows", None, _f32p, _sz, _sz)
@@ -254,6 +259,47 @@ class AttentionLayer:
                     self.len, self.len if pos is None else pos, self.rounding, out)
         _check(rc, "attention_layer")
         self.len += 1
+        return out
+
+
+# ------------------------------------------------------------ Gated DeltaNet ----
+
+def deltanet_conv(weight, x, state, kernel):
+    """conv_step (src/cpu/deltanet.rs:117-131).  state [kernel-1][channels] is updated in place
+    (pass a contiguous f32 array); returns the mixed, SiLU'd channels."""
+    x = _c32(x).reshape(-1)
+    assert state.dtype == np.float32 and state.flags.c_contiguous
+    out = np.empty_like(x)
+    _dn_conv(_c32(weight).reshape(-1), x, state.reshape(-1), x.size, kernel, out)
+    return out
+
+
+def deltanet_step(q, k, v, a, b, a_log, dt_bias, state, z, norm, k_heads, v_heads, k_dim, v_dim, eps):
+    """normalize_qk, the gates, delta_rule and the gated RMSNorm (src/cpu/deltanet.rs:86-112,133-155).
+    state [v_heads][v_dim][k_dim] is updated in place; returns y [v_heads * v_dim]."""
+    assert state.dtype == np.float32 and state.flags.c_contiguous
+    y = np.empty(v_heads * v_dim, np.float32)
+    _dn_step(_c32(q).reshape(-1), _c32(k).reshape(-1), _c32(v).reshape(-1), _c32(a), _c32(b), _c32(a_log),
+             _c32(dt_bias), state.reshape(-1), _c32(z).reshape(-1), _c32(norm), k_heads, v_heads, k_dim, v_dim, eps, y)
+    return y
+
+
+class DeltaNetLayer:
+    """deltanet (src/cpu/deltanet.rs:69-114) with dense projections, state kept between tokens."""
+
+    def __init__(self, cfg, weights):
+        self.cfg = cfg
+        self.w = {k: _c32(v).reshape(-1) for k, v in weights.items()}
+        conv = 2 * cfg["k_heads"] * cfg["k_dim"] + cfg["v_heads"] * cfg["v_dim"]
+        self.conv = np.zeros((cfg["kernel"] - 1) * conv, np.float32)
+        self.recurrent = np.zeros(cfg["v_heads"] * cfg["v_dim"] * cfg["k_dim"], np.float32)
+
+    def step(self, x):
+        c, w = self.cfg, self.w
+        out = np.empty(c["hidden"], np.float32)
+        _dn_layer(_c32(x).reshape(-1), c["hidden"], c["k_heads"], c["v_heads"], c["k_dim"], c["v_dim"], c["kernel"],
+                  c["eps"], w["in_proj_qkv"], w["in_proj_z"], w["in_proj_b"], w["in_proj_a"], w["out_proj"],
+                  w["conv1d"], w["A_log"], w["dt_bias"], w["norm"], self.conv, self.recurrent, out)
         return out
 
 

@@ -1,5 +1,5 @@
 /*
- * CPU oracle for the full-attention hot path: TEST INFRASTRUCTURE ONLY.
+ * CPU oracle for the full-attention hot path and its next rows: TEST INFRASTRUCTURE ONLY.
  *
  * This file restates, in plain C, the reference's CPU algorithms so that the
  * HIP kernels can be checked against them.  It is never linked into or called
@@ -30,6 +30,14 @@
  *   orc_rows / orc_prefill              definition as single-row calls, checked
  *                                       against torch float64 SDPA with a causal
  *                                       mask
+ *   orc_rms_norm / orc_rope             MLX golden vectors ops.json
+ *   orc_deltanet_conv / _step / _layer  MLX golden vectors deltanet.json (six
+ *                                       tokens: outputs, conv state, recurrent
+ *                                       state; src/cpu/deltanet.rs:162-204), an
+ *                                       f64 restatement of the recurrence, its
+ *                                       limits (beta -> 1: S k = v; g -> 0:
+ *                                       S = beta v k^T), the conv as a causal
+ *                                       filter over the input history
  * No function here is "parity unpinned".
  */
 #include <math.h>
@@ -478,6 +486,97 @@ int orc_attention_layer(const float *x, size_t hidden, size_t heads, size_t kv_h
     free(v);
     free(att);
     return rc;
+}
+
+/* ------------------------------------------------------ Gated DeltaNet ---- */
+/* One token of the linear-attention layer, src/cpu/deltanet.rs:69-155.
+ * Pinned by the MLX golden vectors of deltanet.json (six tokens: outputs, conv
+ * state, recurrent state; src/cpu/deltanet.rs:162-204). */
+
+static float silu_f32(float x) { return x * sigmoid_f32(x); }
+
+/* log(1 + e^x) without overflow (src/cpu/ops.rs:46-49). */
+static float softplus_f32(float x) { return fmaxf(x, 0.0f) + log1pf(expf(-fabsf(x))); }
+
+/* conv_step (src/cpu/deltanet.rs:117-131): depthwise causal conv1d over the stored
+ * inputs and `input`, then SiLU; `input` is shifted into the state.
+ * weight [channels][kernel] (last column = newest token), state [kernel-1][channels]
+ * oldest first. */
+void orc_deltanet_conv(const float *weight, const float *input, float *state, size_t channels,
+                       size_t kernel, float *out) {
+    size_t past = kernel - 1; /* >= 1: the reference drains one input from a non-empty state */
+    for (size_t c = 0; c < channels; c++) {
+        const float *w = weight + c * kernel;
+        float old = 0.0f;
+        for (size_t t = 0; t < past; t++) old += w[t] * state[t * channels + c];
+        out[c] = silu_f32(old + w[past] * input[c]);
+    }
+    memmove(state, state + channels, (past - 1) * channels * sizeof(float));
+    memcpy(state + (past - 1) * channels, input, channels * sizeof(float));
+}
+
+/* normalize_qk + the per-head gates + delta_rule + the gated RMSNorm
+ * (src/cpu/deltanet.rs:86-112,133-155): everything between the conv and out_proj.
+ * q, k [k_heads][k_dim] (after the conv), v [v_heads][v_dim], a, b [v_heads],
+ * state [v_heads][v_dim][k_dim] (updated), z [v_heads][v_dim], norm [v_dim],
+ * y [v_heads][v_dim]. */
+void orc_deltanet_step(const float *q_in, const float *k_in, const float *v, const float *a,
+                       const float *b, const float *a_log, const float *dt_bias, float *state,
+                       const float *z, const float *norm, size_t k_heads, size_t v_heads,
+                       size_t k_dim, size_t v_dim, float eps, float *y) {
+    float *q = malloc(k_heads * k_dim * sizeof(float)), *k = malloc(k_heads * k_dim * sizeof(float));
+    float q_scale = 1.0f / sqrtf((float)k_dim);
+    for (size_t h = 0; h < k_heads; h++) {
+        const float *qh = q_in + h * k_dim, *kh = k_in + h * k_dim;
+        float qi = q_scale / sqrtf(dot_f32(qh, qh, k_dim) + eps);
+        float ki = 1.0f / sqrtf(dot_f32(kh, kh, k_dim) + eps);
+        for (size_t i = 0; i < k_dim; i++) q[h * k_dim + i] = qh[i] * qi, k[h * k_dim + i] = kh[i] * ki;
+    }
+    size_t group = v_heads / k_heads;
+    for (size_t h = 0; h < v_heads; h++) {
+        float g = expf(-expf(a_log[h]) * softplus_f32(a[h] + dt_bias[h]));
+        float beta = sigmoid_f32(b[h]);
+        const float *qh = q + (h / group) * k_dim, *kh = k + (h / group) * k_dim;
+        for (size_t i = 0; i < v_dim; i++) {
+            float *row = state + (h * v_dim + i) * k_dim;
+            for (size_t j = 0; j < k_dim; j++) row[j] *= g;
+            float delta = (v[h * v_dim + i] - dot_f32(row, kh, k_dim)) * beta;
+            for (size_t j = 0; j < k_dim; j++) row[j] += kh[j] * delta;
+            y[h * v_dim + i] = dot_f32(row, qh, k_dim);
+        }
+        orc_rms_norm(y + h * v_dim, norm, v_dim, eps);
+        for (size_t i = 0; i < v_dim; i++) y[h * v_dim + i] *= silu_f32(z[h * v_dim + i]);
+    }
+    free(q);
+    free(k);
+}
+
+/* deltanet (src/cpu/deltanet.rs:69-114) with dense f32 projections [out][in]; used
+ * to hold the two functions above against deltanet.json. */
+void orc_deltanet_layer(const float *x, size_t hidden, size_t k_heads, size_t v_heads, size_t k_dim,
+                        size_t v_dim, size_t kernel, float eps, const float *in_proj_qkv,
+                        const float *in_proj_z, const float *in_proj_b, const float *in_proj_a,
+                        const float *out_proj, const float *conv1d, const float *a_log,
+                        const float *dt_bias, const float *norm, float *conv_state,
+                        float *recurrent, float *out) {
+    size_t key = k_heads * k_dim, val = v_heads * v_dim, conv = 2 * key + val;
+    float *qkv = malloc(conv * sizeof(float)), *mixed = malloc(conv * sizeof(float));
+    float *z = malloc(val * sizeof(float)), *y = malloc(val * sizeof(float));
+    float *b = malloc(v_heads * sizeof(float)), *a = malloc(v_heads * sizeof(float));
+    matvec_f32(in_proj_qkv, x, conv, hidden, qkv);
+    matvec_f32(in_proj_z, x, val, hidden, z);
+    matvec_f32(in_proj_b, x, v_heads, hidden, b);
+    matvec_f32(in_proj_a, x, v_heads, hidden, a);
+    orc_deltanet_conv(conv1d, qkv, conv_state, conv, kernel, mixed);
+    orc_deltanet_step(mixed, mixed + key, mixed + 2 * key, a, b, a_log, dt_bias, recurrent, z, norm,
+                      k_heads, v_heads, k_dim, v_dim, eps, y);
+    matvec_f32(out_proj, y, hidden, val, out);
+    free(qkv);
+    free(mixed);
+    free(z);
+    free(y);
+    free(b);
+    free(a);
 }
 
 /* ------------------------------------------------- the reference's inputs ---- */

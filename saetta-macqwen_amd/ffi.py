@@ -7,7 +7,7 @@ LIB_PATH = os.environ.get("SAETTA_HIP_LIB") or os.path.join(_HERE, "lib", "libsa
 
 # Every symbol include/saetta_hip.h declares; tests check the library exports each.
 SYMBOLS = [
-    "saetta_init", "saetta_last_error", "saetta_kv_quantize", "saetta_kv_dequantize", "saetta_kv_dequantize_f32", "saetta_to_half", "saetta_attn_prep_store",
+    "saetta_init", "saetta_last_error", "saetta_kv_quantize", "saetta_kv_dequantize", "saetta_kv_dequantize_f32", "saetta_to_half", "saetta_attn_prep_store", "saetta_deltanet_conv", "saetta_deltanet_step",
     "saetta_part_o_bytes", "saetta_part_ml_bytes", "saetta_attn_decode", "saetta_attn_decode_quant",
     "saetta_attn_rows", "saetta_attn_rows_quant", "saetta_prefill_workspace_bytes", "saetta_attn_prefill", "saetta_attn_prefill_quant",
 ]
@@ -67,6 +67,10 @@ def lib():
         l.saetta_kv_dequantize_f32.restype = i32
         l.saetta_kv_dequantize_f32.argtypes = [vp, i32, QuantRowsC, vp, KvQuantParamsC]
         l.saetta_to_half.restype, l.saetta_to_half.argtypes = i32, [vp, vp, vp, sz]
+        l.saetta_deltanet_conv.restype = i32
+        l.saetta_deltanet_conv.argtypes = [vp, vp, vp, vp, vp, ConvParamsC]
+        l.saetta_deltanet_step.restype = i32
+        l.saetta_deltanet_step.argtypes = [vp] * 12 + [StepParamsC]
         l.saetta_attn_prep_store.restype = i32
         l.saetta_attn_prep_store.argtypes = [vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, QuantRowsC, QuantRowsC, vp,
                                              PrepParamsC, u32, u32, vp]
@@ -96,6 +100,15 @@ def lib():
 class PrepParamsC(ctypes.Structure):
     _fields_ = [("heads", ctypes.c_uint32), ("kv_heads", ctypes.c_uint32), ("dim", ctypes.c_uint32),
                 ("half_dims", ctypes.c_uint32), ("log2_theta", ctypes.c_float), ("eps", ctypes.c_float)]
+
+
+class ConvParamsC(ctypes.Structure):
+    _fields_ = [("channels", ctypes.c_uint32), ("kernel_size", ctypes.c_uint32)]
+
+
+class StepParamsC(ctypes.Structure):
+    _fields_ = [("k_heads", ctypes.c_uint32), ("v_heads", ctypes.c_uint32), ("v_dim", ctypes.c_uint32),
+                ("eps", ctypes.c_float)]
 
 
 def check(rc, what):

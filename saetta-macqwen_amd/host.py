@@ -324,6 +324,31 @@ def record_store(plan, q_and_gate, k, v, q_norm, k_norm, q, keys, values, p, cap
     plan.op("attention_prep_store", launch)
 
 
+def deltanet_conv(plan, x, w, state, out, channels, kernel_size):
+    """Records deltanet_conv (kernels/layers.metal:203-226; conv_step, src/cpu/deltanet.rs:117-131):
+    depthwise causal conv1d + SiLU of one token; `state` [kernel_size - 1][channels] takes x in."""
+    for t, what in ((x, "x"), (w, "w"), (state, "state"), (out, "out")):
+        _need(t, torch.float32, what)
+    if x.numel() < channels or w.numel() < channels * kernel_size or state.numel() < (kernel_size - 1) * channels:
+        raise ValueError("deltanet_conv: buffers too small")
+    p = ffi.ConvParamsC(channels, kernel_size)
+    plan.op("deltanet_conv", lambda s: ffi.check(
+        ffi.lib().saetta_deltanet_conv(s, _ptr(x), _ptr(w), _ptr(state), _ptr(out), p), "deltanet_conv"))
+
+
+def deltanet_step(plan, q, k, v, a, b, a_log, dt_bias, state, z, norm_w, y, k_heads, v_heads, v_dim, eps):
+    """Records deltanet_step (kernels/layers.metal:297-357): normalize_qk, the gates, the delta rule
+    and the gated RMSNorm for every value head (src/cpu/deltanet.rs:86-112,133-155); key dim 128."""
+    ts = (q, k, v, a, b, a_log, dt_bias, state, z, norm_w, y)
+    for t in ts:
+        _need(t, torch.float32, "deltanet_step buffer")
+    if state.numel() < v_heads * v_dim * 128 or q.numel() < k_heads * 128 or v.numel() < v_heads * v_dim:
+        raise ValueError("deltanet_step: buffers too small")
+    p = ffi.StepParamsC(k_heads, v_heads, v_dim, eps)
+    plan.op("deltanet_step", lambda s: ffi.check(
+        ffi.lib().saetta_deltanet_step(s, *[_ptr(t) for t in ts], p), "deltanet_step"))
+
+
 def _median_ms(run, runs):
     """One warm-up, then the median of `runs` event-timed calls, in milliseconds."""
     ts = []

@@ -334,6 +334,34 @@ inline void record_store(plan::Plan &plan, const View &q_and_gate, const View &k
 
 }  // namespace gpu_layers
 
+namespace deltanet {
+
+// Records deltanet_conv (kernels/layers.metal:203-226): depthwise causal conv1d + SiLU of one token;
+// `state` [kernel_size - 1][channels] takes x in.
+inline void conv(plan::Plan &plan, const View &x, const View &w, const View &state, const View &out, size_t channels,
+                 size_t kernel_size) {
+    const saetta_conv_params p{uint32_t(channels), uint32_t(kernel_size)};
+    plan.op("deltanet_conv", [=](hipStream_t s) {
+        check(saetta_deltanet_conv(s, x.ptr<float>(), w.ptr<float>(), state.ptr<float>(), out.ptr<float>(), p), "deltanet_conv");
+    });
+}
+
+// Records deltanet_step (kernels/layers.metal:297-357): normalize_qk, the gates, the delta rule and
+// the gated RMSNorm for every value head; key dim 128.
+inline void step(plan::Plan &plan, const View &q, const View &k, const View &v, const View &a, const View &b, const View &a_log,
+                 const View &dt_bias, const View &state, const View &z, const View &norm_w, const View &y, size_t k_heads,
+                 size_t v_heads, size_t v_dim, float eps) {
+    const saetta_step_params p{uint32_t(k_heads), uint32_t(v_heads), uint32_t(v_dim), eps};
+    plan.op("deltanet_step", [=](hipStream_t s) {
+        check(saetta_deltanet_step(s, q.ptr<float>(), k.ptr<float>(), v.ptr<float>(), a.ptr<float>(), b.ptr<float>(),
+                                   a_log.ptr<float>(), dt_bias.ptr<float>(), state.ptr<float>(), z.ptr<float>(),
+                                   norm_w.ptr<float>(), y.ptr<float>(), p),
+              "deltanet_step");
+    });
+}
+
+}  // namespace deltanet
+
 namespace attention {
 
 constexpr size_t DIM = 256;
