@@ -22,7 +22,9 @@ cpu_baseline = the CPU oracle (a C restatement of the reference's
              single-threaded f32 CPU attention) on one of the layers.
 
 Other workloads (--workload): decode4_150k (4-bit, 150000 tokens), verify2..4
-(2-4 query rows at 32k, 8-bit), prefill (4096-token chunk at position 4096).
+(2-4 query rows at 32k, 8-bit), prefill (4096-token chunk at position 4096),
+deltanet (the Gated DeltaNet decode step over 30 layer states), all (the default
+line with the others under "other_workloads").
 """
 import argparse
 import json
@@ -266,13 +268,94 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8):
     }
 
 
+def bench_deltanet(s, torch, args, layers=30):
+    """Gated DeltaNet decode step (conv + step) over `layers` layer states of their own, the model's
+    shape: 16 key / 32 value heads of 128, conv kernel 4.  Algorithmic bytes per layer: the
+    recurrent state read and written, 2 x 32 x 128 x 128 x 4 B."""
+    import numpy as np
+    import oracle  # parity check and CPU-baseline leg only
+
+    kh, vh, dv, kernel, eps = 16, 32, 128, 4, 1e-6
+    key, val = kh * 128, vh * dv
+    ch = 2 * key + val
+    gen = torch.Generator(device="cuda").manual_seed(7)
+
+    def r(n, scale=1.0):
+        return torch.randn(n, generator=gen, device="cuda") * scale
+
+    x, z, a, b, alog, dtb, w = r(ch), r(val), r(vh), r(vh), r(vh), r(vh), r(ch * kernel, 0.5)
+    norm = 1 + r(dv, 0.1)
+    states = [(torch.zeros((kernel - 1) * ch, device="cuda"), r(vh * dv * 128, 0.1)) for _ in range(layers)]
+    first_state = states[0][1].clone()
+    mixed, y = torch.empty(ch, device="cuda"), torch.empty(val, device="cuda")
+
+    def plan_of(which):
+        plan = s.Plan()
+        for conv, st in states:
+            if which != "step":
+                s.deltanet_conv(plan, x, w, conv, mixed, ch, kernel)
+            if which != "conv":
+                s.deltanet_step(plan, mixed[:key], mixed[key:2 * key], mixed[2 * key:], a, b, alog, dtb, st, z, norm, y,
+                                kh, vh, dv, eps)
+        return plan.build(graph=not args.no_graph)
+
+    # parity of one step against the oracle, before the states are run over many times
+    one = s.Plan()
+    s.deltanet_conv(one, x, w, states[0][0], mixed, ch, kernel)
+    s.deltanet_step(one, mixed[:key], mixed[key:2 * key], mixed[2 * key:], a, b, alog, dtb, states[0][1], z, norm, y,
+                    kh, vh, dv, eps)
+    one.build().run()
+    torch.cuda.synchronize()
+    conv_cpu = np.zeros((kernel - 1, ch), np.float32)
+    st_cpu = first_state.cpu().numpy().copy()
+    c0 = time.perf_counter()
+    m_cpu = oracle.deltanet_conv(w.cpu().numpy().reshape(ch, kernel), x.cpu().numpy(), conv_cpu, kernel)
+    y_cpu = oracle.deltanet_step(m_cpu[:key], m_cpu[key:2 * key], m_cpu[2 * key:], a.cpu().numpy(), b.cpu().numpy(),
+                                 alog.cpu().numpy(), dtb.cpu().numpy(), st_cpu, z.cpu().numpy(), norm.cpu().numpy(),
+                                 kh, vh, 128, dv, eps)
+    cpu_s = time.perf_counter() - c0
+    rel = float(np.sqrt(((y.cpu().numpy() - y_cpu) ** 2).mean() / (y_cpu ** 2).mean()))
+
+    def timed(built):
+        for _ in range(args.warmup):
+            built.run()
+        ts = []
+        for _ in range(max(5, args.steps)):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            built.run()
+            e1.record()
+            e1.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e3 / layers)
+        return median(ts)
+
+    both_us, step_us = timed(plan_of("both")), timed(plan_of("step"))
+    nbytes = 2.0 * vh * dv * 128 * 4
+    achieved = nbytes / step_us / 1e3
+    return {
+        "metric": "Gated DeltaNet decode step, state GB/s",
+        "value": round(nbytes / both_us / 1e3, 1),
+        "unit": "GB/s",
+        "ms_per_step": round(both_us * layers / 1e3, 4),
+        "dtype": "f32",
+        "config": {"workload": f"Gated DeltaNet, one token, conv + step, {layers} layer states per step",
+                   "k_heads": kh, "v_heads": vh, "k_dim": 128, "v_dim": dv, "conv_kernel": kernel, "bytes_per_layer": nbytes},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "deltanet_step_kernel",
+                     "avg_us": round(step_us, 3)},
+        "cpu_baseline": {"value": round(nbytes / cpu_s / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                         "sample": f"one layer, conv + step ({cpu_s * 1e3:.2f} ms)"},
+        "parity_rel_rms_vs_oracle": float(f"{rel:.3e}"),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="decode8_32k",
-                    choices=["decode8_32k", "decode4_150k", "verify2", "verify3", "verify4", "prefill", "all"])
+                    choices=["decode8_32k", "decode4_150k", "verify2", "verify3", "verify4", "prefill", "deltanet", "all"])
     ap.add_argument("--no-graph", action="store_true", help="launch from Python instead of replaying a HIP graph")
     ap.add_argument("--layers", type=int, default=0, help="layer caches per step (default 32; 12 at 150k)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -305,12 +388,14 @@ def main():
             return bench_decode(s, torch, args, 150000, 4, 1, args.layers or 12)
         if workload.startswith("verify"):
             return bench_decode(s, torch, args, 32768, 8, int(workload[-1]), args.layers or 32)
+        if workload == "deltanet":
+            return bench_deltanet(s, torch, args)
         return bench_prefill(s, torch, args)
 
     if args.workload == "all":
         res = one("decode8_32k")
         res["other_workloads"] = {}
-        for w in ["verify2", "verify3", "verify4", "decode4_150k", "prefill"]:
+        for w in ["verify2", "verify3", "verify4", "decode4_150k", "prefill", "deltanet"]:
             torch.cuda.empty_cache()
             r = one(w)
             res["other_workloads"][w] = {k: r[k] for k in ("metric", "value", "unit", "ms_per_step", "roofline",
