@@ -762,12 +762,12 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     }
 }
 
-// One 16-row tile of query rows fits two waves per SIMD (8 per CU, i.e. two
-// workgroups per CU, which is what the split count is sized for); more tiles
-// take the whole register file.
-template <int BITS, bool PACKED>
+// One query row over codes (a single packed tile) fits two waves per SIMD, i.e. two workgroups
+// per CU (attention_partial_kernel_1, for long contexts); the others take the whole register file
+// and run one workgroup per CU.  Which one runs is decided in run_attention.
+template <int BITS>
 __global__ __launch_bounds__(THREADS, 2) void attention_partial_kernel_1(PartialArgs a) {
-    attention_partial_body<BITS, 1, PACKED>(a);
+    attention_partial_body<BITS, 1, true>(a);
 }
 
 template <int BITS, int TILES>
@@ -874,7 +874,7 @@ void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu) {
         if (one_per_cu) {
             kernel = attention_partial_kernel_p<BITS>;
         } else {
-            kernel = attention_partial_kernel_1<BITS, PACKED>;
+            kernel = attention_partial_kernel_1<BITS>;
         }
     } else if constexpr (PACKED) {
         kernel = attention_partial_kernel_p<BITS>;  // f16 cache: its registers do not fit two waves
