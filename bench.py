@@ -23,8 +23,9 @@ cpu_baseline = the CPU oracle (a C restatement of the reference's
 
 Other workloads (--workload): decode4_150k (4-bit, 150000 tokens), verify2..4
 (2-4 query rows at 32k, 8-bit), prefill (4096-token chunk at position 4096),
-deltanet (the Gated DeltaNet decode step over 30 layer states), all (the default
-line with the others under "other_workloads").
+deltanet (the Gated DeltaNet decode step over 30 layer states), deltanet_prefill
+(conv + delta rule + gated norm of a 4096-token chunk of one layer), all (the
+default line with the others under "other_workloads").
 """
 import argparse
 import json
@@ -349,13 +350,99 @@ def bench_deltanet(s, torch, args, layers=30):
     }
 
 
+def bench_deltanet_prefill(s, torch, args, tokens=4096):
+    """A prefill chunk of one Gated DeltaNet layer: deltanet_conv_rows + deltanet_rows over `tokens`
+    tokens in order, the model's shape.  Algorithmic bytes of the rows launch: `mixed` and a, b read,
+    o written, the gated norm's read of o and z and write of y, the state read and written.  The
+    delta rule itself is a chain over the tokens (7 f32 flops per state value and token), so the
+    f32 vector rate is reported beside the HBM fraction."""
+    import numpy as np
+    import oracle  # parity check and CPU-baseline leg only
+
+    kh, vh, dv, kernel, eps = 16, 32, 128, 4, 1e-6
+    key, val = kh * 128, vh * dv
+    ch = 2 * key + val
+    gen = torch.Generator(device="cuda").manual_seed(9)
+
+    def r(*n, scale=1.0):
+        return torch.randn(*n, generator=gen, device="cuda") * scale
+
+    x, z, a, b = r(tokens, ch), r(tokens, val), r(tokens, vh), r(tokens, vh)
+    alog, dtb, w, norm = r(vh), r(vh), r(ch * kernel, scale=0.5), 1 + r(dv, scale=0.1)
+    conv, st = torch.zeros((kernel - 1) * ch, device="cuda"), torch.zeros(vh * dv * 128, device="cuda")
+    mixed, y = torch.empty(tokens, ch, device="cuda"), torch.empty(tokens, val, device="cuda")
+
+    def plan_of(which, n=tokens):
+        plan = s.Plan()
+        if which != "rows":
+            s.deltanet_conv_rows(plan, x, w, conv, mixed, ch, kernel, n)
+        if which != "conv":
+            s.deltanet_rows(plan, mixed, a, b, alog, dtb, st, z, norm, y, kh, vh, dv, n, eps)
+        return plan.build(graph=not args.no_graph)
+
+    # parity of the first tokens against the oracle (token by token), from zero states
+    n_check = 24
+    plan_of("both", n_check).run()
+    torch.cuda.synchronize()
+    conv_cpu, st_cpu = np.zeros((kernel - 1, ch), np.float32), np.zeros(vh * dv * 128, np.float32)
+    xs, zs, as_, bs = (t[:n_check].cpu().numpy() for t in (x, z, a, b))
+    wn, an, dn, nn = w.cpu().numpy().reshape(ch, kernel), alog.cpu().numpy(), dtb.cpu().numpy(), norm.cpu().numpy()
+    c0 = time.perf_counter()
+    want = []
+    for t in range(n_check):
+        m = oracle.deltanet_conv(wn, xs[t], conv_cpu, kernel)
+        want.append(oracle.deltanet_step(m[:key], m[key:2 * key], m[2 * key:], as_[t], bs[t], an, dn, st_cpu, zs[t], nn,
+                                         kh, vh, 128, dv, eps))
+    cpu_s = (time.perf_counter() - c0) / n_check
+    want = np.stack(want)
+    rel = float(np.sqrt(((y[:n_check].cpu().numpy() - want) ** 2).mean() / (want ** 2).mean()))
+    conv.zero_(), st.zero_()
+
+    def timed(built):
+        for _ in range(min(args.warmup, 2)):
+            built.run()
+        ts = []
+        for _ in range(max(5, min(args.steps, 10))):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            built.run()
+            e1.record()
+            e1.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e3)
+        return median(ts)
+
+    both_us, rows_us = timed(plan_of("both")), timed(plan_of("rows"))
+    rows_bytes = 4.0 * (tokens * ch + 2 * tokens * vh + 4 * tokens * val + 2 * vh * dv * 128)
+    conv_bytes = 4.0 * 2 * tokens * ch
+    flops = 7.0 * tokens * vh * dv * 128
+    achieved = rows_bytes / rows_us / 1e3
+    return {
+        "metric": "Gated DeltaNet prefill chunk, tokens/s of one layer",
+        "value": round(tokens / both_us * 1e6, 1),
+        "unit": "tokens/s",
+        "ms_per_step": round(both_us / 1e3, 4),
+        "dtype": "f32",
+        "config": {"workload": f"Gated DeltaNet, {tokens}-token chunk of one layer, conv + delta rule + gated norm",
+                   "k_heads": kh, "v_heads": vh, "k_dim": 128, "v_dim": dv, "conv_kernel": kernel,
+                   "bytes_rows_launch": rows_bytes, "bytes_conv_launch": conv_bytes},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "deltanet_rows_kernel + deltanet_gated_norm_rows_kernel", "avg_us": round(rows_us, 1),
+                     "f32_vector_TFLOPs": round(flops / rows_us / 1e6, 2), "f32_vector_peak_TFLOPs": 157.3},
+        "cpu_baseline": {"value": round(1.0 / cpu_s, 1), "unit": "tokens/s", "cores": 1, "kind": "port",
+                         "sample": f"the first {n_check} tokens, conv + step each ({cpu_s * 1e3:.2f} ms per token)"},
+        "parity_rel_rms_vs_oracle": float(f"{rel:.3e}"),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="decode8_32k",
-                    choices=["decode8_32k", "decode4_150k", "verify2", "verify3", "verify4", "prefill", "deltanet", "all"])
+                    choices=["decode8_32k", "decode4_150k", "verify2", "verify3", "verify4", "prefill", "deltanet",
+                             "deltanet_prefill", "all"])
     ap.add_argument("--no-graph", action="store_true", help="launch from Python instead of replaying a HIP graph")
     ap.add_argument("--layers", type=int, default=0, help="layer caches per step (default 32; 12 at 150k)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -390,12 +477,14 @@ def main():
             return bench_decode(s, torch, args, 32768, 8, int(workload[-1]), args.layers or 32)
         if workload == "deltanet":
             return bench_deltanet(s, torch, args)
+        if workload == "deltanet_prefill":
+            return bench_deltanet_prefill(s, torch, args)
         return bench_prefill(s, torch, args)
 
     if args.workload == "all":
         res = one("decode8_32k")
         res["other_workloads"] = {}
-        for w in ["verify2", "verify3", "verify4", "decode4_150k", "prefill", "deltanet"]:
+        for w in ["verify2", "verify3", "verify4", "decode4_150k", "prefill", "deltanet", "deltanet_prefill"]:
             torch.cuda.empty_cache()
             r = one(w)
             res["other_workloads"][w] = {k: r[k] for k in ("metric", "value", "unit", "ms_per_step", "roofline",

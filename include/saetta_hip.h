@@ -114,6 +114,24 @@ typedef struct saetta_step_params {
     uint32_t v_dim;
     float eps;
 } saetta_step_params;
+/* ConvRowsParams (kernels/prefill.metal:571-576). */
+typedef struct saetta_conv_rows_params {
+    uint32_t channels;
+    uint32_t kernel_size;
+    uint32_t tokens;
+    uint32_t snapshots; /* write the state after each token to `snaps` */
+} saetta_conv_rows_params;
+/* DeltaRowsParams (kernels/prefill.metal:629-637) and RowsStepParams
+ * (src/gpu_layers.rs:563-571); the floats per token of `mixed` follow from
+ * the heads: 2 * k_heads * 128 + v_heads * v_dim. */
+typedef struct saetta_rows_step_params {
+    uint32_t k_heads;
+    uint32_t v_heads;
+    uint32_t v_dim;
+    uint32_t tokens;
+    float eps;
+    uint32_t snapshots; /* write the state after each token to `snaps` */
+} saetta_rows_step_params;
 
 /* The three arrays of one quantized cache, keys or values: QuantRows
  * {data, scales, biases} (src/kv_quant.rs:156-180).  Token p's groups start
@@ -127,9 +145,10 @@ typedef struct saetta_quant_rows {
 
 /* ---- set-up --------------------------------------------------------------- */
 
-/* Checks that the current device is gfx950 and that the kernels load.  Stands
- * where Gpu::new() (src/gpu.rs:233-263) stands for this path.  Optional: every
- * entry point does the same check on first use. */
+/* Checks that the current device is gfx950, loads the kernels and raises their
+ * LDS limits.  Stands where Gpu::new() (src/gpu.rs:233-263) stands for this
+ * path.  Every entry point does the same on first use, but that first use must
+ * not be under stream capture: call this before capturing a graph. */
 int saetta_init(void);
 
 /* Text of the last error on this thread ("" if none). */
@@ -258,6 +277,33 @@ int saetta_deltanet_step(saetta_stream_t stream, const float *q, const float *k,
                          const float *a, const float *b, const float *a_log, const float *dt_bias,
                          float *state, const float *z, const float *norm_w, float *y,
                          saetta_step_params p);
+
+/* ---- Gated DeltaNet, several tokens in order: verify rows and prefill chunks -- */
+
+/* conv over `tokens` tokens: kernels conv_rows2 + conv_state
+ * (kernels/prefill.metal:734-786, recorded by src/prefill.rs:1455-1485) and
+ * deltanet_conv_rows (kernels/layers.metal:510-544).  x, out f32
+ * [tokens][channels]; w and state as for saetta_deltanet_conv; the state ends as
+ * the last kernel_size - 1 inputs.  With snapshots, snaps f32
+ * [tokens][kernel_size - 1][channels] gets the state after each token (what
+ * GpuDeltaNetSnaps.conv holds, src/gpu_layers.rs:819-836); else it may be NULL. */
+int saetta_deltanet_conv_rows(saetta_stream_t stream, const float *x, const float *w, float *state, float *out,
+                              float *snaps, saetta_conv_rows_params p);
+
+/* What saetta_deltanet_step does, for `tokens` tokens one after the other:
+ * kernels delta_prep + delta_rows3 and the gated norm (kernels/prefill.metal:788-1116,
+ * src/prefill.rs:1487-1578), deltanet_step_rows (kernels/layers.metal:546-635,
+ * GpuDeltaNet::record_rows, src/gpu_layers.rs:686-786).  mixed f32
+ * [tokens][2 * k_heads * 128 + v_heads * v_dim] is the conv output: q of every
+ * key head, then k, then v of every value head; unlike delta_prep the call
+ * leaves it (and a, b) unchanged.  a, b f32 [tokens][v_heads]; z, y f32
+ * [tokens][v_heads][v_dim]; state f32 [v_heads][v_dim][128] updated in place.
+ * With snapshots, snaps f32 [tokens][v_heads][v_dim][128] gets the state after
+ * each token (GpuDeltaNetSnaps.recurrent); else it may be NULL.  Key dim 128,
+ * v_dim a multiple of 4 up to 256. */
+int saetta_deltanet_rows(saetta_stream_t stream, const float *mixed, const float *a, const float *b,
+                         const float *a_log, const float *dt_bias, float *state, const float *z,
+                         const float *norm_w, float *y, float *snaps, saetta_rows_step_params p);
 
 /* ---- prefill attention (src/attention_prefill.rs, src/prefill.rs) ---------- */
 

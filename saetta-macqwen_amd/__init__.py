@@ -10,9 +10,11 @@ be checked), every call needs the library and a gfx950 device.
 """
 from . import ffi
 from .host import (GROUP, MAX_ROWS, AttentionRows, Built, DecodeAttention, FlashParams, KvBits, Plan,
-                   PrepParams, QuantRows, TokenParams, attention_prefill, bench, deltanet_conv, deltanet_step, dequantize, quantize, round_trip,
+                   PrepParams, QuantRows, TokenParams, attention_prefill, bench, deltanet_conv, deltanet_conv_rows, deltanet_rows,
+                   deltanet_step, dequantize, quantize, round_trip,
                    record_store, round_trip_as_half, test_slack, to_half)
 
 __all__ = ["ffi", "GROUP", "MAX_ROWS", "AttentionRows", "Built", "DecodeAttention", "FlashParams", "KvBits",
-           "Plan", "PrepParams", "QuantRows", "TokenParams", "attention_prefill", "bench", "deltanet_conv", "deltanet_step", "dequantize", "quantize",
+           "Plan", "PrepParams", "QuantRows", "TokenParams", "attention_prefill", "bench", "deltanet_conv", "deltanet_conv_rows",
+           "deltanet_rows", "deltanet_step", "dequantize", "quantize",
            "record_store", "round_trip", "round_trip_as_half", "test_slack", "to_half"]

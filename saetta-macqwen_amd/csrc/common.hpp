@@ -20,6 +20,20 @@ int ensure_device();
 // Turns the status of the launches since the last call into a return code.
 int launch_status(const char *what);
 
+// One-time set-up of a source file's kernels on the current device: loads their code object and
+// raises their dynamic LDS limits, so that a first launch under stream capture has nothing left to
+// do.  Called from ensure_device(); each returns a hipError_t as int.
+int setup_kv_quant();
+int setup_prep();
+int setup_deltanet();
+int setup_decode();
+int setup_prefill();
+// Loads the code object `kernel` lives in.
+inline int load_kernel(const void *kernel) {
+    hipFuncAttributes attr;
+    return int(hipFuncGetAttributes(&attr, kernel));
+}
+
 inline hipStream_t as_stream(saetta_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }

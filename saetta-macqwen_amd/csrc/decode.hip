@@ -881,12 +881,7 @@ void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu) {
     } else {
         kernel = attention_partial_kernel_n<BITS, TILES>;
     }
-    static bool attr_set = false;
-    if (!attr_set && Sh::LDS_BYTES > 48 * 1024) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, Sh::LDS_BYTES);
-        attr_set = true;
-    }
+    // (the dynamic LDS limit of every variant was raised in setup_decode)
     kernel<<<dim3(a.nsplits, a.kv_heads), THREADS, Sh::LDS_BYTES, stream>>>(a);
 }
 
@@ -951,6 +946,31 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
 }
 
 }  // namespace
+
+namespace {
+template <int BITS, int TILES, bool PACKED>
+int raise_lds(void (*kernel)(PartialArgs)) {
+    if (Shape<BITS, TILES, PACKED>::LDS_BYTES <= 48 * 1024) return 0;
+    return int(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   Shape<BITS, TILES, PACKED>::LDS_BYTES));
+}
+template <int BITS>
+int raise_lds_of_bits() {
+    if (int rc = raise_lds<BITS, 1, true>(attention_partial_kernel_p<BITS>)) return rc;
+    if (int rc = raise_lds<BITS, 1, false>(attention_partial_kernel_n<BITS, 1>)) return rc;
+    if (int rc = raise_lds<BITS, 2, false>(attention_partial_kernel_n<BITS, 2>)) return rc;
+    return raise_lds<BITS, 4, false>(attention_partial_kernel_n<BITS, 4>);
+}
+}  // namespace
+
+int setup_decode() {
+    if (int rc = load_kernel(reinterpret_cast<const void *>(attention_reduce_kernel))) return rc;
+    if (int rc = raise_lds_of_bits<8>()) return rc;
+    if (int rc = raise_lds_of_bits<4>()) return rc;
+    if (int rc = raise_lds_of_bits<16>()) return rc;
+    if (int rc = raise_lds<8, 1, true>(attention_partial_kernel_1<8>)) return rc;
+    return raise_lds<4, 1, true>(attention_partial_kernel_1<4>);
+}
 }  // namespace saetta
 
 using namespace saetta;

@@ -18,6 +18,8 @@
 #include "common.hpp"
 #include "lanes.hpp"
 
+#include <type_traits>
+
 namespace saetta {
 namespace {
 
@@ -113,7 +115,296 @@ __global__ __launch_bounds__(STEP_THREADS) void deltanet_step_kernel(StepArgs a)
     }
 }
 
+
+// ---- several tokens in one launch: verify rows and prefill chunks ------------------------------
+//
+// Reference: conv_rows2 + conv_state, delta_prep + delta_rows3 and the gated norm after them
+// (kernels/prefill.metal:734-1116, recorded by src/prefill.rs:1433-1578), and for verify rows
+// deltanet_conv_rows + deltanet_step_rows (kernels/layers.metal:510-635, src/gpu_layers.rs:686-786).
+// Token t + 1 sees the state token t left, exactly as t single-token calls would.
+
+// One thread per (channel, tile of CONV_TILE tokens).  Input i of the window of token t is
+// x[i] for i >= 0 and the stored state row i + kernel_size - 1 before that; the taps are added
+// oldest first, as the single-token kernel does.
+constexpr uint32_t CONV_TILE = 32;
+
+__device__ __forceinline__ float conv_input(const float *x, const float *state, int i, uint32_t c,
+                                            const saetta_conv_rows_params &p) {
+    return i >= 0 ? x[size_t(i) * p.channels + c] : state[size_t(i + int(p.kernel_size) - 1) * p.channels + c];
+}
+
+__global__ __launch_bounds__(256) void deltanet_conv_rows_kernel(const float *__restrict__ x,
+                                                                 const float *__restrict__ w,
+                                                                 const float *__restrict__ state,
+                                                                 float *__restrict__ out, float *__restrict__ snaps,
+                                                                 saetta_conv_rows_params p) {
+    const uint32_t c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= p.channels) return;
+    const int past = int(p.kernel_size) - 1;
+    const float *wc = w + size_t(c) * p.kernel_size;
+    const uint32_t t_end = min(p.tokens, (blockIdx.y + 1) * CONV_TILE);
+    for (uint32_t t = blockIdx.y * CONV_TILE; t < t_end; t++) {
+        float acc = 0.0f;
+        for (int j = 0; j < past; j++) acc += wc[j] * conv_input(x, state, int(t) - past + j, c, p);
+        out[size_t(t) * p.channels + c] = silu_f(acc + wc[past] * x[size_t(t) * p.channels + c]);
+        if (p.snapshots) {
+            float *snap = snaps + size_t(t) * past * p.channels;
+            for (int j = 0; j < past; j++) snap[size_t(j) * p.channels + c] = conv_input(x, state, int(t) - past + 1 + j, c, p);
+        }
+    }
+}
+
+// After the outputs: the last kernel_size - 1 inputs become the state.  Rows are written in
+// ascending order and row j only reads rows above it (or x), so the shift is safe in place.
+__global__ __launch_bounds__(256) void deltanet_conv_state_kernel(const float *__restrict__ x, float *state,
+                                                                  saetta_conv_rows_params p) {
+    const uint32_t c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= p.channels) return;
+    const int past = int(p.kernel_size) - 1;
+    for (int j = 0; j < past; j++) {
+        state[size_t(j) * p.channels + c] = conv_input(x, state, int(p.tokens) - past + j, c, p);
+    }
+}
+
+// The delta rule over the tokens, in order.  A workgroup owns a few rows of one value head's state
+// for the whole launch: LANES lanes per row, 128 / LANES state values per lane in registers.  The
+// chain from one token to the next (decay, S_i . k, its sum over the row's lanes, delta, update)
+// cannot be shortened, so the rows are spread as wide as the chip: 32 lanes per row make the 4096
+// rows of 32 heads two wavefronts on every SIMD, one running while the other waits on its chain.
+// The q and k of the head's key head are the same for all its rows: they are staged per block of 16
+// tokens in LDS (double buffered; the next block's loads are in flight while this one runs),
+// normalised on the way in; g, beta and v of a block sit in the lanes (lane p of each 16 holds
+// token p's) and reach the others by DPP row broadcasts.
+constexpr int ROWS_TB = 16;  // tokens per staged block
+#ifndef ROWS_LANES_PER_ROW
+#define ROWS_LANES_PER_ROW 16
+#endif
+
+struct RowsArgs {
+    const float *mixed, *a, *b, *a_log, *dt_bias;
+    float *state;
+    float *o;      // [tokens][v_heads][v_dim], before the gated norm
+    float *snaps;  // [tokens] copies of the state, or unused
+    saetta_rows_step_params p;
+    uint32_t channels;
+};
+
+template <int I>
+__device__ __forceinline__ float row_lane(float x) {
+    // value of lane I of every row of 16 lanes
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x150 + I, 0xf, 0xf, true));
+}
+
+template <int I>
+struct TokenLoop {
+    template <class F>
+    static __device__ __forceinline__ void run(F &&f) {
+        f(std::integral_constant<int, I>{});
+        if constexpr (I + 1 < ROWS_TB) TokenLoop<I + 1>::run(f);
+    }
+};
+
+// sum of N float4 products as a tree (N = 1 or 2): two or three dependent additions after the products
+template <int N>
+__device__ __forceinline__ float dot_tree(const float4 (&a)[N], const float4 (&b)[N]) {
+    float sum = (a[0].x * b[0].x + a[0].y * b[0].y) + (a[0].z * b[0].z + a[0].w * b[0].w);
+    if constexpr (N == 2) sum += (a[1].x * b[1].x + a[1].y * b[1].y) + (a[1].z * b[1].z + a[1].w * b[1].w);
+    return sum;
+}
+
+template <bool SNAPS, int LANES>
+__global__ __launch_bounds__(256) void deltanet_rows_kernel(RowsArgs a) {
+    constexpr int PER_LANE = K_DIM / LANES;  // state values per lane: 8 or 4
+    constexpr int F4 = PER_LANE / 4;         // as float4s
+    constexpr int ROWS_PER_WG = 256 / LANES;
+    static_assert(LANES == 16 || LANES == 32, "a row is one or two DPP rows");
+    // a token's q and k: [q | k][float4 of the lane][lane][4] floats, so that the lanes of a row read
+    // contiguous bytes
+    __shared__ __attribute__((aligned(16))) float qk_lds[2][ROWS_TB][2 * K_DIM];
+    __shared__ float gb_lds[2][ROWS_TB][2];
+    __shared__ float o_lds[ROWS_TB][ROWS_PER_WG];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t h = blockIdx.y, part = tid % LANES, row_in_wg = tid / LANES;
+    const uint32_t tok_lane = tid & 15;  // the token of a block whose g, beta and v this lane holds
+    const uint32_t row = blockIdx.x * ROWS_PER_WG + row_in_wg;
+    const uint32_t v_dim = a.p.v_dim, v_heads = a.p.v_heads, tokens = a.p.tokens;
+    const bool live = row < v_dim;
+    const uint32_t kh = h / (v_heads / a.p.k_heads);
+    const uint32_t key_size = a.p.k_heads * K_DIM;
+    const size_t value_size = size_t(v_heads) * v_dim;
+
+    float4 st[F4];
+    float *sp = a.state + (size_t(h) * v_dim + (live ? row : 0)) * K_DIM + part * PER_LANE;
+#pragma unroll
+    for (int c = 0; c < F4; c++) st[c] = live ? reinterpret_cast<const float4 *>(sp)[c] : make_float4(0, 0, 0, 0);
+
+    const float exp_a = expf(a.a_log[h]);
+    const float bias = a.dt_bias[h];
+    const float q_scale = 1.0f / sqrtf(float(K_DIM));
+
+    // ---- one block's inputs, as loaded (registers) --------------------------------------------
+    // thread -> float4 `lane` of token wave + 4 j of the block: lanes 0-31 are q, 32-63 are k
+    float4 raw[ROWS_TB / 4];
+    float ga = 0.0f, gbv = 0.0f;  // a and b of token `tid` (threads 0-15)
+    bool g_real = false;          // that token exists
+    float nv = 0.0f;              // v of token `tok_lane`, this thread's row
+    auto load_block = [&](uint32_t t0) {
+        const uint32_t off = (lane < 32 ? 0 : key_size) + kh * K_DIM + 4 * (lane & 31);
+#pragma unroll
+        for (int j = 0; j < ROWS_TB / 4; j++) {
+            const uint32_t t = t0 + wave + 4 * j;
+            raw[j] = make_float4(0, 0, 0, 0);
+            if (t < tokens) raw[j] = *reinterpret_cast<const float4 *>(a.mixed + size_t(t) * a.channels + off);
+        }
+        g_real = t0 + tid < tokens;
+        if (tid < ROWS_TB && g_real) {
+            ga = a.a[size_t(t0 + tid) * v_heads + h];
+            gbv = a.b[size_t(t0 + tid) * v_heads + h];
+        }
+        nv = 0.0f;
+        if (live && t0 + tok_lane < tokens) {
+            nv = a.mixed[size_t(t0 + tok_lane) * a.channels + 2 * key_size + h * v_dim + row];
+        }
+    };
+    // normalise (src/cpu/deltanet.rs:133-146), compute the gates, and put the block into buffer `buf`
+    auto store_block = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < ROWS_TB / 4; j++) {
+            const float4 x = raw[j];
+            const float ss = group_reduce<32>(dot4(x, x), SumOp());
+            const float inv = (lane < 32 ? q_scale : 1.0f) / sqrtf(ss + a.p.eps);
+            const uint32_t f = lane & 31;  // float4 f of the vector belongs to lane f / F4, its float4 f % F4
+            float *dst = &qk_lds[buf][wave + 4 * j][(lane < 32 ? 0 : K_DIM) + (f % F4) * (LANES * 4) + (f / F4) * 4];
+            *reinterpret_cast<float4 *>(dst) = make_float4(x.x * inv, x.y * inv, x.z * inv, x.w * inv);
+        }
+        if (tid < ROWS_TB) {
+            const float xg = ga + bias;
+            const float softplus = fmaxf(xg, 0.0f) + log1pf(expf(-fabsf(xg)));
+            gb_lds[buf][tid][0] = g_real ? expf(-exp_a * softplus) : 1.0f;
+            gb_lds[buf][tid][1] = g_real ? sigmoid_f(gbv) : 0.0f;
+        }
+    };
+
+    load_block(0);
+    store_block(0);
+    float v_cur = nv;
+    __syncthreads();
+
+    int cur = 0;
+    for (uint32_t t0 = 0; t0 < tokens; t0 += ROWS_TB) {
+        const bool more = t0 + ROWS_TB < tokens;
+        if (more) load_block(t0 + ROWS_TB);
+        const float g_mine = gb_lds[cur][tok_lane][0], b_mine = gb_lds[cur][tok_lane][1];
+        const float v_mine = v_cur;
+
+        // Tokens past the end of a ragged last block are staged as q = k = 0, g = 1, beta = 0: they
+        // leave the state as it is, so the 16 steps run without a branch between them, and token
+        // I + 1's q and k are read from LDS while token I is computed.
+        float4 q_next[F4], k_next[F4];
+        auto read_qk = [&](int i) {
+            const float *qk = qk_lds[cur][i];
+#pragma unroll
+            for (int c = 0; c < F4; c++) {
+                q_next[c] = *reinterpret_cast<const float4 *>(qk + c * (LANES * 4) + part * 4);
+                k_next[c] = *reinterpret_cast<const float4 *>(qk + K_DIM + c * (LANES * 4) + part * 4);
+            }
+        };
+        read_qk(0);
+        float out_mine = 0.0f;  // lane `tok_lane` keeps the output of that token
+        float out_part = 0.0f;  // this lane's share of the previous token's output: its sum over the
+                                // row is not needed by the next token, so it runs beside that token's chain
+        auto token = [&](auto index) {
+            constexpr int I = decltype(index)::value;
+            float4 q[F4], k[F4];
+#pragma unroll
+            for (int c = 0; c < F4; c++) q[c] = q_next[c], k[c] = k_next[c];
+            if constexpr (I + 1 < ROWS_TB) read_qk(I + 1);
+            __builtin_amdgcn_sched_barrier(0);  // the reads stay here, a token ahead of their use
+            if constexpr (I > 0) {
+                const float out = group_reduce<LANES>(out_part, SumOp());
+                out_mine = tok_lane == I - 1 ? out : out_mine;
+            }
+            const float gt = row_lane<I>(g_mine), bt = row_lane<I>(b_mine), vt = row_lane<I>(v_mine);
+#pragma unroll
+            for (int c = 0; c < F4; c++) st[c].x *= gt, st[c].y *= gt, st[c].z *= gt, st[c].w *= gt;
+            const float mem = group_reduce<LANES>(dot_tree<F4>(st, k), SumOp());
+            const float delta = (vt - mem) * bt;
+#pragma unroll
+            for (int c = 0; c < F4; c++) {
+                st[c].x += k[c].x * delta, st[c].y += k[c].y * delta, st[c].z += k[c].z * delta, st[c].w += k[c].w * delta;
+            }
+            out_part = dot_tree<F4>(st, q);
+            if constexpr (SNAPS) {
+                if (live && t0 + I < tokens) {
+                    float *snap = a.snaps + size_t(t0 + I) * v_heads * v_dim * K_DIM +
+                                  (size_t(h) * v_dim + row) * K_DIM + part * PER_LANE;
+#pragma unroll
+                    for (int c = 0; c < F4; c++) reinterpret_cast<float4 *>(snap)[c] = st[c];
+                }
+            }
+        };
+        TokenLoop<0>::run(token);
+        {
+            const float out = group_reduce<LANES>(out_part, SumOp());
+            out_mine = tok_lane == ROWS_TB - 1 ? out : out_mine;
+        }
+        if (part < ROWS_TB) o_lds[part][row_in_wg] = out_mine;
+
+        if (more) {
+            store_block(cur ^ 1);
+            v_cur = nv;
+        }
+        __syncthreads();  // the block's outputs are in o_lds; the next block is staged
+        if (tid < ROWS_TB * ROWS_PER_WG) {
+            // thread -> (token, row): the rows of a token are contiguous
+            const uint32_t ti = tid / ROWS_PER_WG, ri = tid % ROWS_PER_WG;
+            const uint32_t t = t0 + ti, r = blockIdx.x * ROWS_PER_WG + ri;
+            if (t < tokens && r < v_dim) a.o[size_t(t) * value_size + size_t(h) * v_dim + r] = o_lds[ti][ri];
+        }
+        __syncthreads();  // o_lds is free again
+        cur ^= 1;
+    }
+    if (live) {
+#pragma unroll
+        for (int c = 0; c < F4; c++) reinterpret_cast<float4 *>(sp)[c] = st[c];
+    }
+}
+
+// y = o / sqrt(mean(o^2) + eps) * norm_w * silu(z) per (token, value head), in place on y:
+// one wavefront per pair, v_dim up to 256.
+__global__ __launch_bounds__(256) void deltanet_gated_norm_rows_kernel(float *y, const float *__restrict__ z,
+                                                                       const float *__restrict__ norm_w,
+                                                                       uint32_t pairs, uint32_t v_dim, float eps) {
+    const uint32_t pair = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (pair >= pairs) return;
+    float *yp = y + size_t(pair) * v_dim;
+    const float *zp = z + size_t(pair) * v_dim;
+    float o[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t d = lane + 64 * i;
+        o[i] = d < v_dim ? yp[d] : 0.0f;
+    }
+    // the single-token kernel sums 64-lane partials in the same order: lanes first, then the groups of 64
+    float total = 0.0f;
+    {
+        float part_sum[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) part_sum[i] = group_reduce<64>(o[i] * o[i], SumOp());
+#pragma unroll
+        for (int i = 0; i < 4; i++) total += part_sum[i];
+    }
+    const float inv = 1.0f / sqrtf(total / float(v_dim) + eps);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t d = lane + 64 * i;
+        if (d < v_dim) yp[d] = o[i] * (inv * norm_w[d]) * silu_f(zp[d]);
+    }
+}
+
 }  // namespace
+
+int setup_deltanet() { return load_kernel(reinterpret_cast<const void *>(deltanet_step_kernel)); }
 }  // namespace saetta
 
 using namespace saetta;
@@ -146,4 +437,48 @@ extern "C" int saetta_deltanet_step(saetta_stream_t stream, const float *q, cons
     StepArgs args{q, k, v, a, b, a_log, dt_bias, state, z, norm_w, y, p};
     deltanet_step_kernel<<<p.v_heads, STEP_THREADS, 0, as_stream(stream)>>>(args);
     return launch_status("deltanet_step");
+}
+
+extern "C" int saetta_deltanet_conv_rows(saetta_stream_t stream, const float *x, const float *w, float *state,
+                                         float *out, float *snaps, saetta_conv_rows_params p) {
+    SAETTA_REQUIRE(x && w && state && out, SAETTA_E_NULL, "deltanet_conv_rows: null buffer");
+    SAETTA_REQUIRE(!p.snapshots || snaps, SAETTA_E_NULL, "deltanet_conv_rows: snapshots asked for, no buffer");
+    SAETTA_REQUIRE(p.kernel_size >= 2 && p.kernel_size <= 16, SAETTA_E_SHAPE,
+                   "deltanet_conv_rows: kernel size %u (2..16)", p.kernel_size);
+    SAETTA_REQUIRE(p.tokens <= (1u << 20), SAETTA_E_SHAPE, "deltanet_conv_rows: %u tokens", p.tokens);
+    if (int rc = ensure_device()) return rc;
+    if (p.channels == 0 || p.tokens == 0) return SAETTA_OK;
+    const dim3 grid((p.channels + 255) / 256, (p.tokens + CONV_TILE - 1) / CONV_TILE);
+    deltanet_conv_rows_kernel<<<grid, 256, 0, as_stream(stream)>>>(x, w, state, out, snaps, p);
+    deltanet_conv_state_kernel<<<grid.x, 256, 0, as_stream(stream)>>>(x, state, p);
+    return launch_status("deltanet_conv_rows");
+}
+
+extern "C" int saetta_deltanet_rows(saetta_stream_t stream, const float *mixed, const float *a, const float *b,
+                                    const float *a_log, const float *dt_bias, float *state, const float *z,
+                                    const float *norm_w, float *y, float *snaps, saetta_rows_step_params p) {
+    SAETTA_REQUIRE(mixed && a && b && a_log && dt_bias && state && z && norm_w && y, SAETTA_E_NULL,
+                   "deltanet_rows: null buffer");
+    SAETTA_REQUIRE(!p.snapshots || snaps, SAETTA_E_NULL, "deltanet_rows: snapshots asked for, no buffer");
+    SAETTA_REQUIRE(p.k_heads > 0 && p.v_heads > 0 && p.v_heads % p.k_heads == 0, SAETTA_E_SHAPE,
+                   "deltanet_rows: %u value heads over %u key heads", p.v_heads, p.k_heads);
+    SAETTA_REQUIRE(p.v_dim >= 1 && p.v_dim <= 256 && p.v_dim % 4 == 0, SAETTA_E_SHAPE,
+                   "deltanet_rows: value dim %u (a multiple of 4 up to 256); the key dim is 128", p.v_dim);
+    SAETTA_REQUIRE(p.tokens <= (1u << 20), SAETTA_E_SHAPE, "deltanet_rows: %u tokens", p.tokens);
+    SAETTA_REQUIRE(aligned(mixed, 16) && aligned(state, 16) && (!p.snapshots || aligned(snaps, 16)), SAETTA_E_ALIGN,
+                   "deltanet_rows: mixed, the state and the snapshots must be 16-byte aligned");
+    if (int rc = ensure_device()) return rc;
+    if (p.tokens == 0) return SAETTA_OK;
+    const uint32_t channels = 2 * p.k_heads * K_DIM + p.v_heads * p.v_dim;
+    RowsArgs args{mixed, a, b, a_log, dt_bias, state, y, snaps, p, channels};
+    constexpr int LANES = ROWS_LANES_PER_ROW, ROWS_PER_WG = 256 / LANES;
+    const dim3 grid((p.v_dim + ROWS_PER_WG - 1) / ROWS_PER_WG, p.v_heads);
+    if (p.snapshots) {
+        deltanet_rows_kernel<true, LANES><<<grid, 256, 0, as_stream(stream)>>>(args);
+    } else {
+        deltanet_rows_kernel<false, LANES><<<grid, 256, 0, as_stream(stream)>>>(args);
+    }
+    const uint32_t pairs = p.tokens * p.v_heads;
+    deltanet_gated_norm_rows_kernel<<<(pairs + 3) / 4, 256, 0, as_stream(stream)>>>(y, z, norm_w, pairs, p.v_dim, p.eps);
+    return launch_status("deltanet_rows");
 }

@@ -140,6 +140,8 @@ __global__ __launch_bounds__(256) void to_half_kernel(const float *__restrict__ 
 }
 
 }  // namespace
+
+int setup_kv_quant() { return load_kernel(reinterpret_cast<const void *>(kv_quantize_kernel<8>)); }
 }  // namespace saetta
 
 using namespace saetta;

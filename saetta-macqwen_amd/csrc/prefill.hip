@@ -811,18 +811,18 @@ int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kda
     }
     PrefillArgs a{q, static_cast<const unsigned char *>(workspace), q_and_gate, out, p.heads, p.kv_heads, p.pos,
                   p.tokens, p.scale, nblocks};
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(attention_prefill_kernel),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-        attr_set = true;
-    }
     const dim3 grid((p.tokens + TQ - 1) / TQ, p.kv_heads);
     attention_prefill_kernel<<<grid, THREADS, LDS_BYTES, stream>>>(a);
     return launch_status(what);
 }
 
 }  // namespace
+
+int setup_prefill() {
+    if (int rc = load_kernel(reinterpret_cast<const void *>(attention_prefill_kernel))) return rc;
+    return int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_prefill_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
+}
 }  // namespace saetta
 
 using namespace saetta;

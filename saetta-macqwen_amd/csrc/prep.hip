@@ -104,6 +104,8 @@ __global__ __launch_bounds__(256) void attention_prep_store_kernel(PrepArgs a) {
 }
 
 }  // namespace
+
+int setup_prep() { return load_kernel(reinterpret_cast<const void *>(attention_prep_store_kernel<8>)); }
 }  // namespace saetta
 
 using namespace saetta;

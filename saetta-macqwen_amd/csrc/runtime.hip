@@ -38,6 +38,16 @@ int ensure_device() {
             status = SAETTA_E_DEVICE;
             snprintf(why, sizeof why, "device is %s; this library is built for gfx950 only",
                      prop.gcnArchName);
+            return;
+        }
+        int (*const setups[])() = {setup_kv_quant, setup_prep, setup_deltanet, setup_decode, setup_prefill};
+        for (auto setup : setups) {
+            if (int rc = setup()) {
+                status = SAETTA_E_DEVICE;
+                snprintf(why, sizeof why, "kernels do not load: %s", hipGetErrorString(hipError_t(rc)));
+                (void)hipGetLastError();
+                return;
+            }
         }
     });
     if (status != SAETTA_OK) return fail(status, "%s", why);

@@ -106,8 +106,9 @@ class Built:
         self.ops = ops
         self.graph = None
         if graph and ops:
-            # One eager run first: lazy one-time set-up must not happen under capture.
-            self.run()
+            # The library's one-time set-up (code objects, LDS limits) must not happen under capture;
+            # the launches themselves are not run here: a plan may hold ops that advance a state.
+            ffi.check(ffi.lib().saetta_init(), "init")
             torch.cuda.synchronize()
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
@@ -347,6 +348,49 @@ def deltanet_step(plan, q, k, v, a, b, a_log, dt_bias, state, z, norm_w, y, k_he
     p = ffi.StepParamsC(k_heads, v_heads, v_dim, eps)
     plan.op("deltanet_step", lambda s: ffi.check(
         ffi.lib().saetta_deltanet_step(s, *[_ptr(t) for t in ts], p), "deltanet_step"))
+
+
+def deltanet_conv_rows(plan, x, w, state, out, channels, kernel_size, tokens, snaps=None):
+    """Records the conv of `tokens` tokens in order (conv_rows2 + conv_state, kernels/prefill.metal:734-786;
+    deltanet_conv_rows, kernels/layers.metal:510-544): x, out [tokens][channels]; with `snaps`
+    ([tokens][kernel_size - 1][channels]) the state after each token goes there too."""
+    for t, what in ((x, "x"), (w, "w"), (state, "state"), (out, "out")):
+        _need(t, torch.float32, what)
+    if snaps is not None:
+        _need(snaps, torch.float32, "snaps")
+        if snaps.numel() < tokens * (kernel_size - 1) * channels:
+            raise ValueError("deltanet_conv_rows: snapshots too small")
+    if (x.numel() < tokens * channels or out.numel() < tokens * channels or w.numel() < channels * kernel_size
+            or state.numel() < (kernel_size - 1) * channels):
+        raise ValueError("deltanet_conv_rows: buffers too small")
+    p = ffi.ConvRowsParamsC(channels, kernel_size, tokens, int(snaps is not None))
+    plan.op("deltanet_conv_rows", lambda s: ffi.check(
+        ffi.lib().saetta_deltanet_conv_rows(s, _ptr(x), _ptr(w), _ptr(state), _ptr(out),
+                                            _ptr(snaps) if snaps is not None else None, p), "deltanet_conv_rows"))
+
+
+def deltanet_rows(plan, mixed, a, b, a_log, dt_bias, state, z, norm_w, y, k_heads, v_heads, v_dim, tokens, eps,
+                  snaps=None):
+    """Records the step of `tokens` tokens in order (delta_prep + delta_rows3 + gated norm,
+    kernels/prefill.metal:788-1116, src/prefill.rs:1487-1578; deltanet_step_rows,
+    GpuDeltaNet::record_rows, src/gpu_layers.rs:686-786): `mixed` [tokens][q | k | v] is the conv
+    output; with `snaps` ([tokens][v_heads][v_dim][128]) the state after each token goes there too."""
+    ts = (mixed, a, b, a_log, dt_bias, state, z, norm_w, y)
+    for t in ts:
+        _need(t, torch.float32, "deltanet_rows buffer")
+    channels = 2 * k_heads * 128 + v_heads * v_dim
+    if (mixed.numel() < tokens * channels or state.numel() < v_heads * v_dim * 128
+            or y.numel() < tokens * v_heads * v_dim or z.numel() < tokens * v_heads * v_dim
+            or a.numel() < tokens * v_heads or b.numel() < tokens * v_heads):
+        raise ValueError("deltanet_rows: buffers too small")
+    if snaps is not None:
+        _need(snaps, torch.float32, "snaps")
+        if snaps.numel() < tokens * v_heads * v_dim * 128:
+            raise ValueError("deltanet_rows: snapshots too small")
+    p = ffi.RowsStepParamsC(k_heads, v_heads, v_dim, tokens, eps, int(snaps is not None))
+    plan.op("deltanet_rows", lambda s: ffi.check(
+        ffi.lib().saetta_deltanet_rows(s, *[_ptr(t) for t in ts], _ptr(snaps) if snaps is not None else None, p),
+        "deltanet_rows"))
 
 
 def _median_ms(run, runs):

@@ -122,7 +122,9 @@ class Built {
     // one exception: prefill without a caller's workspace allocates.
     Built(Ops ops, const gpu::Gpu &gpu, bool graph) : ops_(std::move(ops)) {
         if (!graph || ops_.empty()) return;
-        for (auto &op : ops_) op.second(gpu.stream());  // once outside the capture: first-call set-up
+        // The library's one-time set-up must not happen under capture; the launches themselves are not
+        // run here: a plan may hold ops that advance a state (the DeltaNet ones do).
+        if (int rc = saetta_init()) throw std::runtime_error(std::string("saetta_init: ") + saetta_last_error() + " (" + std::to_string(rc) + ")");
         gpu.sync();
         hipGraph_t g = nullptr;
         hip_check(hipStreamBeginCapture(gpu.stream(), hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
@@ -357,6 +359,51 @@ inline void step(plan::Plan &plan, const View &q, const View &k, const View &v, 
                                    a_log.ptr<float>(), dt_bias.ptr<float>(), state.ptr<float>(), z.ptr<float>(),
                                    norm_w.ptr<float>(), y.ptr<float>(), p),
               "deltanet_step");
+    });
+}
+
+// Records the conv of `tokens` tokens in order (conv_rows2 + conv_state, kernels/prefill.metal:734-786;
+// deltanet_conv_rows, kernels/layers.metal:510-544).  x, out [tokens][channels]; with `snaps`
+// ([tokens][kernel_size - 1][channels]) the state after each token goes there too.
+inline void conv_rows(plan::Plan &plan, const View &x, const View &w, const View &state, const View &out, size_t channels,
+                      size_t kernel_size, size_t tokens, const View *snaps = nullptr) {
+    const saetta_conv_rows_params p{uint32_t(channels), uint32_t(kernel_size), uint32_t(tokens), snaps ? 1u : 0u};
+    const View sn = snaps ? *snaps : View{};
+    const bool has = snaps != nullptr;
+    plan.op("deltanet_conv_rows", [=](hipStream_t s) {
+        check(saetta_deltanet_conv_rows(s, x.ptr<float>(), w.ptr<float>(), state.ptr<float>(), out.ptr<float>(),
+                                        has ? sn.ptr<float>() : nullptr, p),
+              "deltanet_conv_rows");
+    });
+}
+
+// Records the step of `tokens` tokens in order (delta_prep + delta_rows3 + the gated norm,
+// kernels/prefill.metal:788-1116; deltanet_step_rows, GpuDeltaNet::record_rows, src/gpu_layers.rs:686-786).
+// `mixed` [tokens][q | k | v] is the conv output; with `snaps` ([tokens][v_heads][v_dim][128]) the
+// state after each token goes there too (GpuDeltaNetSnaps, src/gpu_layers.rs:819-836).
+inline void rows(plan::Plan &plan, const View &mixed, const View &a, const View &b, const View &a_log, const View &dt_bias,
+                 const View &state, const View &z, const View &norm_w, const View &y, size_t k_heads, size_t v_heads,
+                 size_t v_dim, size_t tokens, float eps, const View *snaps = nullptr) {
+    const saetta_rows_step_params p{uint32_t(k_heads), uint32_t(v_heads), uint32_t(v_dim), uint32_t(tokens), eps, snaps ? 1u : 0u};
+    const View sn = snaps ? *snaps : View{};
+    const bool has = snaps != nullptr;
+    plan.op("deltanet_rows", [=](hipStream_t s) {
+        check(saetta_deltanet_rows(s, mixed.ptr<float>(), a.ptr<float>(), b.ptr<float>(), a_log.ptr<float>(),
+                                   dt_bias.ptr<float>(), state.ptr<float>(), z.ptr<float>(), norm_w.ptr<float>(),
+                                   y.ptr<float>(), has ? sn.ptr<float>() : nullptr, p),
+              "deltanet_rows");
+    });
+}
+
+// GpuDeltaNetSnaps::record_restore (src/gpu_layers.rs:838-856): the state after row `row` of the
+// last rows call becomes the state; two device copies in stream order.
+inline void restore(plan::Plan &plan, const View &conv_snaps, const View &state_snaps, size_t row, const View &conv,
+                    const View &state, size_t conv_floats, size_t state_floats) {
+    plan.op("copy_u32", [=](hipStream_t s) {
+        hip_check(hipMemcpyAsync(conv.ptr<float>(), conv_snaps.ptr<float>() + row * conv_floats, conv_floats * 4,
+                                 hipMemcpyDeviceToDevice, s), "restore conv");
+        hip_check(hipMemcpyAsync(state.ptr<float>(), state_snaps.ptr<float>() + row * state_floats, state_floats * 4,
+                                 hipMemcpyDeviceToDevice, s), "restore state");
     });
 }
 

@@ -193,6 +193,53 @@ int main() {
         compare(kc, gpu::contents<float>(kb.buffer, KV * DIM), pos, KvBits::Eight);
         compare(vc, v, pos, KvBits::Eight);
     }
+    {   // GpuDeltaNet::record_rows "as m calls of record would" (src/gpu_layers.rs:686-688), the snapshots
+        // and record_restore (src/gpu_layers.rs:838-856; the reference's test at :1063-1095 restores a row
+        // and goes on from there)
+        const size_t kh = 2, vh = 4, dv = 16, kernel = 4, m = 5, key = kh * 128, val = vh * dv, ch = 2 * key + val;
+        const size_t conv_n = (kernel - 1) * ch, state_n = vh * dv * 128;
+        std::vector<float> x(m * ch), z(m * val), a(m * vh), b(m * vh), w(ch * kernel), alog(vh), dtb(vh), norm(dv, 1.0f);
+        orc_noise(x.data(), x.size(), 31), orc_noise(z.data(), z.size(), 32), orc_noise(a.data(), a.size(), 33);
+        orc_noise(b.data(), b.size(), 34), orc_noise(w.data(), w.size(), 35), orc_noise(alog.data(), vh, 36);
+        orc_noise(dtb.data(), vh, 37);
+        View xd(gpu.buffer_from(x)), zd(gpu.buffer_from(z)), ad(gpu.buffer_from(a)), bd(gpu.buffer_from(b));
+        View wd(gpu.buffer_from(w)), al(gpu.buffer_from(alog)), dt(gpu.buffer_from(dtb)), nw(gpu.buffer_from(norm));
+        View conv1(gpu.buffer(conv_n * 4)), st1(gpu.buffer(state_n * 4)), mixed1(gpu.buffer(m * ch * 4)), y1(gpu.buffer(m * val * 4));
+        View conv2(gpu.buffer(conv_n * 4)), st2(gpu.buffer(state_n * 4)), mixed2(gpu.buffer(m * ch * 4)), y2(gpu.buffer(m * val * 4));
+        View csn(gpu.buffer(m * conv_n * 4)), ssn(gpu.buffer(m * state_n * 4));
+        plan::Plan one(gpu), many(gpu);
+        for (size_t t = 0; t < m; t++) {
+            const View mt = mixed1.at(t * ch * 4);
+            deltanet::conv(one, xd.at(t * ch * 4), wd, conv1, mt, ch, kernel);
+            deltanet::step(one, mt, mt.at(key * 4), mt.at(2 * key * 4), ad.at(t * vh * 4), bd.at(t * vh * 4), al, dt, st1,
+                           zd.at(t * val * 4), nw, y1.at(t * val * 4), kh, vh, dv, 1e-6f);
+        }
+        deltanet::conv_rows(many, xd, wd, conv2, mixed2, ch, kernel, m, &csn);
+        deltanet::rows(many, mixed2, ad, bd, al, dt, st2, zd, nw, y2, kh, vh, dv, m, 1e-6f, &ssn);
+        one.build(false).run(gpu);
+        many.build(true).run(gpu);
+        auto worst = [](const std::vector<float> &p, const std::vector<float> &q) {
+            float d = 0;
+            for (size_t i = 0; i < p.size(); i++) d = std::max(d, std::fabs(p[i] - q[i]));
+            return d;
+        };
+        EXPECT(gpu::contents<float>(mixed1.buffer, m * ch) == gpu::contents<float>(mixed2.buffer, m * ch), "conv_rows != m convs");
+        EXPECT(gpu::contents<float>(conv1.buffer, conv_n) == gpu::contents<float>(conv2.buffer, conv_n), "conv state");
+        EXPECT(worst(gpu::contents<float>(y1.buffer, m * val), gpu::contents<float>(y2.buffer, m * val)) < 2e-5f, "rows y");
+        EXPECT(worst(gpu::contents<float>(st1.buffer, state_n), gpu::contents<float>(st2.buffer, state_n)) < 2e-5f, "rows state");
+        EXPECT(gpu::contents<float>(ssn.buffer, state_n, (m - 1) * state_n * 4) == gpu::contents<float>(st2.buffer, state_n),
+               "last snapshot is the state");
+        // accept two rows: restore the state after row 1, then rows 2.. again give the same end state
+        plan::Plan again(gpu);
+        deltanet::restore(again, csn, ssn, 1, conv2, st2, conv_n, state_n);
+        deltanet::conv_rows(again, xd.at(2 * ch * 4), wd, conv2, mixed2, ch, kernel, m - 2);
+        deltanet::rows(again, mixed2, ad.at(2 * vh * 4), bd.at(2 * vh * 4), al, dt, st2, zd.at(2 * val * 4), nw, y2, kh, vh, dv,
+                       m - 2, 1e-6f);
+        again.build(false).run(gpu);
+        EXPECT(gpu::contents<float>(ssn.buffer, state_n, (m - 1) * state_n * 4) == gpu::contents<float>(st2.buffer, state_n),
+               "restore + the remaining rows");
+        EXPECT(gpu::contents<float>(conv1.buffer, conv_n) == gpu::contents<float>(conv2.buffer, conv_n), "restore conv");
+    }
     // shape checks panic (throw) as the reference asserts
     bool threw = false;
     try {

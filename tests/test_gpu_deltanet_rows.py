@@ -1,0 +1,190 @@
+"""Gated DeltaNet over several tokens in one launch (verify rows, prefill chunks) against the oracle.
+
+The oracle runs the tokens one at a time (conv, then step), which is how the reference defines the
+result (`record_rows`: "as m calls of record would", src/gpu_layers.rs:686-688; the chunked prefill
+of src/prefill.rs:1433-1578 against the CPU layer).  Beyond that, properties the oracle is too slow
+for: a 4096-token chunk equals the same tokens in uneven pieces bit for bit, snapshot t equals the
+state a t + 1-token call leaves, and the first rows equal the single-token kernels'.
+Tolerances as for the single-token kernels: 2e-6 on the conv, 2e-5 (relative to the largest value)
+on y and the state; the sums run over 16 lanes of 8 values instead of the CPU's one after the other.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_common import dev, host, oracle, saetta
+
+pytestmark = pytest.mark.gpu
+K_DIM = 128
+EPS = 1e-6
+
+
+class Layer:
+    def __init__(self, k_heads, v_heads, v_dim, kernel, seed):
+        rng = np.random.default_rng(seed)
+        self.k_heads, self.v_heads, self.v_dim, self.kernel = k_heads, v_heads, v_dim, kernel
+        self.key, self.val = k_heads * K_DIM, v_heads * v_dim
+        self.channels = 2 * self.key + self.val
+        self.conv_w = (0.5 * rng.standard_normal((self.channels, kernel))).astype(np.float32)
+        self.a_log = rng.uniform(-1, 1, v_heads).astype(np.float32)
+        self.dt_bias = rng.standard_normal(v_heads).astype(np.float32)
+        self.norm = (1 + 0.1 * rng.standard_normal(v_dim)).astype(np.float32)
+        self.rng = rng
+
+    def inputs(self, tokens):
+        r = self.rng
+        return (r.standard_normal((tokens, self.channels)).astype(np.float32),
+                r.standard_normal((tokens, self.val)).astype(np.float32),
+                r.standard_normal((tokens, self.v_heads)).astype(np.float32),
+                r.standard_normal((tokens, self.v_heads)).astype(np.float32))
+
+    def zero_state(self):
+        return (torch.zeros(self.kernel - 1, self.channels, device="cuda"),
+                torch.zeros(self.v_heads * self.v_dim * K_DIM, device="cuda"))
+
+    def gpu_rows(self, x, z, a, b, conv, state, snapshots=False):
+        """One call over all the tokens of x; returns mixed, y and the snapshots (or None)."""
+        tokens = x.shape[0]
+        xd, zd, ad, bd = (dev(np.ascontiguousarray(t)) for t in (x, z, a, b))
+        mixed = torch.empty(tokens, self.channels, device="cuda")
+        y = torch.empty(tokens, self.val, device="cuda")
+        snaps = None
+        if snapshots:
+            snaps = (torch.full((tokens, self.kernel - 1, self.channels), 7.0, device="cuda"),
+                     torch.full((tokens, self.v_heads * self.v_dim * K_DIM), 7.0, device="cuda"))
+        plan = saetta.Plan()
+        saetta.deltanet_conv_rows(plan, xd, dev(self.conv_w), conv, mixed, self.channels, self.kernel, tokens,
+                                  snaps[0] if snapshots else None)
+        saetta.deltanet_rows(plan, mixed, ad, bd, dev(self.a_log), dev(self.dt_bias), state, zd, dev(self.norm), y,
+                             self.k_heads, self.v_heads, self.v_dim, tokens, EPS, snaps[1] if snapshots else None)
+        assert [n for n, _ in plan.ops] == ["deltanet_conv_rows", "deltanet_rows"]
+        plan.build().run()
+        torch.cuda.synchronize()
+        return mixed, y, snaps
+
+    def cpu_rows(self, x, z, a, b, conv, state):
+        """Token by token through the oracle; conv and state (numpy) are updated in place."""
+        mixed, y, conv_after, state_after = [], [], [], []
+        for t in range(x.shape[0]):
+            m = oracle.deltanet_conv(self.conv_w, x[t], conv, self.kernel)
+            y.append(oracle.deltanet_step(m[:self.key], m[self.key:2 * self.key], m[2 * self.key:], a[t], b[t],
+                                          self.a_log, self.dt_bias, state, z[t], self.norm, self.k_heads,
+                                          self.v_heads, K_DIM, self.v_dim, EPS))
+            mixed.append(m)
+            conv_after.append(conv.copy())
+            state_after.append(state.copy())
+        return np.stack(mixed), np.stack(y), np.stack(conv_after), np.stack(state_after)
+
+
+def close(got, want, rel):
+    return np.abs(got - want).max() <= rel * max(1.0, np.abs(want).max())
+
+
+def check_against_oracle(layer, tokens, pieces, snapshots):
+    x, z, a, b = layer.inputs(tokens)
+    conv_cpu = np.zeros((layer.kernel - 1, layer.channels), np.float32)
+    state_cpu = np.zeros(layer.v_heads * layer.v_dim * K_DIM, np.float32)
+    want_mixed, want_y, want_conv, want_state = layer.cpu_rows(x, z, a, b, conv_cpu, state_cpu)
+    conv, state = layer.zero_state()
+    at = 0
+    for n in pieces:
+        s = slice(at, at + n)
+        mixed, y, snaps = layer.gpu_rows(x[s], z[s], a[s], b[s], conv, state, snapshots)
+        assert close(host(mixed), want_mixed[s], 2e-6), (at, n)
+        assert close(host(y), want_y[s], 2e-5), (at, n)
+        if n:
+            assert np.array_equal(host(conv), want_conv[at + n - 1]), (at, n)
+            assert close(host(state), want_state[at + n - 1], 2e-5), (at, n)
+        if snapshots and n:
+            assert np.array_equal(host(snaps[0]), want_conv[s])
+            assert close(host(snaps[1]), want_state[s], 2e-5)
+            # the last snapshot is the state itself
+            assert np.array_equal(host(snaps[1][n - 1]), host(state))
+        at += n
+    assert at == tokens
+
+
+def test_real_shape_verify_rows_with_snapshots():
+    # configs[4]: 16 key / 32 value heads of 128, conv kernel 4; 1..4 rows as the verify step has
+    layer = Layer(16, 32, 128, 4, seed=11)
+    check_against_oracle(layer, 10, [1, 2, 3, 4], snapshots=True)
+
+
+def test_real_shape_chunk_crosses_token_blocks():
+    # 37 tokens: two full staged blocks of 16 and a ragged one
+    layer = Layer(16, 32, 128, 4, seed=12)
+    check_against_oracle(layer, 37, [37], snapshots=False)
+
+
+@pytest.mark.parametrize("v_dim,kernel,tokens", [(4, 2, 5), (24, 4, 17), (100, 7, 33), (256, 4, 16), (16, 16, 3)])
+def test_other_shapes(v_dim, kernel, tokens):
+    layer = Layer(2, 4, v_dim, kernel, seed=v_dim + kernel)
+    check_against_oracle(layer, tokens, [tokens // 2, tokens - tokens // 2], snapshots=(v_dim <= 100))
+
+
+def test_fewer_tokens_than_conv_taps_keep_the_older_state_rows():
+    layer = Layer(1, 2, 8, 6, seed=3)
+    check_against_oracle(layer, 7, [1, 2, 1, 3], snapshots=True)
+
+
+def test_first_row_equals_the_single_token_kernels():
+    layer = Layer(16, 32, 128, 4, seed=21)
+    x, z, a, b = layer.inputs(1)
+    conv, state = layer.zero_state()
+    state.copy_(torch.randn_like(state) * 0.1)
+    conv.copy_(torch.randn_like(conv))
+    conv1, state1 = conv.clone(), state.clone()
+    mixed, y, _ = layer.gpu_rows(x, z, a, b, conv, state)
+    mixed1, y1 = torch.empty(layer.channels, device="cuda"), torch.empty(layer.val, device="cuda")
+    key = layer.key
+    plan = saetta.Plan()
+    saetta.deltanet_conv(plan, dev(x[0]), dev(layer.conv_w), conv1, mixed1, layer.channels, layer.kernel)
+    saetta.deltanet_step(plan, mixed1[:key], mixed1[key:2 * key], mixed1[2 * key:], dev(a[0]), dev(b[0]),
+                         dev(layer.a_log), dev(layer.dt_bias), state1, dev(z[0]), dev(layer.norm), y1,
+                         layer.k_heads, layer.v_heads, layer.v_dim, EPS)
+    plan.build().run()
+    assert torch.equal(mixed[0], mixed1) and torch.equal(conv, conv1)
+    # the two step kernels add a row's 128 products in different orders
+    assert close(host(y[0]), host(y1), 2e-5) and close(host(state), host(state1), 2e-5)
+
+
+def test_full_chunk_equals_uneven_pieces_bit_for_bit():
+    # 4096 tokens at the real shape: what a prefill chunk is.  The arithmetic of a token does not
+    # depend on where the launch or the staged block starts, so any split gives the same bits.
+    layer = Layer(16, 32, 128, 4, seed=31)
+    tokens = 4096
+    x, z, a, b = layer.inputs(tokens)
+    conv, state = layer.zero_state()
+    _, y, _ = layer.gpu_rows(x, z, a, b, conv, state)
+    conv2, state2 = layer.zero_state()
+    ys, at = [], 0
+    for n in (1, 15, 16, 17, 1000, 3047):
+        s = slice(at, at + n)
+        ys.append(layer.gpu_rows(x[s], z[s], a[s], b[s], conv2, state2)[1])
+        at += n
+    assert at == tokens
+    assert torch.equal(torch.cat(ys), y)
+    assert torch.equal(conv, conv2) and torch.equal(state, state2)
+    assert torch.isfinite(y).all() and float(y.abs().max()) > 0.1
+    # decay keeps the state bounded: |g| < 1 and beta in (0, 1) with unit keys
+    assert float(state.abs().max()) < 1e3
+
+
+def test_rejections():
+    z = torch.zeros(4096, device="cuda")
+    plan = saetta.Plan()
+    saetta.deltanet_rows(plan, z, z, z, z, z, torch.zeros(3 * 8 * 128, device="cuda"), z, z, z, 2, 3, 8, 1, EPS)
+    with pytest.raises(saetta.ffi.SaettaError, match="value heads"):
+        plan.build().run()
+    plan = saetta.Plan()
+    saetta.deltanet_rows(plan, z, z, z, z, z, torch.zeros(2 * 6 * 128, device="cuda"), z, z, z, 1, 2, 6, 1, EPS)
+    with pytest.raises(saetta.ffi.SaettaError, match="multiple of 4"):
+        plan.build().run()
+    with pytest.raises(ValueError):
+        saetta.deltanet_rows(saetta.Plan(), z, z, z, z, z, torch.zeros(10, device="cuda"), z, z, z, 2, 4, 8, 1, EPS)
+    with pytest.raises(ValueError):
+        saetta.deltanet_conv_rows(saetta.Plan(), z, z, z, z, 1024, 4, 8)
+    plan = saetta.Plan()
+    saetta.deltanet_conv_rows(plan, z, z, z, z, 16, 1, 2)
+    with pytest.raises(saetta.ffi.SaettaError, match="kernel size"):
+        plan.build().run()
