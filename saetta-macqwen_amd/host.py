@@ -393,6 +393,94 @@ def deltanet_rows(plan, mixed, a, b, a_log, dt_bias, state, z, norm_w, y, k_head
         "deltanet_rows"))
 
 
+KV_ALIGN = 128  # src/gpu_layers.rs:199: the decode chunk, and a multiple of the prefill key block
+
+
+class GpuKvCache:
+    """GpuKvCache (src/gpu_layers.rs:183-293): the keys and values of one attention layer on the
+    GPU, token p in row p, half values or codes with their scales and biases, plus the decode
+    attention sized for the capacity.  `resize` moves to new buffers and copies every old row that
+    fits; plans recorded with the old buffers must be recorded again, as in the reference."""
+
+    def __init__(self, heads, kv_heads, head_dim, capacity, bits=KvBits.Half, device="cuda"):
+        self.heads, self.kv_heads, self.head_dim, self.bits, self.device = heads, kv_heads, head_dim, bits, device
+        self.capacity = -(-capacity // KV_ALIGN) * KV_ALIGN
+        values = kv_heads * head_dim
+        self.decode = DecodeAttention(heads, kv_heads, head_dim, self.capacity, device)
+        if bits is KvBits.Half:
+            self.quant = None
+            self.keys = torch.zeros(self.capacity * values, dtype=torch.float16, device=device)
+            self.values = torch.zeros(self.capacity * values, dtype=torch.float16, device=device)
+        else:
+            k, v = QuantRows(bits, values, self.capacity, device), QuantRows(bits, values, self.capacity, device)
+            self.quant, self.keys, self.values = (k, v), k.data, v.data
+
+    @classmethod
+    def with_bits(cls, heads, kv_heads, head_dim, capacity, bits, device="cuda"):
+        return cls(heads, kv_heads, head_dim, capacity, bits, device)
+
+    def buffers(self):
+        """Every buffer of the cache; each holds `capacity` rows of equal size (src/gpu_layers.rs:247-253)."""
+        out = [self.keys, self.values]
+        if self.quant:
+            k, v = self.quant
+            out += [k.scales, k.biases, v.scales, v.biases]
+        return out
+
+    def resize(self, capacity):
+        capacity = -(-capacity // KV_ALIGN) * KV_ALIGN
+        old, rows = self.capacity, min(self.capacity, capacity)
+        moved = []
+        for b in self.buffers():
+            per_row = b.numel() // old
+            new = torch.zeros(per_row * capacity, dtype=b.dtype, device=b.device)
+            new[:per_row * rows].copy_(b[:per_row * rows])
+            moved.append(new)
+        torch.cuda.current_stream().synchronize()  # the reference waits for the blit as well
+        self.keys, self.values = moved[0], moved[1]
+        if self.quant:
+            k, v = self.quant
+            k.data, v.data = self.keys, self.values
+            k.scales, k.biases, v.scales, v.biases = moved[2:6]
+            k.capacity = v.capacity = capacity
+        self.decode = DecodeAttention(self.heads, self.kv_heads, self.head_dim, capacity, self.device)
+        self.capacity = capacity
+
+
+class RowBackup:
+    """RowBackup (src/gpu_cache.rs:196-283): a copy of KV rows from..from + n of every attention
+    layer, for a short detour that writes over a long conversation; `restore` puts them back."""
+
+    def __init__(self):
+        self.copy = None
+
+    def bytes(self):
+        return sum(p.numel() * p.element_size() for p in self.copy[0]) if self.copy else 0
+
+    @staticmethod
+    def _parts(caches):
+        return [(b, b.numel() // c.capacity) for c in caches for b in c.buffers()]
+
+    def save(self, caches, start, n):
+        self.copy = None
+        if n == 0 or not caches:
+            return
+        if any(start + n > c.capacity for c in caches):
+            raise ValueError("RowBackup.save: rows past the capacity")
+        self.copy = ([b[start * row:(start + n) * row].clone() for b, row in self._parts(caches)], start, n)
+
+    def restore(self, caches):
+        if not self.copy:
+            return
+        parts, start, n = self.copy
+        self.copy = None
+        for (b, row), saved in zip(self._parts(caches), parts):
+            b[start * row:(start + n) * row].copy_(saved)
+
+    def clear(self):
+        self.copy = None
+
+
 def _median_ms(run, runs):
     """One warm-up, then the median of `runs` event-timed calls, in milliseconds."""
     ts = []

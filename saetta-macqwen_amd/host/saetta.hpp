@@ -19,6 +19,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -585,5 +586,111 @@ inline void encode_quant(const gpu::Gpu &gpu, const View &q, const kv_quant::Qua
 }
 
 }  // namespace attention_prefill
+
+namespace gpu_layers {
+
+constexpr size_t KV_ALIGN = 128;  // src/gpu_layers.rs:199
+
+// GpuKvCache (src/gpu_layers.rs:183-293): keys and values of one attention layer, token p in row p,
+// half values or codes with their scales and biases, and the decode attention sized for the capacity.
+class GpuKvCache {
+  public:
+    gpu::Buffer keys, values;
+    std::unique_ptr<std::pair<kv_quant::QuantRows, kv_quant::QuantRows>> quant;  // Option<(QuantRows, QuantRows)>
+    kv_quant::KvBits bits;
+    size_t capacity;
+    std::unique_ptr<attention::DecodeAttention> decode;
+
+    GpuKvCache(const gpu::Gpu &gpu, size_t heads, size_t kv_heads, size_t head_dim, size_t capacity_,
+               kv_quant::KvBits bits_ = kv_quant::KvBits::Half)
+        : bits(bits_), capacity((capacity_ + KV_ALIGN - 1) / KV_ALIGN * KV_ALIGN), heads_(heads), kv_heads_(kv_heads), head_dim_(head_dim) {
+        const size_t row = kv_heads * head_dim;
+        decode = std::make_unique<attention::DecodeAttention>(gpu, heads, kv_heads, head_dim, capacity);
+        if (bits == kv_quant::KvBits::Half) {
+            keys = gpu.buffer(capacity * row * 2);
+            values = gpu.buffer(capacity * row * 2);
+        } else {
+            quant = std::make_unique<std::pair<kv_quant::QuantRows, kv_quant::QuantRows>>(
+                kv_quant::QuantRows(gpu, bits, row, capacity), kv_quant::QuantRows(gpu, bits, row, capacity));
+            keys = quant->first.data;
+            values = quant->second.data;
+        }
+    }
+    // Every buffer of the cache; each holds `capacity` rows of equal size.
+    std::vector<gpu::Buffer *> buffers() {
+        std::vector<gpu::Buffer *> out{&keys, &values};
+        if (quant) {
+            for (gpu::Buffer *b : {&quant->first.scales, &quant->first.biases, &quant->second.scales, &quant->second.biases}) out.push_back(b);
+        }
+        return out;
+    }
+    // New buffers with room for `capacity_` tokens; every old row that fits is copied over.  Plans
+    // recorded with the old buffers must be recorded again.
+    void resize(const gpu::Gpu &gpu, size_t capacity_) {
+        const size_t cap = (capacity_ + KV_ALIGN - 1) / KV_ALIGN * KV_ALIGN, rows = std::min(capacity, cap);
+        for (gpu::Buffer *b : buffers()) {
+            const size_t row = b->length() / capacity;
+            gpu::Buffer moved = gpu.buffer(row * cap);
+            hip_check(hipMemcpyAsync(moved.get(), b->get(), row * rows, hipMemcpyDeviceToDevice, gpu.stream()), "resize");
+            gpu.sync();  // the old buffer goes when its last handle does
+            *b = moved;
+        }
+        if (quant) {
+            quant->first.data = keys;
+            quant->second.data = values;
+        }
+        decode = std::make_unique<attention::DecodeAttention>(gpu, heads_, kv_heads_, head_dim_, cap);
+        capacity = cap;
+    }
+
+  private:
+    size_t heads_, kv_heads_, head_dim_;
+};
+
+// RowBackup (src/gpu_cache.rs:196-283): a copy of KV rows from..from + n of every attention layer;
+// `restore` puts them back where they came from and frees the copy.
+class RowBackup {
+  public:
+    size_t bytes() const {
+        size_t total = 0;
+        for (auto &b : parts_) total += b.length();
+        return total;
+    }
+    void save(const gpu::Gpu &gpu, const std::vector<GpuKvCache *> &caches, size_t from, size_t n) {
+        clear();
+        if (n == 0) return;
+        for (GpuKvCache *c : caches) {
+            if (from + n > c->capacity) throw std::runtime_error("RowBackup::save: rows past the capacity");
+            for (gpu::Buffer *b : c->buffers()) {
+                const size_t row = b->length() / c->capacity;
+                gpu::Buffer copy = gpu.buffer(n * row);
+                hip_check(hipMemcpyAsync(copy.get(), static_cast<char *>(b->get()) + from * row, n * row, hipMemcpyDeviceToDevice,
+                                         gpu.stream()), "RowBackup::save");
+                parts_.push_back(copy);
+            }
+        }
+        from_ = from, n_ = n;
+    }
+    void restore(const gpu::Gpu &gpu, const std::vector<GpuKvCache *> &caches) {
+        if (parts_.empty()) return;
+        size_t i = 0;
+        for (GpuKvCache *c : caches) {
+            for (gpu::Buffer *b : c->buffers()) {
+                const size_t row = b->length() / c->capacity;
+                hip_check(hipMemcpyAsync(static_cast<char *>(b->get()) + from_ * row, parts_.at(i++).get(), n_ * row,
+                                         hipMemcpyDeviceToDevice, gpu.stream()), "RowBackup::restore");
+            }
+        }
+        gpu.sync();  // the copies are freed below
+        clear();
+    }
+    void clear() { parts_.clear(); }
+
+  private:
+    std::vector<gpu::Buffer> parts_;
+    size_t from_ = 0, n_ = 0;
+};
+
+}  // namespace gpu_layers
 
 }  // namespace saetta

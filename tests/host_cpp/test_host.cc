@@ -240,6 +240,40 @@ int main() {
                "restore + the remaining rows");
         EXPECT(gpu::contents<float>(conv1.buffer, conv_n) == gpu::contents<float>(conv2.buffer, conv_n), "restore conv");
     }
+    {   // GpuKvCache::resize keeps the rows (src/gpu_layers.rs:255-293); RowBackup puts rows back (src/gpu_cache.rs:196-283)
+        gpu_layers::GpuKvCache cache(gpu, HEADS, KV, DIM, 200, KvBits::Eight);
+        EXPECT(cache.capacity == 256 && cache.buffers().size() == 6, "GpuKvCache::with_bits");
+        std::vector<float> x(150 * VALUES);
+        orc_quant_rows(x.data(), 150, VALUES);
+        const View xd(gpu.buffer_from(x));
+        cache.quant->first.encode(gpu, xd, 0, 150);
+        cache.quant->second.encode(gpu, xd, 0, 150);
+        gpu.sync();
+        const auto codes = gpu::contents<uint32_t>(cache.keys, 150 * 8 * 16);
+        const auto scales = gpu::contents<uint16_t>(cache.quant->second.scales, 150 * 8);
+        cache.resize(gpu, 1000);
+        EXPECT(cache.capacity == 1024 && cache.keys.length() == 1024 * 8 * 16 * 4, "resize capacity");
+        EXPECT(gpu::contents<uint32_t>(cache.keys, 150 * 8 * 16) == codes, "resize moved the codes");
+        EXPECT(gpu::contents<uint16_t>(cache.quant->second.scales, 150 * 8) == scales, "resize moved the scales");
+        EXPECT(cache.quant->first.data.get() == cache.keys.get(), "QuantRows follows the cache");
+        compare(cache.quant->first, x, 0, KvBits::Eight);
+        gpu_layers::RowBackup backup;
+        backup.save(gpu, {&cache}, 100, 12);
+        EXPECT(backup.bytes() == 12 * 1088, "RowBackup::bytes %zu", backup.bytes());
+        std::vector<float> other(12 * VALUES, 0.25f);
+        const View od(gpu.buffer_from(other));
+        cache.quant->first.encode(gpu, od, 100, 12);
+        cache.quant->second.encode(gpu, od, 100, 12);
+        gpu.sync();
+        EXPECT(gpu::contents<uint32_t>(cache.keys, 150 * 8 * 16) != codes, "the detour wrote over the rows");
+        backup.restore(gpu, {&cache});
+        EXPECT(backup.bytes() == 0 && gpu::contents<uint32_t>(cache.keys, 150 * 8 * 16) == codes, "RowBackup::restore");
+        EXPECT(gpu::contents<uint16_t>(cache.quant->second.scales, 150 * 8) == scales, "RowBackup::restore scales");
+        cache.resize(gpu, 100);
+        EXPECT(cache.capacity == 128, "shrink");
+        std::vector<float> first(x.begin(), x.begin() + 128 * VALUES);
+        compare(cache.quant->first, first, 0, KvBits::Eight);
+    }
     // shape checks panic (throw) as the reference asserts
     bool threw = false;
     try {
