@@ -125,7 +125,8 @@ __global__ __launch_bounds__(STEP_THREADS) void deltanet_step_kernel(StepArgs a)
 
 // One thread per (channel, tile of CONV_TILE tokens).  Input i of the window of token t is
 // x[i] for i >= 0 and the stored state row i + kernel_size - 1 before that; the taps are added
-// oldest first, as the single-token kernel does.
+// oldest first, as the single-token kernel does.  The window slides in registers (KS taps known
+// at compile time for the common sizes), so every x is loaded once per tile.
 constexpr uint32_t CONV_TILE = 32;
 
 __device__ __forceinline__ float conv_input(const float *x, const float *state, int i, uint32_t c,
@@ -133,6 +134,7 @@ __device__ __forceinline__ float conv_input(const float *x, const float *state, 
     return i >= 0 ? x[size_t(i) * p.channels + c] : state[size_t(i + int(p.kernel_size) - 1) * p.channels + c];
 }
 
+template <int KS>  // taps; 0: any number (read from p), the window is re-read from memory
 __global__ __launch_bounds__(256) void deltanet_conv_rows_kernel(const float *__restrict__ x,
                                                                  const float *__restrict__ w,
                                                                  const float *__restrict__ state,
@@ -142,14 +144,39 @@ __global__ __launch_bounds__(256) void deltanet_conv_rows_kernel(const float *__
     if (c >= p.channels) return;
     const int past = int(p.kernel_size) - 1;
     const float *wc = w + size_t(c) * p.kernel_size;
-    const uint32_t t_end = min(p.tokens, (blockIdx.y + 1) * CONV_TILE);
-    for (uint32_t t = blockIdx.y * CONV_TILE; t < t_end; t++) {
-        float acc = 0.0f;
-        for (int j = 0; j < past; j++) acc += wc[j] * conv_input(x, state, int(t) - past + j, c, p);
-        out[size_t(t) * p.channels + c] = silu_f(acc + wc[past] * x[size_t(t) * p.channels + c]);
-        if (p.snapshots) {
-            float *snap = snaps + size_t(t) * past * p.channels;
-            for (int j = 0; j < past; j++) snap[size_t(j) * p.channels + c] = conv_input(x, state, int(t) - past + 1 + j, c, p);
+    const uint32_t t_begin = blockIdx.y * CONV_TILE, t_end = min(p.tokens, t_begin + CONV_TILE);
+    if constexpr (KS > 0) {
+        float taps[KS], win[KS - 1];
+#pragma unroll
+        for (int j = 0; j < KS; j++) taps[j] = wc[j];
+#pragma unroll
+        for (int j = 0; j < KS - 1; j++) win[j] = conv_input(x, state, int(t_begin) - (KS - 1) + j, c, p);
+        for (uint32_t t = t_begin; t < t_end; t++) {
+            const float xt = x[size_t(t) * p.channels + c];
+            float acc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < KS - 1; j++) acc += taps[j] * win[j];
+            out[size_t(t) * p.channels + c] = silu_f(acc + taps[KS - 1] * xt);
+#pragma unroll
+            for (int j = 0; j + 1 < KS - 1; j++) win[j] = win[j + 1];
+            win[KS - 2] = xt;
+            if (p.snapshots) {
+                float *snap = snaps + size_t(t) * (KS - 1) * p.channels;
+#pragma unroll
+                for (int j = 0; j < KS - 1; j++) snap[size_t(j) * p.channels + c] = win[j];
+            }
+        }
+    } else {
+        for (uint32_t t = t_begin; t < t_end; t++) {
+            float acc = 0.0f;
+            for (int j = 0; j < past; j++) acc += wc[j] * conv_input(x, state, int(t) - past + j, c, p);
+            out[size_t(t) * p.channels + c] = silu_f(acc + wc[past] * x[size_t(t) * p.channels + c]);
+            if (p.snapshots) {
+                float *snap = snaps + size_t(t) * past * p.channels;
+                for (int j = 0; j < past; j++) {
+                    snap[size_t(j) * p.channels + c] = conv_input(x, state, int(t) - past + 1 + j, c, p);
+                }
+            }
         }
     }
 }
@@ -449,7 +476,13 @@ extern "C" int saetta_deltanet_conv_rows(saetta_stream_t stream, const float *x,
     if (int rc = ensure_device()) return rc;
     if (p.channels == 0 || p.tokens == 0) return SAETTA_OK;
     const dim3 grid((p.channels + 255) / 256, (p.tokens + CONV_TILE - 1) / CONV_TILE);
-    deltanet_conv_rows_kernel<<<grid, 256, 0, as_stream(stream)>>>(x, w, state, out, snaps, p);
+    if (p.kernel_size == 4) {
+        deltanet_conv_rows_kernel<4><<<grid, 256, 0, as_stream(stream)>>>(x, w, state, out, snaps, p);
+    } else if (p.kernel_size == 2) {
+        deltanet_conv_rows_kernel<2><<<grid, 256, 0, as_stream(stream)>>>(x, w, state, out, snaps, p);
+    } else {
+        deltanet_conv_rows_kernel<0><<<grid, 256, 0, as_stream(stream)>>>(x, w, state, out, snaps, p);
+    }
     deltanet_conv_state_kernel<<<grid.x, 256, 0, as_stream(stream)>>>(x, state, p);
     return launch_status("deltanet_conv_rows");
 }
