@@ -24,8 +24,9 @@ cpu_baseline = the CPU oracle (a C restatement of the reference's
 Other workloads (--workload): decode4_150k (4-bit, 150000 tokens), verify2..4
 (2-4 query rows at 32k, 8-bit), prefill (4096-token chunk at position 4096),
 deltanet (the Gated DeltaNet decode step over 30 layer states), deltanet_prefill
-(conv + delta rule + gated norm of a 4096-token chunk of one layer), all (the
-default line with the others under "other_workloads").
+(conv + delta rule + gated norm of a 4096-token chunk of one layer), prep_store
+(q/k norm + RoPE + KV store of one token, 32 layers), all (the default line with
+the others under "other_workloads").
 """
 import argparse
 import json
@@ -350,6 +351,73 @@ def bench_deltanet(s, torch, args, layers=30):
     }
 
 
+def bench_prep_store(s, torch, args, layers=32, capacity=32896):
+    """The step before the scores, once per layer: q/k norm + RoPE + the token's key and value into
+    8-bit caches in one launch (attention_prep_store), beside the two kv_quantize launches the
+    reference records after its own prep kernel.  Latency-bound: 21 KB in, 1.1 KB + 16 KB out."""
+    import numpy as np
+    import oracle  # parity check only
+
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    qg = torch.randn(H * 2 * D, generator=gen, device="cuda")
+    k, v = torch.randn(KV * D, generator=gen, device="cuda"), torch.randn(KV * D, generator=gen, device="cuda")
+    qn, kn = 1 + 0.1 * torch.randn(D, generator=gen, device="cuda"), 1 + 0.1 * torch.randn(D, generator=gen, device="cuda")
+    q, kb = torch.empty(H * D, device="cuda"), torch.empty(KV * D, device="cuda")
+    caches = [(s.QuantRows(s.KvBits.Eight, VALUES, capacity), s.QuantRows(s.KvBits.Eight, VALUES, capacity))
+              for _ in range(layers)]
+    p = s.PrepParams(H, KV, D, 64, 1e7, 1e-6)
+    pos = 32768
+
+    def timed(plan):
+        plan.set_params(s.TokenParams(0, pos))
+        built = plan.build(graph=not args.no_graph)
+        for _ in range(args.warmup):
+            built.run()
+        ts = []
+        for _ in range(max(5, args.steps)):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            built.run()
+            e1.record()
+            e1.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e3 / layers)
+        return median(ts)
+
+    two = s.Plan()
+    for kc, vc in caches:
+        kc.record(two, k), vc.record(two, v)
+    two_us = timed(two)
+    fused = s.Plan()  # last: what it stores is checked below
+    for i, (kc, vc) in enumerate(caches):
+        s.record_store(fused, qg, k, v, qn, kn, q, kc, vc, p, capacity, k_back=kb if i == 0 else None)
+    fused_us = timed(fused)
+    # parity: q against the oracle's norm + rope, the stored codes against the oracle's quantizer
+    want_q, _, _ = oracle.attention_prep(qg.cpu().numpy(), k.cpu().numpy(), v.cpu().numpy(), qn.cpu().numpy(),
+                                         kn.cpu().numpy(), H, KV, D, 64, pos, 1e7, 1e-6)
+    torch.cuda.synchronize()
+    rel = float(np.sqrt(((q.cpu().numpy() - want_q.reshape(-1)) ** 2).mean() / (want_q ** 2).mean()))
+    data, scales, biases = oracle.quantize(kb.cpu().numpy().reshape(1, VALUES), 8)
+    kc = caches[0][0]
+    w0 = pos * 8 * 16
+    codes_equal = bool((kc.data[w0:w0 + 8 * 16].cpu().numpy().view(np.uint32) == data.reshape(-1)).all())
+    nbytes = 4.0 * (H * 2 * D + 2 * KV * D + 2 * D) + 4.0 * H * D + 2 * 8 * (64 + 4)
+    return {
+        "metric": "q/k norm + RoPE + KV store, launches per second of one layer",
+        "value": round(1e6 / fused_us, 1),
+        "unit": "layer-tokens/s",
+        "ms_per_step": round(fused_us * layers / 1e3, 4),
+        "dtype": "f32 in, u8 codes + f16 scales out",
+        "config": {"workload": f"attention_prep_store, 8-bit caches, position {pos}, {layers} layers per step",
+                   "bytes_per_layer": nbytes, "two_kv_quantize_launches_us": round(two_us, 3)},
+        "roofline": {"bound": "hbm", "achieved": round(nbytes / fused_us / 1e3, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(nbytes / fused_us / 1e3 / HBM_PEAK_GBS, 6), "traffic": None,
+                     "kernel": "attention_prep_store_kernel", "avg_us": round(fused_us, 3)},
+        "cpu_baseline": None,
+        "parity_rel_rms_vs_oracle": float(f"{rel:.3e}"),
+        "codes_equal_oracle": codes_equal,
+    }
+
+
 def bench_deltanet_prefill(s, torch, args, tokens=4096):
     """A prefill chunk of one Gated DeltaNet layer: deltanet_conv_rows + deltanet_rows over `tokens`
     tokens in order, the model's shape.  Algorithmic bytes of the rows launch: `mixed` and a, b read,
@@ -442,7 +510,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="decode8_32k",
                     choices=["decode8_32k", "decode4_150k", "verify2", "verify3", "verify4", "prefill", "deltanet",
-                             "deltanet_prefill", "all"])
+                             "deltanet_prefill", "prep_store", "all"])
     ap.add_argument("--no-graph", action="store_true", help="launch from Python instead of replaying a HIP graph")
     ap.add_argument("--layers", type=int, default=0, help="layer caches per step (default 32; 12 at 150k)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -479,12 +547,14 @@ def main():
             return bench_deltanet(s, torch, args)
         if workload == "deltanet_prefill":
             return bench_deltanet_prefill(s, torch, args)
+        if workload == "prep_store":
+            return bench_prep_store(s, torch, args)
         return bench_prefill(s, torch, args)
 
     if args.workload == "all":
         res = one("decode8_32k")
         res["other_workloads"] = {}
-        for w in ["verify2", "verify3", "verify4", "decode4_150k", "prefill", "deltanet", "deltanet_prefill"]:
+        for w in ["verify2", "verify3", "verify4", "decode4_150k", "prefill", "deltanet", "deltanet_prefill", "prep_store"]:
             torch.cuda.empty_cache()
             r = one(w)
             res["other_workloads"][w] = {k: r[k] for k in ("metric", "value", "unit", "ms_per_step", "roofline",
