@@ -68,7 +68,8 @@ typedef struct saetta_kv_quant_params {
 typedef struct saetta_decode_params {
     uint32_t heads;
     uint32_t kv_heads;
-    uint32_t capacity; /* tokens the cache has room for */
+    uint32_t capacity; /* tokens the cache has room for: a multiple of 16 (the reference's caches are
+                          multiples of 128, src/gpu_layers.rs:199) */
     float scale;       /* 1/sqrt(256) */
 } saetta_decode_params;
 

@@ -59,9 +59,12 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 constexpr int DIM = SAETTA_HEAD_DIM;
 constexpr int THREADS = 256;
 constexpr int BLOCK = 16;                     // tokens per MFMA block
-constexpr int IT_BLOCKS = 12;                 // blocks per iteration of a workgroup
-constexpr int IT_TOKENS = BLOCK * IT_BLOCKS;  // 192
-constexpr int SC_STRIDE = IT_TOKENS + 4;      // floats; keeps rows on different LDS banks
+// A buffer offset past any cache (their sizes stay below 2^31): the load returns 0 and touches no
+// memory.  With UNCOND, loads that an iteration does not need are issued with it instead of being
+// branched around, so that the number of loads in flight at every wait is known when the kernel is
+// compiled: loads return in order, and a wait whose count is not known has to wait for all of them.
+// (Measured per kernel: it pays for one and two query rows, not for the larger tiles.)
+constexpr int OOB = int(0x80000000u);
 constexpr float NO_SCORE = -1e30f;            // finite "minus infinity" of the running max
 
 // q is multiplied by scale * log2(e) * Q_UP before the hi/lo split so that
@@ -230,8 +233,12 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t bits16) {
 // TILES: 16-row tiles of query rows (rows * 8 heads, rounded up).  PACKED: one
 // verify row; its 8 heads' hi parts are operand rows 0-7 and lo parts rows 8-15
 // of a single tile.  Otherwise hi and lo are two MFMAs into one accumulator.
-template <int BITS, int TILES, bool PACKED>
+// ITB: blocks per iteration of a workgroup (a multiple of 4: one block per wave and round).
+template <int BITS, int TILES, bool PACKED, int ITB>
 struct Shape {
+    static constexpr int IT_BLOCKS = ITB;
+    static constexpr int IT_TOKENS = BLOCK * ITB;
+    static constexpr int SC_STRIDE = IT_TOKENS + 4;  // floats; keeps rows on different LDS banks
     static constexpr bool QUANT = BITS != 16;
     static constexpr int S_ROWS = 16 * TILES;                  // rows of the score buffer
     static constexpr int SOFT_ROWS = PACKED ? 8 : 16 * TILES;  // rows phase B walks
@@ -253,9 +260,11 @@ struct Shape {
     static constexpr int LDS_BYTES = ZSUM_OFF + 4 * S_ROWS * 4;
 };
 
-template <int BITS, int TILES, bool PACKED>
+template <int BITS, int TILES, bool PACKED, int ITB, bool UNCOND>
 __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
-    using Sh = Shape<BITS, TILES, PACKED>;
+    using Sh = Shape<BITS, TILES, PACKED, ITB>;
+    constexpr int IT_BLOCKS = ITB, IT_TOKENS = Sh::IT_TOKENS, SC_STRIDE = Sh::SC_STRIDE;
+    constexpr int KROUNDS = ITB / 4, KSTEPS = ITB / 2;
     constexpr bool QUANT = Sh::QUANT;
     constexpr int PARTS = Sh::PARTS;
     constexpr int RB = row_bytes<BITS>();
@@ -285,7 +294,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
         const int on = l & 15, oj = l >> 4;
         const int g = step >> 1, ab = step & 1;
         const int pair = PACKED ? (on & 7) : 16 * t + on;
-        if (pair < int(real_rows)) {
+        if (PACKED || pair < int(real_rows)) {  // (a single row always has its 8 heads)
             const int row = pair >> 3, head = pair & 7;
             const float *src = a.q + (size_t(row) * a.heads + kv * 8 + head) * DIM + 64 * g + 16 * oj + 8 * ab;
             const float4 f0 = *reinterpret_cast<const float4 *>(src);
@@ -335,26 +344,29 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     // ---- the loads of one iteration ------------------------------------------------
     // Everything an iteration reads is requested before anything is computed: keys first
     // (phase A needs them first), then the small scale/bias rows, then the values.
-    KeyRegs<BITS> kreg[3][4];
-    ValRegs<BITS> vreg[6];
+    KeyRegs<BITS> kreg[KROUNDS][4];
+    ValRegs<BITS> vreg[KSTEPS];
     u32x2 ksr = {0, 0}, kzr = {0, 0}, vsr = {0, 0}, vzr = {0, 0};
     auto blocks_of = [&](uint32_t it) { return min(per_it, blk_end - (blk_begin + it * per_it)); };
     auto load_keys = [&](uint32_t it) {
         const uint32_t base = (blk_begin + it * per_it) * BLOCK, nb = blocks_of(it);
         const int voff = int((base + BLOCK * wave + n) * kvh + kv) * RB + j * key_piece<BITS>();
 #pragma unroll
-        for (int i = 0; i < 3; i++) {
-            if (uint32_t(wave + 4 * i) < nb) {
+        for (int i = 0; i < KROUNDS; i++) {
+            const bool need = uint32_t(wave + 4 * i) < nb;
+            if (UNCOND || need) {
+                const int off = need ? voff : OOB;
 #pragma unroll
-                for (int g = 0; g < 4; g++) kreg[i][g] = load_key<BITS>(k_rsrc, voff, i * 64 * tok_stride, g);
+                for (int g = 0; g < 4; g++) kreg[i][g] = load_key<BITS>(k_rsrc, off, i * 64 * tok_stride, g);
             }
         }
     };
     auto load_scales = [&](uint32_t it) {
         if constexpr (QUANT) {
             const uint32_t base = (blk_begin + it * per_it) * BLOCK;
-            if (tid < IT_TOKENS) {
-                const int voff = int((base + tid) * kvh + kv) * 8;
+            const bool need = uint32_t(tid) < blocks_of(it) * BLOCK;
+            if (UNCOND || need) {
+                const int voff = need ? int((base + tid) * kvh + kv) * 8 : OOB;
                 ksr = __builtin_amdgcn_raw_buffer_load_b64(ks_rsrc, voff, 0, 0);
                 kzr = __builtin_amdgcn_raw_buffer_load_b64(kz_rsrc, voff, 0, 0);
                 vsr = __builtin_amdgcn_raw_buffer_load_b64(vs_rsrc, voff, 0, 0);
@@ -366,22 +378,24 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
         const uint32_t base = (blk_begin + it * per_it) * BLOCK, ksteps = (blocks_of(it) + 1) / 2;
         const int voff = int((base + 8 * j) * kvh + kv) * RB + val_lane_offset<BITS>(wave, n);
 #pragma unroll
-        for (int ks = 0; ks < 6; ks++) {
-            if (uint32_t(ks) < ksteps) {
+        for (int ks = 0; ks < KSTEPS; ks++) {
+            const bool need = uint32_t(ks) < ksteps;
+            if (UNCOND || need) {
+                const int off = need ? voff : OOB;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     const int soff = (32 * ks + e) * tok_stride;
-                    vreg[ks].w[e] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, voff, soff, 0);
+                    vreg[ks].w[e] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, off, soff, 0);
                     if constexpr (BITS == 16) {
-                        vreg[ks].w[8 + e] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, voff + 64, soff, 0);
+                        vreg[ks].w[8 + e] = __builtin_amdgcn_raw_buffer_load_b32(v_rsrc, off + 64, soff, 0);
                     }
                 }
             }
         }
     };
+    load_scales(0);  // first: loads return in order, and the barrier that publishes the scales must not wait for the keys
     load_keys(0);
-    load_scales(0);
-    if constexpr (TILES != 1) load_values(0);
+    load_values(0);
 
     // ---- prologue: query rows to f16 hi/lo operands in LDS ------------------------
     // (while the first iteration's keys are in flight; the values are requested after it)
@@ -432,7 +446,6 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
         }
     }
     __syncthreads();
-    if constexpr (TILES == 1) load_values(0);
 
     // Query operands of a single tile live in registers for the whole kernel.
     half8 q_reg[TILES == 1 ? PARTS * 8 : 1];
@@ -469,7 +482,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
 
     for (uint32_t it = 0; it < n_it; it++) {
         const uint32_t blk0 = blk_begin + it * per_it;
-        const uint32_t nb = min(per_it, blk_end - blk0);  // blocks of this iteration, 1..12
+        const uint32_t nb = min(per_it, blk_end - blk0);  // blocks of this iteration, 1..ITB
         const uint32_t base = blk0 * BLOCK;
         const uint32_t it_tokens = nb * BLOCK;
         const uint32_t ksteps = (nb + 1) / 2;
@@ -507,7 +520,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
                 }
             }
 #pragma unroll
-            for (int i = 0; i < 3; i++) {
+            for (int i = 0; i < KROUNDS; i++) {
                 const int blk = wave + 4 * i;
                 if (uint32_t(blk) >= nb) break;
                 const int tok0 = BLOCK * blk + 4 * j;  // this lane's 4 tokens in C layout
@@ -558,8 +571,8 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
         }
         // The key registers and the scale registers are free: request the next iteration's.
         if (it + 1 < n_it) {
-            load_keys(it + 1);
             load_scales(it + 1);
+            load_keys(it + 1);
         }
         __syncthreads();
 
@@ -656,13 +669,13 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
                 zacc[t] *= alpha_lds[PACKED ? (n & 7) : 16 * t + n];
             }
             if constexpr (PACKED) {
-                half8 phi[6], plo[6];
+                half8 phi[KSTEPS], plo[KSTEPS];
 #pragma unroll
-                for (int ks = 0; ks < 6; ks++) {
+                for (int ks = 0; ks < KSTEPS; ks++) {
                     if (uint32_t(ks) < ksteps) build_p(t, ks, phi[ks], plo[ks]);
                 }
 #pragma unroll
-                for (int ks = 0; ks < 6; ks++) {
+                for (int ks = 0; ks < KSTEPS; ks++) {
                     if (uint32_t(ks) >= ksteps) break;
                     if constexpr (BITS == 16) {
                         // Rows past the context may hold anything, NaN included: 0 * NaN must not reach O.
@@ -682,7 +695,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
                 }
             } else {
 #pragma unroll
-                for (int ks = 0; ks < 6; ks++) {
+                for (int ks = 0; ks < KSTEPS; ks++) {
                     if (uint32_t(ks) >= ksteps) break;
                     half8 phi, plo;
                     build_p(t, ks, phi, plo);
@@ -765,19 +778,26 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
 // One query row over codes (a single packed tile) fits two waves per SIMD, i.e. two workgroups
 // per CU (attention_partial_kernel_1, for long contexts); the others take the whole register file
 // and run one workgroup per CU.  Which one runs is decided in run_attention.
+// Blocks per iteration of each kernel.
+constexpr int ITB_TWO_PER_CU = 12, ITB_ONE_PER_CU = 8;
+template <int TILES>
+constexpr int itb_rows() {
+    return TILES == 1 ? 8 : 12;
+}
+
 template <int BITS>
 __global__ __launch_bounds__(THREADS, 2) void attention_partial_kernel_1(PartialArgs a) {
-    attention_partial_body<BITS, 1, true>(a);
+    attention_partial_body<BITS, 1, true, ITB_TWO_PER_CU, false>(a);
 }
 
 template <int BITS, int TILES>
 __global__ __launch_bounds__(THREADS) void attention_partial_kernel_n(PartialArgs a) {
-    attention_partial_body<BITS, TILES, false>(a);
+    attention_partial_body<BITS, TILES, false, itb_rows<TILES>(), TILES == 1>(a);
 }
 
 template <int BITS>
 __global__ __launch_bounds__(THREADS) void attention_partial_kernel_p(PartialArgs a) {
-    attention_partial_body<BITS, 1, true>(a);
+    attention_partial_body<BITS, 1, true, ITB_ONE_PER_CU, true>(a);
 }
 
 // Merges the splits of one (q head, row) and a 64-dim quarter of the head:
@@ -868,21 +888,25 @@ uint32_t splits_for(uint32_t capacity, uint32_t wanted) {
 
 template <int BITS, int TILES, bool PACKED>
 void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu) {
-    using Sh = Shape<BITS, TILES, PACKED>;
     void (*kernel)(PartialArgs);
+    int lds_bytes;
     if constexpr (TILES == 1 && BITS != 16 && PACKED) {
         if (one_per_cu) {
             kernel = attention_partial_kernel_p<BITS>;
+            lds_bytes = Shape<BITS, TILES, PACKED, ITB_ONE_PER_CU>::LDS_BYTES;
         } else {
             kernel = attention_partial_kernel_1<BITS>;
+            lds_bytes = Shape<BITS, TILES, PACKED, ITB_TWO_PER_CU>::LDS_BYTES;
         }
     } else if constexpr (PACKED) {
         kernel = attention_partial_kernel_p<BITS>;  // f16 cache: its registers do not fit two waves
+        lds_bytes = Shape<BITS, TILES, PACKED, ITB_ONE_PER_CU>::LDS_BYTES;
     } else {
         kernel = attention_partial_kernel_n<BITS, TILES>;
+        lds_bytes = Shape<BITS, TILES, PACKED, itb_rows<TILES>()>::LDS_BYTES;
     }
     // (the dynamic LDS limit of every variant was raised in setup_decode)
-    kernel<<<dim3(a.nsplits, a.kv_heads), THREADS, Sh::LDS_BYTES, stream>>>(a);
+    kernel<<<dim3(a.nsplits, a.kv_heads), THREADS, lds_bytes, stream>>>(a);
 }
 
 template <int BITS>
@@ -910,6 +934,9 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
     // Byte offsets into the cache are 32-bit: capacity * kv_heads * 512 B (the f16 row) must fit.
     SAETTA_REQUIRE(capacity > 0 && uint64_t(capacity) * kv_heads * 512 < (uint64_t(1) << 31), SAETTA_E_SHAPE,
                    "%s: capacity %u out of range", what, capacity);
+    // Whole 16-token blocks are read: the last one must lie inside the cache (the reference's caches
+    // are multiples of 128, src/gpu_layers.rs:199).
+    SAETTA_REQUIRE(capacity % BLOCK == 0, SAETTA_E_SHAPE, "%s: capacity %u is not a multiple of 16", what, capacity);
     SAETTA_REQUIRE(q && kdata && vdata && part_o && part_ml && q_and_gate && out && d_tp, SAETTA_E_NULL,
                    "%s: null buffer", what);
     SAETTA_REQUIRE(bits == 16 || (ks && kz && vs && vz), SAETTA_E_NULL, "%s: null scales or biases", what);
@@ -948,18 +975,19 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
 }  // namespace
 
 namespace {
-template <int BITS, int TILES, bool PACKED>
+template <int BITS, int TILES, bool PACKED, int ITB>
 int raise_lds(void (*kernel)(PartialArgs)) {
-    if (Shape<BITS, TILES, PACKED>::LDS_BYTES <= 48 * 1024) return 0;
+    static_assert(Shape<BITS, TILES, PACKED, ITB>::LDS_BYTES <= 160 * 1024, "LDS of a CU");
+    if (Shape<BITS, TILES, PACKED, ITB>::LDS_BYTES <= 48 * 1024) return 0;
     return int(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   Shape<BITS, TILES, PACKED>::LDS_BYTES));
+                                   Shape<BITS, TILES, PACKED, ITB>::LDS_BYTES));
 }
 template <int BITS>
 int raise_lds_of_bits() {
-    if (int rc = raise_lds<BITS, 1, true>(attention_partial_kernel_p<BITS>)) return rc;
-    if (int rc = raise_lds<BITS, 1, false>(attention_partial_kernel_n<BITS, 1>)) return rc;
-    if (int rc = raise_lds<BITS, 2, false>(attention_partial_kernel_n<BITS, 2>)) return rc;
-    return raise_lds<BITS, 4, false>(attention_partial_kernel_n<BITS, 4>);
+    if (int rc = raise_lds<BITS, 1, true, ITB_ONE_PER_CU>(attention_partial_kernel_p<BITS>)) return rc;
+    if (int rc = raise_lds<BITS, 1, false, itb_rows<1>()>(attention_partial_kernel_n<BITS, 1>)) return rc;
+    if (int rc = raise_lds<BITS, 2, false, itb_rows<2>()>(attention_partial_kernel_n<BITS, 2>)) return rc;
+    return raise_lds<BITS, 4, false, itb_rows<4>()>(attention_partial_kernel_n<BITS, 4>);
 }
 }  // namespace
 
@@ -968,8 +996,8 @@ int setup_decode() {
     if (int rc = raise_lds_of_bits<8>()) return rc;
     if (int rc = raise_lds_of_bits<4>()) return rc;
     if (int rc = raise_lds_of_bits<16>()) return rc;
-    if (int rc = raise_lds<8, 1, true>(attention_partial_kernel_1<8>)) return rc;
-    return raise_lds<4, 1, true>(attention_partial_kernel_1<4>);
+    if (int rc = raise_lds<8, 1, true, ITB_TWO_PER_CU>(attention_partial_kernel_1<8>)) return rc;
+    return raise_lds<4, 1, true, ITB_TWO_PER_CU>(attention_partial_kernel_1<4>);
 }
 }  // namespace saetta
 

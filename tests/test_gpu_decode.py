@@ -166,3 +166,16 @@ def test_shape_checks():
         saetta.DecodeAttention(16, 4, 256, 1024)
     with pytest.raises(ValueError):
         saetta.AttentionRows(16, 2, 1024, 9)
+
+
+def test_capacity_must_be_whole_blocks():
+    # The kernels read whole 16-token blocks; the reference's caches are multiples of 128 (KV_ALIGN).
+    capacity = 1000
+    z = torch.zeros(capacity * VALUES, dtype=torch.float16, device="cuda")
+    q, qg, out = torch.zeros(H * D, device="cuda"), torch.zeros(H * 2 * D, device="cuda"), torch.zeros(H * D, device="cuda")
+    att = saetta.DecodeAttention(H, KV, D, capacity)
+    plan = saetta.Plan()
+    att.record(plan, q, z, z, qg, out)
+    plan.set_params(saetta.TokenParams(0, 10))
+    with pytest.raises(saetta.ffi.SaettaError, match="multiple of 16"):
+        plan.build().run()
