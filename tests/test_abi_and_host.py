@@ -70,6 +70,20 @@ def test_bad_arguments_are_rejected_before_any_launch():
     rp = ffi.RowsParamsC(16, 2, 1024, 0.0625, 9, 8)
     assert lib.saetta_attn_rows_quant(None, 8, 16, rows, rows, 16, 16, 16, 16, rp, 16, 3) == -2
     assert b"9 rows" in lib.saetta_last_error()
+    odd = ffi.DecodeParamsC(16, 2, 1000, 0.0625)
+    assert lib.saetta_attn_decode_quant(None, 8, 16, rows, rows, 16, 16, 16, 16, odd, 16, 3) == -2
+    assert b"multiple of 16" in lib.saetta_last_error()
+    # Gated DeltaNet: heads must divide, v_dim a multiple of 4 for several tokens, snapshots need a buffer
+    sp = ffi.RowsStepParamsC(2, 3, 8, 1, 1e-6, 0)
+    assert lib.saetta_deltanet_rows(None, *([16] * 9), None, sp) == -2
+    assert b"value heads" in lib.saetta_last_error()
+    sp = ffi.RowsStepParamsC(1, 2, 6, 1, 1e-6, 0)
+    assert lib.saetta_deltanet_rows(None, *([16] * 9), None, sp) == -2
+    sp = ffi.RowsStepParamsC(1, 2, 8, 1, 1e-6, 1)
+    assert lib.saetta_deltanet_rows(None, *([16] * 9), None, sp) == -3  # snapshots asked for, no buffer
+    cp = ffi.ConvRowsParamsC(64, 1, 4, 0)
+    assert lib.saetta_deltanet_conv_rows(None, 16, 16, 16, 16, None, cp) == -2
+    assert b"kernel size" in lib.saetta_last_error()
     fp = ffi.FlashParamsC(16, 2, 0, 1, 0.0625)
     assert lib.saetta_attn_prefill_quant(None, 16, 16, rows, rows, 16, 16, fp, None, 0) == -1
     assert lib.saetta_attn_prefill_quant(None, 8, 16, rows, rows, 16, 16, fp, 8, 1 << 30) == -4  # workspace alignment
