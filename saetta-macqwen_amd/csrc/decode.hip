@@ -47,6 +47,8 @@
 #include "common.hpp"
 #include "lanes.hpp"
 
+#include <cstdlib>
+
 namespace saetta {
 namespace {
 
@@ -65,6 +67,11 @@ constexpr int BLOCK = 16;                     // tokens per MFMA block
 // compiled: loads return in order, and a wait whose count is not known has to wait for all of them.
 // (Measured per kernel: it pays for one and two query rows, not for the larger tiles.)
 constexpr int OOB = int(0x80000000u);
+// s_waitcnt operand that waits for the vector memory counter only (gfx9 encoding: vmcnt in bits
+// 3:0 and 15:14, the other counters at their maxima).
+constexpr int vmcnt_only(int n) {
+    return (n & 15) | 0x70 | 0xf00 | ((n >> 4) << 14);
+}
 constexpr float NO_SCORE = -1e30f;            // finite "minus infinity" of the running max
 
 // q is multiplied by scale * log2(e) * Q_UP before the hi/lo split so that
@@ -258,10 +265,34 @@ struct Shape {
     static constexpr int QZ_OFF = ALPHA_OFF + S_ROWS * 4;                   // [tile][hi, lo][lane] half8
     static constexpr int ZSUM_OFF = QZ_OFF + TILES * 2 * 64 * 16;           // [wave][S_ROWS] f32
     static constexpr int LDS_BYTES = ZSUM_OFF + 4 * S_ROWS * 4;
+    // With loader waves (8-bit codes only): four slots of one iteration's key and value codes each.
+    // Keys: per block [16 pieces of 16 bytes][16 tokens]; values: token rows of 256 bytes in groups
+    // of four, the groups 32 bytes apart so that the four lane groups of a value read hit
+    // different banks.
+    static constexpr int DMA_SLOTS = 16 / ITB;  // 256 tokens of codes in LDS
+    static constexpr int K_SLOT_BYTES = ITB * 4096;
+    static constexpr int V_GROUP_BYTES = 4 * 256 + 32;
+    static constexpr int V_SLOT_BYTES = ITB * 4 * V_GROUP_BYTES;
+    // The teams share the query operands (the first array and qz); a further team's other arrays
+    // start where the first team's end, its own (unused) query area lying over them.
+    static constexpr int TEAM_SHIFT = LDS_BYTES - Q_BYTES;
+    static constexpr int dma_k_off(int teams) { return (LDS_BYTES + (teams - 1) * TEAM_SHIFT + 1023) / 1024 * 1024; }
+    static constexpr int dma_lds_bytes(int teams) {
+        return dma_k_off(teams) + DMA_SLOTS * (K_SLOT_BYTES + V_SLOT_BYTES);
+    }
 };
 
-template <int BITS, int TILES, bool PACKED, int ITB, bool UNCOND>
+// DMA: the workgroup has four more waves that do nothing but move key and value codes from global
+// memory into LDS (global_load_lds, no registers), slot by slot, as far ahead as the slots allow; a
+// wave that requests loads stands still while the request queues are full, and these waves have
+// nothing else to do.  The four computing waves take their operands from LDS instead.
+// TEAMS (with DMA): groups of four computing waves; in every round team t takes iteration
+// TEAMS * round + t, all in step (the barriers are the workgroup's), and team 0 merges the teams'
+// results at the end.
+template <int BITS, int TILES, bool PACKED, int ITB, bool UNCOND, bool DMA = false, int TEAMS = 1>
 __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
+    static_assert(TEAMS == 1 || (DMA && TEAMS == 2), "teams need the loader waves");
+    static_assert(!DMA || (BITS == 8 && PACKED && (ITB == 4 || ITB == 8)), "loader waves: one row over 8-bit codes, 64- or 128-token iterations");
     using Sh = Shape<BITS, TILES, PACKED, ITB>;
     constexpr int IT_BLOCKS = ITB, IT_TOKENS = Sh::IT_TOKENS, SC_STRIDE = Sh::SC_STRIDE;
     constexpr int KROUNDS = ITB / 4, KSTEPS = ITB / 2;
@@ -269,17 +300,21 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     constexpr int PARTS = Sh::PARTS;
     constexpr int RB = row_bytes<BITS>();
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    // team: 0 .. TEAMS - 1 compute, TEAMS = the loader waves; tid and wave are the team's own
+    const int team = DMA ? int(threadIdx.x) / THREADS : 0;
+    const int tid = DMA ? int(threadIdx.x) % THREADS : int(threadIdx.x), lane = tid & 63, wave = tid >> 6;
+    unsigned char *lds_team = lds_raw + (DMA && team < TEAMS ? team * Sh::TEAM_SHIFT : 0);
+    constexpr int K_OFF = Sh::dma_k_off(TEAMS), V_OFF = K_OFF + Sh::DMA_SLOTS * Sh::K_SLOT_BYTES;
     half8 *q_lds = reinterpret_cast<half8 *>(lds_raw + Sh::Q_OFF);
-    float *s_lds = reinterpret_cast<float *>(lds_raw + Sh::S_OFF);
-    uint16_t *ks_lds = reinterpret_cast<uint16_t *>(lds_raw + Sh::KS_OFF);
-    uint16_t *kz_lds = reinterpret_cast<uint16_t *>(lds_raw + Sh::KZ_OFF);
-    uint16_t *vs_lds = reinterpret_cast<uint16_t *>(lds_raw + Sh::VS_OFF);
-    uint16_t *vz_lds = reinterpret_cast<uint16_t *>(lds_raw + Sh::VZ_OFF);
-    float *alpha_lds = reinterpret_cast<float *>(lds_raw + Sh::ALPHA_OFF);
+    float *s_lds = reinterpret_cast<float *>(lds_team + Sh::S_OFF);
+    uint16_t *ks_lds = reinterpret_cast<uint16_t *>(lds_team + Sh::KS_OFF);
+    uint16_t *kz_lds = reinterpret_cast<uint16_t *>(lds_team + Sh::KZ_OFF);
+    uint16_t *vs_lds = reinterpret_cast<uint16_t *>(lds_team + Sh::VS_OFF);
+    uint16_t *vz_lds = reinterpret_cast<uint16_t *>(lds_team + Sh::VZ_OFF);
+    float *alpha_lds = reinterpret_cast<float *>(lds_team + Sh::ALPHA_OFF);
     _Float16 *qz_lds = reinterpret_cast<_Float16 *>(lds_raw + Sh::QZ_OFF);
-    float *zsum_lds = reinterpret_cast<float *>(lds_raw + Sh::ZSUM_OFF);
+    float *zsum_lds = reinterpret_cast<float *>(lds_team + Sh::ZSUM_OFF);
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, j = lane >> 4;
     const uint32_t split = blockIdx.x, kv = blockIdx.y;
     const uint32_t kvh = a.kv_heads;
@@ -308,8 +343,10 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     };
     float q_early[TILES == 1 ? 2 : 1][8];
     if constexpr (TILES == 1) {
-        load_q_item(tid, q_early[0]);
-        load_q_item(tid + THREADS, q_early[1]);
+        if (team < TEAMS) {
+            load_q_item(tid, q_early[0]);
+            load_q_item(tid + THREADS, q_early[1]);
+        }
     }
 
     // ---- the context and this workgroup's share of it -----------------------------
@@ -331,6 +368,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     const uint32_t range = blk_end - blk_begin;
     const uint32_t n_it = (range + IT_BLOCKS - 1) / IT_BLOCKS;
     const uint32_t per_it = (range + n_it - 1) / n_it;
+    const uint32_t n_rounds = (n_it + TEAMS - 1) / TEAMS;
 
     const uint32_t cap_rows = a.capacity * kvh;
     const __amdgpu_buffer_rsrc_t k_rsrc = make_rsrc(a.kdata, cap_rows * RB);
@@ -341,14 +379,89 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     const __amdgpu_buffer_rsrc_t vz_rsrc = make_rsrc(a.vbiases, QUANT ? cap_rows * 8 : 0);
     const int tok_stride = int(kvh) * RB;  // bytes between tokens of one kv head
 
+    if constexpr (DMA) {
+        if (team == TEAMS) {
+            // ---- a loader wave: block L of every iteration, keys then values ----------------
+            const uint32_t L = __builtin_amdgcn_readfirstlane(wave);
+            const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(lds_raw));
+            auto dma = [&](uint32_t lds_addr, uint32_t voff, const void *src) {
+                asm volatile("s_mov_b32 m0, %0\n"
+                             "s_nop 0\n"
+                             "global_load_lds_dwordx4 %1, %2\n"
+                             :
+                             : "s"(lds_addr), "v"(voff), "s"(src)
+                             : "memory", "m0");
+            };
+            const uint32_t last_row = a.capacity - 1;  // (global loads are not bounds checked)
+            constexpr int PER_REQUEST = 8 * KROUNDS;  // loads of one iteration, per loader wave
+            auto request = [&](uint32_t it) {
+                const uint32_t slot = it % Sh::DMA_SLOTS;
+                // keys of every round first: phase A needs them first
+#pragma unroll
+                for (int r = 0; r < KROUNDS; r++) {
+                    const uint32_t blk = L + 4 * r, base = (blk_begin + it * per_it + blk) * BLOCK;
+                    // lane -> (piece lane / 16 of the instruction's four, token lane % 16)
+                    const uint32_t ktok = min(base + (lane & 15), last_row);
+                    const uint32_t kvoff = (ktok * kvh + kv) * RB + (lane >> 4) * 16;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        dma(lds0 + K_OFF + slot * Sh::K_SLOT_BYTES + blk * 4096 + i * 1024, kvoff + 64 * i, a.kdata);
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < KROUNDS; r++) {
+                    const uint32_t blk = L + 4 * r, base = (blk_begin + it * per_it + blk) * BLOCK;
+                    // lane -> (token lane / 16 of the instruction's four, piece lane % 16)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const uint32_t vtok = min(base + 4 * i + (lane >> 4), last_row);
+                        dma(lds0 + V_OFF + slot * Sh::V_SLOT_BYTES + (4 * blk + i) * Sh::V_GROUP_BYTES,
+                            (vtok * kvh + kv) * RB + (lane & 15) * 16, a.vdata);
+                    }
+                }
+            };
+            uint32_t requested = min(n_it, uint32_t(Sh::DMA_SLOTS));
+            for (uint32_t it = 0; it < requested; it++) request(it);
+            __builtin_amdgcn_s_barrier();  // the computing waves' barrier after the query prologue
+            for (uint32_t round = 0; round < n_rounds; round++) {
+                // the round's iterations are in LDS when at most the later ones' loads are in flight
+                const uint32_t last = min(round * TEAMS + TEAMS - 1, n_it - 1);
+                const uint32_t later = requested - 1 - last;
+                static_assert(PER_REQUEST * (Sh::DMA_SLOTS - 1) < 64, "vmcnt is 6 bits");
+                if (Sh::DMA_SLOTS > 3 && later >= 3) {
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(PER_REQUEST * 3 < 64 ? PER_REQUEST * 3 : 63));
+                } else if (Sh::DMA_SLOTS > 2 && later == 2) {
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(PER_REQUEST * 2 < 64 ? PER_REQUEST * 2 : 63));
+                } else if (later == 1) {
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(PER_REQUEST));
+                } else {
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+                }
+                __builtin_amdgcn_s_barrier();  // "scales visible": the round may start
+                // every computing wave is past phase C of the round before: its slots take the next
+                if (round >= 1) {
+#pragma unroll
+                    for (int t = 0; t < TEAMS; t++) {
+                        if (requested < n_it) request(requested++);
+                    }
+                }
+                __builtin_amdgcn_s_barrier();  // scores done
+                __builtin_amdgcn_s_barrier();  // probabilities done
+            }
+            if constexpr (TEAMS > 1) __builtin_amdgcn_s_barrier();  // the teams' merge
+            return;
+        }
+    }
+
     // ---- the loads of one iteration ------------------------------------------------
     // Everything an iteration reads is requested before anything is computed: keys first
     // (phase A needs them first), then the small scale/bias rows, then the values.
     KeyRegs<BITS> kreg[KROUNDS][4];
     ValRegs<BITS> vreg[KSTEPS];
     u32x2 ksr = {0, 0}, kzr = {0, 0}, vsr = {0, 0}, vzr = {0, 0};
-    auto blocks_of = [&](uint32_t it) { return min(per_it, blk_end - (blk_begin + it * per_it)); };
+    auto blocks_of = [&](uint32_t it) { return it < n_it ? min(per_it, blk_end - (blk_begin + it * per_it)) : 0u; };
     auto load_keys = [&](uint32_t it) {
+        if constexpr (DMA) return;
         const uint32_t base = (blk_begin + it * per_it) * BLOCK, nb = blocks_of(it);
         const int voff = int((base + BLOCK * wave + n) * kvh + kv) * RB + j * key_piece<BITS>();
 #pragma unroll
@@ -375,6 +488,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
         }
     };
     auto load_values = [&](uint32_t it) {
+        if constexpr (DMA) return;
         const uint32_t base = (blk_begin + it * per_it) * BLOCK, ksteps = (blocks_of(it) + 1) / 2;
         const int voff = int((base + 8 * j) * kvh + kv) * RB + val_lane_offset<BITS>(wave, n);
 #pragma unroll
@@ -393,9 +507,9 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
             }
         }
     };
-    load_scales(0);  // first: loads return in order, and the barrier that publishes the scales must not wait for the keys
-    load_keys(0);
-    load_values(0);
+    load_scales(team);  // first: loads return in order, and the barrier that publishes the scales must not wait for the keys
+    load_keys(team);
+    load_values(team);
 
     // ---- prologue: query rows to f16 hi/lo operands in LDS ------------------------
     // (while the first iteration's keys are in flight; the values are requested after it)
@@ -480,9 +594,10 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
         for (int e = 0; e < 4; e++) acc[t][e] = floatx4{0, 0, 0, 0};
     }
 
-    for (uint32_t it = 0; it < n_it; it++) {
+    for (uint32_t round = 0; round < n_rounds; round++) {
+        const uint32_t it = round * TEAMS + team;  // (a team without an iteration in the last round idles through it)
         const uint32_t blk0 = blk_begin + it * per_it;
-        const uint32_t nb = min(per_it, blk_end - blk0);  // blocks of this iteration, 1..ITB
+        const uint32_t nb = blocks_of(it);  // blocks of this iteration, 0..ITB
         const uint32_t base = blk0 * BLOCK;
         const uint32_t it_tokens = nb * BLOCK;
         const uint32_t ksteps = (nb + 1) / 2;
@@ -502,6 +617,18 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
             }
         }
         __syncthreads();  // scales visible; the previous iteration's phase C is over
+        if constexpr (DMA) {
+            // this wave's block: the lane's piece j of each group, its token n
+            const unsigned char *kb = lds_raw + K_OFF + (it % Sh::DMA_SLOTS) * Sh::K_SLOT_BYTES + wave * 4096;
+#pragma unroll
+            for (int i = 0; i < KROUNDS; i++) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const u32x4 v = *reinterpret_cast<const u32x4 *>(kb + i * 4 * 4096 + (4 * g + j) * 256 + n * 16);
+                    kreg[i][g].w[0] = v.x, kreg[i][g].w[1] = v.y, kreg[i][g].w[2] = v.z, kreg[i][g].w[3] = v.w;
+                }
+            }
+        }
 
         // ---- phase A: scores -------------------------------------------------------
 #pragma unroll
@@ -570,9 +697,9 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
             }
         }
         // The key registers and the scale registers are free: request the next iteration's.
-        if (it + 1 < n_it) {
-            load_scales(it + 1);
-            load_keys(it + 1);
+        if (it + TEAMS < n_it) {
+            load_scales(it + TEAMS);
+            load_keys(it + TEAMS);
         }
         __syncthreads();
 
@@ -661,7 +788,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
 #pragma unroll
         for (int t = 0; t < TILES; t++) {
             // Rescale what was summed so far.  Accumulator rows (C layout) are 4j..4j+3.
-            if (it > 0) {
+            if (round > 0) {
                 const int arow = PACKED ? ((4 * j) & 7) : 16 * t + 4 * j;
                 const floatx4 al = *reinterpret_cast<const floatx4 *>(alpha_lds + arow);
 #pragma unroll
@@ -673,6 +800,17 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ks++) {
                     if (uint32_t(ks) < ksteps) build_p(t, ks, phi[ks], plo[ks]);
+                }
+                if constexpr (DMA) {
+                    const unsigned char *vb = lds_raw + V_OFF + (it % Sh::DMA_SLOTS) * Sh::V_SLOT_BYTES + 64 * wave + 4 * n;
+#pragma unroll
+                    for (int ks = 0; ks < KSTEPS; ks++) {
+#pragma unroll
+                        for (int e = 0; e < 8; e++) {
+                            const int tk = 32 * ks + 8 * j + e;  // token of the iteration
+                            vreg[ks].w[e] = *reinterpret_cast<const uint32_t *>(vb + (tk >> 2) * Sh::V_GROUP_BYTES + (tk & 3) * 256);
+                        }
+                    }
                 }
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ks++) {
@@ -716,9 +854,56 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
                 }
             }
         }
-        if (it + 1 < n_it) load_values(it + 1);
+        if (it + TEAMS < n_it) load_values(it + TEAMS);
     }
 
+    if constexpr (TEAMS > 1) {
+        // ---- epilogue with teams: every team finishes its own (m, l, O), team 1 hands its to team 0
+        // through LDS (the key slots are free by now), team 0 merges and writes the partial.
+        static_assert(TEAMS == 1 || (TILES == 1 && PACKED && QUANT), "teams: one row over codes");
+        l_part = group_reduce<Sh::TPR>(l_part, SumOp());
+        float *x_ml = reinterpret_cast<float *>(lds_raw + K_OFF);             // [team][m of 8 heads, l of 8 heads]
+        floatx4 *x_o = reinterpret_cast<floatx4 *>(lds_raw + K_OFF + 1024);  // [thread][4 rows]
+        if (b_part == 0) x_ml[team * 16 + b_row] = m_run, x_ml[team * 16 + 8 + b_row] = l_part;
+        {
+            const float z = across_rows<16, 64>(zacc[0], SumOp());
+            if (j == 0 && n < 8) zsum_lds[wave * Sh::S_ROWS + n] = z;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+        constexpr float unscale = code_up<BITS>() / P_UP;
+        floatx4 mine[4];  // head 4j + i (j < 2), dims 64 wave + 4n .. + 3
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float zb = zsum_lds[wave * Sh::S_ROWS + ((4 * j + i) & 7)] * (1.0f / P_UP);
+#pragma unroll
+            for (int e = 0; e < 4; e++) mine[i][e] = across_rows<32, 64>(acc[0][e][i], SumOp()) * unscale + zb;
+        }
+        if (team == 1 && j < 2) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) x_o[tid * 4 + i] = mine[i];
+        }
+        __syncthreads();
+        if (team != 0) return;
+        if (b_part == 0) {
+            const float m0 = x_ml[b_row], m1 = x_ml[16 + b_row], mm = fmaxf(m0, m1);
+            const float l = x_ml[8 + b_row] * __builtin_amdgcn_exp2f(m0 - mm) + x_ml[24 + b_row] * __builtin_amdgcn_exp2f(m1 - mm);
+            const size_t slot = size_t(split) * a.heads + kv * 8 + b_row;
+            *reinterpret_cast<floatx2 *>(a.part_ml + 2 * slot) = floatx2{mm, l};
+        }
+        if (j < 2) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int head = 4 * j + i;
+                const float m0 = x_ml[head], m1 = x_ml[16 + head], mm = fmaxf(m0, m1);
+                const float f0 = __builtin_amdgcn_exp2f(m0 - mm), f1 = __builtin_amdgcn_exp2f(m1 - mm);
+                const floatx4 other = x_o[tid * 4 + i];
+                const size_t slot = size_t(split) * a.heads + kv * 8 + head;
+                *reinterpret_cast<floatx4 *>(a.part_o + slot * DIM + 64 * wave + 4 * n) = mine[i] * f0 + other * f1;
+            }
+        }
+        return;
+    }
     // ---- epilogue: one partial per (row, head) ------------------------------------
     // m and l from the phase B threads.
     l_part = group_reduce<Sh::TPR>(l_part, SumOp());
@@ -793,6 +978,12 @@ __global__ __launch_bounds__(THREADS, 2) void attention_partial_kernel_1(Partial
 template <int BITS, int TILES>
 __global__ __launch_bounds__(THREADS) void attention_partial_kernel_n(PartialArgs a) {
     attention_partial_body<BITS, TILES, false, itb_rows<TILES>(), TILES == 1>(a);
+}
+
+// One query row over 8-bit codes with loader waves: 4 computing + 4 loading waves.
+constexpr int ITB_DMA = 4, TEAMS_DMA = 2;
+__global__ __launch_bounds__((TEAMS_DMA + 1) * THREADS) void attention_partial_kernel_d(PartialArgs a) {
+    attention_partial_body<8, 1, true, ITB_DMA, true, true, TEAMS_DMA>(a);
 }
 
 template <int BITS>
@@ -886,10 +1077,30 @@ uint32_t splits_for(uint32_t capacity, uint32_t wanted) {
     return s ? s : 1;
 }
 
+// One row over 8-bit codes: from this capacity on the kernel with loader waves is the faster one
+// (measured, per layer with the merge: 10.0 against 11.0 us at 4k tokens, equal at 32k, 20.9
+// against 22.3 at 50k, 35.5 against 36.5 at 131k).
+constexpr uint32_t LOADERS_FROM = 24 * 1024;
+
+bool loaders_enabled() {  // SAETTA_DECODE_LOADERS=0 keeps to the kernels without loader waves
+    static const bool on = [] {
+        const char *e = getenv("SAETTA_DECODE_LOADERS");
+        return !e || e[0] != '0';
+    }();
+    return on;
+}
+
 template <int BITS, int TILES, bool PACKED>
-void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu) {
+void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu, bool loaders) {
     void (*kernel)(PartialArgs);
     int lds_bytes;
+    if constexpr (TILES == 1 && BITS == 8 && PACKED) {
+        if (loaders) {
+            attention_partial_kernel_d<<<dim3(a.nsplits, a.kv_heads), (TEAMS_DMA + 1) * THREADS,
+                                         Shape<8, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA), stream>>>(a);
+            return;
+        }
+    }
     if constexpr (TILES == 1 && BITS != 16 && PACKED) {
         if (one_per_cu) {
             kernel = attention_partial_kernel_p<BITS>;
@@ -910,15 +1121,15 @@ void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu) {
 }
 
 template <int BITS>
-void launch_partial_rows(hipStream_t stream, const PartialArgs &a, bool one_per_cu) {
+void launch_partial_rows(hipStream_t stream, const PartialArgs &a, bool one_per_cu, bool loaders) {
     if (a.rows == 1) {
-        launch_partial<BITS, 1, true>(stream, a, one_per_cu);
+        launch_partial<BITS, 1, true>(stream, a, one_per_cu, loaders);
     } else if (a.rows == 2) {
-        launch_partial<BITS, 1, false>(stream, a, one_per_cu);
+        launch_partial<BITS, 1, false>(stream, a, one_per_cu, loaders);
     } else if (a.rows <= 4) {
-        launch_partial<BITS, 2, false>(stream, a, one_per_cu);
+        launch_partial<BITS, 2, false>(stream, a, one_per_cu, loaders);
     } else {
-        launch_partial<BITS, 4, false>(stream, a, one_per_cu);
+        launch_partial<BITS, 4, false>(stream, a, one_per_cu, loaders);
     }
 }
 
@@ -952,17 +1163,20 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
     // which pays only for long contexts: up to 64k tokens the shorter merge of half as many partials
     // is worth more (measured: 19.4 against 20.6 us per layer at 32k, 28.3 against 29.7 at 64k,
     // but 44 against 35 at 146k, 4-bit).  Both stages derive the same number from the same arguments.
-    const bool one_per_cu = rows >= 2 || bits == 16 || capacity <= 80 * 1024;
+    // One row over 8-bit codes in a cache of 24k tokens and more goes to the kernel with loader waves,
+    // which is a one-workgroup-per-CU kernel at every length.
+    const bool loaders = rows == 1 && bits == 8 && capacity >= LOADERS_FROM && loaders_enabled();
+    const bool one_per_cu = rows >= 2 || bits == 16 || capacity <= 80 * 1024 || loaders;
     if (one_per_cu && nsplits > MAX_SPLITS / 2) nsplits = MAX_SPLITS / 2;
     if (stages & SAETTA_STAGE_PARTIAL) {
         PartialArgs a{q,     kdata,    vdata,    ks,    kz,   vs,      vz,   part_o, part_ml,
                       heads, kv_heads, capacity, scale, rows, nsplits, d_tp, decode_len ? 1u : 0u};
         if (bits == 8) {
-            launch_partial_rows<8>(stream, a, one_per_cu);
+            launch_partial_rows<8>(stream, a, one_per_cu, loaders);
         } else if (bits == 4) {
-            launch_partial_rows<4>(stream, a, one_per_cu);
+            launch_partial_rows<4>(stream, a, one_per_cu, loaders);
         } else {
-            launch_partial_rows<16>(stream, a, one_per_cu);
+            launch_partial_rows<16>(stream, a, one_per_cu, loaders);
         }
     }
     if (stages & SAETTA_STAGE_REDUCE) {
@@ -993,6 +1207,12 @@ int raise_lds_of_bits() {
 
 int setup_decode() {
     if (int rc = load_kernel(reinterpret_cast<const void *>(attention_reduce_kernel))) return rc;
+    static_assert(Shape<8, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA) <= 160 * 1024, "LDS of a CU");
+    if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_partial_kernel_d),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         Shape<8, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA)))) {
+        return rc;
+    }
     if (int rc = raise_lds_of_bits<8>()) return rc;
     if (int rc = raise_lds_of_bits<4>()) return rc;
     if (int rc = raise_lds_of_bits<16>()) return rc;
