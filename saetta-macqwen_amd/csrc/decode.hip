@@ -602,21 +602,27 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
         const uint32_t it_tokens = nb * BLOCK;
         const uint32_t ksteps = (nb + 1) / 2;
 
-        // Scales and biases of the iteration's tokens to LDS: thread = token, 4 groups each.
+        // Scales and biases of the iteration's tokens to LDS: thread = token, 4 groups each.  The key
+        // ones before the barrier (phase A reads them); the value ones after it: a wave may still be
+        // reading the previous iteration's in its phase C until every wave has arrived here.
+        if constexpr (QUANT) {
+            if (tid < IT_TOKENS) {
+                *reinterpret_cast<u32x2 *>(ks_lds + 4 * tid) = ksr;
+                *reinterpret_cast<u32x2 *>(kz_lds + 4 * tid) = kzr;
+            }
+        }
+        __syncthreads();  // key scales visible; the previous iteration's phase C is over
         if constexpr (QUANT) {
             if (tid < IT_TOKENS) {
                 // Tokens past the context or the iteration get value scale 0 and bias 0, so that
                 // whatever their rows hold stays out of O (their probabilities are 0 as well).
                 if (uint32_t(tid) >= it_tokens || base + tid >= max_len) vsr = u32x2{0, 0}, vzr = u32x2{0, 0};
-                *reinterpret_cast<u32x2 *>(ks_lds + 4 * tid) = ksr;
-                *reinterpret_cast<u32x2 *>(kz_lds + 4 * tid) = kzr;
                 vs_lds[0 * IT_TOKENS + tid] = uint16_t(vsr.x), vs_lds[1 * IT_TOKENS + tid] = uint16_t(vsr.x >> 16);
                 vs_lds[2 * IT_TOKENS + tid] = uint16_t(vsr.y), vs_lds[3 * IT_TOKENS + tid] = uint16_t(vsr.y >> 16);
                 vz_lds[0 * IT_TOKENS + tid] = uint16_t(vzr.x), vz_lds[1 * IT_TOKENS + tid] = uint16_t(vzr.x >> 16);
                 vz_lds[2 * IT_TOKENS + tid] = uint16_t(vzr.y), vz_lds[3 * IT_TOKENS + tid] = uint16_t(vzr.y >> 16);
             }
         }
-        __syncthreads();  // scales visible; the previous iteration's phase C is over
         if constexpr (DMA) {
             // this wave's block: the lane's piece j of each group, its token n
             const unsigned char *kb = lds_raw + K_OFF + (it % Sh::DMA_SLOTS) * Sh::K_SLOT_BYTES + wave * 4096;
