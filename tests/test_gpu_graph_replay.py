@@ -1,0 +1,82 @@
+"""Plans replayed from a HIP graph (the counterpart of the reference's indirect command buffer,
+src/plan.rs:229-235; tests/plan.rs:27-45 asks that serial == replay exactly).  A graph is replayed
+several times, with eager work of the program between the replays and another position each time,
+and every replay is checked against the same launches run eagerly."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_common import D, H, KV, VALUES, dev, host, oracle, saetta
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("kind,capacity", [(saetta.KvBits.Eight, 4096), (saetta.KvBits.Eight, 32768),
+                                           (saetta.KvBits.Four, 4096), (saetta.KvBits.Half, 4096)])
+def test_token_step_replays_bit_for_bit(kind, capacity):
+    # one token of an attention layer: store (norm, rope, append) then decode, at the plan's position
+    rng = np.random.default_rng(capacity + kind.value)
+    qg, k, v = (dev(rng.standard_normal(n).astype(np.float32)) for n in (H * 2 * D, KV * D, KV * D))
+    qn, kn = dev(np.ones(D, np.float32)), dev(np.ones(D, np.float32))
+    cache = saetta.GpuKvCache.with_bits(H, KV, D, capacity, kind)
+    fill = dev(oracle.noise(capacity * VALUES, 3).reshape(capacity, VALUES))
+    if kind is saetta.KvBits.Half:
+        cache.keys.copy_(fill.flatten().half()), cache.values.copy_(fill.flatten().half())
+        keys, values = cache.keys, cache.values
+    else:
+        keys, values = cache.quant
+        keys.encode(fill, 0, capacity), values.encode(fill, 0, capacity)
+    q, out = torch.empty(H * D, device="cuda"), torch.empty(H * D, device="cuda")
+    plan = saetta.Plan()
+    saetta.record_store(plan, qg, k, v, qn, kn, q, keys, values, saetta.PrepParams(H, KV, D, 64, 1e7, 1e-6), capacity)
+    if kind is saetta.KvBits.Half:
+        cache.decode.record(plan, q, keys, values, qg, out)
+    else:
+        cache.decode.record_quant(plan, q, keys, values, qg, out)
+    eager, graph = plan.build(), plan.build(graph=True)
+    assert graph.graph is not None
+    for pos in (0, 17, 1000, capacity - 1, 5):
+        plan.set_params(saetta.TokenParams(0, pos))
+        eager.run()
+        want = out.clone()
+        out.fill_(float("nan"))
+        scratch = torch.randn(1 << 16, device="cuda").sum()  # the program's own eager work between replays
+        graph.run()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), pos
+        assert torch.isfinite(scratch)
+
+
+def test_deltanet_rows_replay_advances_the_state_like_eager_runs():
+    kh, vh, dv, kernel, m = 2, 4, 32, 4, 3
+    key, val = kh * 128, vh * dv
+    ch = 2 * key + val
+    g = torch.Generator(device="cuda").manual_seed(5)
+
+    def r(*n):
+        return torch.randn(*n, generator=g, device="cuda")
+
+    x, z, a, b = r(m, ch), r(m, val), r(m, vh), r(m, vh)
+    w, alog, dtb, norm = 0.5 * r(ch * kernel), r(vh), r(vh), 1 + 0.1 * r(dv)
+
+    def run(graph, replays):
+        conv, st = torch.zeros((kernel - 1) * ch, device="cuda"), torch.zeros(vh * dv * 128, device="cuda")
+        mixed, y = torch.empty(m, ch, device="cuda"), torch.empty(m, val, device="cuda")
+        plan = saetta.Plan()
+        saetta.deltanet_conv_rows(plan, x, w, conv, mixed, ch, kernel, m)
+        saetta.deltanet_rows(plan, mixed, a, b, alog, dtb, st, z, norm, y, kh, vh, dv, m, 1e-6)
+        built = plan.build(graph=graph)  # building a graph must not run the plan: the state would move
+        assert not st.any()
+        ys = []
+        for _ in range(replays):
+            built.run()
+            torch.cuda.synchronize()
+            ys.append(y.clone())
+        return ys, conv, st
+
+    want_y, want_conv, want_st = run(False, 4)
+    got_y, got_conv, got_st = run(True, 4)
+    for u, v in zip(got_y, want_y):
+        assert torch.equal(u, v)
+    assert torch.equal(got_conv, want_conv) and torch.equal(got_st, want_st)
+    assert not torch.equal(want_y[0], want_y[1])  # the state did move between the runs
