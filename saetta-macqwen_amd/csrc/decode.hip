@@ -14,7 +14,7 @@
 // memory when the kernel runs) is cut into 16-token blocks and the blocks are
 // dealt evenly to the `nsplits` workgroups of each kv head, so every
 // workgroup streams the same number of bytes whatever the position is.  A
-// workgroup walks its range in iterations of up to 192 tokens, keeps an
+// workgroup walks its range in iterations of 64 to 192 tokens, keeps an
 // online softmax per query row, and writes one unnormalised partial (o, m, l)
 // per (row, q head); a second kernel merges the partials and applies the gate.
 //
@@ -41,9 +41,20 @@
 // or for a single row the hi and lo parts share one 16-row tile), which keeps
 // the result within ~1e-6 of an f32 evaluation.
 //
-// All cache reads are buffer loads with the cache's size as the bound: rows
-// past the capacity read as 0 instead of faulting, and the per-lane address is
-// one 32-bit offset plus scalar and immediate parts.
+// All cache reads of the register kernels are buffer loads with the cache's
+// size as the bound: rows past the capacity read as 0 instead of faulting, and
+// the per-lane address is one 32-bit offset plus scalar and immediate parts.
+//
+// Kernels (one body, attention_partial_body, behind template switches):
+//   attention_partial_kernel_p   one query row, one workgroup per CU (all registers)
+//   attention_partial_kernel_1   one query row over codes, two workgroups per CU (long 4-bit caches)
+//   attention_partial_kernel_n   2 rows (1 tile), 3-4 rows (2 tiles), 5-8 rows (4 tiles)
+//   attention_partial_kernel_d   one query row over 8-bit codes in large caches: four more waves
+//                                move the codes into LDS (global_load_lds), two teams of four
+//                                computing waves take alternate 64-token iterations
+//   attention_reduce_kernel      the merge of the splits and the gate
+// Which one runs is decided in run_attention from the launch arguments alone, so that the partial
+// and the reduce stage of a step agree on the number of splits.
 #include "common.hpp"
 #include "lanes.hpp"
 
