@@ -279,6 +279,17 @@ int saetta_deltanet_step(saetta_stream_t stream, const float *q, const float *k,
                          float *state, const float *z, const float *norm_w, float *y,
                          saetta_step_params p);
 
+/* saetta_deltanet_conv and saetta_deltanet_step of one token as one call of two
+ * launches (GpuDeltaNet::record, src/gpu_layers.rs:633-684, records the two
+ * kernels one after the other; nothing else reads the conv output): 32 state
+ * rows per workgroup instead of a head, each workgroup computing the conv
+ * outputs it needs, then the gated norm and the shift of x into the conv state.
+ * Arguments as for the two calls; cp.channels = 2 * k_heads * 128 + v_heads * v_dim. */
+int saetta_deltanet_token(saetta_stream_t stream, const float *x, const float *w, float *conv_state,
+                          const float *a, const float *b, const float *a_log, const float *dt_bias,
+                          float *state, const float *z, const float *norm_w, float *y,
+                          saetta_conv_params cp, saetta_step_params sp);
+
 /* ---- Gated DeltaNet, several tokens in order: verify rows and prefill chunks -- */
 
 /* conv over `tokens` tokens: kernels conv_rows2 + conv_state

@@ -429,6 +429,134 @@ __global__ __launch_bounds__(256) void deltanet_gated_norm_rows_kernel(float *y,
     }
 }
 
+
+// ---- one token, conv and step together ---------------------------------------------------------
+//
+// The two kernels above cost a launch each and the step runs on 32 workgroups.  Here a workgroup
+// takes 16 rows of one value head's state (grid 8 x 32 at the model's shape), computes the conv
+// outputs it needs itself (q and k of its key head, v of its rows: the conv state is only read), and
+// leaves what needs the whole head or the whole layer to a small second launch: the gated norm over
+// the head's outputs and the shift of the new input into the conv state.
+constexpr int TOKEN_ROWS = 16;  // state rows per workgroup
+constexpr int TOKEN_SETS = TOKEN_ROWS / 16;
+
+struct TokenArgs {
+    const float *x, *w;
+    float *conv_state;
+    const float *a, *b, *a_log, *dt_bias;
+    float *state;
+    const float *z, *norm_w;
+    float *y;
+    saetta_conv_params cp;
+    saetta_step_params sp;
+};
+
+__global__ __launch_bounds__(256) void deltanet_token_kernel(TokenArgs a) {
+    __shared__ __attribute__((aligned(16))) float qk_lds[2 * K_DIM];  // conv output: q then k, as [half][part][4]
+    __shared__ float v_lds[TOKEN_ROWS];
+    const uint32_t tid = threadIdx.x, part = tid & 15, row_in_set = tid >> 4;
+    const uint32_t h = blockIdx.y, r0 = blockIdx.x * TOKEN_ROWS;
+    const uint32_t v_dim = a.sp.v_dim, kh = h / (a.sp.v_heads / a.sp.k_heads);
+    const uint32_t key_size = a.sp.k_heads * K_DIM, channels = a.cp.channels, past = a.cp.kernel_size - 1;
+
+    // the state rows of this thread (sets of 16 rows), requested before anything else
+    float4 st[TOKEN_SETS][2];
+    float *sp[TOKEN_SETS];
+    bool live[TOKEN_SETS];
+#pragma unroll
+    for (int s = 0; s < TOKEN_SETS; s++) {
+        const uint32_t row = r0 + 16 * s + row_in_set;
+        live[s] = row < v_dim;
+        sp[s] = a.state + (size_t(h) * v_dim + (live[s] ? row : 0)) * K_DIM + part * 8;
+        st[s][0] = live[s] ? reinterpret_cast<const float4 *>(sp[s])[0] : make_float4(0, 0, 0, 0);
+        st[s][1] = live[s] ? reinterpret_cast<const float4 *>(sp[s])[1] : make_float4(0, 0, 0, 0);
+    }
+    // conv_step (src/cpu/deltanet.rs:117-131) of one channel: the stored inputs oldest first, the new one last
+    // (every load of a channel is requested before the first is used: up to 15 stored inputs)
+    auto conv = [&](uint32_t c) {
+        const float *wc = a.w + size_t(c) * a.cp.kernel_size;
+        float ws[15], cs[15];
+#pragma unroll
+        for (uint32_t t = 0; t < 15; t++) {
+            ws[t] = t < past ? wc[t] : 0.0f;
+            cs[t] = t < past ? a.conv_state[size_t(t) * channels + c] : 0.0f;
+        }
+        const float wx = wc[past], xc = a.x[c];
+        float old = 0.0f;
+#pragma unroll
+        for (uint32_t t = 0; t < 15; t++) {
+            if (t < past) old += ws[t] * cs[t];
+        }
+        return silu_f(old + wx * xc);
+    };
+    {
+        // threads 0-127: q channel tid, threads 128-255: k channel tid - 128 of the key head
+        const uint32_t e = tid & 127;
+        const float v = conv((tid < 128 ? 0 : key_size) + kh * K_DIM + e);
+        // element e of a vector belongs to part e / 8, its value e % 8: float4 (e % 8) / 4 of the part
+        qk_lds[(tid < 128 ? 0 : K_DIM) + ((e & 7) >> 2) * 64 + (e >> 3) * 4 + (e & 3)] = v;
+        if (tid < TOKEN_ROWS && r0 + tid < v_dim) v_lds[tid] = conv(2 * key_size + h * v_dim + r0 + tid);
+    }
+    const float xg = a.a[h] + a.dt_bias[h];
+    const float softplus = fmaxf(xg, 0.0f) + log1pf(expf(-fabsf(xg)));
+    const float g = expf(-expf(a.a_log[h]) * softplus);
+    const float beta = sigmoid_f(a.b[h]);
+    __syncthreads();
+    float4 q[2], k[2];
+    q[0] = *reinterpret_cast<const float4 *>(qk_lds + part * 4);
+    q[1] = *reinterpret_cast<const float4 *>(qk_lds + 64 + part * 4);
+    k[0] = *reinterpret_cast<const float4 *>(qk_lds + K_DIM + part * 4);
+    k[1] = *reinterpret_cast<const float4 *>(qk_lds + K_DIM + 64 + part * 4);
+    // normalize_qk (src/cpu/deltanet.rs:133-146)
+    const float qi = (1.0f / sqrtf(float(K_DIM))) / sqrtf(group_reduce<16>(dot4(q[0], q[0]) + dot4(q[1], q[1]), SumOp()) + a.sp.eps);
+    const float ki = 1.0f / sqrtf(group_reduce<16>(dot4(k[0], k[0]) + dot4(k[1], k[1]), SumOp()) + a.sp.eps);
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+        q[c].x *= qi, q[c].y *= qi, q[c].z *= qi, q[c].w *= qi;
+        k[c].x *= ki, k[c].y *= ki, k[c].z *= ki, k[c].w *= ki;
+    }
+#pragma unroll
+    for (int s = 0; s < TOKEN_SETS; s++) {
+        const uint32_t row = r0 + 16 * s + row_in_set;
+#pragma unroll
+        for (int c = 0; c < 2; c++) st[s][c].x *= g, st[s][c].y *= g, st[s][c].z *= g, st[s][c].w *= g;
+        const float mem = group_reduce<16>(dot4(st[s][0], k[0]) + dot4(st[s][1], k[1]), SumOp());
+        const float delta = (v_lds[16 * s + row_in_set] - mem) * beta;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            st[s][c].x += k[c].x * delta, st[s][c].y += k[c].y * delta, st[s][c].z += k[c].z * delta, st[s][c].w += k[c].w * delta;
+        }
+        const float o = group_reduce<16>(dot4(st[s][0], q[0]) + dot4(st[s][1], q[1]), SumOp());
+        if (live[s]) {
+            reinterpret_cast<float4 *>(sp[s])[0] = st[s][0];
+            reinterpret_cast<float4 *>(sp[s])[1] = st[s][1];
+            if (part == 0) a.y[size_t(h) * v_dim + row] = o;  // before the norm
+        }
+    }
+}
+
+// After it: block b < v_heads norms head b (y = o / sqrt(mean(o^2) + eps) * norm_w * silu(z), in
+// place), and every block shifts the new input into its slice of the conv state.
+__global__ __launch_bounds__(256) void deltanet_token_tail_kernel(TokenArgs a) {
+    __shared__ float partial[4];
+    const uint32_t tid = threadIdx.x, b = blockIdx.x;
+    const uint32_t v_dim = a.sp.v_dim, channels = a.cp.channels, past = a.cp.kernel_size - 1;
+    for (uint32_t c = b * 256 + tid; c < channels; c += gridDim.x * 256) {
+        for (uint32_t t = 0; t + 1 < past; t++) a.conv_state[size_t(t) * channels + c] = a.conv_state[size_t(t + 1) * channels + c];
+        a.conv_state[size_t(past - 1) * channels + c] = a.x[c];
+    }
+    if (b < a.sp.v_heads) {
+        const size_t at = size_t(b) * v_dim + tid;
+        const float o = tid < v_dim ? a.y[at] : 0.0f;
+        const float sq = group_reduce<64>(o * o, SumOp());
+        if ((tid & 63) == 0) partial[tid >> 6] = sq;
+        __syncthreads();
+        const float total = partial[0] + partial[1] + partial[2] + partial[3];
+        const float inv = 1.0f / sqrtf(total / float(v_dim) + a.sp.eps);
+        if (tid < v_dim) a.y[at] = o * (inv * a.norm_w[tid]) * silu_f(a.z[at]);
+    }
+}
+
 }  // namespace
 
 int setup_deltanet() { return load_kernel(reinterpret_cast<const void *>(deltanet_step_kernel)); }
@@ -514,4 +642,27 @@ extern "C" int saetta_deltanet_rows(saetta_stream_t stream, const float *mixed, 
     const uint32_t pairs = p.tokens * p.v_heads;
     deltanet_gated_norm_rows_kernel<<<(pairs + 3) / 4, 256, 0, as_stream(stream)>>>(y, z, norm_w, pairs, p.v_dim, p.eps);
     return launch_status("deltanet_rows");
+}
+
+extern "C" int saetta_deltanet_token(saetta_stream_t stream, const float *x, const float *w, float *conv_state,
+                                     const float *a, const float *b, const float *a_log, const float *dt_bias,
+                                     float *state, const float *z, const float *norm_w, float *y,
+                                     saetta_conv_params cp, saetta_step_params sp) {
+    SAETTA_REQUIRE(x && w && conv_state && a && b && a_log && dt_bias && state && z && norm_w && y, SAETTA_E_NULL,
+                   "deltanet_token: null buffer");
+    SAETTA_REQUIRE(cp.kernel_size >= 2 && cp.kernel_size <= 16, SAETTA_E_SHAPE, "deltanet_token: kernel size %u (2..16)",
+                   cp.kernel_size);
+    SAETTA_REQUIRE(sp.k_heads > 0 && sp.v_heads > 0 && sp.v_heads % sp.k_heads == 0, SAETTA_E_SHAPE,
+                   "deltanet_token: %u value heads over %u key heads", sp.v_heads, sp.k_heads);
+    SAETTA_REQUIRE(sp.v_dim >= 1 && sp.v_dim <= 256, SAETTA_E_SHAPE, "deltanet_token: value dim %u (1..256); the key dim is 128",
+                   sp.v_dim);
+    SAETTA_REQUIRE(cp.channels == 2 * sp.k_heads * K_DIM + sp.v_heads * sp.v_dim, SAETTA_E_SHAPE,
+                   "deltanet_token: %u channels, the heads make %u", cp.channels, 2 * sp.k_heads * K_DIM + sp.v_heads * sp.v_dim);
+    SAETTA_REQUIRE(aligned(state, 16), SAETTA_E_ALIGN, "deltanet_token: the state must be 16-byte aligned");
+    if (int rc = ensure_device()) return rc;
+    TokenArgs args{x, w, conv_state, a, b, a_log, dt_bias, state, z, norm_w, y, cp, sp};
+    deltanet_token_kernel<<<dim3((sp.v_dim + TOKEN_ROWS - 1) / TOKEN_ROWS, sp.v_heads), 256, 0, as_stream(stream)>>>(args);
+    const uint32_t blocks = sp.v_heads > 32 ? sp.v_heads : 32;
+    deltanet_token_tail_kernel<<<blocks, 256, 0, as_stream(stream)>>>(args);
+    return launch_status("deltanet_token");
 }

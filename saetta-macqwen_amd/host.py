@@ -350,6 +350,23 @@ def deltanet_step(plan, q, k, v, a, b, a_log, dt_bias, state, z, norm_w, y, k_he
         ffi.lib().saetta_deltanet_step(s, *[_ptr(t) for t in ts], p), "deltanet_step"))
 
 
+def deltanet_token(plan, x, w, conv_state, a, b, a_log, dt_bias, state, z, norm_w, y, k_heads, v_heads, v_dim,
+                   kernel_size, eps):
+    """Records one token of a Gated DeltaNet layer, conv and step (GpuDeltaNet::record,
+    src/gpu_layers.rs:633-684) as one call of two launches: what deltanet_conv + deltanet_step give,
+    without the conv output in between."""
+    ts = (x, w, conv_state, a, b, a_log, dt_bias, state, z, norm_w, y)
+    for t in ts:
+        _need(t, torch.float32, "deltanet_token buffer")
+    channels = 2 * k_heads * 128 + v_heads * v_dim
+    if (x.numel() < channels or w.numel() < channels * kernel_size or conv_state.numel() < (kernel_size - 1) * channels
+            or state.numel() < v_heads * v_dim * 128 or y.numel() < v_heads * v_dim or z.numel() < v_heads * v_dim):
+        raise ValueError("deltanet_token: buffers too small")
+    cp, sp = ffi.ConvParamsC(channels, kernel_size), ffi.StepParamsC(k_heads, v_heads, v_dim, eps)
+    plan.op("deltanet_token", lambda s: ffi.check(
+        ffi.lib().saetta_deltanet_token(s, *[_ptr(t) for t in ts], cp, sp), "deltanet_token"))
+
+
 def deltanet_conv_rows(plan, x, w, state, out, channels, kernel_size, tokens, snaps=None):
     """Records the conv of `tokens` tokens in order (conv_rows2 + conv_state, kernels/prefill.metal:734-786;
     deltanet_conv_rows, kernels/layers.metal:510-544): x, out [tokens][channels]; with `snaps`

@@ -363,6 +363,22 @@ inline void step(plan::Plan &plan, const View &q, const View &k, const View &v, 
     });
 }
 
+// One token, conv and step as one call of two launches with the state rows spread over more
+// workgroups: what conv + step give, without the conv output in between (GpuDeltaNet::record,
+// src/gpu_layers.rs:633-684).
+inline void token(plan::Plan &plan, const View &x, const View &w, const View &conv_state, const View &a, const View &b,
+                  const View &a_log, const View &dt_bias, const View &state, const View &z, const View &norm_w, const View &y,
+                  size_t k_heads, size_t v_heads, size_t v_dim, size_t kernel_size, float eps) {
+    const saetta_conv_params cp{uint32_t(2 * k_heads * 128 + v_heads * v_dim), uint32_t(kernel_size)};
+    const saetta_step_params sp{uint32_t(k_heads), uint32_t(v_heads), uint32_t(v_dim), eps};
+    plan.op("deltanet_token", [=](hipStream_t s) {
+        check(saetta_deltanet_token(s, x.ptr<float>(), w.ptr<float>(), conv_state.ptr<float>(), a.ptr<float>(), b.ptr<float>(),
+                                    a_log.ptr<float>(), dt_bias.ptr<float>(), state.ptr<float>(), z.ptr<float>(),
+                                    norm_w.ptr<float>(), y.ptr<float>(), cp, sp),
+              "deltanet_token");
+    });
+}
+
 // Records the conv of `tokens` tokens in order (conv_rows2 + conv_state, kernels/prefill.metal:734-786;
 // deltanet_conv_rows, kernels/layers.metal:510-544).  x, out [tokens][channels]; with `snaps`
 // ([tokens][kernel_size - 1][channels]) the state after each token goes there too.

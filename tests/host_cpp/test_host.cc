@@ -214,6 +214,27 @@ int main() {
             deltanet::step(one, mt, mt.at(key * 4), mt.at(2 * key * 4), ad.at(t * vh * 4), bd.at(t * vh * 4), al, dt, st1,
                            zd.at(t * val * 4), nw, y1.at(t * val * 4), kh, vh, dv, 1e-6f);
         }
+        {   // deltanet::token == conv then step
+            View conv3(gpu.buffer(conv_n * 4)), st3(gpu.buffer(state_n * 4)), y3(gpu.buffer(m * val * 4));
+            plan::Plan fused(gpu);
+            for (size_t t = 0; t < m; t++) {
+                deltanet::token(fused, xd.at(t * ch * 4), wd, conv3, ad.at(t * vh * 4), bd.at(t * vh * 4), al, dt, st3,
+                                zd.at(t * val * 4), nw, y3.at(t * val * 4), kh, vh, dv, kernel, 1e-6f);
+            }
+            one.build(false).run(gpu);
+            fused.build(true).run(gpu);
+            auto worst3 = [](const std::vector<float> &p, const std::vector<float> &q) {
+                float d = 0;
+                for (size_t i = 0; i < p.size(); i++) d = std::max(d, std::fabs(p[i] - q[i]));
+                return d;
+            };
+            EXPECT(gpu::contents<float>(conv1.buffer, conv_n) == gpu::contents<float>(conv3.buffer, conv_n), "token: conv state");
+            EXPECT(worst3(gpu::contents<float>(y1.buffer, m * val), gpu::contents<float>(y3.buffer, m * val)) < 2e-5f, "token: y");
+            EXPECT(worst3(gpu::contents<float>(st1.buffer, state_n), gpu::contents<float>(st3.buffer, state_n)) < 2e-5f, "token: state");
+            // `one` ran here: start its states again for the comparison below
+            hip_check(hipMemset(conv1.ptr<void>(), 0, conv_n * 4), "memset");
+            hip_check(hipMemset(st1.ptr<void>(), 0, state_n * 4), "memset");
+        }
         deltanet::conv_rows(many, xd, wd, conv2, mixed2, ch, kernel, m, &csn);
         deltanet::rows(many, mixed2, ad, bd, al, dt, st2, zd, nw, y2, kh, vh, dv, m, 1e-6f, &ssn);
         one.build(false).run(gpu);

@@ -72,3 +72,40 @@ def test_conv_kernel_sizes_and_rejections():
         plan.build().run()
     with pytest.raises(ValueError):
         saetta.deltanet_step(saetta.Plan(), z, z, z, z, z, z, z, torch.zeros(10, device="cuda"), z, z, z, 2, 4, 8, 1e-6)
+
+
+@pytest.mark.parametrize("k_heads,v_heads,v_dim,kernel", [(16, 32, 128, 4), (2, 4, 24, 4), (1, 2, 200, 7), (1, 1, 1, 2)])
+def test_token_call_matches_conv_then_step(k_heads, v_heads, v_dim, kernel):
+    # saetta_deltanet_token: the same token step in two launches with the rows spread over more
+    # workgroups; against the oracle over several tokens, states carried on both sides.
+    rng = np.random.default_rng(v_dim + kernel)
+    eps = 1e-6
+    key, val = k_heads * K_DIM, v_heads * v_dim
+    channels = 2 * key + val
+    conv_w = (0.5 * rng.standard_normal((channels, kernel))).astype(np.float32)
+    a_log = rng.uniform(-1, 1, v_heads).astype(np.float32)
+    dt_bias = rng.standard_normal(v_heads).astype(np.float32)
+    norm = (1 + 0.1 * rng.standard_normal(v_dim)).astype(np.float32)
+    conv_cpu = np.zeros((kernel - 1, channels), np.float32)
+    state_cpu = np.zeros(v_heads * v_dim * K_DIM, np.float32)
+    conv_gpu, state_gpu = dev(conv_cpu.copy()), dev(state_cpu.copy())
+    x_d, z_d, y = torch.empty(channels, device="cuda"), torch.empty(val, device="cuda"), torch.empty(val, device="cuda")
+    a_d, b_d = torch.empty(v_heads, device="cuda"), torch.empty(v_heads, device="cuda")
+    plan = saetta.Plan()
+    saetta.deltanet_token(plan, x_d, dev(conv_w), conv_gpu, a_d, b_d, dev(a_log), dev(dt_bias), state_gpu, z_d,
+                          dev(norm), y, k_heads, v_heads, v_dim, kernel, eps)
+    built = plan.build(graph=True)
+    for t in range(5):
+        x = rng.standard_normal(channels).astype(np.float32)
+        z = rng.standard_normal(val).astype(np.float32)
+        a = rng.standard_normal(v_heads).astype(np.float32)
+        b = rng.standard_normal(v_heads).astype(np.float32)
+        for dst, src in ((x_d, x), (z_d, z), (a_d, a), (b_d, b)):
+            dst.copy_(torch.from_numpy(src))
+        built.run()
+        m = oracle.deltanet_conv(conv_w, x, conv_cpu, kernel)
+        want_y = oracle.deltanet_step(m[:key], m[key:2 * key], m[2 * key:], a, b, a_log, dt_bias, state_cpu, z, norm,
+                                      k_heads, v_heads, K_DIM, v_dim, eps)
+        assert np.array_equal(host(conv_gpu).reshape(kernel - 1, channels), conv_cpu), t
+        assert np.abs(host(y) - want_y).max() <= 2e-5 * max(1.0, np.abs(want_y).max()), t
+        assert np.abs(host(state_gpu) - state_cpu).max() <= 2e-5 * max(1.0, np.abs(state_cpu).max()), t
