@@ -346,7 +346,7 @@ def bench_deltanet(s, torch, args, layers=30):
                    "conv_then_step_us": round(both_us, 3), "step_kernel_alone_us": round(step_us, 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "deltanet_token_kernel + deltanet_token_tail_kernel", "avg_us": round(token_us, 3)},
+                     "kernel": "deltanet_rows_small_kernel + deltanet_rows_small_tail_kernel", "avg_us": round(token_us, 3)},
         "cpu_baseline": {"value": round(nbytes / cpu_s / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
                          "sample": f"one layer, conv + step ({cpu_s * 1e3:.2f} ms)"},
         "parity_rel_rms_vs_oracle": float(f"{rel:.3e}"),

@@ -133,6 +133,16 @@ typedef struct saetta_rows_step_params {
     float eps;
     uint32_t snapshots; /* write the state after each token to `snaps` */
 } saetta_rows_step_params;
+/* RowsStepParams (src/gpu_layers.rs:563-571), field for field. */
+typedef struct saetta_rows_fused_params {
+    uint32_t k_heads;
+    uint32_t v_heads;
+    uint32_t v_dim;
+    uint32_t kernel_size;
+    float eps;
+    uint32_t rows;      /* 0..8 */
+    uint32_t snapshots; /* write the states after each row to the snapshot buffers */
+} saetta_rows_fused_params;
 
 /* The three arrays of one quantized cache, keys or values: QuantRows
  * {data, scales, biases} (src/kv_quant.rs:156-180).  Token p's groups start
@@ -316,6 +326,19 @@ int saetta_deltanet_conv_rows(saetta_stream_t stream, const float *x, const floa
 int saetta_deltanet_rows(saetta_stream_t stream, const float *mixed, const float *a, const float *b,
                          const float *a_log, const float *dt_bias, float *state, const float *z,
                          const float *norm_w, float *y, float *snaps, saetta_rows_step_params p);
+
+/* Kernel deltanet_rows (recorded by GpuDeltaNet::record_rows with DN_SIMDS = 0,
+ * src/gpu_layers.rs:737-757): conv and step of up to 8 rows as one op, what
+ * saetta_deltanet_conv_rows + saetta_deltanet_rows give, in two launches
+ * instead of four; the call for the verify step.  x f32 [rows][channels] is the
+ * qkv projection (channels = 2 * k_heads * 128 + v_heads * v_dim); a, b f32
+ * [rows][v_heads]; z, y f32 [rows][v_heads][v_dim]; conv_state, state as above.
+ * With snapshots: conv_snaps f32 [rows][kernel_size - 1][channels], state_snaps
+ * f32 [rows][v_heads][v_dim][128]; else both may be NULL. */
+int saetta_deltanet_rows_fused(saetta_stream_t stream, const float *x, const float *w, float *conv_state,
+                               const float *a, const float *b, const float *a_log, const float *dt_bias,
+                               float *state, const float *z, const float *norm_w, float *y,
+                               float *conv_snaps, float *state_snaps, saetta_rows_fused_params p);
 
 /* ---- prefill attention (src/attention_prefill.rs, src/prefill.rs) ---------- */
 

@@ -1,4 +1,12 @@
-// Gated DeltaNet (linear attention), one token: the conv and the step after it.
+// Gated DeltaNet (linear attention): the conv and the step after it, for one token, for up to 8
+// rows of a verify step, and for the tokens of a prefill chunk in order.
+//
+// Kernels:
+//   deltanet_conv_kernel, deltanet_step_kernel          one token, the reference's two ops
+//   deltanet_conv_rows_kernel, deltanet_conv_state_kernel,
+//   deltanet_rows_kernel, deltanet_gated_norm_rows_kernel   any number of tokens in order (prefill chunks)
+//   deltanet_rows_small_kernel, deltanet_rows_small_tail_kernel
+//                                                       conv and step together for 1..8 tokens
 //
 // Reference: kernels deltanet_conv and deltanet_step (kernels/layers.metal:198-226,290-357),
 // recorded by GpuDeltaNet (src/gpu_layers.rs:573-1000); CPU definition src/cpu/deltanet.rs:69-155:
@@ -430,131 +438,218 @@ __global__ __launch_bounds__(256) void deltanet_gated_norm_rows_kernel(float *y,
 }
 
 
-// ---- one token, conv and step together ---------------------------------------------------------
+// ---- up to 8 tokens, conv and step together (the verify step) -----------------------------------
 //
-// The two kernels above cost a launch each and the step runs on 32 workgroups.  Here a workgroup
-// takes 16 rows of one value head's state (grid 8 x 32 at the model's shape), computes the conv
-// outputs it needs itself (q and k of its key head, v of its rows: the conv state is only read), and
-// leaves what needs the whole head or the whole layer to a small second launch: the gated norm over
-// the head's outputs and the shift of the new input into the conv state.
-constexpr int TOKEN_ROWS = 16;  // state rows per workgroup
-constexpr int TOKEN_SETS = TOKEN_ROWS / 16;
+// Reference: kernel deltanet_rows (kernels/layers.metal, recorded by GpuDeltaNet::record_rows with
+// DN_SIMDS = 0, src/gpu_layers.rs:737-757): conv, q/k norm, gates, delta rule, gated norm for m rows
+// in one op, with the states after every row to the snapshot buffers; with one row, what
+// GpuDeltaNet::record does (src/gpu_layers.rs:633-684).  The separate conv and step kernels above
+// cost a launch each and the step runs on 32 workgroups.  Here a workgroup takes 16 rows of one value
+// head's state (grid 8 x 32 at the model's shape), computes the conv outputs it needs itself for all
+// the tokens (q and k of its key head, v of its rows: the conv state is only read) and walks the
+// tokens; what needs the whole head or the whole layer is a small second launch: the gated norm over
+// a head's outputs, the new conv state and the conv snapshots.
+constexpr int SMALL_ROWS_MAX = 8;
 
-struct TokenArgs {
+struct SmallRowsArgs {
     const float *x, *w;
     float *conv_state;
     const float *a, *b, *a_log, *dt_bias;
     float *state;
     const float *z, *norm_w;
-    float *y;
-    saetta_conv_params cp;
-    saetta_step_params sp;
+    float *y, *conv_snaps, *state_snaps;
+    saetta_rows_fused_params p;
+    uint32_t channels;
 };
 
-__global__ __launch_bounds__(256) void deltanet_token_kernel(TokenArgs a) {
-    __shared__ __attribute__((aligned(16))) float qk_lds[2 * K_DIM];  // conv output: q then k, as [half][part][4]
-    __shared__ float v_lds[TOKEN_ROWS];
-    const uint32_t tid = threadIdx.x, part = tid & 15, row_in_set = tid >> 4;
-    const uint32_t h = blockIdx.y, r0 = blockIdx.x * TOKEN_ROWS;
-    const uint32_t v_dim = a.sp.v_dim, kh = h / (a.sp.v_heads / a.sp.k_heads);
-    const uint32_t key_size = a.sp.k_heads * K_DIM, channels = a.cp.channels, past = a.cp.kernel_size - 1;
-
-    // the state rows of this thread (sets of 16 rows), requested before anything else
-    float4 st[TOKEN_SETS][2];
-    float *sp[TOKEN_SETS];
-    bool live[TOKEN_SETS];
+// out[t] of channel c for t < tokens.  The stored inputs and the new ones are one sequence in
+// registers, the stored ones ending at index 14, x[t] at 15 + t; the taps are right-aligned the same
+// way (the newest at 15), so that out[t] = sum_k taps[k] * seq[t + k] with constant indices: the
+// unused leading taps are zeros, which leaves the sum (oldest first, the new input last, as the
+// single-token kernel adds them) unchanged.  Every load is requested before the first is used.
+template <typename F>
+__device__ __forceinline__ void conv_small(const SmallRowsArgs &a, uint32_t c, F &&emit) {
+    const uint32_t past = a.p.kernel_size - 1, tokens = a.p.rows;
+    const float *wc = a.w + size_t(c) * a.p.kernel_size;
+    float taps[16], seq[15 + SMALL_ROWS_MAX];
 #pragma unroll
-    for (int s = 0; s < TOKEN_SETS; s++) {
-        const uint32_t row = r0 + 16 * s + row_in_set;
-        live[s] = row < v_dim;
-        sp[s] = a.state + (size_t(h) * v_dim + (live[s] ? row : 0)) * K_DIM + part * 8;
-        st[s][0] = live[s] ? reinterpret_cast<const float4 *>(sp[s])[0] : make_float4(0, 0, 0, 0);
-        st[s][1] = live[s] ? reinterpret_cast<const float4 *>(sp[s])[1] : make_float4(0, 0, 0, 0);
-    }
-    // conv_step (src/cpu/deltanet.rs:117-131) of one channel: the stored inputs oldest first, the new one last
-    // (every load of a channel is requested before the first is used: up to 15 stored inputs)
-    auto conv = [&](uint32_t c) {
-        const float *wc = a.w + size_t(c) * a.cp.kernel_size;
-        float ws[15], cs[15];
+    for (uint32_t k = 0; k < 16; k++) taps[k] = k + past >= 15 ? wc[k + past - 15] : 0.0f;
 #pragma unroll
-        for (uint32_t t = 0; t < 15; t++) {
-            ws[t] = t < past ? wc[t] : 0.0f;
-            cs[t] = t < past ? a.conv_state[size_t(t) * channels + c] : 0.0f;
-        }
-        const float wx = wc[past], xc = a.x[c];
-        float old = 0.0f;
+    for (uint32_t k = 0; k < 15; k++) seq[k] = k + past >= 15 ? a.conv_state[size_t(k + past - 15) * a.channels + c] : 0.0f;
 #pragma unroll
-        for (uint32_t t = 0; t < 15; t++) {
-            if (t < past) old += ws[t] * cs[t];
-        }
-        return silu_f(old + wx * xc);
-    };
-    {
-        // threads 0-127: q channel tid, threads 128-255: k channel tid - 128 of the key head
-        const uint32_t e = tid & 127;
-        const float v = conv((tid < 128 ? 0 : key_size) + kh * K_DIM + e);
-        // element e of a vector belongs to part e / 8, its value e % 8: float4 (e % 8) / 4 of the part
-        qk_lds[(tid < 128 ? 0 : K_DIM) + ((e & 7) >> 2) * 64 + (e >> 3) * 4 + (e & 3)] = v;
-        if (tid < TOKEN_ROWS && r0 + tid < v_dim) v_lds[tid] = conv(2 * key_size + h * v_dim + r0 + tid);
-    }
-    const float xg = a.a[h] + a.dt_bias[h];
-    const float softplus = fmaxf(xg, 0.0f) + log1pf(expf(-fabsf(xg)));
-    const float g = expf(-expf(a.a_log[h]) * softplus);
-    const float beta = sigmoid_f(a.b[h]);
-    __syncthreads();
-    float4 q[2], k[2];
-    q[0] = *reinterpret_cast<const float4 *>(qk_lds + part * 4);
-    q[1] = *reinterpret_cast<const float4 *>(qk_lds + 64 + part * 4);
-    k[0] = *reinterpret_cast<const float4 *>(qk_lds + K_DIM + part * 4);
-    k[1] = *reinterpret_cast<const float4 *>(qk_lds + K_DIM + 64 + part * 4);
-    // normalize_qk (src/cpu/deltanet.rs:133-146)
-    const float qi = (1.0f / sqrtf(float(K_DIM))) / sqrtf(group_reduce<16>(dot4(q[0], q[0]) + dot4(q[1], q[1]), SumOp()) + a.sp.eps);
-    const float ki = 1.0f / sqrtf(group_reduce<16>(dot4(k[0], k[0]) + dot4(k[1], k[1]), SumOp()) + a.sp.eps);
+    for (uint32_t t = 0; t < SMALL_ROWS_MAX; t++) seq[15 + t] = t < tokens ? a.x[size_t(t) * a.channels + c] : 0.0f;
 #pragma unroll
-    for (int c = 0; c < 2; c++) {
-        q[c].x *= qi, q[c].y *= qi, q[c].z *= qi, q[c].w *= qi;
-        k[c].x *= ki, k[c].y *= ki, k[c].z *= ki, k[c].w *= ki;
-    }
+    for (uint32_t t = 0; t < SMALL_ROWS_MAX; t++) {
+        if (t < tokens) {
+            float acc = 0.0f;
 #pragma unroll
-    for (int s = 0; s < TOKEN_SETS; s++) {
-        const uint32_t row = r0 + 16 * s + row_in_set;
-#pragma unroll
-        for (int c = 0; c < 2; c++) st[s][c].x *= g, st[s][c].y *= g, st[s][c].z *= g, st[s][c].w *= g;
-        const float mem = group_reduce<16>(dot4(st[s][0], k[0]) + dot4(st[s][1], k[1]), SumOp());
-        const float delta = (v_lds[16 * s + row_in_set] - mem) * beta;
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
-            st[s][c].x += k[c].x * delta, st[s][c].y += k[c].y * delta, st[s][c].z += k[c].z * delta, st[s][c].w += k[c].w * delta;
-        }
-        const float o = group_reduce<16>(dot4(st[s][0], q[0]) + dot4(st[s][1], q[1]), SumOp());
-        if (live[s]) {
-            reinterpret_cast<float4 *>(sp[s])[0] = st[s][0];
-            reinterpret_cast<float4 *>(sp[s])[1] = st[s][1];
-            if (part == 0) a.y[size_t(h) * v_dim + row] = o;  // before the norm
+            for (uint32_t k = 0; k < 15; k++) acc += taps[k] * seq[t + k];
+            emit(t, silu_f(acc + taps[15] * seq[t + 15]));
         }
     }
 }
 
-// After it: block b < v_heads norms head b (y = o / sqrt(mean(o^2) + eps) * norm_w * silu(z), in
-// place), and every block shifts the new input into its slice of the conv state.
-__global__ __launch_bounds__(256) void deltanet_token_tail_kernel(TokenArgs a) {
-    __shared__ float partial[4];
-    const uint32_t tid = threadIdx.x, b = blockIdx.x;
-    const uint32_t v_dim = a.sp.v_dim, channels = a.cp.channels, past = a.cp.kernel_size - 1;
-    for (uint32_t c = b * 256 + tid; c < channels; c += gridDim.x * 256) {
-        for (uint32_t t = 0; t + 1 < past; t++) a.conv_state[size_t(t) * channels + c] = a.conv_state[size_t(t + 1) * channels + c];
-        a.conv_state[size_t(past - 1) * channels + c] = a.x[c];
+// Waves 0-3 hold the 16 state rows (16 lanes a row) and compute the conv of the key head's q and k
+// channels; wave 4 computes the conv of the 16 value channels and wave 5 the gates, so that no wave
+// waits for memory twice before the first barrier.  Then the q/k norms of every token at once (one
+// group of 16 lanes per token and vector), and the tokens in order with the next token's operands
+// fetched from LDS while the current one's chain of sums runs.
+constexpr int SMALL_THREADS = 384;
+
+template <bool SNAPS>
+__global__ __launch_bounds__(SMALL_THREADS) void deltanet_rows_small_kernel(SmallRowsArgs a) {
+    __shared__ __attribute__((aligned(16))) float qk_lds[SMALL_ROWS_MAX][2 * K_DIM];  // per token: q then k, as [half][part][4]
+    __shared__ float v_lds[SMALL_ROWS_MAX][16];
+    __shared__ float gb_lds[SMALL_ROWS_MAX][2];   // decay, beta
+    __shared__ float inv_lds[SMALL_ROWS_MAX][2];  // what q and k are multiplied by
+    const uint32_t tid = threadIdx.x, part = tid & 15, row_in_wg = (tid >> 4) & 15;
+    const uint32_t h = blockIdx.y, r0 = blockIdx.x * 16, row = r0 + row_in_wg;
+    const uint32_t v_dim = a.p.v_dim, v_heads = a.p.v_heads, tokens = a.p.rows;
+    const uint32_t kh = h / (v_heads / a.p.k_heads), key_size = a.p.k_heads * K_DIM;
+    const bool live = tid < 256 && row < v_dim;
+    float *sp = a.state + (size_t(h) * v_dim + (live ? row : 0)) * K_DIM + part * 8;
+    float4 st[2];
+    st[0] = live ? reinterpret_cast<const float4 *>(sp)[0] : make_float4(0, 0, 0, 0);
+    st[1] = live ? reinterpret_cast<const float4 *>(sp)[1] : make_float4(0, 0, 0, 0);
+    if (tid < 256) {
+        const uint32_t e = tid & 127;
+        const uint32_t slot = (tid < 128 ? 0 : K_DIM) + ((e & 7) >> 2) * 64 + (e >> 3) * 4 + (e & 3);
+        conv_small(a, (tid < 128 ? 0 : key_size) + kh * K_DIM + e, [&](uint32_t t, float v) { qk_lds[t][slot] = v; });
+    } else if (tid < 320) {
+        const uint32_t i = tid - 256;
+        if (i < 16 && r0 + i < v_dim) {
+            conv_small(a, 2 * key_size + h * v_dim + r0 + i, [&](uint32_t t, float v) { v_lds[t][i] = v; });
+        }
+    } else {
+        const uint32_t t = tid - 320;
+        if (t < tokens) {
+            const float xg = a.a[size_t(t) * v_heads + h] + a.dt_bias[h];
+            const float softplus = fmaxf(xg, 0.0f) + log1pf(expf(-fabsf(xg)));
+            gb_lds[t][0] = expf(-expf(a.a_log[h]) * softplus);
+            gb_lds[t][1] = sigmoid_f(a.b[size_t(t) * v_heads + h]);
+        }
     }
-    if (b < a.sp.v_heads) {
-        const size_t at = size_t(b) * v_dim + tid;
-        const float o = tid < v_dim ? a.y[at] : 0.0f;
-        const float sq = group_reduce<64>(o * o, SumOp());
-        if ((tid & 63) == 0) partial[tid >> 6] = sq;
-        __syncthreads();
-        const float total = partial[0] + partial[1] + partial[2] + partial[3];
-        const float inv = 1.0f / sqrtf(total / float(v_dim) + a.sp.eps);
-        if (tid < v_dim) a.y[at] = o * (inv * a.norm_w[tid]) * silu_f(a.z[at]);
+    __syncthreads();
+    if (tid < 256) {
+        // normalize_qk (src/cpu/deltanet.rs:133-146): group (tid / 16) takes token (group % 8), q or k
+        const uint32_t t = row_in_wg & 7, which = row_in_wg >> 3;
+        if (t < tokens) {
+            const float4 lo = *reinterpret_cast<const float4 *>(qk_lds[t] + which * K_DIM + part * 4);
+            const float4 hi = *reinterpret_cast<const float4 *>(qk_lds[t] + which * K_DIM + 64 + part * 4);
+            const float sum = group_reduce<16>(dot4(lo, lo) + dot4(hi, hi), SumOp());
+            const float scale = which == 0 ? 1.0f / sqrtf(float(K_DIM)) : 1.0f;
+            if (part == 0) inv_lds[t][which] = scale / sqrtf(sum + a.p.eps);
+        }
     }
+    __syncthreads();
+    if (tid >= 256) return;
+    const size_t value_size = size_t(v_heads) * v_dim;
+    float4 qn[2], kn[2];
+    float gn, bn, vn, qin, kin;
+    auto fetch = [&](uint32_t t) {
+        qn[0] = *reinterpret_cast<const float4 *>(qk_lds[t] + part * 4);
+        qn[1] = *reinterpret_cast<const float4 *>(qk_lds[t] + 64 + part * 4);
+        kn[0] = *reinterpret_cast<const float4 *>(qk_lds[t] + K_DIM + part * 4);
+        kn[1] = *reinterpret_cast<const float4 *>(qk_lds[t] + K_DIM + 64 + part * 4);
+        gn = gb_lds[t][0], bn = gb_lds[t][1], vn = v_lds[t][row_in_wg];
+        qin = inv_lds[t][0], kin = inv_lds[t][1];
+    };
+    fetch(0);
+    for (uint32_t t = 0; t < tokens; t++) {
+        float4 q[2], k[2];
+        const float g = gn, beta = bn, v = vn, qi = qin, ki = kin;
+#pragma unroll
+        for (int c = 0; c < 2; c++) q[c] = qn[c], k[c] = kn[c];
+        if (t + 1 < tokens) fetch(t + 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            q[c].x *= qi, q[c].y *= qi, q[c].z *= qi, q[c].w *= qi;
+            k[c].x *= ki, k[c].y *= ki, k[c].z *= ki, k[c].w *= ki;
+            st[c].x *= g, st[c].y *= g, st[c].z *= g, st[c].w *= g;
+        }
+        const float mem = group_reduce<16>(dot4(st[0], k[0]) + dot4(st[1], k[1]), SumOp());
+        const float delta = (v - mem) * beta;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            st[c].x += k[c].x * delta, st[c].y += k[c].y * delta, st[c].z += k[c].z * delta, st[c].w += k[c].w * delta;
+        }
+        const float o = group_reduce<16>(dot4(st[0], q[0]) + dot4(st[1], q[1]), SumOp());
+        if (live) {
+            if (part == 0) a.y[size_t(t) * value_size + size_t(h) * v_dim + row] = o;  // before the norm
+            if constexpr (SNAPS) {
+                float *snap = a.state_snaps + size_t(t) * v_heads * v_dim * K_DIM + (size_t(h) * v_dim + row) * K_DIM + part * 8;
+                reinterpret_cast<float4 *>(snap)[0] = st[0];
+                reinterpret_cast<float4 *>(snap)[1] = st[1];
+            }
+        }
+    }
+    if (live) reinterpret_cast<float4 *>(sp)[0] = st[0], reinterpret_cast<float4 *>(sp)[1] = st[1];
+}
+
+// After it.  Block b owns 16 channels of the conv: entry j of the conv state after token t is place
+// t + 1 + j of (stored inputs, new inputs); the snapshots are written first, then, past a barrier
+// (the entries are moved in place), the state after the last token.  The first blocks also norm the
+// (token, head) pairs, one wave each, in place on y.
+constexpr int TAIL_CHANNELS = 16;
+
+__global__ __launch_bounds__(256) void deltanet_rows_small_tail_kernel(SmallRowsArgs a) {
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t v_dim = a.p.v_dim, tokens = a.p.rows, past = a.p.kernel_size - 1, channels = a.channels;
+    const uint32_t pair = blockIdx.x * 4 + (tid >> 6), pairs = tokens * a.p.v_heads;
+    const bool has_pair = pair < pairs;
+    float o[4];
+    if (has_pair) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t d = lane + 64 * i;
+            o[i] = d < v_dim ? a.y[size_t(pair) * v_dim + d] : 0.0f;
+        }
+    }
+    const uint32_t c = blockIdx.x * TAIL_CHANNELS + (tid & 15);
+    const float *stored = a.conv_state, *fresh = a.x;
+    auto place = [&](uint32_t at) {  // `at` in (stored inputs, new inputs)
+        return at < past ? stored[size_t(at) * channels + c] : fresh[size_t(at - past) * channels + c];
+    };
+    if (c < channels) {
+        if (a.p.snapshots) {
+            float *__restrict__ snaps = a.conv_snaps;
+#pragma unroll 2
+            for (uint32_t e = tid >> 4; e < tokens * past; e += 16) {  // e = t * past + j
+                snaps[size_t(e) * channels + c] = place(e / past + 1 + e % past);
+            }
+        }
+    }
+    const uint32_t j = tid >> 4;  // past <= 15 < 16 entries a block can move at once
+    const bool moves = c < channels && j < past;
+    const float moved = moves ? place(tokens + j) : 0.0f;
+    __syncthreads();
+    if (moves) a.conv_state[size_t(j) * channels + c] = moved;
+    if (has_pair) {
+        float *yp = a.y + size_t(pair) * v_dim;
+        const float *zp = a.z + size_t(pair) * v_dim;
+        float total = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) total += group_reduce<64>(o[i] * o[i], SumOp());
+        const float inv = 1.0f / sqrtf(total / float(v_dim) + a.p.eps);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t d = lane + 64 * i;
+            if (d < v_dim) yp[d] = o[i] * (inv * a.norm_w[d]) * silu_f(zp[d]);
+        }
+    }
+}
+
+void launch_small_rows(const SmallRowsArgs &args, hipStream_t stream) {
+    const saetta_rows_fused_params &p = args.p;
+    const dim3 grid((p.v_dim + 15) / 16, p.v_heads);
+    if (p.snapshots) {
+        deltanet_rows_small_kernel<true><<<grid, SMALL_THREADS, 0, stream>>>(args);
+    } else {
+        deltanet_rows_small_kernel<false><<<grid, SMALL_THREADS, 0, stream>>>(args);
+    }
+    const uint32_t pair_blocks = (p.rows * p.v_heads + 3) / 4, chan_blocks = (args.channels + TAIL_CHANNELS - 1) / TAIL_CHANNELS;
+    deltanet_rows_small_tail_kernel<<<pair_blocks > chan_blocks ? pair_blocks : chan_blocks, 256, 0, stream>>>(args);
 }
 
 }  // namespace
@@ -660,9 +755,33 @@ extern "C" int saetta_deltanet_token(saetta_stream_t stream, const float *x, con
                    "deltanet_token: %u channels, the heads make %u", cp.channels, 2 * sp.k_heads * K_DIM + sp.v_heads * sp.v_dim);
     SAETTA_REQUIRE(aligned(state, 16), SAETTA_E_ALIGN, "deltanet_token: the state must be 16-byte aligned");
     if (int rc = ensure_device()) return rc;
-    TokenArgs args{x, w, conv_state, a, b, a_log, dt_bias, state, z, norm_w, y, cp, sp};
-    deltanet_token_kernel<<<dim3((sp.v_dim + TOKEN_ROWS - 1) / TOKEN_ROWS, sp.v_heads), 256, 0, as_stream(stream)>>>(args);
-    const uint32_t blocks = sp.v_heads > 32 ? sp.v_heads : 32;
-    deltanet_token_tail_kernel<<<blocks, 256, 0, as_stream(stream)>>>(args);
+    const saetta_rows_fused_params p{sp.k_heads, sp.v_heads, sp.v_dim, cp.kernel_size, sp.eps, 1, 0};
+    SmallRowsArgs args{x, w, conv_state, a, b, a_log, dt_bias, state, z, norm_w, y, nullptr, nullptr, p, cp.channels};
+    launch_small_rows(args, as_stream(stream));
     return launch_status("deltanet_token");
+}
+
+extern "C" int saetta_deltanet_rows_fused(saetta_stream_t stream, const float *x, const float *w, float *conv_state,
+                                          const float *a, const float *b, const float *a_log, const float *dt_bias,
+                                          float *state, const float *z, const float *norm_w, float *y,
+                                          float *conv_snaps, float *state_snaps, saetta_rows_fused_params p) {
+    SAETTA_REQUIRE(x && w && conv_state && a && b && a_log && dt_bias && state && z && norm_w && y, SAETTA_E_NULL,
+                   "deltanet_rows_fused: null buffer");
+    SAETTA_REQUIRE(!p.snapshots || (conv_snaps && state_snaps), SAETTA_E_NULL,
+                   "deltanet_rows_fused: snapshots asked for, no buffers");
+    SAETTA_REQUIRE(p.rows <= SMALL_ROWS_MAX, SAETTA_E_SHAPE, "deltanet_rows_fused: %u rows (up to 8)", p.rows);
+    SAETTA_REQUIRE(p.kernel_size >= 2 && p.kernel_size <= 16, SAETTA_E_SHAPE,
+                   "deltanet_rows_fused: kernel size %u (2..16)", p.kernel_size);
+    SAETTA_REQUIRE(p.k_heads > 0 && p.v_heads > 0 && p.v_heads % p.k_heads == 0, SAETTA_E_SHAPE,
+                   "deltanet_rows_fused: %u value heads over %u key heads", p.v_heads, p.k_heads);
+    SAETTA_REQUIRE(p.v_dim >= 1 && p.v_dim <= 256, SAETTA_E_SHAPE,
+                   "deltanet_rows_fused: value dim %u (1..256); the key dim is 128", p.v_dim);
+    SAETTA_REQUIRE(aligned(state, 16) && (!p.snapshots || aligned(state_snaps, 16)), SAETTA_E_ALIGN,
+                   "deltanet_rows_fused: the state and its snapshots must be 16-byte aligned");
+    if (int rc = ensure_device()) return rc;
+    if (p.rows == 0) return SAETTA_OK;
+    const uint32_t channels = 2 * p.k_heads * K_DIM + p.v_heads * p.v_dim;
+    SmallRowsArgs args{x, w, conv_state, a, b, a_log, dt_bias, state, z, norm_w, y, conv_snaps, state_snaps, p, channels};
+    launch_small_rows(args, as_stream(stream));
+    return launch_status("deltanet_rows_fused");
 }

@@ -7,7 +7,7 @@ LIB_PATH = os.environ.get("SAETTA_HIP_LIB") or os.path.join(_HERE, "lib", "libsa
 
 # Every symbol include/saetta_hip.h declares; tests check the library exports each.
 SYMBOLS = [
-    "saetta_init", "saetta_last_error", "saetta_kv_quantize", "saetta_kv_dequantize", "saetta_kv_dequantize_f32", "saetta_to_half", "saetta_attn_prep_store", "saetta_deltanet_conv", "saetta_deltanet_step", "saetta_deltanet_conv_rows", "saetta_deltanet_rows", "saetta_deltanet_token",
+    "saetta_init", "saetta_last_error", "saetta_kv_quantize", "saetta_kv_dequantize", "saetta_kv_dequantize_f32", "saetta_to_half", "saetta_attn_prep_store", "saetta_deltanet_conv", "saetta_deltanet_step", "saetta_deltanet_conv_rows", "saetta_deltanet_rows", "saetta_deltanet_token", "saetta_deltanet_rows_fused",
     "saetta_part_o_bytes", "saetta_part_ml_bytes", "saetta_attn_decode", "saetta_attn_decode_quant",
     "saetta_attn_rows", "saetta_attn_rows_quant", "saetta_prefill_workspace_bytes", "saetta_attn_prefill", "saetta_attn_prefill_quant",
 ]
@@ -73,6 +73,8 @@ def lib():
         l.saetta_deltanet_step.argtypes = [vp] * 12 + [StepParamsC]
         l.saetta_deltanet_token.restype = i32
         l.saetta_deltanet_token.argtypes = [vp] * 12 + [ConvParamsC, StepParamsC]
+        l.saetta_deltanet_rows_fused.restype = i32
+        l.saetta_deltanet_rows_fused.argtypes = [vp] * 14 + [RowsFusedParamsC]
         l.saetta_deltanet_conv_rows.restype = i32
         l.saetta_deltanet_conv_rows.argtypes = [vp] * 6 + [ConvRowsParamsC]
         l.saetta_deltanet_rows.restype = i32
@@ -125,6 +127,12 @@ class ConvRowsParamsC(ctypes.Structure):
 class RowsStepParamsC(ctypes.Structure):
     _fields_ = [("k_heads", ctypes.c_uint32), ("v_heads", ctypes.c_uint32), ("v_dim", ctypes.c_uint32),
                 ("tokens", ctypes.c_uint32), ("eps", ctypes.c_float), ("snapshots", ctypes.c_uint32)]
+
+
+class RowsFusedParamsC(ctypes.Structure):
+    _fields_ = [("k_heads", ctypes.c_uint32), ("v_heads", ctypes.c_uint32), ("v_dim", ctypes.c_uint32),
+                ("kernel_size", ctypes.c_uint32), ("eps", ctypes.c_float), ("rows", ctypes.c_uint32),
+                ("snapshots", ctypes.c_uint32)]
 
 
 def check(rc, what):

@@ -410,6 +410,38 @@ def deltanet_rows(plan, mixed, a, b, a_log, dt_bias, state, z, norm_w, y, k_head
         "deltanet_rows"))
 
 
+def deltanet_rows_fused(plan, x, w, conv_state, a, b, a_log, dt_bias, state, z, norm_w, y, k_heads, v_heads, v_dim,
+                        kernel_size, rows, eps, conv_snaps=None, state_snaps=None):
+    """Records up to 8 rows of a Gated DeltaNet layer, conv and step, as one call of two launches
+    (kernel deltanet_rows, GpuDeltaNet::record_rows with DN_SIMDS = 0, src/gpu_layers.rs:737-757):
+    x, z [rows][...] as for deltanet_conv_rows + deltanet_rows, which this equals; with the two
+    snapshot buffers the conv and delta states after each row go there too."""
+    ts = (x, w, conv_state, a, b, a_log, dt_bias, state, z, norm_w, y)
+    for t in ts:
+        _need(t, torch.float32, "deltanet_rows_fused buffer")
+    if rows > MAX_ROWS:
+        raise ValueError(f"deltanet_rows_fused: {rows} rows (up to {MAX_ROWS})")
+    if (conv_snaps is None) != (state_snaps is None):
+        raise ValueError("deltanet_rows_fused: both snapshot buffers or neither")
+    channels = 2 * k_heads * 128 + v_heads * v_dim
+    if (x.numel() < rows * channels or w.numel() < channels * kernel_size
+            or conv_state.numel() < (kernel_size - 1) * channels or state.numel() < v_heads * v_dim * 128
+            or y.numel() < rows * v_heads * v_dim or z.numel() < rows * v_heads * v_dim
+            or a.numel() < rows * v_heads or b.numel() < rows * v_heads):
+        raise ValueError("deltanet_rows_fused: buffers too small")
+    if conv_snaps is not None:
+        _need(conv_snaps, torch.float32, "conv_snaps")
+        _need(state_snaps, torch.float32, "state_snaps")
+        if conv_snaps.numel() < rows * (kernel_size - 1) * channels or state_snaps.numel() < rows * v_heads * v_dim * 128:
+            raise ValueError("deltanet_rows_fused: snapshots too small")
+    p = ffi.RowsFusedParamsC(k_heads, v_heads, v_dim, kernel_size, eps, rows, int(conv_snaps is not None))
+    plan.op("deltanet_rows_fused", lambda s: ffi.check(
+        ffi.lib().saetta_deltanet_rows_fused(s, *[_ptr(t) for t in ts],
+                                             _ptr(conv_snaps) if conv_snaps is not None else None,
+                                             _ptr(state_snaps) if state_snaps is not None else None, p),
+        "deltanet_rows_fused"))
+
+
 KV_ALIGN = 128  # src/gpu_layers.rs:199: the decode chunk, and a multiple of the prefill key block
 
 

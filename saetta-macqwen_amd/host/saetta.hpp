@@ -379,6 +379,27 @@ inline void token(plan::Plan &plan, const View &x, const View &w, const View &co
     });
 }
 
+// Up to 8 rows, conv and step as one call of two launches (kernel deltanet_rows, GpuDeltaNet::record_rows
+// with DN_SIMDS = 0, src/gpu_layers.rs:737-757): what conv_rows + rows give.  With the two snapshot
+// buffers the conv and delta states after each row go there too.
+inline void rows_fused(plan::Plan &plan, const View &x, const View &w, const View &conv_state, const View &a, const View &b,
+                       const View &a_log, const View &dt_bias, const View &state, const View &z, const View &norm_w,
+                       const View &y, size_t k_heads, size_t v_heads, size_t v_dim, size_t kernel_size, size_t rows, float eps,
+                       const View *conv_snaps = nullptr, const View *state_snaps = nullptr) {
+    if ((conv_snaps == nullptr) != (state_snaps == nullptr)) throw std::runtime_error("deltanet_rows_fused: both snapshot buffers or neither");
+    const bool has = conv_snaps != nullptr;
+    const saetta_rows_fused_params p{uint32_t(k_heads), uint32_t(v_heads), uint32_t(v_dim), uint32_t(kernel_size), eps,
+                                     uint32_t(rows), has ? 1u : 0u};
+    const View cs = has ? *conv_snaps : View{}, ss = has ? *state_snaps : View{};
+    plan.op("deltanet_rows_fused", [=](hipStream_t s) {
+        check(saetta_deltanet_rows_fused(s, x.ptr<float>(), w.ptr<float>(), conv_state.ptr<float>(), a.ptr<float>(),
+                                         b.ptr<float>(), a_log.ptr<float>(), dt_bias.ptr<float>(), state.ptr<float>(),
+                                         z.ptr<float>(), norm_w.ptr<float>(), y.ptr<float>(), has ? cs.ptr<float>() : nullptr,
+                                         has ? ss.ptr<float>() : nullptr, p),
+              "deltanet_rows_fused");
+    });
+}
+
 // Records the conv of `tokens` tokens in order (conv_rows2 + conv_state, kernels/prefill.metal:734-786;
 // deltanet_conv_rows, kernels/layers.metal:510-544).  x, out [tokens][channels]; with `snaps`
 // ([tokens][kernel_size - 1][channels]) the state after each token goes there too.

@@ -250,6 +250,20 @@ int main() {
         EXPECT(worst(gpu::contents<float>(st1.buffer, state_n), gpu::contents<float>(st2.buffer, state_n)) < 2e-5f, "rows state");
         EXPECT(gpu::contents<float>(ssn.buffer, state_n, (m - 1) * state_n * 4) == gpu::contents<float>(st2.buffer, state_n),
                "last snapshot is the state");
+        if (m <= 8) {   // deltanet::rows_fused == conv_rows + rows, snapshots included
+            View conv4(gpu.buffer(conv_n * 4)), st4(gpu.buffer(state_n * 4)), y4(gpu.buffer(m * val * 4));
+            View csn4(gpu.buffer(m * conv_n * 4)), ssn4(gpu.buffer(m * state_n * 4));
+            plan::Plan both(gpu);
+            deltanet::rows_fused(both, xd, wd, conv4, ad, bd, al, dt, st4, zd, nw, y4, kh, vh, dv, kernel, m, 1e-6f, &csn4, &ssn4);
+            both.build(true).run(gpu);
+            EXPECT(gpu::contents<float>(conv2.buffer, conv_n) == gpu::contents<float>(conv4.buffer, conv_n), "rows_fused: conv state");
+            EXPECT(gpu::contents<float>(csn.buffer, m * conv_n) == gpu::contents<float>(csn4.buffer, m * conv_n), "rows_fused: conv snapshots");
+            EXPECT(worst(gpu::contents<float>(y2.buffer, m * val), gpu::contents<float>(y4.buffer, m * val)) < 2e-5f, "rows_fused: y");
+            EXPECT(worst(gpu::contents<float>(ssn.buffer, m * state_n), gpu::contents<float>(ssn4.buffer, m * state_n)) < 2e-5f,
+                   "rows_fused: state snapshots");
+            EXPECT(gpu::contents<float>(ssn4.buffer, state_n, (m - 1) * state_n * 4) == gpu::contents<float>(st4.buffer, state_n),
+                   "rows_fused: last snapshot is the state");
+        }
         // accept two rows: restore the state after row 1, then rows 2.. again give the same end state
         plan::Plan again(gpu);
         deltanet::restore(again, csn, ssn, 1, conv2, st2, conv_n, state_n);
