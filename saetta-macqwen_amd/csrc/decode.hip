@@ -49,7 +49,7 @@
 //   attention_partial_kernel_p   one query row, one workgroup per CU (all registers)
 //   attention_partial_kernel_1   one query row over codes, two workgroups per CU (long 4-bit caches)
 //   attention_partial_kernel_n   2 rows (1 tile), 3-4 rows (2 tiles), 5-8 rows (4 tiles)
-//   attention_partial_kernel_d   one query row over 8-bit codes in large caches: four more waves
+//   attention_partial_kernel_d   one query row over codes in large caches: four more waves
 //                                move the codes into LDS (global_load_lds), two teams of four
 //                                computing waves take alternate 64-token iterations
 //   attention_reduce_kernel      the merge of the splits and the gate
@@ -276,14 +276,19 @@ struct Shape {
     static constexpr int QZ_OFF = ALPHA_OFF + S_ROWS * 4;                   // [tile][hi, lo][lane] half8
     static constexpr int ZSUM_OFF = QZ_OFF + TILES * 2 * 64 * 16;           // [wave][S_ROWS] f32
     static constexpr int LDS_BYTES = ZSUM_OFF + 4 * S_ROWS * 4;
-    // With loader waves (8-bit codes only): four slots of one iteration's key and value codes each.
-    // Keys: per block [16 pieces of 16 bytes][16 tokens]; values: token rows of 256 bytes in groups
-    // of four, the groups 32 bytes apart so that the four lane groups of a value read hit
-    // different banks.
+    // With loader waves (codes only): four slots of one iteration's key and value codes each.  A
+    // load instruction brings 64 pieces of 16 bytes; a (token, kv head) row is PIECES of them.
+    // Keys: per block [piece][16 tokens]; values: whole token rows, as many as one instruction
+    // brings (four of 256 bytes, eight of 128), these groups 32 bytes apart so that the four lane
+    // groups of a value read hit different banks.
+    static constexpr int PIECES = row_bytes<BITS>() / 16;
+    static constexpr int DMA_PER_BLOCK = PIECES / 4;   // load instructions per block of keys, and of values
+    static constexpr int V_GROUP_TOKENS = 64 / PIECES;
     static constexpr int DMA_SLOTS = 16 / ITB;  // 256 tokens of codes in LDS
-    static constexpr int K_SLOT_BYTES = ITB * 4096;
-    static constexpr int V_GROUP_BYTES = 4 * 256 + 32;
-    static constexpr int V_SLOT_BYTES = ITB * 4 * V_GROUP_BYTES;
+    static constexpr int K_BLOCK_BYTES = BLOCK * row_bytes<BITS>();
+    static constexpr int K_SLOT_BYTES = ITB * K_BLOCK_BYTES;
+    static constexpr int V_GROUP_BYTES = 1024 + 32;
+    static constexpr int V_SLOT_BYTES = ITB * DMA_PER_BLOCK * V_GROUP_BYTES;
     // The teams share the query operands (the first array and qz); a further team's other arrays
     // start where the first team's end, its own (unused) query area lying over them.
     static constexpr int TEAM_SHIFT = LDS_BYTES - Q_BYTES;
@@ -303,7 +308,7 @@ struct Shape {
 template <int BITS, int TILES, bool PACKED, int ITB, bool UNCOND, bool DMA = false, int TEAMS = 1>
 __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     static_assert(TEAMS == 1 || (DMA && TEAMS == 2), "teams need the loader waves");
-    static_assert(!DMA || (BITS == 8 && PACKED && (ITB == 4 || ITB == 8)), "loader waves: one row over 8-bit codes, 64- or 128-token iterations");
+    static_assert(!DMA || (BITS != 16 && PACKED && (ITB == 4 || ITB == 8)), "loader waves: one row over codes, 64- or 128-token iterations");
     using Sh = Shape<BITS, TILES, PACKED, ITB>;
     constexpr int IT_BLOCKS = ITB, IT_TOKENS = Sh::IT_TOKENS, SC_STRIDE = Sh::SC_STRIDE;
     constexpr int KROUNDS = ITB / 4, KSTEPS = ITB / 2;
@@ -404,7 +409,8 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
                              : "memory", "m0");
             };
             const uint32_t last_row = a.capacity - 1;  // (global loads are not bounds checked)
-            constexpr int PER_REQUEST = 8 * KROUNDS;  // loads of one iteration, per loader wave
+            constexpr int PER_BLOCK = Sh::DMA_PER_BLOCK;
+            constexpr int PER_REQUEST = 2 * PER_BLOCK * KROUNDS;  // loads of one iteration, per loader wave
             auto request = [&](uint32_t it) {
                 const uint32_t slot = it % Sh::DMA_SLOTS;
                 // keys of every round first: phase A needs them first
@@ -415,19 +421,19 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
                     const uint32_t ktok = min(base + (lane & 15), last_row);
                     const uint32_t kvoff = (ktok * kvh + kv) * RB + (lane >> 4) * 16;
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        dma(lds0 + K_OFF + slot * Sh::K_SLOT_BYTES + blk * 4096 + i * 1024, kvoff + 64 * i, a.kdata);
+                    for (int i = 0; i < PER_BLOCK; i++) {
+                        dma(lds0 + K_OFF + slot * Sh::K_SLOT_BYTES + blk * Sh::K_BLOCK_BYTES + i * 1024, kvoff + 64 * i, a.kdata);
                     }
                 }
 #pragma unroll
                 for (int r = 0; r < KROUNDS; r++) {
                     const uint32_t blk = L + 4 * r, base = (blk_begin + it * per_it + blk) * BLOCK;
-                    // lane -> (token lane / 16 of the instruction's four, piece lane % 16)
+                    // lane -> (token lane / PIECES of the instruction's group, piece lane % PIECES)
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const uint32_t vtok = min(base + 4 * i + (lane >> 4), last_row);
-                        dma(lds0 + V_OFF + slot * Sh::V_SLOT_BYTES + (4 * blk + i) * Sh::V_GROUP_BYTES,
-                            (vtok * kvh + kv) * RB + (lane & 15) * 16, a.vdata);
+                    for (int i = 0; i < PER_BLOCK; i++) {
+                        const uint32_t vtok = min(base + Sh::V_GROUP_TOKENS * i + lane / Sh::PIECES, last_row);
+                        dma(lds0 + V_OFF + slot * Sh::V_SLOT_BYTES + (PER_BLOCK * blk + i) * Sh::V_GROUP_BYTES,
+                            (vtok * kvh + kv) * RB + (lane % Sh::PIECES) * 16, a.vdata);
                     }
                 }
             };
@@ -636,13 +642,20 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
         }
         if constexpr (DMA) {
             // this wave's block: the lane's piece j of each group, its token n
-            const unsigned char *kb = lds_raw + K_OFF + (it % Sh::DMA_SLOTS) * Sh::K_SLOT_BYTES + wave * 4096;
+            const unsigned char *kb = lds_raw + K_OFF + (it % Sh::DMA_SLOTS) * Sh::K_SLOT_BYTES + wave * Sh::K_BLOCK_BYTES;
 #pragma unroll
             for (int i = 0; i < KROUNDS; i++) {
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
-                    const u32x4 v = *reinterpret_cast<const u32x4 *>(kb + i * 4 * 4096 + (4 * g + j) * 256 + n * 16);
-                    kreg[i][g].w[0] = v.x, kreg[i][g].w[1] = v.y, kreg[i][g].w[2] = v.z, kreg[i][g].w[3] = v.w;
+                    if constexpr (BITS == 8) {
+                        const u32x4 v = *reinterpret_cast<const u32x4 *>(kb + i * 4 * Sh::K_BLOCK_BYTES + (4 * g + j) * 256 + n * 16);
+                        kreg[i][g].w[0] = v.x, kreg[i][g].w[1] = v.y, kreg[i][g].w[2] = v.z, kreg[i][g].w[3] = v.w;
+                    } else {
+                        // 8 bytes: half (j % 2) of piece 2 g + j / 2
+                        const u32x2 v = *reinterpret_cast<const u32x2 *>(kb + i * 4 * Sh::K_BLOCK_BYTES + (2 * g + (j >> 1)) * 256 +
+                                                                         n * 16 + (j & 1) * 8);
+                        kreg[i][g].w[0] = v.x, kreg[i][g].w[1] = v.y;
+                    }
                 }
             }
         }
@@ -819,13 +832,14 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
                     if (uint32_t(ks) < ksteps) build_p(t, ks, phi[ks], plo[ks]);
                 }
                 if constexpr (DMA) {
-                    const unsigned char *vb = lds_raw + V_OFF + (it % Sh::DMA_SLOTS) * Sh::V_SLOT_BYTES + 64 * wave + 4 * n;
+                    const unsigned char *vb = lds_raw + V_OFF + (it % Sh::DMA_SLOTS) * Sh::V_SLOT_BYTES + val_lane_offset<BITS>(wave, n);
 #pragma unroll
                     for (int ks = 0; ks < KSTEPS; ks++) {
 #pragma unroll
                         for (int e = 0; e < 8; e++) {
                             const int tk = 32 * ks + 8 * j + e;  // token of the iteration
-                            vreg[ks].w[e] = *reinterpret_cast<const uint32_t *>(vb + (tk >> 2) * Sh::V_GROUP_BYTES + (tk & 3) * 256);
+                            vreg[ks].w[e] = *reinterpret_cast<const uint32_t *>(vb + (tk / Sh::V_GROUP_TOKENS) * Sh::V_GROUP_BYTES +
+                                                                                (tk % Sh::V_GROUP_TOKENS) * RB);
                         }
                     }
                 }
@@ -997,10 +1011,11 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel_n(PartialArg
     attention_partial_body<BITS, TILES, false, itb_rows<TILES>(), TILES == 1>(a);
 }
 
-// One query row over 8-bit codes with loader waves: 4 computing + 4 loading waves.
+// One query row over codes with loader waves: two teams of 4 computing waves + 4 loading waves.
 constexpr int ITB_DMA = 4, TEAMS_DMA = 2;
+template <int BITS>
 __global__ __launch_bounds__((TEAMS_DMA + 1) * THREADS) void attention_partial_kernel_d(PartialArgs a) {
-    attention_partial_body<8, 1, true, ITB_DMA, true, true, TEAMS_DMA>(a);
+    attention_partial_body<BITS, 1, true, ITB_DMA, true, true, TEAMS_DMA>(a);
 }
 
 template <int BITS>
@@ -1098,6 +1113,10 @@ uint32_t splits_for(uint32_t capacity, uint32_t wanted) {
 // (measured, per layer with the merge: 10.0 against 11.0 us at 4k tokens, equal at 32k, 20.9
 // against 22.3 at 50k, 35.5 against 36.5 at 131k).
 constexpr uint32_t LOADERS_FROM = 24 * 1024;
+// 4-bit codes: the same kernel from the same capacity (15.0 against 16.8 us at 32k, 29.5 against 31.6
+// at 131k), up to where the two-workgroups-per-CU kernel streams faster than the loader kernel's
+// two teams get through their iterations (29.1 against 28.5 us at 150k, 40.9 against 39.3 at 200k).
+constexpr uint32_t LOADERS_4BIT_UP_TO = 136 * 1024;
 
 bool loaders_enabled() {  // SAETTA_DECODE_LOADERS=0 keeps to the kernels without loader waves
     static const bool on = [] {
@@ -1111,10 +1130,10 @@ template <int BITS, int TILES, bool PACKED>
 void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu, bool loaders) {
     void (*kernel)(PartialArgs);
     int lds_bytes;
-    if constexpr (TILES == 1 && BITS == 8 && PACKED) {
+    if constexpr (TILES == 1 && BITS != 16 && PACKED) {
         if (loaders) {
-            attention_partial_kernel_d<<<dim3(a.nsplits, a.kv_heads), (TEAMS_DMA + 1) * THREADS,
-                                         Shape<8, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA), stream>>>(a);
+            attention_partial_kernel_d<BITS><<<dim3(a.nsplits, a.kv_heads), (TEAMS_DMA + 1) * THREADS,
+                                               Shape<BITS, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA), stream>>>(a);
             return;
         }
     }
@@ -1180,9 +1199,10 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
     // which pays only for long contexts: up to 64k tokens the shorter merge of half as many partials
     // is worth more (measured: 19.4 against 20.6 us per layer at 32k, 28.3 against 29.7 at 64k,
     // but 44 against 35 at 146k, 4-bit).  Both stages derive the same number from the same arguments.
-    // One row over 8-bit codes in a cache of 24k tokens and more goes to the kernel with loader waves,
-    // which is a one-workgroup-per-CU kernel at every length.
-    const bool loaders = rows == 1 && bits == 8 && capacity >= LOADERS_FROM && loaders_enabled();
+    // One row over codes in a cache of 24k tokens and more (4-bit: up to 136k) goes to the kernel with
+    // loader waves, which is a one-workgroup-per-CU kernel at every length.
+    const bool loaders = rows == 1 && bits != 16 && capacity >= LOADERS_FROM && (bits == 8 || capacity <= LOADERS_4BIT_UP_TO) &&
+                         loaders_enabled();
     const bool one_per_cu = rows >= 2 || bits == 16 || capacity <= 80 * 1024 || loaders;
     if (one_per_cu && nsplits > MAX_SPLITS / 2) nsplits = MAX_SPLITS / 2;
     if (stages & SAETTA_STAGE_PARTIAL) {
@@ -1225,9 +1245,14 @@ int raise_lds_of_bits() {
 int setup_decode() {
     if (int rc = load_kernel(reinterpret_cast<const void *>(attention_reduce_kernel))) return rc;
     static_assert(Shape<8, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA) <= 160 * 1024, "LDS of a CU");
-    if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_partial_kernel_d),
+    if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_partial_kernel_d<8>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize,
                                          Shape<8, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA)))) {
+        return rc;
+    }
+    if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_partial_kernel_d<4>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         Shape<4, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA)))) {
         return rc;
     }
     if (int rc = raise_lds_of_bits<8>()) return rc;

@@ -181,9 +181,10 @@ def test_capacity_must_be_whole_blocks():
         plan.build().run()
 
 
-def test_large_eight_bit_cache_one_row():
-    # One row over 8-bit codes in a cache of 24k tokens and more runs the kernel whose extra waves
-    # move the codes into LDS and whose two teams of computing waves take alternate 64-token
+@pytest.mark.parametrize("kind", [saetta.KvBits.Eight, saetta.KvBits.Four])
+def test_large_cache_of_codes_one_row(kind):
+    # One row over codes in a cache of 24k tokens and more runs the kernel whose extra waves move
+    # the codes into LDS and whose two teams of computing waves take alternate 64-token
     # iterations.  Lengths: less than one block; one team idle; both teams, even and odd numbers of
     # iterations; more iterations than LDS slots (the slots are refilled); the whole capacity.  The
     # rows past each length are poisoned.
@@ -195,8 +196,8 @@ def test_large_eight_bit_cache_one_row():
     qg = rng.standard_normal(H * 2 * D).astype(np.float32)
     att = saetta.DecodeAttention(H, KV, D, capacity)
     for length in [1, 100, 2049, 8200, 16400, 33000, 50001, 81920]:
-        kc, vc, kf, vf = cache_pair(k[:length], v[:length], saetta.KvBits.Eight, capacity, poison=True)
-        got = run_decode(att, saetta.KvBits.Eight, dev(q), kc, vc, dev(qg), length)
+        kc, vc, kf, vf = cache_pair(k[:length], v[:length], kind, capacity, poison=True)
+        got = run_decode(att, kind, dev(q), kc, vc, dev(qg), length)
         assert np.isfinite(got).all(), length
         worst = np.abs(got - oracle.attention_f64(q, kf, vf, qg, length, threads=8)).max()
         assert worst < MAX_ABS_F64, (length, worst)
