@@ -168,6 +168,19 @@ def bench_decode(s, torch, args, ctx, bits, rows, layers):
     torch.cuda.synchronize()
     rel_rms = oracle.rel_rms(out[0].cpu().numpy(), ref)
 
+    # Quantize-on-append of 4 new tokens into every layer's K and V caches (two launches per
+    # layer, rows ctx .. ctx + 3; last, because it writes over the rows the check above read).
+    import ctypes
+    new_tokens = 4
+    x_new = torch.randn(new_tokens, VALUES, device="cuda")
+    append = s.Plan()
+    for k, v in caches:
+        for rows_q in (k, v):
+            p = s.ffi.KvQuantParamsC(rows_q.per_token * new_tokens, rows_q.per_token)
+            append.op(f"kv_quantize_{bits}", lambda st, c=rows_q.c(), p=p: s.ffi.check(
+                s.ffi.lib().saetta_kv_quantize(st, bits, ctypes.c_void_p(x_new.data_ptr()), c, p, None, ctx), "kv_quantize"))
+    append_us, _ = kernel_us(append.build(graph))
+
     name = f"decode attention, {bits}-bit KV, ctx {ctx}, {rows} query row(s), {layers} layer caches per step"
     return {
         "metric": f"decode attn HBM GB/s @{ctx // 1024}k ctx {bits}-bit KV",
@@ -176,7 +189,8 @@ def bench_decode(s, torch, args, ctx, bits, rows, layers):
         "ms_per_step": round(ms_per_step, 4),
         "dtype": "u8 codes, f16 MFMA, f32 accumulate",
         "config": {"workload": name, "heads": H, "kv_heads": KV, "head_dim": D, "ctx": ctx, "kv_bits": bits,
-                   "rows": rows, "layers_per_step": layers, "bytes_per_layer": layer_bytes},
+                   "rows": rows, "layers_per_step": layers, "bytes_per_layer": layer_bytes,
+                   "append_4_tokens_k_and_v_us_per_layer": round(append_us, 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("decode8_32k") if (ctx, bits, rows) == (32768, 8, 1) else None,
                      "kernel": "attention_partial_kernel", "avg_us": round(part_us, 3),
