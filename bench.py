@@ -347,6 +347,20 @@ def bench_deltanet(s, torch, args, layers=30):
         return median(ts)
 
     both_us, step_us, token_us = timed(plan_of("both")), timed(plan_of("step")), timed(plan_of("token"))
+
+    # The verify step of the same layers: 4 rows with the conv and delta states after every row
+    # (what an MTP verify asks for), as one call of two launches and as the pair of calls for chunks.
+    m = 4
+    xm, zm, am, bm = r(m * ch), r(m * val), r(m * vh), r(m * vh)
+    mixed_m, ym = torch.empty(m * ch, device="cuda"), torch.empty(m * val, device="cuda")
+    csn, ssn = torch.empty(m * (kernel - 1) * ch, device="cuda"), torch.empty(m * vh * dv * 128, device="cuda")
+    fused, pair = s.Plan(), s.Plan()
+    for conv, st in states:
+        s.deltanet_rows_fused(fused, xm, w, conv, am, bm, alog, dtb, st, zm, norm, ym, kh, vh, dv, kernel, m, eps, csn, ssn)
+        s.deltanet_conv_rows(pair, xm, w, conv, mixed_m, ch, kernel, m, csn)
+        s.deltanet_rows(pair, mixed_m, am, bm, alog, dtb, st, zm, norm, ym, kh, vh, dv, m, eps, ssn)
+    verify_us = timed(fused.build(graph=not args.no_graph))
+    verify_pair_us = timed(pair.build(graph=not args.no_graph))
     nbytes = 2.0 * vh * dv * 128 * 4
     achieved = nbytes / token_us / 1e3
     return {
@@ -357,7 +371,8 @@ def bench_deltanet(s, torch, args, layers=30):
         "dtype": "f32",
         "config": {"workload": f"Gated DeltaNet, one token, conv + step (deltanet_token), {layers} layer states per step",
                    "k_heads": kh, "v_heads": vh, "k_dim": 128, "v_dim": dv, "conv_kernel": kernel, "bytes_per_layer": nbytes,
-                   "conv_then_step_us": round(both_us, 3), "step_kernel_alone_us": round(step_us, 3)},
+                   "conv_then_step_us": round(both_us, 3), "verify_4_rows_with_snapshots_us": round(verify_us, 3),
+                   "verify_4_rows_as_conv_rows_then_rows_us": round(verify_pair_us, 3), "step_kernel_alone_us": round(step_us, 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "kernel": "deltanet_rows_small_kernel + deltanet_rows_small_tail_kernel", "avg_us": round(token_us, 3)},
