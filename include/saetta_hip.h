@@ -157,9 +157,10 @@ typedef struct saetta_quant_rows {
 /* ---- set-up --------------------------------------------------------------- */
 
 /* Checks that the current device is gfx950, loads the kernels and raises their
- * LDS limits.  Stands where Gpu::new() (src/gpu.rs:233-263) stands for this
- * path.  Every entry point does the same on first use, but that first use must
- * not be under stream capture: call this before capturing a graph. */
+ * LDS limits; once per device.  Stands where Gpu::new() (src/gpu.rs:233-263)
+ * stands for this path.  Every entry point does the same on its first use on a
+ * device, but that first use must not be under stream capture: call this, with
+ * the device current, before capturing a graph. */
 int saetta_init(void);
 
 /* Text of the last error on this thread ("" if none). */

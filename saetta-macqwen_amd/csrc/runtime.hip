@@ -19,38 +19,52 @@ int fail(int code, const char *fmt, ...) {
     return code;
 }
 
+// The set-up of a device (its architecture checked, the code objects loaded, the kernels' LDS
+// limits raised) runs once per device, the first time a call finds that device current.
+namespace {
+constexpr int MAX_DEVICES = 64;
+struct DeviceSetup {
+    std::once_flag once;
+    int status = SAETTA_OK;
+    char why[256] = "";
+};
+DeviceSetup g_devices[MAX_DEVICES];
+}  // namespace
+
 int ensure_device() {
-    static std::once_flag once;
-    static int status = SAETTA_OK;
-    static char why[256] = "";
-    std::call_once(once, [] {
-        int dev = 0;
-        hipError_t e = hipGetDevice(&dev);
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(SAETTA_E_DEVICE, "no HIP device: %s", hipGetErrorString(e));
+    }
+    if (dev < 0 || dev >= MAX_DEVICES) return fail(SAETTA_E_DEVICE, "device index %d (up to %d)", dev, MAX_DEVICES - 1);
+    DeviceSetup &d = g_devices[dev];
+    std::call_once(d.once, [&d, dev] {
         hipDeviceProp_t prop;
-        if (e == hipSuccess) e = hipGetDeviceProperties(&prop, dev);
+        hipError_t e = hipGetDeviceProperties(&prop, dev);
         if (e != hipSuccess) {
-            status = SAETTA_E_DEVICE;
-            snprintf(why, sizeof why, "no HIP device: %s", hipGetErrorString(e));
+            d.status = SAETTA_E_DEVICE;
+            snprintf(d.why, sizeof d.why, "no HIP device: %s", hipGetErrorString(e));
             (void)hipGetLastError();
             return;
         }
         if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
-            status = SAETTA_E_DEVICE;
-            snprintf(why, sizeof why, "device is %s; this library is built for gfx950 only",
-                     prop.gcnArchName);
+            d.status = SAETTA_E_DEVICE;
+            snprintf(d.why, sizeof d.why, "device is %s; this library is built for gfx950 only", prop.gcnArchName);
             return;
         }
         int (*const setups[])() = {setup_kv_quant, setup_prep, setup_deltanet, setup_decode, setup_prefill};
         for (auto setup : setups) {
             if (int rc = setup()) {
-                status = SAETTA_E_DEVICE;
-                snprintf(why, sizeof why, "kernels do not load: %s", hipGetErrorString(hipError_t(rc)));
+                d.status = SAETTA_E_DEVICE;
+                snprintf(d.why, sizeof d.why, "kernels do not load: %s", hipGetErrorString(hipError_t(rc)));
                 (void)hipGetLastError();
                 return;
             }
         }
     });
-    if (status != SAETTA_OK) return fail(status, "%s", why);
+    if (d.status != SAETTA_OK) return fail(d.status, "%s", d.why);
     return SAETTA_OK;
 }
 
