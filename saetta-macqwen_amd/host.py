@@ -1,7 +1,8 @@
 """Host-side objects of the path, named as in the reference.
 
   kv_quant.rs           KvBits, GROUP, QuantRows (new / record / record_at / encode / encode_dequantize)
-  plan.rs               TokenParams, Plan (params / op / set_params / build), Built.run
+  plan.rs               TokenParams, Plan (params / op / constant / set_params / len / is_empty / run_serial /
+                        kernels / build / build_where), Built (run / run_timed / commit)
   attention.rs          DecodeAttention (new / record / record_quant, pub kernel)
   rows.rs               MAX_ROWS, AttentionRows (new / record / record_quant)
   attention_prefill.rs  FlashParams, KERNELS, DEFAULT, KEY_BLOCK, encode
@@ -13,6 +14,7 @@ view with an offset); a Metal encoder is a HIP stream.  Shape violations raise
 import ctypes
 import enum
 import math
+import time
 
 import torch
 
@@ -90,6 +92,38 @@ class Plan:
         self.params.copy_(host, non_blocking=True)
         self._keep = host
 
+    def __len__(self):
+        return len(self.ops)
+
+    def len(self):
+        return len(self.ops)
+
+    def is_empty(self):
+        return not self.ops
+
+    def constant(self, data):
+        """Plan::constant (src/plan.rs:128-141): a device buffer holding `data`, for values that never
+        change between tokens."""
+        return torch.as_tensor(data).to(self.params.device)
+
+    def run_serial(self, stream=None):
+        """Plan::run_serial (src/plan.rs:157-168): every op launched one after the other on the
+        stream, outside any graph, then a wait; the wall time in seconds."""
+        start = time.perf_counter()
+        s = _stream(stream)
+        for _, launch in self.ops:
+            launch(s)
+        torch.cuda.synchronize()
+        return time.perf_counter() - start
+
+    def kernels(self):
+        """Plan::kernels (src/plan.rs:171-181): each kernel name with how many ops use it, in order
+        of first use."""
+        out = {}
+        for kernel, _ in self.ops:
+            out[kernel] = out.get(kernel, 0) + 1
+        return list(out.items())
+
     def build(self, graph=False):
         """Plan::build (src/plan.rs:229-235).  graph=True captures the launches into a HIP
         graph, the counterpart of the reference's indirect command buffer: one submission
@@ -118,12 +152,34 @@ class Built:
             self.graph = g
 
     def run(self, stream=None):
+        """Enqueues the recorded launches (one graph launch, or one by one) and returns without
+        waiting: the stream orders what follows, as for any torch op.  Built::commit
+        (src/plan.rs:254-256) without the Pending; `run_timed` is the reference's waiting `run`."""
         if self.graph is not None:
             self.graph.replay()
             return
         s = _stream(stream)
         for _, launch in self.ops:
             launch(s)
+
+    def run_timed(self, stream=None):
+        """Built::run_timed (src/plan.rs:249-251): runs, waits, and returns (wall seconds, the
+        GPU's own seconds between the first launch and the end of the last, from two events)."""
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start = time.perf_counter()
+        e0.record()
+        self.run(stream)
+        e1.record()
+        e1.synchronize()
+        return time.perf_counter() - start, e0.elapsed_time(e1) * 1e-3
+
+    def commit(self, stream=None):
+        """Built::commit (src/plan.rs:254-256): `run` without the wait; the event returned waits
+        for it (`.synchronize()`)."""
+        self.run(stream)
+        done = torch.cuda.Event()
+        done.record()
+        return done
 
 
 class QuantRows:

@@ -20,6 +20,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <chrono>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -136,11 +137,39 @@ class Built {
         hip_check(hipGraphDestroy(g), "hipGraphDestroy");
         exec_ = std::shared_ptr<hipGraphExec>(e, [](hipGraphExec_t x) { (void)hipGraphExecDestroy(x); });
     }
-    void run(const gpu::Gpu &gpu) const {
+    // Replays the recorded launches and waits (Built::run, src/plan.rs:241-243); the wall time in seconds.
+    double run(const gpu::Gpu &gpu) const { return run_timed(gpu).first; }
+    // `run`, also returning the GPU's own time between the first launch and the end of the last,
+    // in seconds (Built::run_timed, src/plan.rs:249-251), from two events on the stream.
+    std::pair<double, double> run_timed(const gpu::Gpu &gpu) const {
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+        hip_check(hipEventCreate(&e0), "hipEventCreate");
+        hip_check(hipEventCreate(&e1), "hipEventCreate");
+        const auto start = std::chrono::steady_clock::now();
+        hip_check(hipEventRecord(e0, gpu.stream()), "hipEventRecord");
         enqueue(gpu);
-        gpu.sync();
+        hip_check(hipEventRecord(e1, gpu.stream()), "hipEventRecord");
+        hip_check(hipEventSynchronize(e1), "hipEventSynchronize");
+        const double wall = std::chrono::duration<double>(std::chrono::steady_clock::now() - start).count();
+        float ms = 0.0f;
+        hip_check(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
+        return {wall, double(ms) * 1e-3};
     }
-    // Replays without waiting, for timing many runs back to back.
+    // `run` without the wait (Built::commit, src/plan.rs:254-256): what is returned waits for it.
+    struct Pending {
+        std::shared_ptr<ihipEvent_t> done;
+        void wait() const { hip_check(hipEventSynchronize(done.get()), "hipEventSynchronize"); }
+    };
+    Pending commit(const gpu::Gpu &gpu) const {
+        hipEvent_t e = nullptr;
+        hip_check(hipEventCreate(&e), "hipEventCreate");
+        enqueue(gpu);
+        hip_check(hipEventRecord(e, gpu.stream()), "hipEventRecord");
+        return Pending{std::shared_ptr<ihipEvent_t>(e, [](hipEvent_t x) { (void)hipEventDestroy(x); })};
+    }
+    // Replays without waiting and without an event, for timing many runs back to back.
     void enqueue(const gpu::Gpu &gpu) const {
         if (exec_) {
             hip_check(hipGraphLaunch(exec_.get(), gpu.stream()), "hipGraphLaunch");
@@ -165,6 +194,35 @@ class Plan {
     void set_params(TokenParams tp) {
         hip_check(hipMemcpyAsync(params.ptr<void>(), &tp, sizeof tp, hipMemcpyHostToDevice, gpu_.stream()), "set_params");
         gpu_.sync();
+    }
+    const gpu::Gpu &gpu() const { return gpu_; }
+    size_t len() const { return ops_.size(); }
+    bool is_empty() const { return ops_.empty(); }
+    // A buffer holding `data`, for values that never change between tokens (Plan::constant, src/plan.rs:128-141).
+    template <typename T>
+    View constant(const std::vector<T> &data) const {
+        return View(gpu_.buffer_from(data));
+    }
+    // Launches every op one after the other on the stream, outside any graph, and waits
+    // (Plan::run_serial, src/plan.rs:157-168); the wall time in seconds.
+    double run_serial() const {
+        const auto start = std::chrono::steady_clock::now();
+        for (auto &op : ops_) op.second(gpu_.stream());
+        gpu_.sync();
+        return std::chrono::duration<double>(std::chrono::steady_clock::now() - start).count();
+    }
+    // Each kernel name with how many ops use it, in order of first use (Plan::kernels, src/plan.rs:171-181).
+    std::vector<std::pair<std::string, size_t>> kernels() const {
+        std::vector<std::pair<std::string, size_t>> out;
+        for (auto &op : ops_) {
+            auto it = std::find_if(out.begin(), out.end(), [&](const auto &k) { return k.first == op.first; });
+            if (it == out.end()) {
+                out.emplace_back(op.first, 1);
+            } else {
+                it->second++;
+            }
+        }
+        return out;
     }
     Built build(bool graph = false) const { return Built(ops_, gpu_, graph); }
     // Only the launches whose kernel name `keep` accepts (Plan::build_where, src/plan.rs:237-273).

@@ -74,6 +74,26 @@ int main() {
             plan.set_params(plan::token_params(0, 41));
             built.run(gpu);
             compare(cache, x, 41, bits);
+            // serial == replay (tests/plan.rs:27-45), and the rest of Plan and Built
+            QuantRows second(gpu, bits, VALUES, 64);
+            second.record(plan, xb);
+            EXPECT(plan.len() == 2 && !plan.is_empty() && plan::Plan(gpu).is_empty(), "Plan::len");
+            const auto kernels = plan.kernels();
+            EXPECT(kernels.size() == 1 && kernels[0].second == 2 && kernels[0].first.rfind("kv_quantize", 0) == 0, "Plan::kernels");
+            plan.set_params(plan::token_params(0, 7));
+            EXPECT(plan.run_serial() > 0.0, "Plan::run_serial");
+            compare(second, x, 7, bits);
+            auto graph = plan.build(true);
+            plan.set_params(plan::token_params(0, 50));
+            const auto timed = graph.run_timed(gpu);
+            EXPECT(timed.first > 0.0 && timed.second > 0.0 && timed.second <= timed.first, "Built::run_timed %g %g", timed.first, timed.second);
+            compare(second, x, 50, bits);
+            compare(cache, x, 50, bits);
+            plan.set_params(plan::token_params(0, 60));
+            graph.commit(gpu).wait();
+            compare(second, x, 60, bits);
+            const View c = plan.constant(std::vector<float>{1.5f, 2.5f});
+            EXPECT(gpu::contents<float>(c.buffer, 2) == (std::vector<float>{1.5f, 2.5f}), "Plan::constant");
         }
         {  // dequantize_matches_cpu
             const size_t tokens = 9;

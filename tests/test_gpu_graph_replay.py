@@ -80,3 +80,33 @@ def test_deltanet_rows_replay_advances_the_state_like_eager_runs():
         assert torch.equal(u, v)
     assert torch.equal(got_conv, want_conv) and torch.equal(got_st, want_st)
     assert not torch.equal(want_y[0], want_y[1])  # the state did move between the runs
+
+
+def test_serial_and_replay_agree_on_a_chain():
+    # tests/plan.rs:27-45: 100 dependent ops each add 1, then one adds the token position, which the
+    # device reads from the plan's TokenParams when it runs; run serially, then replayed from the
+    # graph at another position.
+    n = 1024
+    data = torch.zeros(n, device="cuda")
+    plan = saetta.Plan()
+    for _ in range(100):
+        plan.op("add_one", lambda s: data.add_(1.0))
+    plan.op("add_position", lambda s: data.add_(plan.params[1]))
+    assert len(plan) == 101 and plan.len() == 101 and not plan.is_empty() and saetta.Plan().is_empty()
+    assert plan.kernels() == [("add_one", 100), ("add_position", 1)]
+    built = plan.build(graph=True)
+    plan.set_params(saetta.TokenParams(0, 7))
+    assert plan.run_serial() > 0.0
+    assert bool((data == 107.0).all())
+    plan.set_params(saetta.TokenParams(0, 1000))
+    wall, gpu_seconds = built.run_timed()
+    assert bool((data == 1207.0).all())
+    assert wall > 0.0 and 0.0 < gpu_seconds <= wall
+    # commit does not wait; what it returns does
+    built.commit().synchronize()
+    assert bool((data == 2307.0).all())
+    # only the ops of one kernel (Plan::build_where)
+    plan.build_where(lambda k: k == "add_position").run()
+    assert bool((data == 3307.0).all())
+    two = plan.constant([1.5, 2.5])
+    assert two.is_cuda and two.tolist() == [1.5, 2.5]
