@@ -490,16 +490,12 @@ constexpr int LDS_BYTES = 8 * MERGE_WAVE_BYTES > 8 * PART_BYTES ? 8 * MERGE_WAVE
 __device__ __forceinline__ uint32_t k_slot(uint32_t b) { return (b & 3) * PART_BYTES; }
 __device__ __forceinline__ uint32_t v_slot(uint32_t b) { return (4 + (b & 3)) * PART_BYTES; }
 
-__global__ __launch_bounds__(THREADS, 2) void attention_prefill_kernel(PrefillArgs a) {
-    extern __shared__ __attribute__((aligned(1024))) unsigned char tiles[];
-
+// One tile of TQ tokens x 8 heads of kv head `kv` against the keys it sees.
+__device__ __forceinline__ void prefill_tile(const PrefillArgs &a, unsigned char *tiles, uint32_t tile, uint32_t kv) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, hf = lane >> 5;
     const int group = wave & 3, parity = wave >> 2;  // the wave's rows; which key blocks it takes
-    const uint32_t kv = blockIdx.y;
-    const uint32_t ntiles = (a.tokens + TQ - 1) / TQ;
-    const uint32_t tile = ntiles - 1 - blockIdx.x;  // the tiles with the most keys start first
     const uint32_t tok0 = tile * TQ + 4 * group;    // this wave's first token
     const float c = a.scale * 1.4426950408889634f;  // scores are kept in units of log2(e)
 
@@ -744,6 +740,21 @@ __global__ __launch_bounds__(THREADS, 2) void attention_prefill_kernel(PrefillAr
     }
 }
 
+// A workgroup takes tiles until there are none left: with more tiles than workgroups (one per CU:
+// the LDS ring fills a CU), the next tile starts without a new workgroup having to be dispatched.
+// Tiles are numbered from the one with the most keys down, the kv heads side by side, and handed
+// out boustrophedon: round 0 gives workgroup w tile w, round 1 tile 2 G - 1 - w, ... so that every
+// workgroup gets the same amount of keys to within a tile.
+__global__ __launch_bounds__(THREADS, 2) void attention_prefill_kernel(PrefillArgs a) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char tiles[];
+    const uint32_t ntiles = (a.tokens + TQ - 1) / TQ, total = ntiles * a.kv_heads, G = gridDim.x;
+    for (uint32_t first = 0, round = 0; first < total; first += G, round++) {
+        const uint32_t idx = first + ((round & 1) ? G - 1 - blockIdx.x : blockIdx.x);
+        if (round) __syncthreads();  // the last tile's merge has been read: the next tile's keys may land on it
+        if (idx < total) prefill_tile(a, tiles, ntiles - 1 - idx / a.kv_heads, idx % a.kv_heads);
+    }
+}
+
 // Workspace the library owns when the caller passes none: grown on demand, one per device.
 struct OwnedWorkspace {
     void *ptr = nullptr;
@@ -811,8 +822,14 @@ int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kda
     }
     PrefillArgs a{q, static_cast<const unsigned char *>(workspace), q_and_gate, out, p.heads, p.kv_heads, p.pos,
                   p.tokens, p.scale, nblocks};
-    const dim3 grid((p.tokens + TQ - 1) / TQ, p.kv_heads);
-    attention_prefill_kernel<<<grid, THREADS, LDS_BYTES, stream>>>(a);
+    // one workgroup per CU at most: a workgroup's LDS ring fills a CU, and further tiles are taken in the kernel
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+        (void)hipGetLastError();
+        cus = 256;
+    }
+    const uint32_t total = (p.tokens + TQ - 1) / TQ * p.kv_heads;
+    attention_prefill_kernel<<<dim3(total < uint32_t(cus) ? total : uint32_t(cus)), THREADS, LDS_BYTES, stream>>>(a);
     return launch_status(what);
 }
 
