@@ -39,6 +39,18 @@ __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf
 __device__ __forceinline__ float silu_f(float x) { return x * sigmoid_f(x); }
 __device__ __forceinline__ float dot4(float4 a, float4 b) { return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w; }
 
+// The gates of a token and head: g = exp(-exp(A_log) softplus(a + dt_bias)), beta = sigmoid(b), with
+// the hardware's exp2 and log2 (the library routines are some 150 instructions, and in the kernels
+// below the gates sit in one wave's path): log1p(e) as e - e^2 / 2 below 2^-10 and log(1 + e)
+// above; the errors stay near 1e-7.
+__device__ __forceinline__ void fast_gates(float a_plus_bias, float exp_a_log, float b, float &g, float &beta) {
+    const float e = __expf(-fabsf(a_plus_bias));
+    const float log1p_e = e < 0x1p-10f ? e * (1.0f - 0.5f * e) : __logf(1.0f + e);
+    const float softplus = fmaxf(a_plus_bias, 0.0f) + log1p_e;
+    g = __expf(-exp_a_log * softplus);
+    beta = __builtin_amdgcn_rcpf(1.0f + __expf(-b));
+}
+
 __global__ __launch_bounds__(256) void deltanet_conv_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                             float *__restrict__ state, float *__restrict__ out,
                                                             saetta_conv_params p) {
@@ -307,16 +319,16 @@ __global__ __launch_bounds__(256) void deltanet_rows_kernel(RowsArgs a) {
         for (int j = 0; j < ROWS_TB / 4; j++) {
             const float4 x = raw[j];
             const float ss = group_reduce<32>(dot4(x, x), SumOp());
-            const float inv = (lane < 32 ? q_scale : 1.0f) / sqrtf(ss + a.p.eps);
+            const float inv = (lane < 32 ? q_scale : 1.0f) * __builtin_amdgcn_rsqf(ss + a.p.eps);
             const uint32_t f = lane & 31;  // float4 f of the vector belongs to lane f / F4, its float4 f % F4
             float *dst = &qk_lds[buf][wave + 4 * j][(lane < 32 ? 0 : K_DIM) + (f % F4) * (LANES * 4) + (f / F4) * 4];
             *reinterpret_cast<float4 *>(dst) = make_float4(x.x * inv, x.y * inv, x.z * inv, x.w * inv);
         }
         if (tid < ROWS_TB) {
-            const float xg = ga + bias;
-            const float softplus = fmaxf(xg, 0.0f) + log1pf(expf(-fabsf(xg)));
-            gb_lds[buf][tid][0] = g_real ? expf(-exp_a * softplus) : 1.0f;
-            gb_lds[buf][tid][1] = g_real ? sigmoid_f(gbv) : 0.0f;
+            float g, beta;
+            fast_gates(ga + bias, exp_a, gbv, g, beta);
+            gb_lds[buf][tid][0] = g_real ? g : 1.0f;
+            gb_lds[buf][tid][1] = g_real ? beta : 0.0f;
         }
     };
 
@@ -523,10 +535,8 @@ __global__ __launch_bounds__(SMALL_THREADS) void deltanet_rows_small_kernel(Smal
     } else {
         const uint32_t t = tid - 320;
         if (t < tokens) {
-            const float xg = a.a[size_t(t) * v_heads + h] + a.dt_bias[h];
-            const float softplus = fmaxf(xg, 0.0f) + log1pf(expf(-fabsf(xg)));
-            gb_lds[t][0] = expf(-expf(a.a_log[h]) * softplus);
-            gb_lds[t][1] = sigmoid_f(a.b[size_t(t) * v_heads + h]);
+            fast_gates(a.a[size_t(t) * v_heads + h] + a.dt_bias[h], __expf(a.a_log[h]), a.b[size_t(t) * v_heads + h],
+                       gb_lds[t][0], gb_lds[t][1]);
         }
     }
     __syncthreads();
@@ -538,7 +548,7 @@ __global__ __launch_bounds__(SMALL_THREADS) void deltanet_rows_small_kernel(Smal
             const float4 hi = *reinterpret_cast<const float4 *>(qk_lds[t] + which * K_DIM + 64 + part * 4);
             const float sum = group_reduce<16>(dot4(lo, lo) + dot4(hi, hi), SumOp());
             const float scale = which == 0 ? 1.0f / sqrtf(float(K_DIM)) : 1.0f;
-            if (part == 0) inv_lds[t][which] = scale / sqrtf(sum + a.p.eps);
+            if (part == 0) inv_lds[t][which] = scale * __builtin_amdgcn_rsqf(sum + a.p.eps);
         }
     }
     __syncthreads();
