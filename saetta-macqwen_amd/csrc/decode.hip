@@ -1096,7 +1096,7 @@ __global__ __launch_bounds__(256) void attention_reduce_kernel(ReduceArgs a) {
         float o = 0.0f;
 #pragma unroll
         for (int i = 0; i < 16; i++) o += o_lds[i][d >> 2][d & 3];
-        a.out[qh * DIM + 64 * quarter + d] = o / total * (1.0f / (1.0f + expf(-g)));
+        a.out[qh * DIM + 64 * quarter + d] = o * __builtin_amdgcn_rcpf(total) * __builtin_amdgcn_rcpf(1.0f + __expf(-g));
     }
 }
 
