@@ -84,6 +84,20 @@ def test_bad_arguments_are_rejected_before_any_launch():
     cp = ffi.ConvRowsParamsC(64, 1, 4, 0)
     assert lib.saetta_deltanet_conv_rows(None, 16, 16, 16, 16, None, cp) == -2
     assert b"kernel size" in lib.saetta_last_error()
+    # ... the fused call takes up to 8 rows, conv kernels of 2..16 taps, and both snapshot buffers or neither
+    fused = ffi.RowsFusedParamsC(1, 2, 8, 4, 1e-6, 9, 0)
+    assert lib.saetta_deltanet_rows_fused(None, *([16] * 11), None, None, fused) == -2
+    assert b"9 rows" in lib.saetta_last_error()
+    fused = ffi.RowsFusedParamsC(1, 2, 8, 17, 1e-6, 2, 0)
+    assert lib.saetta_deltanet_rows_fused(None, *([16] * 11), None, None, fused) == -2
+    assert b"kernel size" in lib.saetta_last_error()
+    fused = ffi.RowsFusedParamsC(1, 2, 8, 4, 1e-6, 2, 1)
+    assert lib.saetta_deltanet_rows_fused(None, *([16] * 11), 16, None, fused) == -3
+    fused = ffi.RowsFusedParamsC(1, 2, 8, 4, 1e-6, 2, 0)
+    assert lib.saetta_deltanet_rows_fused(None, *([16] * 7), 12, *([16] * 3), None, None, fused) == -4  # the state's alignment
+    token_c, token_s = ffi.ConvParamsC(100, 4), ffi.StepParamsC(1, 2, 8, 1e-6)
+    assert lib.saetta_deltanet_token(None, *([16] * 11), token_c, token_s) == -2
+    assert b"channels" in lib.saetta_last_error()
     fp = ffi.FlashParamsC(16, 2, 0, 1, 0.0625)
     assert lib.saetta_attn_prefill_quant(None, 16, 16, rows, rows, 16, 16, fp, None, 0) == -1
     assert lib.saetta_attn_prefill_quant(None, 8, 16, rows, rows, 16, 16, fp, 8, 1 << 30) == -4  # workspace alignment
