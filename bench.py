@@ -21,7 +21,8 @@ roofline   = the same bytes per launch of the partial kernel over that kernel's
 cpu_baseline = the CPU oracle (a C restatement of the reference's
              single-threaded f32 CPU attention) on one of the layers.
 
-Other workloads (--workload): decode4_150k (4-bit, 150000 tokens), verify2..4
+Other workloads (--workload): decode4_150k (4-bit, 150000 tokens), decode16_4k
+(half cache, 4096 tokens: the reference's own CPU-runnable case), verify2..4
 (2-4 query rows at 32k, 8-bit), prefill (4096-token chunk at position 4096),
 deltanet (the Gated DeltaNet decode step over 30 layer states), deltanet_prefill
 (conv + delta rule + gated norm of a 4096-token chunk of one layer), prep_store
@@ -58,12 +59,19 @@ def median(xs):
 
 def make_decode_workload(s, torch, ctx, bits, rows, layers, seed=1234):
     """LAYERS caches of ctx + rows tokens, quantized on the device from N(0,1)."""
-    kind = {8: s.KvBits.Eight, 4: s.KvBits.Four}[bits]
+    kind = {8: s.KvBits.Eight, 4: s.KvBits.Four, 16: s.KvBits.Half}[bits]
     capacity = (ctx + rows + 127) // 128 * 128
     gen = torch.Generator(device="cuda").manual_seed(seed)
     caches = []
     chunk = 8192
-    for _ in range(layers):
+    for _ in range(layers if bits == 16 else 0):
+        # a half cache: [capacity][kv heads][256] f16, the rows past the context left at zero
+        k = torch.zeros(capacity, VALUES, dtype=torch.float16, device="cuda")
+        v = torch.zeros(capacity, VALUES, dtype=torch.float16, device="cuda")
+        k[:ctx + rows] = torch.randn(ctx + rows, VALUES, generator=gen, device="cuda").to(torch.float16)
+        v[:ctx + rows] = torch.randn(ctx + rows, VALUES, generator=gen, device="cuda").to(torch.float16)
+        caches.append((k, v))
+    for _ in range(0 if bits == 16 else layers):
         k, v = s.QuantRows(kind, VALUES, capacity), s.QuantRows(kind, VALUES, capacity)
         for rows_q in (k, v):
             for start in range(0, ctx + rows, chunk):
@@ -85,21 +93,22 @@ def bench_decode(s, torch, args, ctx, bits, rows, layers):
 
     kind, capacity, caches, q, qg, out = make_decode_workload(s, torch, ctx, bits, rows, layers)
     plan = s.Plan()
+    half = bits == 16
     if rows == 1:
         att = s.DecodeAttention(H, KV, D, capacity)
         for k, v in caches:
-            att.record_quant(plan, q[0], k, v, qg[0], out[0])
+            (att.record if half else att.record_quant)(plan, q[0], k, v, qg[0], out[0])
         plan.set_params(s.TokenParams(0, ctx))  # position ctx: sees ctx + 1 tokens
     else:
         att = s.AttentionRows(H, KV, capacity, rows)
         tp = s.TokenParams(0, ctx).as_tensor("cuda")
         for k, v in caches:
-            att.record_quant(plan, rows, q, k, v, qg, out, [tp] * rows)
+            (att.record if half else att.record_quant)(plan, rows, q, k, v, qg, out, [tp] * rows)
     graph = not args.no_graph
     built = plan.build(graph)
     partial_only = plan.build_where(lambda name: "partial" in name, graph)
     reduce_only = plan.build_where(lambda name: "reduce" in name, graph)
-    bytes_per_token = {8: 1088, 4: 576}[bits]
+    bytes_per_token = {8: 1088, 4: 576, 16: 2048}[bits]
     layer_bytes = (ctx + rows) * bytes_per_token
 
     for _ in range(args.warmup):
@@ -142,7 +151,10 @@ def bench_decode(s, torch, args, ctx, bits, rows, layers):
                                  rows_q.scales[:groups].cpu().numpy().view(np.uint16),
                                  rows_q.biases[:groups].cpu().numpy().view(np.uint16), bits)
 
-    kf, vf = deq(k0), deq(v0)
+    if half:
+        kf, vf = k0[:n_tok].float().cpu().numpy().reshape(-1), v0[:n_tok].float().cpu().numpy().reshape(-1)
+    else:
+        kf, vf = deq(k0), deq(v0)
     qh, qgh = q[0].cpu().numpy(), qg[0].cpu().numpy()
     threads_all = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
 
@@ -160,10 +172,11 @@ def bench_decode(s, torch, args, ctx, bits, rows, layers):
     # The GPU's answer for the same layer, checked against the oracle while we are here.
     check = s.Plan()
     if rows == 1:
-        att.record_quant(check, q[0], k0, v0, qg[0], out[0])
+        (att.record if half else att.record_quant)(check, q[0], k0, v0, qg[0], out[0])
         check.set_params(s.TokenParams(0, ctx))
     else:
-        att.record_quant(check, rows, q, k0, v0, qg, out, [s.TokenParams(0, ctx).as_tensor("cuda")] * rows)
+        (att.record if half else att.record_quant)(check, rows, q, k0, v0, qg, out,
+                                                    [s.TokenParams(0, ctx).as_tensor("cuda")] * rows)
     check.build().run()
     torch.cuda.synchronize()
     rel_rms = oracle.rel_rms(out[0].cpu().numpy(), ref)
@@ -174,12 +187,12 @@ def bench_decode(s, torch, args, ctx, bits, rows, layers):
     new_tokens = 4
     x_new = torch.randn(new_tokens, VALUES, device="cuda")
     append = s.Plan()
-    for k, v in caches:
+    for k, v in ([] if half else caches):
         for rows_q in (k, v):
             p = s.ffi.KvQuantParamsC(rows_q.per_token * new_tokens, rows_q.per_token)
             append.op(f"kv_quantize_{bits}", lambda st, c=rows_q.c(), p=p: s.ffi.check(
                 s.ffi.lib().saetta_kv_quantize(st, bits, ctypes.c_void_p(x_new.data_ptr()), c, p, None, ctx), "kv_quantize"))
-    append_us, _ = kernel_us(append.build(graph))
+    append_us = kernel_us(append.build(graph))[0] if not half else 0.0
 
     name = f"decode attention, {bits}-bit KV, ctx {ctx}, {rows} query row(s), {layers} layer caches per step"
     return {
@@ -187,10 +200,10 @@ def bench_decode(s, torch, args, ctx, bits, rows, layers):
         "value": round(value, 1),
         "unit": "GB/s",
         "ms_per_step": round(ms_per_step, 4),
-        "dtype": "u8 codes, f16 MFMA, f32 accumulate",
+        "dtype": "f16 cache, f16 MFMA, f32 accumulate" if half else "u8 codes, f16 MFMA, f32 accumulate",
         "config": {"workload": name, "heads": H, "kv_heads": KV, "head_dim": D, "ctx": ctx, "kv_bits": bits,
                    "rows": rows, "layers_per_step": layers, "bytes_per_layer": layer_bytes,
-                   "append_4_tokens_k_and_v_us_per_layer": round(append_us, 3)},
+                   "append_4_tokens_k_and_v_us_per_layer": None if half else round(append_us, 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("decode8_32k") if (ctx, bits, rows) == (32768, 8, 1) else None,
                      "kernel": "attention_partial_kernel", "avg_us": round(part_us, 3),
@@ -540,7 +553,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="decode8_32k",
-                    choices=["decode8_32k", "decode4_150k", "verify2", "verify3", "verify4", "prefill", "deltanet",
+                    choices=["decode8_32k", "decode4_150k", "decode16_4k", "verify2", "verify3", "verify4", "prefill", "deltanet",
                              "deltanet_prefill", "prep_store", "all"])
     ap.add_argument("--no-graph", action="store_true", help="launch from Python instead of replaying a HIP graph")
     ap.add_argument("--layers", type=int, default=0, help="layer caches per step (default 32; 12 at 150k)")
@@ -572,6 +585,8 @@ def main():
             return bench_decode(s, torch, args, 32768, 8, 1, args.layers or 32)
         if workload == "decode4_150k":
             return bench_decode(s, torch, args, 150000, 4, 1, args.layers or 12)
+        if workload == "decode16_4k":
+            return bench_decode(s, torch, args, 4096, 16, 1, args.layers or 32)
         if workload.startswith("verify"):
             return bench_decode(s, torch, args, 32768, 8, int(workload[-1]), args.layers or 32)
         if workload == "deltanet":
@@ -585,7 +600,7 @@ def main():
     if args.workload == "all":
         res = one("decode8_32k")
         res["other_workloads"] = {}
-        for w in ["verify2", "verify3", "verify4", "decode4_150k", "prefill", "deltanet", "deltanet_prefill", "prep_store"]:
+        for w in ["verify2", "verify3", "verify4", "decode4_150k", "decode16_4k", "prefill", "deltanet", "deltanet_prefill", "prep_store"]:
             torch.cuda.empty_cache()
             r = one(w)
             res["other_workloads"][w] = {k: r[k] for k in ("metric", "value", "unit", "ms_per_step", "roofline",
