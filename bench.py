@@ -49,7 +49,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # rocprofv3 --pmc, each scaled by what the same counter reads for a 256 MiB copy in the same run;
 # the runs are summarised in profiles/*_hbm_traffic.txt).  Counters cannot be read inside this
 # script, so the figures are carried here for the workloads they were measured on.
-MEASURED_TRAFFIC = {"decode8_32k": 38.2e6, "prefill": 376.4e6}
+MEASURED_TRAFFIC = {"decode8_32k": 38.2e6, "prefill": 376.4e6, "decode4_150k": 91.7e6, "verify4": 45.1e6}
 
 
 def median(xs):
@@ -205,7 +205,8 @@ def bench_decode(s, torch, args, ctx, bits, rows, layers):
                    "rows": rows, "layers_per_step": layers, "bytes_per_layer": layer_bytes,
                    "append_4_tokens_k_and_v_us_per_layer": None if half else round(append_us, 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("decode8_32k") if (ctx, bits, rows) == (32768, 8, 1) else None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get({(32768, 8, 1): "decode8_32k", (150000, 4, 1): "decode4_150k",
+                                                      (32768, 8, 4): "verify4"}.get((ctx, bits, rows))),
                      "kernel": "attention_partial_kernel", "avg_us": round(part_us, 3),
                      "min_us": round(part_us_min, 3), "reduce_kernel_us": round(red_us, 3)},
         "cpu_baseline": {"value": round(layer_bytes / cpu1 / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
