@@ -34,6 +34,27 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name)
 
 
+def test_header_is_plain_c():
+    # The boundary is a C ABI: the header must compile as C99 on its own (a Rust, Go or C binding reads it).
+    header = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "saetta_hip.h")
+    done = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", "c", header],
+                          capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr
+    # ... and the parameter blocks the mirrors build by hand have the sizes the compiler gives them
+    probe = ('#include "%s"\n#include <stdio.h>\nint main(void) { printf("%%zu %%zu %%zu %%zu %%zu\\n", '
+             'sizeof(saetta_rows_fused_params), sizeof(saetta_rows_step_params), sizeof(saetta_conv_rows_params), '
+             'sizeof(saetta_step_params), sizeof(saetta_conv_params)); return 0; }\n') % header
+    import tempfile
+    with tempfile.TemporaryDirectory() as d:
+        src, exe = os.path.join(d, "probe.c"), os.path.join(d, "probe")
+        with open(src, "w") as f:
+            f.write(probe)
+        subprocess.run(["gcc", "-std=c99", src, "-o", exe], check=True)
+        sizes = [int(x) for x in subprocess.run([exe], capture_output=True, text=True, check=True).stdout.split()]
+    assert sizes == [ctypes.sizeof(ffi.RowsFusedParamsC), ctypes.sizeof(ffi.RowsStepParamsC), ctypes.sizeof(ffi.ConvRowsParamsC),
+                     ctypes.sizeof(ffi.StepParamsC), ctypes.sizeof(ffi.ConvParamsC)]
+
+
 def test_parameter_blocks_match_the_reference_layout():
     # TokenParams (src/plan.rs:16-35) is 4 x u32; DecodeParams 3 x u32 + f32 (src/attention.rs:19-26);
     # RowsAttentionParams adds rows, splits (src/rows.rs:307-317); FlashParams 4 x u32 + f32
