@@ -206,6 +206,12 @@ size_t saetta_part_ml_bytes(uint32_t heads, uint32_t capacity, uint32_t rows);
 #define SAETTA_STAGE_PARTIAL 1u
 #define SAETTA_STAGE_REDUCE 2u
 #define SAETTA_STAGE_ALL 3u
+/* Or-ed into `stages`: keep to the kernels that load the cache into registers, also where the
+ * library would pick the kernel whose extra waves stage the codes in LDS.  The counterpart of
+ * DecodeAttention.kernel (src/attention.rs:36-38), which switches the reference between its two
+ * kernel families.  The partial and the reduce stage of one step must be called with the same
+ * flag: the number of splits follows from it. */
+#define SAETTA_STAGE_NO_LOADERS 4u
 
 /* DecodeAttention::record (src/attention.rs:73-92): one query token over a
  * half cache.  q f32 [heads][256]; keys, values f16 [capacity][kv_heads][256];

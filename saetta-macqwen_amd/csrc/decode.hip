@@ -58,8 +58,6 @@
 #include "common.hpp"
 #include "lanes.hpp"
 
-#include <cstdlib>
-
 namespace saetta {
 namespace {
 
@@ -1118,14 +1116,6 @@ constexpr uint32_t LOADERS_FROM = 24 * 1024;
 // two teams get through their iterations (29.1 against 28.5 us at 150k, 40.9 against 39.3 at 200k).
 constexpr uint32_t LOADERS_4BIT_UP_TO = 136 * 1024;
 
-bool loaders_enabled() {  // SAETTA_DECODE_LOADERS=0 keeps to the kernels without loader waves
-    static const bool on = [] {
-        const char *e = getenv("SAETTA_DECODE_LOADERS");
-        return !e || e[0] != '0';
-    }();
-    return on;
-}
-
 template <int BITS, int TILES, bool PACKED>
 void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu, bool loaders) {
     void (*kernel)(PartialArgs);
@@ -1201,8 +1191,10 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
     // but 44 against 35 at 146k, 4-bit).  Both stages derive the same number from the same arguments.
     // One row over codes in a cache of 24k tokens and more (4-bit: up to 136k) goes to the kernel with
     // loader waves, which is a one-workgroup-per-CU kernel at every length.
+    // SAETTA_STAGE_NO_LOADERS keeps to the register kernels (the caller's choice of kernel family,
+    // as DecodeAttention.kernel is in the reference, src/attention.rs:36-38).
     const bool loaders = rows == 1 && bits != 16 && capacity >= LOADERS_FROM && (bits == 8 || capacity <= LOADERS_4BIT_UP_TO) &&
-                         loaders_enabled();
+                         !(stages & SAETTA_STAGE_NO_LOADERS);
     const bool one_per_cu = rows >= 2 || bits == 16 || capacity <= 80 * 1024 || loaders;
     if (one_per_cu && nsplits > MAX_SPLITS / 2) nsplits = MAX_SPLITS / 2;
     if (stages & SAETTA_STAGE_PARTIAL) {

@@ -12,7 +12,7 @@ SYMBOLS = [
     "saetta_attn_rows", "saetta_attn_rows_quant", "saetta_prefill_workspace_bytes", "saetta_attn_prefill", "saetta_attn_prefill_quant",
 ]
 
-STAGE_PARTIAL, STAGE_REDUCE, STAGE_ALL = 1, 2, 3
+STAGE_PARTIAL, STAGE_REDUCE, STAGE_ALL, STAGE_NO_LOADERS = 1, 2, 3, 4
 
 
 class TokenParamsC(ctypes.Structure):

@@ -302,9 +302,15 @@ class DecodeAttention:
                                   device=device)
         self.part_ml = torch.empty(l.saetta_part_ml_bytes(heads, capacity, 1) // 4, dtype=torch.float32,
                                    device=device)
-        # The reference switches between a vector and a matrix kernel here; this
-        # build has one kernel per cache kind and keeps the field for callers.
+        # The reference switches between its two kernel families here (src/attention.rs:36-38).
+        # "attention_partial_mma": the library picks, which for one row over codes in a large
+        # cache is the kernel with loader waves; "attention_partial": the register kernels only.
         self.kernel = "attention_partial_mma"
+
+    def _flags(self):
+        if self.kernel not in ("attention_partial_mma", "attention_partial"):
+            raise ValueError(f"no decode attention kernel {self.kernel}")
+        return 0 if self.kernel == "attention_partial_mma" else ffi.STAGE_NO_LOADERS
 
     def _params(self):
         return ffi.DecodeParamsC(self.heads, self.kv_heads, self.capacity, 1.0 / math.sqrt(DIM))
@@ -312,12 +318,12 @@ class DecodeAttention:
     def record(self, plan, q, keys, values, q_and_gate, out):
         _need(q, torch.float32, "q"), _need(keys, torch.float16, "keys"), _need(values, torch.float16, "values")
         _need(q_and_gate, torch.float32, "q_and_gate"), _need(out, torch.float32, "out")
-        p, tp, po, pml = self._params(), plan.params, self.part_o, self.part_ml
+        p, tp, po, pml, flags = self._params(), plan.params, self.part_o, self.part_ml, self._flags()
 
         def launch(stage):
             def f(s):
                 ffi.check(ffi.lib().saetta_attn_decode(s, _ptr(q), _ptr(keys), _ptr(values), _ptr(po), _ptr(pml),
-                                                       _ptr(q_and_gate), _ptr(out), p, _ptr(tp), stage),
+                                                       _ptr(q_and_gate), _ptr(out), p, _ptr(tp), stage | flags),
                           "attn_decode")
             return f
 
@@ -329,12 +335,12 @@ class DecodeAttention:
             raise ValueError("a half cache goes through record")
         _need(q, torch.float32, "q"), _need(q_and_gate, torch.float32, "q_and_gate"), _need(out, torch.float32, "out")
         p, tp, po, pml, bits = self._params(), plan.params, self.part_o, self.part_ml, keys.bits.value
-        kc, vc = keys.c(), values.c()
+        kc, vc, flags = keys.c(), values.c(), self._flags()
 
         def launch(stage):
             def f(s):
                 ffi.check(ffi.lib().saetta_attn_decode_quant(s, bits, _ptr(q), kc, vc, _ptr(po), _ptr(pml),
-                                                             _ptr(q_and_gate), _ptr(out), p, _ptr(tp), stage),
+                                                             _ptr(q_and_gate), _ptr(out), p, _ptr(tp), stage | flags),
                           "attn_decode_quant")
             return f
 

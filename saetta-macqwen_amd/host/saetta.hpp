@@ -518,17 +518,20 @@ class DecodeAttention {
         part_o_ = gpu.buffer(saetta_part_o_bytes(uint32_t(heads), uint32_t(capacity), 1));
         part_ml_ = gpu.buffer(saetta_part_ml_bytes(uint32_t(heads), uint32_t(capacity), 1));
     }
+    // "attention_partial_mma": the library picks (the kernel with loader waves for one row over
+    // codes in a large cache); "attention_partial": the register kernels only (src/attention.rs:36-38).
     std::string kernel = "attention_partial_mma";
 
     void record(plan::Plan &plan, const View &q, const View &keys, const View &values, const View &q_and_gate, const View &out) const {
         const auto p = params();
+        const uint32_t flags = this->flags();
         const View tp = plan.params;
         const gpu::Buffer po = part_o_, pml = part_ml_;
         auto launch = [=](uint32_t stage) {
             return [=](hipStream_t s) {
                 check(saetta_attn_decode(s, q.ptr<float>(), keys.ptr<uint16_t>(), values.ptr<uint16_t>(), static_cast<float *>(po.get()),
                                          static_cast<float *>(pml.get()), q_and_gate.ptr<float>(), out.ptr<float>(), p,
-                                         tp.ptr<saetta_token_params>(), stage),
+                                         tp.ptr<saetta_token_params>(), stage | flags),
                       "attn_decode");
             };
         };
@@ -543,11 +546,12 @@ class DecodeAttention {
         const gpu::Buffer po = part_o_, pml = part_ml_;
         const kv_quant::QuantRows k = keys, v = values;
         const int nbits = int(kv_quant::bits(keys.bits));
+        const uint32_t flags = this->flags();
         auto launch = [=](uint32_t stage) {
             return [=](hipStream_t s) {
                 check(saetta_attn_decode_quant(s, nbits, q.ptr<float>(), k.c(), v.c(), static_cast<float *>(po.get()),
                                                static_cast<float *>(pml.get()), q_and_gate.ptr<float>(), out.ptr<float>(), p,
-                                               tp.ptr<saetta_token_params>(), stage),
+                                               tp.ptr<saetta_token_params>(), stage | flags),
                       "attn_decode_quant");
             };
         };
@@ -556,6 +560,11 @@ class DecodeAttention {
     }
 
   private:
+    uint32_t flags() const {
+        if (kernel == "attention_partial_mma") return 0;
+        if (kernel == "attention_partial") return SAETTA_STAGE_NO_LOADERS;
+        throw std::runtime_error("no decode attention kernel " + kernel);
+    }
     saetta_decode_params params() const {
         return saetta_decode_params{uint32_t(heads_), uint32_t(kv_heads_), uint32_t(capacity_), 1.0f / std::sqrt(float(DIM))};
     }

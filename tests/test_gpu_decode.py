@@ -98,12 +98,14 @@ def test_verify_rows_match_single_row_decodes(kind, m):
             assert np.abs(one - got[r]).max() < 1e-4
 
 
-@pytest.mark.parametrize("kind", [saetta.KvBits.Eight, saetta.KvBits.Four])
-def test_long_context_with_outlier_channels(kind):
-    # configs[1]/[3] in shape: 8-bit at 32768 + m rows, 4-bit with 1 % of channels x8; the new
-    # tokens are quantized on the device into the rows after the context.
-    rng = np.random.default_rng(8)
-    ctx, m = (32768, 4) if kind is saetta.KvBits.Eight else (20000, 1)
+@pytest.mark.parametrize("kind,m", [(saetta.KvBits.Eight, 2), (saetta.KvBits.Eight, 3), (saetta.KvBits.Eight, 4),
+                                    (saetta.KvBits.Four, 1)])
+def test_long_context_with_outlier_channels(kind, m):
+    # configs[1] in full: 8-bit at 32768 + m rows for m = 2, 3, 4 (m = 1 at this size is in
+    # test_large_cache_of_codes_one_row); 4-bit at 20000 with 1 % of channels x8; the new tokens are
+    # quantized on the device into the rows after the context.
+    rng = np.random.default_rng(8 + m)
+    ctx = 32768 if kind is saetta.KvBits.Eight else 20000
     capacity = -(-(ctx + m) // 128) * 128
     k = rng.standard_normal((ctx + m, VALUES)).astype(np.float32)
     v = rng.standard_normal((ctx + m, VALUES)).astype(np.float32)
@@ -130,6 +132,79 @@ def test_long_context_with_outlier_channels(kind):
     want64 = oracle.rows(q, kf, vf, ctx, m, q_and_gate=qg, threads=8, f64=True)
     # Outlier channels carry values 8x larger: the absolute bound scales with them.
     assert np.abs(got - want64).max() < MAX_ABS_F64 * max(1.0, np.abs(want64).max())
+
+
+def poison_from(cache, bits, token):
+    """Everything from row `token` on as uninitialised memory might look: NaN scales, Inf biases,
+    all-ones codes."""
+    cache.scales[token * 8:] = float("nan")
+    cache.biases[token * 8:] = float("inf")
+    cache.data[token * 8 * 2 * bits:] = -1
+
+
+def test_four_bit_150k_tokens_with_append():
+    # configs[3] in full: one query token over 150 000 cached tokens of 4-bit codes with 1 % of the
+    # channels scaled x8, capacity 150 016, the step's 4 new tokens quantized on the device into
+    # the rows after them.  A one-row launch over 4-bit codes in a cache this large takes the
+    # two-workgroups-per-CU kernel and 256 splits.  Then two shorter contexts in the same cache
+    # (fewer blocks than splits; ragged iterations), the rows past them poisoned.
+    kind, bits, ctx, new = saetta.KvBits.Four, 4, 150000, 4
+    capacity = 150016
+    rng = np.random.default_rng(150)
+    k = rng.standard_normal((ctx + new, VALUES)).astype(np.float32)
+    v = rng.standard_normal((ctx + new, VALUES)).astype(np.float32)
+    ch = rng.choice(VALUES, 5, replace=False)
+    k[:, ch] *= 8
+    v[:, ch] *= 8
+    q = rng.standard_normal(H * D).astype(np.float32)
+    qg = rng.standard_normal(H * 2 * D).astype(np.float32)
+    kc, vc, kf, vf = cache_pair(k[:ctx], v[:ctx], kind, capacity)
+    kc.encode(dev(k[ctx:].reshape(-1)), ctx, new)
+    vc.encode(dev(v[ctx:].reshape(-1)), ctx, new)
+    # the appended rows are the oracle quantizer's rows, bit for bit
+    for cache, x in ((kc, k), (vc, v)):
+        data, scales, biases = oracle.quantize(x[ctx:], bits)
+        assert np.array_equal(host(cache.data[ctx * 64:(ctx + new) * 64]).view(np.uint32), data.reshape(-1))
+        assert np.array_equal(host(cache.scales[ctx * 8:(ctx + new) * 8]).view(np.uint16), scales.reshape(-1))
+        assert np.array_equal(host(cache.biases[ctx * 8:(ctx + new) * 8]).view(np.uint16), biases.reshape(-1))
+    kf = np.concatenate([kf, oracle.round_trip(k[ctx:], bits)])
+    vf = np.concatenate([vf, oracle.round_trip(v[ctx:], bits)])
+    att = saetta.DecodeAttention(H, KV, D, capacity)
+    for length in (ctx + new, 70001, 1):
+        poison_from(kc, bits, length), poison_from(vc, bits, length)
+        got = run_decode(att, kind, dev(q), kc, vc, dev(qg), length)
+        assert np.isfinite(got).all(), length
+        want64 = oracle.attention_f64(q, kf, vf, qg, length, threads=8)
+        worst = np.abs(got - want64).max()
+        assert worst < MAX_ABS_F64 * max(1.0, np.abs(want64).max()), (length, worst)
+        want32 = oracle.attend(q, kf, vf, length, q_and_gate=qg, threads=8)
+        assert oracle.rel_rms(got, want32) < REL_RMS, length
+
+
+@pytest.mark.parametrize("kind", [saetta.KvBits.Eight, saetta.KvBits.Four])
+@pytest.mark.parametrize("capacity", [81920, 98304])
+def test_register_kernels_one_row_over_codes(kind, capacity):
+    # DecodeAttention.kernel = "attention_partial" (the reference's switch between its kernel
+    # families, src/attention.rs:36-38) keeps one row over codes on the kernels that load the cache
+    # into registers: one workgroup per CU up to 80k tokens of capacity, two per CU and 256 splits
+    # above.  Same lengths and poisoned tails as for the kernel with loader waves.
+    rng = np.random.default_rng(78)
+    k = (rng.standard_normal((capacity, VALUES)) * 2.0).astype(np.float32)
+    v = rng.standard_normal((capacity, VALUES)).astype(np.float32)
+    q = rng.standard_normal(H * D).astype(np.float32)
+    qg = rng.standard_normal(H * 2 * D).astype(np.float32)
+    att = saetta.DecodeAttention(H, KV, D, capacity)
+    att.kernel = "attention_partial"
+    kc, vc, kf, vf = cache_pair(k, v, kind, capacity, poison=False)
+    for length in [capacity, 50001, 33000, 4100, 100, 1]:
+        poison_from(kc, kind.value, length), poison_from(vc, kind.value, length)
+        got = run_decode(att, kind, dev(q), kc, vc, dev(qg), length)
+        assert np.isfinite(got).all(), length
+        worst = np.abs(got - oracle.attention_f64(q, kf, vf, qg, length, threads=8)).max()
+        assert worst < MAX_ABS_F64, (length, worst)
+    att.kernel = "attention_partial_simd"
+    with pytest.raises(ValueError):
+        run_decode(att, kind, dev(q), kc, vc, dev(qg), 10)
 
 
 def test_one_plan_serves_every_position():
