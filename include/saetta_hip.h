@@ -235,6 +235,24 @@ int saetta_attn_decode_quant(saetta_stream_t stream, int bits, const float *q,
                              saetta_decode_params p, const saetta_token_params *d_tp,
                              uint32_t stages);
 
+/* saetta_attn_decode_quant without the part_o / part_ml arguments, for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): the partials go to a buffer that is part of the library's code object, 4 MiB + 32 KiB
+ * per device (saetta_static_scratch_bytes), and the call allocates nothing.  It has no counterpart
+ * in the reference, whose DecodeAttention::new allocates its scratch (src/attention.rs:58-64).
+ * Limit: p.heads <= 16 (any capacity: a launch never uses more than 256 splits); more is rejected
+ * with SAETTA_E_SCRATCH.  Same kernels, same results, bit for bit, as saetta_attn_decode_quant.
+ * All calls on one device share the one buffer: between the partial stage of a call and its reduce
+ * stage no other call of this entry point may run on that device, so calls from different streams
+ * or threads that overlap on a device race.  Nothing in the buffer needs clearing: every slot the
+ * reduce stage reads was written by the partial stage of the same call.  saetta_init (or any
+ * earlier call on the device) must have run outside stream capture. */
+size_t saetta_static_scratch_bytes(void);
+int saetta_attn_decode_quant_static(saetta_stream_t stream, int bits, const float *q,
+                                    saetta_quant_rows keys, saetta_quant_rows values,
+                                    const float *q_and_gate, float *out, saetta_decode_params p,
+                                    const saetta_token_params *d_tp, uint32_t stages);
+
 /* AttentionRows::record (src/rows.rs:369-412): p.rows query tokens over a
  * half cache; row r is at position d_tp->position + r and sees
  * min(d_tp->position + r + 1, capacity) tokens.  q f32 [rows][heads][256],

@@ -1038,6 +1038,19 @@ struct ReduceArgs {
 
 constexpr uint32_t MAX_SPLITS = 256;  // workgroups per kv head: 2 kv heads fill 512 slots of 256 CUs
 
+// Partials of saetta_attn_decode_quant_static, the entry point that allocates nothing: room for one
+// query row, 16 q heads and the most splits a launch uses: part_o f32 [256][16][256] (4 MiB), then
+// part_ml f32 [256][16][2] (32 KiB).  Every device the library runs on holds its own copy of the
+// array at its own address, until the process ends.  In host code the array's name is only a
+// stand-in for hipGetSymbolAddress, never a device address: setup_decode asks for the address once
+// per device and everything else uses g_static_scratch[device].
+constexpr uint32_t STATIC_MAX_HEADS = 16;
+constexpr size_t STATIC_PART_O_FLOATS = size_t(MAX_SPLITS) * STATIC_MAX_HEADS * DIM;
+constexpr size_t STATIC_PART_ML_FLOATS = size_t(MAX_SPLITS) * STATIC_MAX_HEADS * 2;
+static __device__ __align__(256) float scratch[STATIC_PART_O_FLOATS + STATIC_PART_ML_FLOATS];
+constexpr int STATIC_MAX_DEVICES = 64;
+float *g_static_scratch[STATIC_MAX_DEVICES] = {};
+
 __global__ __launch_bounds__(256) void attention_reduce_kernel(ReduceArgs a) {
     __shared__ float w_lds[MAX_SPLITS];
     __shared__ float red[8];
@@ -1236,6 +1249,15 @@ int raise_lds_of_bits() {
 
 int setup_decode() {
     if (int rc = load_kernel(reinterpret_cast<const void *>(attention_reduce_kernel))) return rc;
+    {
+        // (runs once per device, with that device current)
+        int dev = 0;
+        if (hipError_t e = hipGetDevice(&dev)) return int(e);
+        if (dev < 0 || dev >= STATIC_MAX_DEVICES) return int(hipErrorInvalidDevice);
+        float *ptr = nullptr;
+        if (hipError_t e = hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch))) return int(e);
+        g_static_scratch[dev] = ptr;
+    }
     static_assert(Shape<8, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA) <= 160 * 1024, "LDS of a CU");
     if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_partial_kernel_d<8>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1283,6 +1305,31 @@ extern "C" int saetta_attn_decode_quant(saetta_stream_t stream, int bits, const 
     return run_attention(as_stream(stream), bits, q, keys.data, values.data, keys.scales, keys.biases,
                          values.scales, values.biases, part_o, part_ml, q_and_gate, out, p.heads,
                          p.kv_heads, p.capacity, p.scale, 1, 0, d_tp, true, stages, "attn_decode_quant");
+}
+
+extern "C" size_t saetta_static_scratch_bytes(void) { return sizeof(float) * (STATIC_PART_O_FLOATS + STATIC_PART_ML_FLOATS); }
+
+extern "C" int saetta_attn_decode_quant_static(saetta_stream_t stream, int bits, const float *q,
+                                               saetta_quant_rows keys, saetta_quant_rows values,
+                                               const float *q_and_gate, float *out, saetta_decode_params p,
+                                               const saetta_token_params *d_tp, uint32_t stages) {
+    SAETTA_REQUIRE(bits == 8 || bits == 4, SAETTA_E_BITS, "attn_decode_quant_static: bits %d (8 or 4)", bits);
+    // What the partials of this launch need against what the static array holds (the number of
+    // splits never exceeds 256, so only the heads can outgrow it).
+    const size_t need = saetta_part_o_bytes(p.heads, p.capacity, 1) + saetta_part_ml_bytes(p.heads, p.capacity, 1);
+    SAETTA_REQUIRE(p.heads <= STATIC_MAX_HEADS && need <= saetta_static_scratch_bytes(), SAETTA_E_SCRATCH,
+                   "attn_decode_quant_static: %u heads need %zu bytes of partials, the static scratch holds %zu "
+                   "(up to %u heads); use saetta_attn_decode_quant with scratch of the caller's",
+                   p.heads, need, saetta_static_scratch_bytes(), STATIC_MAX_HEADS);
+    if (int rc = ensure_device()) return rc;
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev)) return fail(int(e), "attn_decode_quant_static: %s", hipGetErrorString(e));
+    float *part_o = (dev >= 0 && dev < STATIC_MAX_DEVICES) ? g_static_scratch[dev] : nullptr;
+    SAETTA_REQUIRE(part_o, SAETTA_E_DEVICE, "attn_decode_quant_static: no static scratch on device %d", dev);
+    return run_attention(as_stream(stream), bits, q, keys.data, values.data, keys.scales, keys.biases,
+                         values.scales, values.biases, part_o, part_o + STATIC_PART_O_FLOATS, q_and_gate, out,
+                         p.heads, p.kv_heads, p.capacity, p.scale, 1, 0, d_tp, true, stages,
+                         "attn_decode_quant_static");
 }
 
 extern "C" int saetta_attn_rows(saetta_stream_t stream, const float *q, const uint16_t *keys,

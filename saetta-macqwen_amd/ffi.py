@@ -9,7 +9,7 @@ LIB_PATH = os.environ.get("SAETTA_HIP_LIB") or os.path.join(_HERE, "lib", "libsa
 SYMBOLS = [
     "saetta_init", "saetta_last_error", "saetta_kv_quantize", "saetta_kv_dequantize", "saetta_kv_dequantize_f32", "saetta_to_half", "saetta_attn_prep_store", "saetta_deltanet_conv", "saetta_deltanet_step", "saetta_deltanet_conv_rows", "saetta_deltanet_rows", "saetta_deltanet_token", "saetta_deltanet_rows_fused",
     "saetta_part_o_bytes", "saetta_part_ml_bytes", "saetta_attn_decode", "saetta_attn_decode_quant",
-    "saetta_attn_rows", "saetta_attn_rows_quant", "saetta_prefill_workspace_bytes", "saetta_attn_prefill", "saetta_attn_prefill_quant",
+    "saetta_attn_rows", "saetta_attn_rows_quant", "saetta_static_scratch_bytes", "saetta_attn_decode_quant_static", "saetta_prefill_workspace_bytes", "saetta_attn_prefill", "saetta_attn_prefill_quant",
 ]
 
 STAGE_PARTIAL, STAGE_REDUCE, STAGE_ALL, STAGE_NO_LOADERS = 1, 2, 3, 4
@@ -89,6 +89,9 @@ def lib():
         l.saetta_attn_decode_quant.restype = i32
         l.saetta_attn_decode_quant.argtypes = [vp, i32, vp, QuantRowsC, QuantRowsC, vp, vp, vp, vp,
                                                DecodeParamsC, vp, u32]
+        l.saetta_static_scratch_bytes.restype, l.saetta_static_scratch_bytes.argtypes = sz, []
+        l.saetta_attn_decode_quant_static.restype = i32
+        l.saetta_attn_decode_quant_static.argtypes = [vp, i32, vp, QuantRowsC, QuantRowsC, vp, vp, DecodeParamsC, vp, u32]
         l.saetta_attn_rows.restype = i32
         l.saetta_attn_rows.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, RowsParamsC, vp, u32]
         l.saetta_attn_rows_quant.restype = i32
