@@ -194,8 +194,14 @@ def bench_decode(s, torch, args, ctx, bits, rows, layers):
                 s.ffi.lib().saetta_kv_quantize(st, bits, ctypes.c_void_p(x_new.data_ptr()), c, p, None, ctx), "kv_quantize"))
     append_us = kernel_us(append.build(graph))[0] if not half else 0.0
 
+    # The floor of a launch of this size: a plain read of the same bytes by 256 workgroups.
+    del caches, k0, v0
+    torch.cuda.empty_cache()
+    reader, empty_us = reader_floor(s, torch, args, layer_bytes, layers) if not args.no_reader_floor else ({}, None)
+    reader_us = min(reader.values()) if reader else None
+
     name = f"decode attention, {bits}-bit KV, ctx {ctx}, {rows} query row(s), {layers} layer caches per step"
-    return {
+    res = {
         "metric": f"decode attn HBM GB/s @{ctx // 1024}k ctx {bits}-bit KV",
         "value": round(value, 1),
         "unit": "GB/s",
@@ -203,18 +209,94 @@ def bench_decode(s, torch, args, ctx, bits, rows, layers):
         "dtype": "f16 cache, f16 MFMA, f32 accumulate" if half else "u8 codes, f16 MFMA, f32 accumulate",
         "config": {"workload": name, "heads": H, "kv_heads": KV, "head_dim": D, "ctx": ctx, "kv_bits": bits,
                    "rows": rows, "layers_per_step": layers, "bytes_per_layer": layer_bytes,
-                   "append_4_tokens_k_and_v_us_per_layer": None if half else round(append_us, 3)},
+                   "append_4_tokens_k_and_v_us_per_layer": None if half else round(append_us, 3),
+                   "inputs": "K, V, q, gate ~ N(0,1) from torch's device generator (Philox, seed 1234), not the "
+                             "reference tests' LCG + Box-Muller stream; caches quantized on the device by the "
+                             "library's quantizer" + ("; channels 7, 101, 230, 333, 460 of the 512 scaled x8 as "
+                                                      "outlier channels" if bits == 4 else "")},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get({(32768, 8, 1): "decode8_32k", (150000, 4, 1): "decode4_150k",
                                                       (32768, 8, 4): "verify4"}.get((ctx, bits, rows))),
                      "kernel": "attention_partial_kernel", "avg_us": round(part_us, 3),
-                     "min_us": round(part_us_min, 3), "reduce_kernel_us": round(red_us, 3)},
+                     "min_us": round(part_us_min, 3), "reduce_kernel_us": round(red_us, 3),
+                     "reader_us": reader_us, "reader_variants_us": reader, "empty_launch_us": empty_us,
+                     "frac_of_reader": round(reader_us / part_us, 4) if reader_us else None},
         "cpu_baseline": {"value": round(layer_bytes / cpu1 / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
                          "sample": f"one of the {layers} layer caches, full shape, median of repeats; "
                                    f"{cpu1 * 1e3:.1f} ms per layer",
                          "all_cores": {"value": round(layer_bytes / cpun / 1e9, 4), "cores": threads_all,
                                        "ms": round(cpun * 1e3, 2)}},
         "parity_rel_rms_vs_oracle": float(f"{rel_rms:.3e}"),
+    }
+    return res
+
+
+_calib = None
+
+
+def calib_lib(s):
+    """The calibration kernels (a plain streaming read): a library of their own beside the product's."""
+    global _calib
+    if _calib is None:
+        import ctypes
+        path = os.path.join(os.path.dirname(s.ffi.LIB_PATH), "libsaetta_calib.so")
+        _calib = ctypes.CDLL(path)
+        _calib.saetta_calib_read.restype = ctypes.c_int
+        _calib.saetta_calib_read.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint32,
+                                             ctypes.c_uint32, ctypes.c_void_p]
+    return _calib
+
+
+def reader_floor(s, torch, args, nbytes, layers, workgroups=256):
+    """How long one launch of `workgroups` workgroups takes to READ nbytes from HBM and do nothing
+    else: `layers` buffers of their own (as the layer caches are), one launch each, replayed from a
+    HIP graph and timed with events like the attention kernels.  Returns {variant: us per launch}
+    and the time of an empty launch in the same setting (a read of 16 bytes per workgroup)."""
+    import ctypes
+    lib = calib_lib(s)
+    nbytes = nbytes // 16 * 16
+    bufs = [torch.full((nbytes // 4,), -1, dtype=torch.int32, device="cuda") for _ in range(layers)]
+    sink = torch.zeros(1024, dtype=torch.int32, device="cuda")
+    names = {0: "256 threads x 8 loads", 1: "512 x 4", 2: "1024 x 4", 3: "1024 x 2"}
+
+    def timed(variant, size):
+        plan = s.Plan()
+        for b in bufs:
+            plan.op("calib_read", lambda st, b=b: s.ffi.check(lib.saetta_calib_read(
+                st, ctypes.c_void_p(b.data_ptr()), size, workgroups, variant, ctypes.c_void_p(sink.data_ptr())), "calib_read"))
+        built = plan.build(graph=not args.no_graph)
+        for _ in range(args.warmup):
+            built.run()
+        ts = []
+        for _ in range(max(5, args.steps)):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            built.run()
+            e1.record()
+            e1.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e3 / layers)
+        return median(ts)
+
+    out = {names[v]: round(timed(v, nbytes), 3) for v in names}
+    empty = round(timed(0, 16 * workgroups), 3)
+    assert int(sink.sum().item()) == 0
+    return out, empty
+
+
+def bench_reader_floor(s, torch, args, ctx=32768, layers=32):
+    nbytes = (ctx + 1) * 1088
+    variants, empty = reader_floor(s, torch, args, nbytes, layers)
+    best = min(variants.values())
+    return {
+        "metric": "plain streaming read of one layer's KV bytes, GB/s",
+        "value": round(nbytes / best / 1e3, 1), "unit": "GB/s", "ms_per_step": round(best * layers / 1e3, 4),
+        "dtype": "u32x4 loads",
+        "config": {"workload": f"calibration: one launch of 256 workgroups reads {nbytes} bytes and computes nothing, "
+                               f"{layers} buffers per step", "us_per_launch": variants, "empty_launch_us": empty},
+        "roofline": {"bound": "hbm", "achieved": round(nbytes / best / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(nbytes / best / 1e3 / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "calib_read_kernel",
+                     "avg_us": best},
+        "cpu_baseline": None,
     }
 
 
@@ -262,7 +344,7 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8):
     kern_us = median(ts)
     achieved = flops / (kern_us * 1e-6) / 1e12
     # CPU baseline on a bounded sample: the last `sample` tokens of the chunk (the longest rows).
-    sample = 8
+    sample = 512  # about 7 s on one core
     groups = (pos + tokens) * 8
 
     def deq(rows_q):
@@ -287,7 +369,10 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8):
         "dtype": "f16 MFMA, f32 softmax state",
         "config": {"workload": f"causal prefill chunk of {tokens} tokens at position {pos}, {bits}-bit KV cache "
                                "read in place, chunk K/V quantized on append inside the step",
-                   "heads": H, "kv_heads": KV, "head_dim": D, "flops": flops},
+                   "heads": H, "kv_heads": KV, "head_dim": D, "flops": flops,
+                   "timing": "value: wall time of steps (2 x kv_quantize of the chunk + prepare + attention); "
+                             "roofline: median of event-timed prepare + attention calls",
+                   "inputs": "q (through bf16), K, V, gate ~ N(0,1) from torch's device generator (Philox, seed 99)"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC.get("prefill") if (tokens, pos, bits) == (4096, 4096, 8) else None,
@@ -553,11 +638,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="decode8_32k",
+    ap.add_argument("--workload", default="default",
                     choices=["decode8_32k", "decode4_150k", "decode16_4k", "verify2", "verify3", "verify4", "prefill", "deltanet",
-                             "deltanet_prefill", "prep_store", "all"])
+                             "deltanet_prefill", "prep_store", "reader_floor", "default", "all"])
     ap.add_argument("--no-graph", action="store_true", help="launch from Python instead of replaying a HIP graph")
     ap.add_argument("--layers", type=int, default=0, help="layer caches per step (default 32; 12 at 150k)")
+    ap.add_argument("--no-reader-floor", action="store_true", help="skip the plain-read calibration of the decode workloads")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run a plain device copy of 256 MiB (three times): a kernel of known traffic for a "
                          "hardware-counter run of the same command to be scaled by")
@@ -596,17 +682,25 @@ def main():
             return bench_deltanet_prefill(s, torch, args)
         if workload == "prep_store":
             return bench_prep_store(s, torch, args)
+        if workload == "reader_floor":
+            return bench_reader_floor(s, torch, args)
         return bench_prefill(s, torch, args)
 
-    if args.workload == "all":
+    if args.workload in ("default", "all"):
+        # Both halves of the metric in one line: the decode record at the top level, the
+        # prefill-chunk record (same keys) under "prefill".
         res = one("decode8_32k")
+        res["metric"] = "decode attn HBM GB/s @32k ctx 8-bit KV; prefill-chunk attn TFLOP/s"
+        torch.cuda.empty_cache()
+        res["prefill"] = one("prefill")
+    if args.workload == "all":
         res["other_workloads"] = {}
-        for w in ["verify2", "verify3", "verify4", "decode4_150k", "decode16_4k", "prefill", "deltanet", "deltanet_prefill", "prep_store"]:
+        for w in ["verify2", "verify3", "verify4", "decode4_150k", "decode16_4k", "deltanet", "deltanet_prefill", "prep_store"]:
             torch.cuda.empty_cache()
             r = one(w)
             res["other_workloads"][w] = {k: r[k] for k in ("metric", "value", "unit", "ms_per_step", "roofline",
                                                             "parity_rel_rms_vs_oracle")}
-    else:
+    elif args.workload != "default":
         res = one(args.workload)
     res.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
                 "scaling": "weak", "vs_baseline": None, "data": "synthetic"})
