@@ -60,7 +60,8 @@ def median(xs):
 def make_decode_workload(s, torch, ctx, bits, rows, layers, seed=1234):
     """LAYERS caches of ctx + rows tokens, quantized on the device from N(0,1)."""
     kind = {8: s.KvBits.Eight, 4: s.KvBits.Four, 16: s.KvBits.Half}[bits]
-    capacity = (ctx + rows + 127) // 128 * 128
+    # room for the query rows' tokens and for the 4 tokens the append timing writes at ctx .. ctx + 3
+    capacity = (ctx + max(rows, 4) + 127) // 128 * 128
     gen = torch.Generator(device="cuda").manual_seed(seed)
     caches = []
     chunk = 8192
@@ -185,6 +186,7 @@ def bench_decode(s, torch, args, ctx, bits, rows, layers):
     # layer, rows ctx .. ctx + 3; last, because it writes over the rows the check above read).
     import ctypes
     new_tokens = 4
+    assert ctx + new_tokens <= capacity, "the appended rows must lie inside the caches"
     x_new = torch.randn(new_tokens, VALUES, device="cuda")
     append = s.Plan()
     for k, v in ([] if half else caches):
@@ -643,6 +645,7 @@ def main():
                              "deltanet_prefill", "prep_store", "reader_floor", "default", "all"])
     ap.add_argument("--no-graph", action="store_true", help="launch from Python instead of replaying a HIP graph")
     ap.add_argument("--layers", type=int, default=0, help="layer caches per step (default 32; 12 at 150k)")
+    ap.add_argument("--ctx", type=int, default=0, help="context length of the decode and verify workloads (default: the workload's own)")
     ap.add_argument("--no-reader-floor", action="store_true", help="skip the plain-read calibration of the decode workloads")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run a plain device copy of 256 MiB (three times): a kernel of known traffic for a "
@@ -669,13 +672,13 @@ def main():
 
     def one(workload):
         if workload == "decode8_32k":
-            return bench_decode(s, torch, args, 32768, 8, 1, args.layers or 32)
+            return bench_decode(s, torch, args, args.ctx or 32768, 8, 1, args.layers or 32)
         if workload == "decode4_150k":
             return bench_decode(s, torch, args, 150000, 4, 1, args.layers or 12)
         if workload == "decode16_4k":
             return bench_decode(s, torch, args, 4096, 16, 1, args.layers or 32)
         if workload.startswith("verify"):
-            return bench_decode(s, torch, args, 32768, 8, int(workload[-1]), args.layers or 32)
+            return bench_decode(s, torch, args, args.ctx or 32768, 8, int(workload[-1]), args.layers or 32)
         if workload == "deltanet":
             return bench_deltanet(s, torch, args)
         if workload == "deltanet_prefill":
