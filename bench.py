@@ -259,7 +259,8 @@ def reader_floor(s, torch, args, nbytes, layers, workgroups=256):
     nbytes = nbytes // 16 * 16
     bufs = [torch.full((nbytes // 4,), -1, dtype=torch.int32, device="cuda") for _ in range(layers)]
     sink = torch.zeros(1024, dtype=torch.int32, device="cuda")
-    names = {0: "256 threads x 8 loads", 1: "512 x 4", 2: "1024 x 4", 3: "1024 x 2"}
+    names = {0: "256 threads x 8 loads", 1: "512 x 4", 2: "1024 x 4", 3: "1024 x 2",
+             4: "to LDS, 4 waves", 5: "to LDS, 8 waves", 6: "to LDS, 12 waves", 7: "to LDS, 16 waves"}
 
     def timed(variant, size):
         plan = s.Plan()

@@ -29,9 +29,39 @@ __global__ __launch_bounds__(THREADS) void calib_read_kernel(const u32x4 *src, s
     // never true for the data bench.py fills in (all ones), but the compiler cannot know
     if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[blockIdx.x] = acc.x;
 }
+
+// The same read through the path the decode kernel uses: workgroup w brings its share into LDS
+// with global_load_lds_dwordx4 (1 KB per instruction, no registers), WAVES waves each issuing
+// every WAVES-th instruction of the share back to back, then waiting for all of them.  The share
+// must fit the 160 KB of LDS (it does for 256 workgroups and one layer's 35 MB).
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void calib_dma_kernel(const unsigned char *src, size_t bytes, uint32_t *sink) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    const size_t per = (bytes / 1024 + gridDim.x - 1) / gridDim.x;  // instructions per workgroup
+    const size_t begin = per * blockIdx.x * 1024;
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(lds_raw));
+    const unsigned char *base = src + begin;
+    const size_t last = bytes - begin >= 16 ? bytes - begin - 16 : 0;  // loads past the buffer's end read its last 16 bytes
+    if (begin >= bytes) return;
+    for (uint32_t i = wave; i < per; i += WAVES) {
+        size_t off = size_t(i) * 1024 + lane * 16;
+        off = off < last ? off : last;
+        asm volatile("s_mov_b32 m0, %0\n"
+                     "s_nop 0\n"
+                     "global_load_lds_dwordx4 %1, %2\n"
+                     :
+                     : "s"(lds0 + i * 1024), "v"(uint32_t(off)), "s"(base)
+                     : "memory", "m0");
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const uint32_t v = *reinterpret_cast<const uint32_t *>(lds_raw + threadIdx.x * 4);
+    if (v == 0x9e3779b9u) sink[blockIdx.x] = v;
+}
 }  // namespace
 
-// variant: 0 = 256 threads x 8 loads in flight, 1 = 512 x 4, 2 = 1024 x 4, 3 = 1024 x 2
+// variant: 0 = 256 threads x 8 loads in flight, 1 = 512 x 4, 2 = 1024 x 4, 3 = 1024 x 2; 4..7 = to LDS with 4, 8, 12, 16 waves
 extern "C" int saetta_calib_read(void *stream, const void *src, size_t bytes, uint32_t workgroups, uint32_t variant,
                                  void *sink) {
     if (!src || !sink || bytes % 16 || !workgroups || (reinterpret_cast<uintptr_t>(src) & 15)) return -1;
@@ -44,6 +74,18 @@ extern "C" int saetta_calib_read(void *stream, const void *src, size_t bytes, ui
         case 1: calib_read_kernel<512, 4><<<workgroups, 512, 0, s>>>(p, n16, k); break;
         case 2: calib_read_kernel<1024, 4><<<workgroups, 1024, 0, s>>>(p, n16, k); break;
         case 3: calib_read_kernel<1024, 2><<<workgroups, 1024, 0, s>>>(p, n16, k); break;
+        case 4: case 5: case 6: case 7: {
+            // LDS-DMA readers: 4, 8, 12, 16 waves
+            const size_t lds = ((bytes / 1024 + workgroups - 1) / workgroups) * 1024;
+            if (lds > 160 * 1024) return -2;
+            const unsigned char *b = static_cast<const unsigned char *>(src);
+            void (*kern)(const unsigned char *, size_t, uint32_t *) =
+                variant == 4 ? calib_dma_kernel<4> : variant == 5 ? calib_dma_kernel<8> : variant == 6 ? calib_dma_kernel<12> : calib_dma_kernel<16>;
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)) return -3;
+            const int waves = variant == 4 ? 4 : variant == 5 ? 8 : variant == 6 ? 12 : 16;
+            kern<<<workgroups, waves * 64, lds < 4096 ? 4096 : lds, s>>>(b, bytes, k);
+            break;
+        }
         default: return -1;
     }
     return int(hipGetLastError());

@@ -1021,6 +1021,598 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel_p(PartialArg
     attention_partial_body<BITS, 1, true, ITB_ONE_PER_CU, true>(a);
 }
 
+// ---- one query row over codes, keys first ---------------------------------------------------------
+// attention_partial_kernel_s: the workgroup's share is taken in rounds of up to 17 blocks of 16
+// tokens whose codes all lie in LDS at once (17: a context of 128 x 256 tokens and a few more still
+// is one round).  The KEYS of a round are requested before its values, so they are there when half
+// of the round's bytes are, and everything that does not need a value code runs while the values
+// are still on their way: the scores of all the tokens, their softmax (every block relative to its
+// own maximum, by the wave that computed its scores; the blocks are joined by one factor per block
+// and head), and the probability operands P * value scale.  When the last values land, what is left
+// is one k-step of O += P V per wave (8 LDS reads, 16 byte permutes, 4 MFMAs), the merge of two
+// waves and the store.
+// Eight computing waves and four loader waves that move codes from global memory straight into LDS
+// (global_load_lds, no registers): two request the round's scales, biases and keys, and two, once
+// those requests are out, the values.  A loader waits for its own loads in order and raises a
+// counter in LDS when a part of the keys, or a 64-token slot of the values, has landed.  In phase A
+// computing wave w takes the blocks w and w + 8 (wave 0 also block 16); in phase C waves 2g and
+// 2g + 1 share quantization group g (dims 64g .. 64g + 63) and take alternate k-steps of 32 tokens,
+// so that each of the round's value slots gives every wave one k-step.
+// A wave that requests more than the memory pipeline takes stands still until it is accepted, so a
+// wave that requests values cannot tell anybody that earlier data is there: that is why the keys and
+// the values have different requesters, and why the waves meet through counters in LDS and not
+// through s_barrier (which would wait for the loaders to finish requesting).  LDS executes a wave's
+// instructions in order, so data written before a counter is raised is there when the counter is
+// seen.  Every wait on a counter is bounded (SPIN_LIMIT polls), so every wave ends whatever happens.
+// Longer shares take further rounds with an online softmax between the rounds.
+template <int BITS>
+struct KeysFirst {
+    static constexpr int LOADERS = 4, WAVES = 8;            // loader waves (keys: 0, 1; values: 2, 3), then the computing waves
+    static constexpr int K_LOADERS = 2, V_LOADERS = 2;
+    static constexpr int RB_ = BITS * 32;                   // bytes of a (token, kv head) row of codes
+    static constexpr int ROUND_BLOCKS = 17, ROUND_TOKENS = ROUND_BLOCKS * BLOCK;
+    static constexpr int KSTEPS = (ROUND_BLOCKS + 1) / 2;   // of 32 tokens; the last one is half there
+    static constexpr int SLOTS = (KSTEPS + 1) / 2;          // value slots of 64 tokens: 5, the last one block 16 alone
+    static constexpr int PIECES = RB_ / 16;
+    static constexpr int PER_BLOCK = PIECES / 4;            // load instructions per block of keys, and of values: 4 | 2
+    static constexpr int V_GROUP_TOKENS = 64 / PIECES;      // token rows one load instruction brings: 4 | 8
+    static constexpr int K_BLOCK_BYTES = BLOCK * RB_;       // [64-byte piece][token]: what one load instruction brings
+    static constexpr int V_GROUP_BYTES = 1024 + 32;         // whole token rows; 8 banks between the groups of the four lane groups
+    static constexpr int K_LOADS = 8 * PER_BLOCK;           // per key-loader wave: blocks 0-15, half of them before the other
+    static constexpr int V_LOADS = 8 * PER_BLOCK;           // per value-loader wave: slots 0-3
+    static constexpr int SC_LOADS = 16;                     // scales and biases of a key loader's 128 tokens: 4 arrays x 2 planes x 2
+    static constexpr int X_LOADS = 8 + PER_BLOCK;           // block 16: its scales and biases (4 arrays x 2 planes) and its keys
+    static_assert(SC_LOADS + K_LOADS + X_LOADS < 64, "vmcnt is 6 bits");
+    // LDS map, in bytes.  The scores of a block (its probabilities relative to the block's maximum,
+    // [head][token] f32, 512 bytes) lie over the block's own keys, which only the wave that writes
+    // them has read.
+    static constexpr int Q_OFF = 0;                                // [k-step][lane] half8
+    static constexpr int QZ_OFF = Q_OFF + 8 * 64 * 16;             // [hi, lo][lane][k-step] f16
+    // scales and biases: per array two planes of one dword per token, the f16 of groups (0, 1) and of (2, 3)
+    static constexpr int SB_OFF = QZ_OFF + 2 * 64 * 16;            // [ks | kz | vs | vz][plane][token] u32
+    static constexpr int SB_ARRAY = 2 * ROUND_TOKENS * 4;
+    static constexpr int BSTRIDE = 20;                             // blocks 17-19 never exist: maximum "none", sum 0
+    static constexpr int BMAX_OFF = SB_OFF + 4 * SB_ARRAY;         // [head][block] f32: the block's maximum score
+    static constexpr int BSUM_OFF = BMAX_OFF + 8 * BSTRIDE * 4;    // [head][block] f32: sum of 2^(score - maximum)
+    static constexpr int ZS_OFF = BSUM_OFF + 8 * BSTRIDE * 4;      // [wave][head] f32
+    static constexpr int SYNC_OFF = ZS_OFF + WAVES * 8 * 4;        // 32 counters, u32
+    static constexpr int K_OFF = (SYNC_OFF + 32 * 4 + 255) / 256 * 256;
+    static constexpr int V_OFF = K_OFF + ROUND_BLOCKS * K_BLOCK_BYTES;
+    static constexpr int LDS_BYTES = V_OFF + ROUND_BLOCKS * PER_BLOCK * V_GROUP_BYTES;
+    static constexpr int X_OFF = K_OFF;                            // the pairs' merge lies over the keys
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS of a CU");
+    // the counters
+    static constexpr int C_KEYS = 0;    // key loaders that have requested the first round's keys
+    static constexpr int C_QUERY = 1;   // computing waves that have written their query operands
+    static constexpr int C_SCORES = 2;  // ... written their scores (8 per round)
+    static constexpr int C_BUILT = 3;   // ... built their probability operands (8 per round)
+    static constexpr int C_DONE = 4;    // ... are through with the round's values (8 per round)
+    static constexpr int C_LENGTH = 5;  // (not a counter: the context length, for every wave)
+    static constexpr int C_KPART = 8;   // [3]: key loaders whose blocks 0-7 and scales | blocks 8-15 | block 16 have landed (2 per round)
+    static constexpr int C_SLOT = 12;   // [5]: value loaders whose values of slot s have landed (2 per round)
+    static constexpr int C_MERGE = 20;  // [4]: wave 2g + 1 has written its sums for wave 2g
+    static constexpr uint32_t SPIN_LIMIT = 1u << 20;
+};
+
+template <int BITS>
+__global__ __launch_bounds__((KeysFirst<BITS>::LOADERS + KeysFirst<BITS>::WAVES) * 64) void attention_partial_kernel_s(PartialArgs a) {
+    using W = KeysFirst<BITS>;
+    constexpr int RB = W::RB_, RT = W::ROUND_TOKENS, RBK = W::ROUND_BLOCKS;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    const int lane = threadIdx.x & 63;
+    const int wave_all = __builtin_amdgcn_readfirstlane(int(threadIdx.x) >> 6);
+    const int n = lane & 15, j = lane >> 4;
+    const uint32_t split = blockIdx.x, kv = blockIdx.y, kvh = a.kv_heads;
+    const bool loader = wave_all < W::LOADERS;
+    const int wave = wave_all - W::LOADERS;          // computing waves: 0..7
+    uint32_t *sync_lds = reinterpret_cast<uint32_t *>(lds_raw + W::SYNC_OFF);
+    const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(lds_raw));
+
+    // ---- query values: requested first (computing waves: thread = (k-step, lane) item) ----------
+    float qv[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (!loader) {
+        const int step = wave, g = step >> 1, ab = step & 1;
+        const float *src = a.q + (size_t(kv) * 8 + (n & 7)) * DIM + 64 * g + 16 * j + 8 * ab;
+        const float4 f0 = *reinterpret_cast<const float4 *>(src);
+        const float4 f1 = *reinterpret_cast<const float4 *>(src + 4);
+        qv[0] = f0.x, qv[1] = f0.y, qv[2] = f0.z, qv[3] = f0.w, qv[4] = f1.x, qv[5] = f1.y, qv[6] = f1.z, qv[7] = f1.w;
+    }
+
+    // ---- the context and this workgroup's share of it -----------------------------
+    // One wave of the workgroup reads the context length and hands it on through LDS.  The counters
+    // start at zero behind the same barrier, the only s_barrier of the kernel, before anybody
+    // requests anything of the cache.
+    if (threadIdx.x < 32) sync_lds[threadIdx.x] = threadIdx.x == W::C_LENGTH ? a.tp->kv_len : 0u;
+    __syncthreads();
+    const uint32_t max_len = min(uint32_t(__builtin_amdgcn_readfirstlane(sync_lds[W::C_LENGTH])), a.capacity);
+    const uint32_t nblocks = (max_len + BLOCK - 1) / BLOCK;
+    uint32_t blk_begin, blk_end;
+    if (nblocks <= a.nsplits) {
+        blk_begin = split;
+        blk_end = split + 1;
+        if (split >= nblocks) return;
+    } else {
+        blk_begin = split * nblocks / a.nsplits;
+        blk_end = (split + 1) * nblocks / a.nsplits;
+    }
+    const uint32_t limit = min(max_len, blk_end * BLOCK);  // tokens of this share end here
+    const uint32_t last_tok = limit - 1;                   // rows past it are never read: loads are clamped to it
+    const uint32_t range = blk_end - blk_begin;
+    const uint32_t n_rounds = (range + RBK - 1) / RBK;
+    auto blocks_of = [&](uint32_t round) { return min(range - round * RBK, uint32_t(RBK)); };
+
+    auto dma = [&](uint32_t lds_addr, uint32_t voff, const void *src) {
+        asm volatile("s_mov_b32 m0, %0\n"
+                     "s_nop 0\n"
+                     "global_load_lds_dwordx4 %1, %2\n"
+                     :
+                     : "s"(lds_addr), "v"(voff), "s"(src)
+                     : "memory", "m0");
+    };
+    auto dma4 = [&](uint32_t lds_addr, uint32_t voff, const void *src) {
+        asm volatile("s_mov_b32 m0, %0\n"
+                     "s_nop 0\n"
+                     "global_load_lds_dword %1, %2\n"
+                     :
+                     : "s"(lds_addr), "v"(voff), "s"(src)
+                     : "memory", "m0");
+    };
+    // counters: raised by one lane after the wave's LDS writes (LDS takes a wave's instructions in
+    // order); a waiting wave polls, a bounded number of times
+    auto raise = [&](int c) {
+        asm volatile("" ::: "memory");
+        if (lane == 0) __hip_atomic_fetch_add(sync_lds + c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        asm volatile("" ::: "memory");
+    };
+    auto peek = [&](int c) {
+        asm volatile("" ::: "memory");
+        const uint32_t v = __hip_atomic_load(sync_lds + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        asm volatile("" ::: "memory");
+        return uint32_t(__builtin_amdgcn_readfirstlane(v));
+    };
+    auto await = [&](int c, uint32_t want) {
+        asm volatile("" ::: "memory");
+        for (uint32_t i = 0; i < W::SPIN_LIMIT; i++) {
+            const uint32_t v = __hip_atomic_load(sync_lds + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (__builtin_amdgcn_readfirstlane(v) >= want) break;
+            __builtin_amdgcn_s_sleep(1);
+        }
+        asm volatile("" ::: "memory");
+    };
+
+    if (loader && wave_all < W::K_LOADERS) {
+        // ---- a key-loader wave: scales and biases of tokens 128 L .. 128 L + 127, keys of blocks L, L + 2, ...;
+        // loader 0 then block 16 with its scales and biases ----
+        const uint32_t L = uint32_t(wave_all);
+        const void *sb_src[4] = {a.kscales, a.kbiases, a.vscales, a.vbiases};
+        for (uint32_t round = 0; round < n_rounds; round++) {
+            const uint32_t base = (blk_begin + round * RBK) * BLOCK, nb = blocks_of(round);
+            // the round before: its scales are read until every wave has built its operands, its keys until every wave has its scores
+            if (round > 0) await(W::C_BUILT, W::WAVES * round);
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                // a dword per lane and load: the token's four f16 of an array go to two planes
+                const uint32_t voff = (min(base + 128 * L + 64 * h + lane, last_tok) * kvh + kv) * 8;
+#pragma unroll
+                for (int arr = 0; arr < 4; arr++) {
+#pragma unroll
+                    for (int pl = 0; pl < 2; pl++) dma4(lds0 + W::SB_OFF + arr * W::SB_ARRAY + (pl * RT + 128 * L + 64 * h) * 4, voff + 4 * pl, sb_src[arr]);
+                }
+            }
+            auto request_block = [&](uint32_t blk) {
+                // lane -> (token lane / 4, 16 bytes lane % 4 of the token's 64-byte piece i): four
+                // neighbouring lanes read 64 contiguous bytes
+                const uint32_t tok = min(base + BLOCK * blk + (lane >> 2), last_tok);
+                const uint32_t voff = (tok * kvh + kv) * RB + (lane & 3) * 16;
+#pragma unroll
+                for (int i = 0; i < W::PER_BLOCK; i++) dma(lds0 + W::K_OFF + blk * W::K_BLOCK_BYTES + i * 1024, voff + 64 * i, a.kdata);
+            };
+#pragma unroll
+            for (int r = 0; r < 8; r++) {
+                if (L + 2 * r < nb) request_block(L + 2 * r);
+            }
+            const bool extra = nb == uint32_t(RBK) && L == 0;
+            if (extra) {
+                if (lane < BLOCK) {
+                    const uint32_t voff = (min(base + 256 + lane, last_tok) * kvh + kv) * 8;
+#pragma unroll
+                    for (int arr = 0; arr < 4; arr++) {
+#pragma unroll
+                        for (int pl = 0; pl < 2; pl++) dma4(lds0 + W::SB_OFF + arr * W::SB_ARRAY + (pl * RT + 256) * 4, voff + 4 * pl, sb_src[arr]);
+                    }
+                }
+                request_block(16);
+            }
+            if (round == 0) raise(W::C_KEYS);
+            // loads return in order (a round of less than 16 blocks: all at once)
+            if (extra) {
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(W::K_LOADS / 2 + W::X_LOADS));
+                raise(W::C_KPART + 0);
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(W::X_LOADS));
+                raise(W::C_KPART + 1);
+            } else if (nb >= 16) {
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(W::K_LOADS / 2));
+                raise(W::C_KPART + 0);
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+                raise(W::C_KPART + 1);
+            } else {
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+                raise(W::C_KPART + 0);
+                raise(W::C_KPART + 1);
+            }
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+            raise(W::C_KPART + 2);
+        }
+        return;
+    }
+    if (loader) {
+        // ---- a value-loader wave: blocks L, L + 2, ... of every round, two of them in each 64-token slot;
+        // loader 0 then block 16 (slot 4) ----
+        const uint32_t L = uint32_t(wave_all) - W::K_LOADERS;
+        for (uint32_t round = 0; round < n_rounds; round++) {
+            const uint32_t base = (blk_begin + round * RBK) * BLOCK, nb = blocks_of(round);
+            // the keys of the first round have been requested | every wave is through with the values before
+            if (round == 0) {
+                await(W::C_KEYS, W::K_LOADERS);
+            } else {
+                await(W::C_DONE, W::WAVES * round);
+            }
+            auto request_block = [&](uint32_t blk) {
+#pragma unroll
+                for (int i = 0; i < W::PER_BLOCK; i++) {
+                    // lane -> (token lane / PIECES of the instruction's group, piece lane % PIECES)
+                    const uint32_t tok = min(base + BLOCK * blk + W::V_GROUP_TOKENS * i + lane / W::PIECES, last_tok);
+                    dma(lds0 + W::V_OFF + (W::PER_BLOCK * blk + i) * W::V_GROUP_BYTES, (tok * kvh + kv) * RB + (lane % W::PIECES) * 16, a.vdata);
+                }
+            };
+#pragma unroll
+            for (int r = 0; r < 8; r++) {
+                if (L + 2 * r < nb) request_block(L + 2 * r);
+            }
+            const bool extra = nb == uint32_t(RBK) && L == 0;
+            if (extra) request_block(16);
+            // loads return in order (a round of less than 16 blocks: all at once)
+            if (extra) {
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(W::V_LOADS * 3 / 4 + W::PER_BLOCK));
+                raise(W::C_SLOT + 0);
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(W::V_LOADS * 2 / 4 + W::PER_BLOCK));
+                raise(W::C_SLOT + 1);
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(W::V_LOADS * 1 / 4 + W::PER_BLOCK));
+                raise(W::C_SLOT + 2);
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(W::PER_BLOCK));
+                raise(W::C_SLOT + 3);
+            } else if (nb >= 16) {
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(W::V_LOADS * 3 / 4));
+                raise(W::C_SLOT + 0);
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(W::V_LOADS * 2 / 4));
+                raise(W::C_SLOT + 1);
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(W::V_LOADS * 1 / 4));
+                raise(W::C_SLOT + 2);
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+                raise(W::C_SLOT + 3);
+            } else {
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+                raise(W::C_SLOT + 0);
+                raise(W::C_SLOT + 1);
+                raise(W::C_SLOT + 2);
+                raise(W::C_SLOT + 3);
+            }
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+            raise(W::C_SLOT + 4);
+        }
+        return;
+    }
+
+    // ---- computing waves ------------------------------------------------------------------------
+    half8 *q_lds = reinterpret_cast<half8 *>(lds_raw + W::Q_OFF);
+    _Float16 *qz_lds = reinterpret_cast<_Float16 *>(lds_raw + W::QZ_OFF);
+    const uint32_t *sb_lds = reinterpret_cast<const uint32_t *>(lds_raw + W::SB_OFF);
+    float *bmax_lds = reinterpret_cast<float *>(lds_raw + W::BMAX_OFF);
+    float *bsum_lds = reinterpret_cast<float *>(lds_raw + W::BSUM_OFF);
+    float *zs_lds = reinterpret_cast<float *>(lds_raw + W::ZS_OFF);
+    // the scores of block b: [head][token] f32 over the block's keys
+    auto s_block = [&](int b) { return reinterpret_cast<float *>(lds_raw + W::K_OFF + b * W::K_BLOCK_BYTES); };
+
+    // ---- prologue: the query row to f16 hi/lo operands in LDS (operand row n: head n & 7, hi part in
+    // rows 0-7 and lo part in rows 8-15 of the one tile) ---------------------------------------------
+    {
+        const float qmul = a.scale * 1.4426950408889634f * Q_UP;
+        half8 op;
+        float sum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            _Float16 h, lw;
+            split_hi_lo(qv[key_slot_dim<BITS>(e)] * qmul, h, lw);
+            const _Float16 x = n < 8 ? h : lw;
+            op[e] = x;
+            sum += (float)x;
+        }
+        q_lds[wave * 64 + lane] = op;
+        // key bias term: slot `k-step` of this lane in the B operand of one more MFMA, as hi and lo halves
+        _Float16 h, lw;
+        split_hi_lo(sum * (1.0f / Q_UP), h, lw);
+        qz_lds[(0 * 64 + lane) * 8 + wave] = h;
+        qz_lds[(1 * 64 + lane) * 8 + wave] = lw;
+        // blocks that never exist
+        if (wave == 0 && lane < 8 * (W::BSTRIDE - RBK)) {
+            const int idx = (lane / (W::BSTRIDE - RBK)) * W::BSTRIDE + RBK + lane % (W::BSTRIDE - RBK);
+            bmax_lds[idx] = NO_SCORE, bsum_lds[idx] = 0.0f;
+        }
+    }
+    raise(W::C_QUERY);
+
+    // ---- running state -------------------------------------------------------------
+    const int g = wave >> 1, b2 = wave & 1;  // phase C: the wave's group and which k-steps of a slot
+    float m_run = NO_SCORE;
+    float l_run = 0.0f;    // sum of P of head n & 7 (wave 0 keeps it)
+    float zacc = 0.0f;     // sum of P * P_UP * value bias of group g over this lane's tokens
+    floatx4 acc[4];        // [tile of 16 dims 4n' + e]: rows 4j .. 4j+3 (operand rows), column n'
+#pragma unroll
+    for (int e = 0; e < 4; e++) acc[e] = floatx4{0, 0, 0, 0};
+    await(W::C_QUERY, W::WAVES);
+
+    for (uint32_t round = 0; round < n_rounds; round++) {
+        const uint32_t base = (blk_begin + round * RBK) * BLOCK, nb = blocks_of(round);
+        const bool more = round + 1 < n_rounds;
+        const bool extra = nb == uint32_t(RBK);  // the round has block 16
+
+        // ---- phase A: scores of blocks wave, wave + 8 (and wave 0: 16) --------------------------
+        // (the query operands are read again in every round: they are not needed between the scores
+        // of one round and the next, and the registers are)
+        {
+            half8 q_reg[8], qz_reg[2];
+#pragma unroll
+            for (int i = 0; i < 8; i++) q_reg[i] = q_lds[i * 64 + lane];
+            qz_reg[0] = *reinterpret_cast<const half8 *>(qz_lds + lane * 8);
+            qz_reg[1] = *reinterpret_cast<const half8 *>(qz_lds + (64 + lane) * 8);
+            const int parts = (wave == 0 && extra) ? 3 : 2;
+#pragma unroll 1
+            for (int part = 0; part < parts; part++) {
+                await(W::C_KPART + part, W::K_LOADERS * (round + 1));  // this part of the keys is in LDS (first: and the scales)
+                const int blk = wave + 8 * part;
+                const unsigned char *kb = lds_raw + W::K_OFF + blk * W::K_BLOCK_BYTES;
+                KeyRegs<BITS> kreg[4];
+#pragma unroll
+                for (int gg = 0; gg < 4; gg++) {
+                    if constexpr (BITS == 8) {
+                        // the group's 64 bytes of token n are piece gg: 16 bytes j of them
+                        const u32x4 v = *reinterpret_cast<const u32x4 *>(kb + gg * 1024 + n * 64 + j * 16);
+                        kreg[gg].w[0] = v.x, kreg[gg].w[1] = v.y, kreg[gg].w[2] = v.z, kreg[gg].w[3] = v.w;
+                    } else {
+                        // the group's 32 bytes of token n are half gg % 2 of piece gg / 2: 8 bytes j of them
+                        const u32x2 v = *reinterpret_cast<const u32x2 *>(kb + (gg >> 1) * 1024 + n * 64 + (gg & 1) * 32 + j * 8);
+                        kreg[gg].w[0] = v.x, kreg[gg].w[1] = v.y;
+                    }
+                }
+                const int tok0 = BLOCK * blk + 4 * j;  // this lane's 4 tokens of the round in C layout
+                const uint32_t *sb_w = sb_lds + BLOCK * blk;  // the block's dwords of groups (0, 1); + RT: groups (2, 3)
+                floatx4 s;
+                {
+                    // bias term: slot e of every lane group belongs to group e / 2 of token n
+                    const u32x2 zr = {sb_w[W::SB_ARRAY / 4 + n], sb_w[W::SB_ARRAY / 4 + RT + n]};
+                    const half8 zop = as_half8(perm(0, zr.x, 0x01000100u), perm(0, zr.x, 0x03020302u), perm(0, zr.y, 0x01000100u),
+                                               perm(0, zr.y, 0x03020302u));
+                    s = floatx4{0, 0, 0, 0};
+                    s = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz_reg[0], s, 0, 0, 0);
+                    s = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz_reg[1], s, 0, 0, 0);
+                }
+                floatx4 r[4];
+#pragma unroll
+                for (int gg = 0; gg < 4; gg++) {
+                    r[gg] = floatx4{0, 0, 0, 0};
+#pragma unroll
+                    for (int ab = 0; ab < 2; ab++) {
+                        r[gg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(key_operand<BITS>(kreg[gg], ab), q_reg[gg * 2 + ab], r[gg], 0, 0, 0);
+                    }
+                }
+                // scales of the lane's tokens 4j .. 4j+3 of the block: groups (0, 1) and groups (2, 3)
+                const u32x4 s01 = *reinterpret_cast<const u32x4 *>(sb_w + 4 * j);
+                const u32x4 s23 = *reinterpret_cast<const u32x4 *>(sb_w + RT + 4 * j);
+                const uint32_t sw[8] = {s01.x, s23.x, s01.y, s23.y, s01.z, s23.z, s01.w, s23.w};
+                constexpr float C1 = code_up<BITS>() / Q_UP;
+#pragma unroll
+                for (int tk = 0; tk < 4; tk++) {
+                    float d = 0.0f;
+#pragma unroll
+                    for (int gg = 0; gg < 4; gg++) d += half_bits_to_float(sw[2 * tk + (gg >> 1)] >> (16 * (gg & 1))) * r[gg][tk];
+                    float v = s[tk] + d * C1;
+                    v += dpp<0x128>(v);  // row_ror 8: the other part (hi | lo) of the same head
+                    s[tk] = base + tok0 + tk < limit ? v : NO_SCORE;  // (also whatever a block past the share left in LDS)
+                }
+                // the block's softmax relative to its own maximum, per head
+                float cm = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+                cm = across_rows<16, 64>(cm, MaxOp());
+                float sum = 0.0f;
+#pragma unroll
+                for (int tk = 0; tk < 4; tk++) {
+                    s[tk] = s[tk] > 0.5f * NO_SCORE ? __builtin_amdgcn_exp2f(s[tk] - cm) : 0.0f;
+                    sum += s[tk];
+                }
+                sum = across_rows<16, 64>(sum, SumOp());
+                // over the block's own keys (every lane of the wave has its key registers by now)
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                if (n < 8) *reinterpret_cast<floatx4 *>(s_block(blk) + n * BLOCK + 4 * j) = s;
+                if (j == 0 && n < 8) bmax_lds[n * W::BSTRIDE + blk] = cm, bsum_lds[n * W::BSTRIDE + blk] = sum;
+            }
+            if (wave == 0 && !extra && j == 0 && n < 8) bmax_lds[n * W::BSTRIDE + 16] = NO_SCORE, bsum_lds[n * W::BSTRIDE + 16] = 0.0f;
+        }
+        raise(W::C_SCORES);
+        await(W::C_SCORES, W::WAVES * (round + 1));
+
+        // ---- the round's maximum per head, and what was summed so far brought to it -------------
+        float nm = m_run;
+        {
+            const floatx4 *bmx = reinterpret_cast<const floatx4 *>(bmax_lds + (n & 7) * W::BSTRIDE);
+#pragma unroll
+            for (int i = 0; i < W::BSTRIDE / 4; i++) {
+                const floatx4 w = bmx[i];
+                nm = fmaxf(nm, fmaxf(fmaxf(w[0], w[1]), fmaxf(w[2], w[3])));
+            }
+        }
+        const float al = __builtin_amdgcn_exp2f(m_run - nm);  // (first round: 2^(-1e30 - nm) = 0, and nothing to scale)
+        if (round > 0) {
+            zacc *= al;
+            // accumulator rows 4j + i are heads (4j + i) & 7: lane h (j = 0, n = h) holds head h's factor
+            floatx4 al4;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                al4[i] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(4 * ((4 * j + i) & 7), __builtin_bit_cast(int, al)));
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[e] *= al4;
+        }
+        m_run = nm;
+        if (wave == 0) {
+            // the round's sum of P of head n & 7: lane group j adds blocks 5j .. 5j + 4
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < W::BSTRIDE / 4; i++) {
+                const int b = (W::BSTRIDE / 4) * j + i;
+                sum += bsum_lds[(n & 7) * W::BSTRIDE + b] * __builtin_amdgcn_exp2f(bmax_lds[(n & 7) * W::BSTRIDE + b] - nm);  // (a block that is not there: sum 0)
+            }
+            l_run = l_run * al + across_rows<16, 64>(sum, SumOp());
+        }
+
+        // ---- probability operands of this wave's k-steps: P * value scale of group g, hi part in
+        // operand rows 0-7 and lo part in rows 8-15.  The two lanes of a head (n and n + 8) make four of
+        // the lane group's eight tokens each, both parts, and exchange what the other one feeds. ----
+        half8 p_op[W::SLOTS];
+        {
+            const int hh = n >> 3;  // this lane makes tokens 8j + 4 hh .. + 3 of a k-step
+            const int sh = 16 * (g & 1);
+            const bool fifth = extra && b2 == 0;  // k-step 8: block 16 (lane groups 0 and 1; the others repeat them with factor 0)
+#pragma unroll
+            for (int sl = 0; sl < W::SLOTS; sl++) {
+                if (sl == 4 && !fifth) {
+                    p_op[sl] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+                    continue;
+                }
+                const int ks = 2 * sl + b2;  // tokens 32 ks ..: blocks 2 ks and 2 ks + 1
+                const int jj = sl == 4 ? (j & 1) : j;
+                const int blk = 2 * ks + (jj >> 1);
+                const floatx4 pt = *reinterpret_cast<const floatx4 *>(s_block(blk) + (n & 7) * BLOCK + 8 * (jj & 1) + 4 * hh);
+                // value scales and biases of group g: half g % 2 of the tokens' dwords of groups (g, g ^ 1).
+                // (Tokens past the share have probability 0 and the scales of the share's last token:
+                // every load is clamped to it, so nothing but cache rows in use is ever read.)
+                const uint32_t *vsp = sb_lds + 2 * (W::SB_ARRAY / 4) + (g >> 1) * RT + 32 * ks + 8 * jj + 4 * hh;
+                const u32x4 sv = *reinterpret_cast<const u32x4 *>(vsp);
+                const u32x4 zv = *reinterpret_cast<const u32x4 *>(vsp + W::SB_ARRAY / 4);
+                // 2^(block maximum - round maximum) * P_UP (2^8, so that the lo part stays a normal f16)
+                const float f = __builtin_amdgcn_exp2f(bmax_lds[(n & 7) * W::BSTRIDE + 2 * ks + (j >> 1)] - nm + 8.0f);
+                const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w}, zw[4] = {zv.x, zv.y, zv.z, zv.w};
+                float x[4], lo[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float p = pt[e] * f;
+                    zacc += p * half_bits_to_float(zw[e] >> sh);
+                    x[e] = p * half_bits_to_float(sw[e] >> sh);
+                    lo[e] = x[e] - __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x[e]) & 0xffffe000u);
+                }
+                // round toward zero: exact truncation to the hi part
+                const uint32_t hi0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x[0], x[1]));
+                const uint32_t hi1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x[2], x[3]));
+                const uint32_t lo0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo[0], lo[1]));
+                const uint32_t lo1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo[2], lo[3]));
+                // the hi lane (n < 8) feeds hi parts and wants the other lane's hi parts of tokens 4-7; the lo
+                // lane feeds lo parts and wants the other lane's lo parts of tokens 0-3
+                const uint32_t send0 = hh ? hi0 : lo0, send1 = hh ? hi1 : lo1;
+                const uint32_t recv0 = uint32_t(__builtin_amdgcn_update_dpp(0, int(send0), 0x128, 0xf, 0xf, false));  // row_ror 8
+                const uint32_t recv1 = uint32_t(__builtin_amdgcn_update_dpp(0, int(send1), 0x128, 0xf, 0xf, false));
+                uint32_t o[4] = {hh ? recv0 : hi0, hh ? recv1 : hi1, hh ? lo0 : recv0, hh ? lo1 : recv1};
+                // (pinned: left alone, the compiler moves an operand's arithmetic down to its use, behind the wait for the values)
+                asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]));
+                p_op[sl] = as_half8(o[0], o[1], o[2], o[3]);
+            }
+        }
+        if (more) raise(W::C_BUILT);  // this wave is through with the round's scores, scales and biases
+
+        // ---- phase C: O += P V, one k-step per value slot as the slots land ---------------------
+        const unsigned char *vb = lds_raw + W::V_OFF + val_lane_offset<BITS>(g, n);
+        auto read_values = [&](int sl, ValRegs<BITS> &vreg) {
+            const int jj = sl == 4 ? (j & 1) : j;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const int tk = 32 * (2 * sl + b2) + 8 * jj + e;
+                vreg.w[e] = *reinterpret_cast<const uint32_t *>(vb + (tk / W::V_GROUP_TOKENS) * W::V_GROUP_BYTES + (tk % W::V_GROUP_TOKENS) * RB);
+            }
+        };
+        auto add_values = [&](int sl, const ValRegs<BITS> &vreg) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p_op[sl], val_operand<BITS>(vreg, e, n), acc[e], 0, 0, 0);
+            }
+        };
+        const bool fifth = extra && b2 == 0;
+        if (peek(W::C_SLOT + 3) >= W::V_LOADERS * (round + 1)) {
+            // slots 0-3 are there already (the slots land in order): every read at once
+            ValRegs<BITS> vreg[4];
+#pragma unroll
+            for (int sl = 0; sl < 4; sl++) read_values(sl, vreg[sl]);
+#pragma unroll
+            for (int sl = 0; sl < 4; sl++) add_values(sl, vreg[sl]);
+        } else {
+#pragma unroll
+            for (int sl = 0; sl < 4; sl++) {
+                await(W::C_SLOT + sl, W::V_LOADERS * (round + 1));  // value slot sl is in LDS
+                ValRegs<BITS> vreg;
+                read_values(sl, vreg);
+                add_values(sl, vreg);
+            }
+        }
+        if (fifth) {
+            await(W::C_SLOT + 4, W::V_LOADERS * (round + 1));
+            ValRegs<BITS> vreg;
+            read_values(4, vreg);
+            add_values(4, vreg);
+        }
+        if (more) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the value codes are in registers
+            raise(W::C_DONE);
+        }
+    }
+
+    // ---- epilogue: the two waves of a group add up, wave 2g writes the partial ---------------------
+    {
+        // the head's bias sum: over the four lane groups and the two lanes of the head
+        float z = across_rows<16, 64>(zacc, SumOp());
+        z += dpp<0x128>(z);
+        if (j == 0 && n < 8) zs_lds[wave * 8 + n] = z;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+    constexpr float unscale = code_up<BITS>() / P_UP;
+    floatx4 mine[4];  // head 4j + i (j < 2), dims 64 g + 4n .. + 3
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float zb = zs_lds[wave * 8 + ((4 * j + i) & 7)] * (1.0f / P_UP);
+#pragma unroll
+        for (int e = 0; e < 4; e++) mine[i][e] = across_rows<32, 64>(acc[e][i], SumOp()) * unscale + zb;
+    }
+    // (the key area is free: the key loaders request nothing after the last round, and every wave is
+    // past the last round's scores, having built its operands from them)
+    floatx4 *x_o = reinterpret_cast<floatx4 *>(lds_raw + W::X_OFF);  // [group][lane < 32][4 rows]
+    if (b2 == 1) {
+        if (j < 2) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) x_o[(g * 32 + lane) * 4 + i] = mine[i];
+        }
+        raise(W::C_MERGE + g);
+        return;
+    }
+    await(W::C_MERGE + g, 1);
+    if (wave == 0 && j == 0 && n < 8) {
+        const size_t slot = size_t(split) * a.heads + kv * 8 + n;
+        *reinterpret_cast<floatx2 *>(a.part_ml + 2 * slot) = floatx2{m_run, l_run};
+    }
+    if (j < 2) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const size_t slot = size_t(split) * a.heads + kv * 8 + 4 * j + i;
+            *reinterpret_cast<floatx4 *>(a.part_o + slot * DIM + 64 * g + 4 * n) = mine[i] + x_o[(g * 32 + lane) * 4 + i];
+        }
+    }
+}
+
 // Merges the splits of one (q head, row) and a 64-dim quarter of the head:
 // weights 2^(m_c - M), then the gate.  256 threads: first one thread per split
 // for the weights, then (16 dim quads) x (16 slices of splits) for the sums.
@@ -1130,10 +1722,15 @@ constexpr uint32_t LOADERS_FROM = 24 * 1024;
 constexpr uint32_t LOADERS_4BIT_UP_TO = 136 * 1024;
 
 template <int BITS, int TILES, bool PACKED>
-void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu, bool loaders) {
+void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu, bool loaders, bool keys_first) {
     void (*kernel)(PartialArgs);
     int lds_bytes;
     if constexpr (TILES == 1 && BITS != 16 && PACKED) {
+        if (loaders && keys_first) {
+            using W = KeysFirst<BITS>;
+            attention_partial_kernel_s<BITS><<<dim3(a.nsplits, a.kv_heads), (W::LOADERS + W::WAVES) * 64, W::LDS_BYTES, stream>>>(a);
+            return;
+        }
         if (loaders) {
             attention_partial_kernel_d<BITS><<<dim3(a.nsplits, a.kv_heads), (TEAMS_DMA + 1) * THREADS,
                                                Shape<BITS, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA), stream>>>(a);
@@ -1160,15 +1757,15 @@ void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu, b
 }
 
 template <int BITS>
-void launch_partial_rows(hipStream_t stream, const PartialArgs &a, bool one_per_cu, bool loaders) {
+void launch_partial_rows(hipStream_t stream, const PartialArgs &a, bool one_per_cu, bool loaders, bool keys_first) {
     if (a.rows == 1) {
-        launch_partial<BITS, 1, true>(stream, a, one_per_cu, loaders);
+        launch_partial<BITS, 1, true>(stream, a, one_per_cu, loaders, keys_first);
     } else if (a.rows == 2) {
-        launch_partial<BITS, 1, false>(stream, a, one_per_cu, loaders);
+        launch_partial<BITS, 1, false>(stream, a, one_per_cu, loaders, keys_first);
     } else if (a.rows <= 4) {
-        launch_partial<BITS, 2, false>(stream, a, one_per_cu, loaders);
+        launch_partial<BITS, 2, false>(stream, a, one_per_cu, loaders, keys_first);
     } else {
-        launch_partial<BITS, 4, false>(stream, a, one_per_cu, loaders);
+        launch_partial<BITS, 4, false>(stream, a, one_per_cu, loaders, keys_first);
     }
 }
 
@@ -1209,16 +1806,17 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
     const bool loaders = rows == 1 && bits != 16 && capacity >= LOADERS_FROM && (bits == 8 || capacity <= LOADERS_4BIT_UP_TO) &&
                          !(stages & SAETTA_STAGE_NO_LOADERS);
     const bool one_per_cu = rows >= 2 || bits == 16 || capacity <= 80 * 1024 || loaders;
+    const bool keys_first = loaders && !(stages & 8u);
     if (one_per_cu && nsplits > MAX_SPLITS / 2) nsplits = MAX_SPLITS / 2;
     if (stages & SAETTA_STAGE_PARTIAL) {
         PartialArgs a{q,     kdata,    vdata,    ks,    kz,   vs,      vz,   part_o, part_ml,
                       heads, kv_heads, capacity, scale, rows, nsplits, d_tp, decode_len ? 1u : 0u};
         if (bits == 8) {
-            launch_partial_rows<8>(stream, a, one_per_cu, loaders);
+            launch_partial_rows<8>(stream, a, one_per_cu, loaders, keys_first);
         } else if (bits == 4) {
-            launch_partial_rows<4>(stream, a, one_per_cu, loaders);
+            launch_partial_rows<4>(stream, a, one_per_cu, loaders, keys_first);
         } else {
-            launch_partial_rows<16>(stream, a, one_per_cu, loaders);
+            launch_partial_rows<16>(stream, a, one_per_cu, loaders, keys_first);
         }
     }
     if (stages & SAETTA_STAGE_REDUCE) {
@@ -1267,6 +1865,14 @@ int setup_decode() {
     if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_partial_kernel_d<4>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize,
                                          Shape<4, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA)))) {
+        return rc;
+    }
+    if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_partial_kernel_s<8>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, KeysFirst<8>::LDS_BYTES))) {
+        return rc;
+    }
+    if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_partial_kernel_s<4>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, KeysFirst<4>::LDS_BYTES))) {
         return rc;
     }
     if (int rc = raise_lds_of_bits<8>()) return rc;
