@@ -675,7 +675,7 @@ def main():
         if workload == "decode8_32k":
             return bench_decode(s, torch, args, args.ctx or 32768, 8, 1, args.layers or 32)
         if workload == "decode4_150k":
-            return bench_decode(s, torch, args, 150000, 4, 1, args.layers or 12)
+            return bench_decode(s, torch, args, args.ctx or 150000, 4, 1, args.layers or 12)
         if workload == "decode16_4k":
             return bench_decode(s, torch, args, 4096, 16, 1, args.layers or 32)
         if workload.startswith("verify"):

@@ -1138,8 +1138,10 @@ __global__ __launch_bounds__((KeysFirst<BITS>::LOADERS + KeysFirst<BITS>::WAVES)
     const uint32_t limit = min(max_len, blk_end * BLOCK);  // tokens of this share end here
     const uint32_t last_tok = limit - 1;                   // rows past it are never read: loads are clamped to it
     const uint32_t range = blk_end - blk_begin;
+    // rounds of equal size (to within a block), none longer than 17 blocks
     const uint32_t n_rounds = (range + RBK - 1) / RBK;
-    auto blocks_of = [&](uint32_t round) { return min(range - round * RBK, uint32_t(RBK)); };
+    const uint32_t per_round = (range + n_rounds - 1) / n_rounds;
+    auto blocks_of = [&](uint32_t round) { return min(range - round * per_round, per_round); };
 
     auto dma = [&](uint32_t lds_addr, uint32_t voff, const void *src) {
         asm volatile("s_mov_b32 m0, %0\n"
@@ -1186,7 +1188,7 @@ __global__ __launch_bounds__((KeysFirst<BITS>::LOADERS + KeysFirst<BITS>::WAVES)
         const uint32_t L = uint32_t(wave_all);
         const void *sb_src[4] = {a.kscales, a.kbiases, a.vscales, a.vbiases};
         for (uint32_t round = 0; round < n_rounds; round++) {
-            const uint32_t base = (blk_begin + round * RBK) * BLOCK, nb = blocks_of(round);
+            const uint32_t base = (blk_begin + round * per_round) * BLOCK, nb = blocks_of(round);
             // the round before: its scales are read until every wave has built its operands, its keys until every wave has its scores
             if (round > 0) await(W::C_BUILT, W::WAVES * round);
 #pragma unroll
@@ -1250,7 +1252,7 @@ __global__ __launch_bounds__((KeysFirst<BITS>::LOADERS + KeysFirst<BITS>::WAVES)
         // loader 0 then block 16 (slot 4) ----
         const uint32_t L = uint32_t(wave_all) - W::K_LOADERS;
         for (uint32_t round = 0; round < n_rounds; round++) {
-            const uint32_t base = (blk_begin + round * RBK) * BLOCK, nb = blocks_of(round);
+            const uint32_t base = (blk_begin + round * per_round) * BLOCK, nb = blocks_of(round);
             // the keys of the first round have been requested | every wave is through with the values before
             if (round == 0) {
                 await(W::C_KEYS, W::K_LOADERS);
@@ -1352,9 +1354,10 @@ __global__ __launch_bounds__((KeysFirst<BITS>::LOADERS + KeysFirst<BITS>::WAVES)
     await(W::C_QUERY, W::WAVES);
 
     for (uint32_t round = 0; round < n_rounds; round++) {
-        const uint32_t base = (blk_begin + round * RBK) * BLOCK, nb = blocks_of(round);
+        const uint32_t base = (blk_begin + round * per_round) * BLOCK, nb = blocks_of(round);
         const bool more = round + 1 < n_rounds;
         const bool extra = nb == uint32_t(RBK);  // the round has block 16
+        const uint32_t round_limit = min(limit, base + nb * BLOCK);  // tokens of this round end here
 
         // ---- phase A: scores of blocks wave, wave + 8 (and wave 0: 16) --------------------------
         // (the query operands are read again in every round: they are not needed between the scores
@@ -1417,7 +1420,7 @@ __global__ __launch_bounds__((KeysFirst<BITS>::LOADERS + KeysFirst<BITS>::WAVES)
                     for (int gg = 0; gg < 4; gg++) d += half_bits_to_float(sw[2 * tk + (gg >> 1)] >> (16 * (gg & 1))) * r[gg][tk];
                     float v = s[tk] + d * C1;
                     v += dpp<0x128>(v);  // row_ror 8: the other part (hi | lo) of the same head
-                    s[tk] = base + tok0 + tk < limit ? v : NO_SCORE;  // (also whatever a block past the share left in LDS)
+                    s[tk] = base + tok0 + tk < round_limit ? v : NO_SCORE;  // (also whatever a block past the round left in LDS)
                 }
                 // the block's softmax relative to its own maximum, per head
                 float cm = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
@@ -1720,6 +1723,8 @@ constexpr uint32_t LOADERS_FROM = 24 * 1024;
 // at 131k), up to where the two-workgroups-per-CU kernel streams faster than the loader kernel's
 // two teams get through their iterations (29.1 against 28.5 us at 150k, 40.9 against 39.3 at 200k).
 constexpr uint32_t LOADERS_4BIT_UP_TO = 136 * 1024;
+// Which of the two: see run_attention.
+constexpr uint32_t KEYS_FIRST_ONE_ROUND = 17 * BLOCK * (MAX_SPLITS / 2), KEYS_FIRST_AGAIN_FROM = 60000, KEYS_FIRST_4BIT_UP_TO = 100 * 1024;
 
 template <int BITS, int TILES, bool PACKED>
 void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu, bool loaders, bool keys_first) {
@@ -1806,7 +1811,13 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
     const bool loaders = rows == 1 && bits != 16 && capacity >= LOADERS_FROM && (bits == 8 || capacity <= LOADERS_4BIT_UP_TO) &&
                          !(stages & SAETTA_STAGE_NO_LOADERS);
     const bool one_per_cu = rows >= 2 || bits == 16 || capacity <= 80 * 1024 || loaders;
-    const bool keys_first = loaders && !(stages & 8u);
+    // Of the two kernels with loader waves, the one that takes the keys first wins wherever a share
+    // is one round (up to 17 blocks of 16 tokens per split: 10.1 against 12.5 us at 32k tokens, 8-bit;
+    // 10.2 against 11.7, 4-bit) and again from about four rounds on (17.1 against 18.6 us at 64k, 29.7
+    // against 31.1 at 131k, 8-bit); with two or three short rounds the ring of slots is ahead (14.1
+    // against 15.6 us at 40k), and so it is for 4-bit codes above 100k tokens (28.0 against 29.3 at 131k).
+    const bool keys_first = loaders && (capacity <= KEYS_FIRST_ONE_ROUND || (capacity >= KEYS_FIRST_AGAIN_FROM &&
+                                                                               (bits == 8 || capacity <= KEYS_FIRST_4BIT_UP_TO)));
     if (one_per_cu && nsplits > MAX_SPLITS / 2) nsplits = MAX_SPLITS / 2;
     if (stages & SAETTA_STAGE_PARTIAL) {
         PartialArgs a{q,     kdata,    vdata,    ks,    kz,   vs,      vz,   part_o, part_ml,

@@ -256,21 +256,27 @@ def test_capacity_must_be_whole_blocks():
         plan.build().run()
 
 
+@pytest.mark.parametrize("capacity", [81920, 49152, 34816])
 @pytest.mark.parametrize("kind", [saetta.KvBits.Eight, saetta.KvBits.Four])
-def test_large_cache_of_codes_one_row(kind):
-    # One row over codes in a cache of 24k tokens and more runs the kernel whose extra waves move
-    # the codes into LDS and whose two teams of computing waves take alternate 64-token
-    # iterations.  Lengths: less than one block; one team idle; both teams, even and odd numbers of
-    # iterations; more iterations than LDS slots (the slots are refilled); the whole capacity.  The
-    # rows past each length are poisoned.
-    capacity = 81920
+def test_large_cache_of_codes_one_row(kind, capacity):
+    # One row over codes in a cache of 24k tokens and more runs one of the two kernels whose extra
+    # waves move the codes into LDS.  Capacity 49152: the ring of four 64-token slots with two teams
+    # of computing waves on alternate iterations.  Lengths: less than one block; one team idle; both
+    # teams, even and odd numbers of iterations; more iterations than slots (the slots are refilled);
+    # the whole capacity.  Capacities 81920 and 34816: the kernel that takes a share in rounds of up to
+    # 17 blocks with the keys requested first.  Lengths: a single block; rounds of fewer than 16
+    # blocks; shares of 16 and of 17 blocks side by side (33000 tokens, and the whole of 34816: every
+    # share has block 16); two and three rounds, the last one short.  The rows past each length are
+    # poisoned.
     rng = np.random.default_rng(77)
     k = (rng.standard_normal((capacity, VALUES)) * 2.0).astype(np.float32)
     v = rng.standard_normal((capacity, VALUES)).astype(np.float32)
     q = rng.standard_normal(H * D).astype(np.float32)
     qg = rng.standard_normal(H * 2 * D).astype(np.float32)
     att = saetta.DecodeAttention(H, KV, D, capacity)
-    for length in [1, 100, 2049, 8200, 16400, 33000, 50001, 81920]:
+    for length in [1, 100, 2049, 8200, 16400, 33000, 34816, 50001, 81920]:
+        if length > capacity:
+            continue
         kc, vc, kf, vf = cache_pair(k[:length], v[:length], kind, capacity, poison=True)
         got = run_decode(att, kind, dev(q), kc, vc, dev(qg), length)
         assert np.isfinite(got).all(), length
