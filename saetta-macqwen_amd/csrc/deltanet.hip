@@ -694,6 +694,14 @@ extern "C" int saetta_deltanet_step(saetta_stream_t stream, const float *q, cons
     SAETTA_REQUIRE(aligned(q, 16) && aligned(k, 16) && aligned(state, 16), SAETTA_E_ALIGN,
                    "deltanet_step: q, k and the state must be 16-byte aligned");
     if (int rc = ensure_device()) return rc;
+    // q, k and v as the conv leaves them (one array, q | k | v: what the reference's layer passes,
+    // src/cpu/deltanet.rs:80-83) take the kernels of saetta_deltanet_rows with one token: 8 workgroups
+    // per value head instead of one.  deltanet_step_kernel is kept for vectors that lie apart.
+    const size_t key_size = size_t(p.k_heads) * K_DIM;
+    if (k == q + key_size && v == k + key_size && p.v_dim % 4 == 0) {
+        const saetta_rows_step_params rp{p.k_heads, p.v_heads, p.v_dim, 1, p.eps, 0};
+        return saetta_deltanet_rows(stream, q, a, b, a_log, dt_bias, state, z, norm_w, y, nullptr, rp);
+    }
     StepArgs args{q, k, v, a, b, a_log, dt_bias, state, z, norm_w, y, p};
     deltanet_step_kernel<<<p.v_heads, STEP_THREADS, 0, as_stream(stream)>>>(args);
     return launch_status("deltanet_step");

@@ -760,7 +760,8 @@ struct OwnedWorkspace {
     void *ptr = nullptr;
     size_t bytes = 0;
 };
-OwnedWorkspace g_owned[16];
+constexpr int OWNED_DEVICES = 64;  // as many devices as the library's set-up admits
+OwnedWorkspace g_owned[OWNED_DEVICES];
 std::mutex g_owned_mutex;
 
 size_t workspace_bytes(uint32_t pos, uint32_t tokens, uint32_t kv_heads) {
@@ -786,16 +787,25 @@ int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kda
     if (int rc = ensure_device()) return rc;
     if (p.tokens == 0) return SAETTA_OK;
     const size_t need = workspace_bytes(p.pos, p.tokens, p.kv_heads);
+    // The library's own workspace is held under its lock until the launches that use it are queued:
+    // a second host thread that has to grow it waits for them (hipDeviceSynchronize) before it frees.
+    std::unique_lock<std::mutex> owned_lock(g_owned_mutex, std::defer_lock);
     if (workspace) {
         SAETTA_REQUIRE(workspace_size >= need, SAETTA_E_SCRATCH, "%s: workspace of %zu bytes, %zu needed", what,
                        workspace_size, need);
     } else {
-        // No workspace given: use (and grow) the library's own.  This allocates, so it cannot be
-        // used under stream capture; work queued on other streams must not share it.
+        // No workspace given: use (and grow) the library's own.  This may allocate, which a stream
+        // under capture cannot do; work queued on other streams must not share it.
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) (void)hipGetLastError();
+        SAETTA_REQUIRE(capturing == hipStreamCaptureStatusNone, SAETTA_E_SCRATCH,
+                       "%s: a stream under capture needs a workspace of the caller's (%zu bytes, saetta_prefill_workspace_bytes)",
+                       what, need);
         int dev = 0;
-        (void)hipGetDevice(&dev);
-        std::lock_guard<std::mutex> lock(g_owned_mutex);
-        OwnedWorkspace &w = g_owned[dev & 15];
+        if (hipError_t e = hipGetDevice(&dev)) return fail(int(e), "%s: %s", what, hipGetErrorString(e));
+        SAETTA_REQUIRE(dev >= 0 && dev < OWNED_DEVICES, SAETTA_E_DEVICE, "%s: device index %d (up to %d)", what, dev, OWNED_DEVICES - 1);
+        owned_lock.lock();
+        OwnedWorkspace &w = g_owned[dev];
         if (w.bytes < need) {
             if (w.ptr) {
                 (void)hipDeviceSynchronize();

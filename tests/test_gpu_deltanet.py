@@ -62,6 +62,30 @@ def test_other_value_dims(v_dim):
     run_tokens(2, 4, v_dim, 4, 3, seed=v_dim)
 
 
+def test_step_with_vectors_apart():
+    # q, k and v in buffers of their own take deltanet_step_kernel (one workgroup per value head);
+    # as slices of the conv's output (the tests above) the same call runs the rows kernels.
+    rng = np.random.default_rng(11)
+    k_heads, v_heads, v_dim, eps = 16, 32, 128, 1e-6
+    key, val = k_heads * K_DIM, v_heads * v_dim
+    a_log = rng.uniform(-1, 1, v_heads).astype(np.float32)
+    dt_bias = rng.standard_normal(v_heads).astype(np.float32)
+    norm = (1 + 0.1 * rng.standard_normal(v_dim)).astype(np.float32)
+    state_cpu = (0.1 * rng.standard_normal(v_heads * v_dim * K_DIM)).astype(np.float32)
+    state_gpu = dev(state_cpu.copy())
+    q, k = rng.standard_normal(key).astype(np.float32), rng.standard_normal(key).astype(np.float32)
+    v, z = rng.standard_normal(val).astype(np.float32), rng.standard_normal(val).astype(np.float32)
+    a, b = rng.standard_normal(v_heads).astype(np.float32), rng.standard_normal(v_heads).astype(np.float32)
+    y = torch.empty(val, device="cuda")
+    plan = saetta.Plan()
+    saetta.deltanet_step(plan, dev(q), dev(k), dev(v), dev(a), dev(b), dev(a_log), dev(dt_bias), state_gpu, dev(z),
+                         dev(norm), y, k_heads, v_heads, v_dim, eps)
+    plan.build().run()
+    want_y = oracle.deltanet_step(q, k, v, a, b, a_log, dt_bias, state_cpu, z, norm, k_heads, v_heads, K_DIM, v_dim, eps)
+    assert np.abs(host(y) - want_y).max() <= 2e-5 * max(1.0, np.abs(want_y).max())
+    assert np.abs(host(state_gpu) - state_cpu).max() <= 2e-5 * max(1.0, np.abs(state_cpu).max())
+
+
 def test_conv_kernel_sizes_and_rejections():
     run_tokens(1, 1, 16, 2, 3, seed=5)
     run_tokens(1, 2, 16, 7, 9, seed=6)
