@@ -352,6 +352,20 @@ int saetta_deltanet_rows(saetta_stream_t stream, const float *mixed, const float
                          const float *a_log, const float *dt_bias, float *state, const float *z,
                          const float *norm_w, float *y, float *snaps, saetta_rows_step_params p);
 
+/* The same call with a workspace of the caller's (the reference's encode_deltanet
+ * works in buffers of the prefill's own, src/prefill.rs:1433-1578): from 128 tokens
+ * on, without snapshots and with v_dim a multiple of 16, the delta rule runs in
+ * blocks of 64 tokens on the matrix cores and keeps per-block matrices in
+ * `workspace` (saetta_deltanet_rows_workspace_bytes(p) bytes, 16-byte aligned; 0
+ * bytes: the call runs token by token and takes no workspace).  With workspace
+ * NULL this is saetta_deltanet_rows, which uses a workspace the library owns and
+ * grows with hipMalloc (under stream capture it falls back to token by token). */
+size_t saetta_deltanet_rows_workspace_bytes(saetta_rows_step_params p);
+int saetta_deltanet_rows_ws(saetta_stream_t stream, const float *mixed, const float *a, const float *b,
+                            const float *a_log, const float *dt_bias, float *state, const float *z,
+                            const float *norm_w, float *y, float *snaps, saetta_rows_step_params p,
+                            void *workspace, size_t workspace_size);
+
 /* Kernel deltanet_rows (recorded by GpuDeltaNet::record_rows with DN_SIMDS = 0,
  * src/gpu_layers.rs:737-757): conv and step of up to 8 rows as one op, what
  * saetta_deltanet_conv_rows + saetta_deltanet_rows give, in two launches

@@ -26,8 +26,18 @@ int launch_status(const char *what);
 int setup_kv_quant();
 int setup_prep();
 int setup_deltanet();
+int setup_deltanet_chunk();
 int setup_decode();
 int setup_prefill();
+// The chunked delta rule (deltanet_chunk.hip): the workspace a call needs (0: the call keeps to the
+// token-by-token kernels), and the call itself (the delta rule only; the gated norm follows as for the
+// token-by-token kernels) with a workspace of the caller's or the library's own (which may allocate).
+size_t deltanet_chunk_workspace_bytes(const saetta_rows_step_params &p);
+int run_deltanet_chunk(hipStream_t stream, const float *mixed, const float *a, const float *b, const float *a_log,
+                       const float *dt_bias, float *state, float *o, const saetta_rows_step_params &p, uint32_t channels,
+                       void *workspace);
+int run_deltanet_chunk_owned(hipStream_t stream, const float *mixed, const float *a, const float *b, const float *a_log,
+                             const float *dt_bias, float *state, float *o, const saetta_rows_step_params &p, uint32_t channels);
 // Loads the code object `kernel` lives in.
 inline int load_kernel(const void *kernel) {
     hipFuncAttributes attr;

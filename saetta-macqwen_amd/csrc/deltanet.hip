@@ -24,6 +24,7 @@
 // rows are requested before the first is used, and the dot products are reductions over 32 lanes
 // by DPP moves (no LDS).
 #include "common.hpp"
+#include "deltanet_gates.hpp"
 #include "lanes.hpp"
 
 #include <type_traits>
@@ -38,18 +39,6 @@ constexpr int MAX_ROWS_PER_LANE = 8;  // v_dim up to 256
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 __device__ __forceinline__ float silu_f(float x) { return x * sigmoid_f(x); }
 __device__ __forceinline__ float dot4(float4 a, float4 b) { return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w; }
-
-// The gates of a token and head: g = exp(-exp(A_log) softplus(a + dt_bias)), beta = sigmoid(b), with
-// the hardware's exp2 and log2 (the library routines are some 150 instructions, and in the kernels
-// below the gates sit in one wave's path): log1p(e) as e - e^2 / 2 below 2^-10 and log(1 + e)
-// above; the errors stay near 1e-7.
-__device__ __forceinline__ void fast_gates(float a_plus_bias, float exp_a_log, float b, float &g, float &beta) {
-    const float e = __expf(-fabsf(a_plus_bias));
-    const float log1p_e = e < 0x1p-10f ? e * (1.0f - 0.5f * e) : __logf(1.0f + e);
-    const float softplus = fmaxf(a_plus_bias, 0.0f) + log1p_e;
-    g = __expf(-exp_a_log * softplus);
-    beta = __builtin_amdgcn_rcpf(1.0f + __expf(-b));
-}
 
 __global__ __launch_bounds__(256) void deltanet_conv_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                             float *__restrict__ state, float *__restrict__ out,
@@ -664,7 +653,10 @@ void launch_small_rows(const SmallRowsArgs &args, hipStream_t stream) {
 
 }  // namespace
 
-int setup_deltanet() { return load_kernel(reinterpret_cast<const void *>(deltanet_step_kernel)); }
+int setup_deltanet() {
+    if (int rc = load_kernel(reinterpret_cast<const void *>(deltanet_step_kernel))) return rc;
+    return setup_deltanet_chunk();
+}
 }  // namespace saetta
 
 using namespace saetta;
@@ -728,9 +720,18 @@ extern "C" int saetta_deltanet_conv_rows(saetta_stream_t stream, const float *x,
     return launch_status("deltanet_conv_rows");
 }
 
+extern "C" size_t saetta_deltanet_rows_workspace_bytes(saetta_rows_step_params p) { return deltanet_chunk_workspace_bytes(p); }
+
 extern "C" int saetta_deltanet_rows(saetta_stream_t stream, const float *mixed, const float *a, const float *b,
                                     const float *a_log, const float *dt_bias, float *state, const float *z,
                                     const float *norm_w, float *y, float *snaps, saetta_rows_step_params p) {
+    return saetta_deltanet_rows_ws(stream, mixed, a, b, a_log, dt_bias, state, z, norm_w, y, snaps, p, nullptr, 0);
+}
+
+extern "C" int saetta_deltanet_rows_ws(saetta_stream_t stream, const float *mixed, const float *a, const float *b,
+                                       const float *a_log, const float *dt_bias, float *state, const float *z,
+                                       const float *norm_w, float *y, float *snaps, saetta_rows_step_params p,
+                                       void *workspace, size_t workspace_size) {
     SAETTA_REQUIRE(mixed && a && b && a_log && dt_bias && state && z && norm_w && y, SAETTA_E_NULL,
                    "deltanet_rows: null buffer");
     SAETTA_REQUIRE(!p.snapshots || snaps, SAETTA_E_NULL, "deltanet_rows: snapshots asked for, no buffer");
@@ -744,13 +745,32 @@ extern "C" int saetta_deltanet_rows(saetta_stream_t stream, const float *mixed, 
     if (int rc = ensure_device()) return rc;
     if (p.tokens == 0) return SAETTA_OK;
     const uint32_t channels = 2 * p.k_heads * K_DIM + p.v_heads * p.v_dim;
-    RowsArgs args{mixed, a, b, a_log, dt_bias, state, y, snaps, p, channels};
-    constexpr int LANES = ROWS_LANES_PER_ROW, ROWS_PER_WG = 256 / LANES;
-    const dim3 grid((p.v_dim + ROWS_PER_WG - 1) / ROWS_PER_WG, p.v_heads);
-    if (p.snapshots) {
-        deltanet_rows_kernel<true, LANES><<<grid, 256, 0, as_stream(stream)>>>(args);
+    // A prefill chunk (128 tokens and more, no snapshots): the delta rule in blocks of 64 tokens on the
+    // matrix cores, with a workspace of the caller's or, outside stream capture, the library's own.
+    const size_t need = deltanet_chunk_workspace_bytes(p);
+    bool blocks = need > 0;
+    if (blocks && workspace) {
+        SAETTA_REQUIRE(workspace_size >= need && aligned(workspace, 16), SAETTA_E_SCRATCH,
+                       "deltanet_rows: workspace of %zu bytes, %zu needed (16-byte aligned)", workspace_size, need);
+    } else if (blocks) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(as_stream(stream), &capturing) != hipSuccess) (void)hipGetLastError();
+        blocks = capturing == hipStreamCaptureStatusNone;  // (the library's own workspace may have to grow)
+    }
+    if (blocks) {
+        if (int rc = workspace ? run_deltanet_chunk(as_stream(stream), mixed, a, b, a_log, dt_bias, state, y, p, channels, workspace)
+                               : run_deltanet_chunk_owned(as_stream(stream), mixed, a, b, a_log, dt_bias, state, y, p, channels)) {
+            return rc;
+        }
     } else {
-        deltanet_rows_kernel<false, LANES><<<grid, 256, 0, as_stream(stream)>>>(args);
+        RowsArgs args{mixed, a, b, a_log, dt_bias, state, y, snaps, p, channels};
+        constexpr int LANES = ROWS_LANES_PER_ROW, ROWS_PER_WG = 256 / LANES;
+        const dim3 grid((p.v_dim + ROWS_PER_WG - 1) / ROWS_PER_WG, p.v_heads);
+        if (p.snapshots) {
+            deltanet_rows_kernel<true, LANES><<<grid, 256, 0, as_stream(stream)>>>(args);
+        } else {
+            deltanet_rows_kernel<false, LANES><<<grid, 256, 0, as_stream(stream)>>>(args);
+        }
     }
     const uint32_t pairs = p.tokens * p.v_heads;
     deltanet_gated_norm_rows_kernel<<<(pairs + 3) / 4, 256, 0, as_stream(stream)>>>(y, z, norm_w, pairs, p.v_dim, p.eps);

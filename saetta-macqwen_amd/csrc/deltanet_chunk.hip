@@ -1,0 +1,580 @@
+// Gated DeltaNet over the tokens of a prefill chunk on the matrix cores: the delta rule in its
+// chunked form, blocks of 64 tokens.
+//
+// What it computes is what deltanet_rows_kernel computes token by token (the reference's definition:
+// src/cpu/deltanet.rs:69-155, delta_rule :148-155; the kernels it stands for: delta_prep + delta_rows3,
+// kernels/prefill.metal:788-1116): per value head, with state S [v_dim][128],
+//     S <- g_t S;  u_t = beta_t (v_t - S k_t);  S += u_t k_t^T;  o_t = S q_t.
+// Inside a block of C = 64 tokens, with c_t = sum_{r <= t} log g_r and S0 the state before the block,
+//     S_t = e^{c_t} S0 + sum_{s <= t} e^{c_t - c_s} u_s k_s^T,
+// so the u_t solve a triangular system that does not involve the state's rows one by one:
+//     (I + A) U = diag(beta) (V - diag(e^c) K S0^T),   A_ts = beta_t e^{c_t - c_s} (k_t . k_s)  (s < t)
+//     O = diag(e^c) Q S0^T + M U,                       M_ts = e^{c_t - c_s} (q_t . k_s)         (s <= t)
+//     S1^T = e^{c_last} S0^T + K^T diag(e^{c_last - c}) U
+// (U, V, O: [C][v_dim]; K, Q: [C][128], normalised as the reference does).  Two kernels:
+//   deltanet_chunk_prepare_kernel   one workgroup per (block, value head), all blocks at once: the
+//       normalised q and k, A and M (64 x 64 x 128 products), T = (I + A)^-1 diag(beta) by forward
+//       substitution, and the decay factors, to a workspace;
+//   deltanet_chunk_chain_kernel     one workgroup per (16 value dims, value head) walks the blocks in
+//       order with its slice of the state in registers: five small products per block.
+// All products run on v_mfma_f32_16x16x32_f16 with every operand split into an f16 hi and lo part
+// (hi * hi + hi * lo + lo * hi: about 2^-21 relative, against 2^-24 of the f32 chain; f32 MFMA has an
+// eighth of the rate per k and wants one LDS read per operand element).  The exponents e^{c_t - c_s}
+// never exceed 1.  The output differs from the token-by-token kernels' by rounding only (tests hold it
+// to 1e-4 of the largest value over a 4096-token chunk).
+#include "common.hpp"
+#include "deltanet_gates.hpp"
+#include "lanes.hpp"
+
+#include <mutex>
+
+namespace saetta {
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int K_DIM = 128;
+constexpr int C = 64;                 // tokens per block
+constexpr int KROW = K_DIM + 8;       // f16 per row of a q / k image: 272 bytes, so that 16 rows' 16-byte reads fall on all banks
+constexpr int TROW = C + 8;           // f16 per row of a T / M image: 144 bytes, likewise
+constexpr int K_IMG = C * KROW * 2;   // bytes: 17408 = 17 load instructions of 1 KB
+constexpr int T_IMG = C * TROW * 2;   // bytes: 9216 = 9 load instructions
+constexpr int KTROW = C + 8;          // f16 per row of the keys' image by key dim, [128][72]
+constexpr int X_IMG = K_DIM * KTROW * 2;  // bytes: 18432 = 18 load instructions
+constexpr int DV = 16;                // value dims per workgroup of the chain kernel (32: 317 against 253 us per 4096 tokens)
+constexpr float Q_SCALE = 0.08838834764831845f;  // 1 / sqrt(128), the reference's factor on q
+static_assert(K_IMG % 1024 == 0 && T_IMG % 1024 == 0, "images are whole load instructions");
+
+// Workspace, per block: per key head the images kh | kl | qh | ql and the keys by key dim xh | xl, then
+// per value head th | tl | mh | ml and 128 floats: e^{c_t} and e^{c_last - c_t}.
+static_assert(X_IMG % 1024 == 0, "images are whole load instructions");
+constexpr size_t KHEAD_BYTES = 4 * size_t(K_IMG) + 2 * size_t(X_IMG);
+constexpr size_t VHEAD_BYTES = 4 * size_t(T_IMG) + 2 * C * sizeof(float);
+__host__ __device__ inline size_t block_bytes(uint32_t k_heads, uint32_t v_heads) { return k_heads * KHEAD_BYTES + v_heads * VHEAD_BYTES; }
+
+struct ChunkArgs {
+    const float *mixed, *a, *b, *a_log, *dt_bias;
+    float *state;
+    float *o;  // [tokens][v_heads][v_dim], before the gated norm
+    unsigned char *ws;
+    uint32_t k_heads, v_heads, v_dim, tokens, channels;
+    float eps;
+};
+
+__device__ __forceinline__ void split2(float x, _Float16 &hi, _Float16 &lo) {
+    hi = (_Float16)x;
+    lo = (_Float16)(x - (float)hi);
+}
+
+// acc += A B with both operands in hi and lo parts
+__device__ __forceinline__ floatx4 mma3(half8 ah, half8 al, half8 bh, half8 bl, floatx4 acc) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, bh, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bl, acc, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bh, acc, 0, 0, 0);
+}
+
+// ---- prepare: everything of a block that does not depend on the state ------------------------------
+// LDS: the four q / k images; once the products are taken, A (f32, over kh), the M images (over kl) and
+// later the T images (over qh) are staged over them, so that they leave as whole 16-byte stores.
+constexpr int PREP_LDS = 4 * K_IMG + 2 * C * 4;
+constexpr int AROW = C + 4;  // f32 per row of A in LDS: [t][q * 16 + m] holds A_t,s of s = 4m + q
+static_assert(C * AROW * 4 <= K_IMG && 2 * T_IMG <= K_IMG + K_IMG, "the staged matrices fit over the images");
+
+__global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    _Float16 *kh = reinterpret_cast<_Float16 *>(lds), *kl = kh + C * KROW, *qh = kl + C * KROW, *ql = qh + C * KROW;
+    float *a_lds = reinterpret_cast<float *>(lds);                        // over kh
+    _Float16 *m_lds = reinterpret_cast<_Float16 *>(lds + K_IMG);           // mh | ml over kl (and the start of qh)
+    _Float16 *t_lds = reinterpret_cast<_Float16 *>(lds + 2 * K_IMG + T_IMG);  // th | tl over the rest of qh and ql
+    float *cum_lds = reinterpret_cast<float *>(lds + 4 * K_IMG), *beta_lds = cum_lds + C;
+    static_assert(K_IMG + 2 * T_IMG <= 2 * K_IMG + T_IMG && 2 * K_IMG + 3 * T_IMG <= 4 * K_IMG, "M and T do not overlap");
+    const uint32_t blk = blockIdx.x, h = blockIdx.y, group = a.v_heads / a.k_heads, khd = h / group;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), n = lane & 15, j = lane >> 4;
+    const uint32_t key_size = a.k_heads * K_DIM;
+    unsigned char *ws_blk = a.ws + size_t(blk) * block_bytes(a.k_heads, a.v_heads);
+    unsigned char *ws_k = ws_blk + khd * KHEAD_BYTES;
+    unsigned char *ws_v = ws_blk + a.k_heads * KHEAD_BYTES + h * VHEAD_BYTES;
+    const bool writer = h % group == 0;  // one value head of the key head's group keeps the q / k images
+
+    // ---- q and k of the block's tokens, normalised (src/cpu/deltanet.rs:133-146), as hi and lo parts ----
+    {
+        const uint32_t t = tid >> 2, part = tid & 3, tok = blk * C + t;
+        float4 qv[8], kv[8];
+        float qs = 0.0f, ks = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            qv[i] = kv[i] = make_float4(0, 0, 0, 0);
+            if (tok < a.tokens) {
+                const float *row = a.mixed + size_t(tok) * a.channels + khd * K_DIM + 32 * part + 4 * i;
+                qv[i] = *reinterpret_cast<const float4 *>(row);
+                kv[i] = *reinterpret_cast<const float4 *>(row + key_size);
+            }
+            qs += qv[i].x * qv[i].x + qv[i].y * qv[i].y + qv[i].z * qv[i].z + qv[i].w * qv[i].w;
+            ks += kv[i].x * kv[i].x + kv[i].y * kv[i].y + kv[i].z * kv[i].z + kv[i].w * kv[i].w;
+        }
+        qs = group_reduce<4>(qs, SumOp());
+        ks = group_reduce<4>(ks, SumOp());
+        const bool real = tok < a.tokens;
+        // (q's factor 1 / sqrt(128) is applied to the output: at unit length the lo parts stay clear of the f16 underflow)
+        const float qi = real ? __builtin_amdgcn_rsqf(qs + a.eps) : 0.0f;
+        const float ki = real ? __builtin_amdgcn_rsqf(ks + a.eps) : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) {
+            half8 a_qh, a_ql, a_kh, a_kl;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float4 qq = qv[i + e / 4], kk = kv[i + e / 4];
+                const float qf = (e % 4 == 0 ? qq.x : e % 4 == 1 ? qq.y : e % 4 == 2 ? qq.z : qq.w) * qi;
+                const float kf = (e % 4 == 0 ? kk.x : e % 4 == 1 ? kk.y : e % 4 == 2 ? kk.z : kk.w) * ki;
+                _Float16 hi, lo;
+                split2(qf, hi, lo);
+                a_qh[e] = hi, a_ql[e] = lo;
+                split2(kf, hi, lo);
+                a_kh[e] = hi, a_kl[e] = lo;
+            }
+            const int at = t * KROW + 32 * part + 4 * i;
+            *reinterpret_cast<half8 *>(kh + at) = a_kh, *reinterpret_cast<half8 *>(kl + at) = a_kl;
+            *reinterpret_cast<half8 *>(qh + at) = a_qh, *reinterpret_cast<half8 *>(ql + at) = a_ql;
+            if (writer) {
+                _Float16 *g = reinterpret_cast<_Float16 *>(ws_k) + at;
+                *reinterpret_cast<half8 *>(g) = a_kh, *reinterpret_cast<half8 *>(g + C * KROW) = a_kl;
+                *reinterpret_cast<half8 *>(g + 2 * C * KROW) = a_qh, *reinterpret_cast<half8 *>(g + 3 * C * KROW) = a_ql;
+            }
+        }
+    }
+    // ---- the gates: c_t = sum of log g up to t, beta_t (tokens past the end: g = 1, beta = 0) ----
+    if (tid < C) {
+        const uint32_t tok = blk * C + tid;
+        float lg = 0.0f, beta = 0.0f;
+        if (tok < a.tokens) {
+            float g;
+            fast_gates(a.a[size_t(tok) * a.v_heads + h] + a.dt_bias[h], __expf(a.a_log[h]), a.b[size_t(tok) * a.v_heads + h], g, beta, &lg);
+        }
+        // inclusive sum over the 64 lanes
+        float c = lg;
+#pragma unroll
+        for (int d = 1; d < 64; d *= 2) {
+            const float up = __shfl_up(c, d, 64);
+            if (int(lane) >= d) c += up;
+        }
+        cum_lds[tid] = c, beta_lds[tid] = beta;
+        const float last = __shfl(c, 63, 64);
+        float *gam = reinterpret_cast<float *>(ws_v + 4 * T_IMG);
+        gam[tid] = __expf(c), gam[C + tid] = __expf(last - c);
+    }
+    __syncthreads();
+
+    // ---- k . k and q . k: rows 16 wave .. + 15, the column tiles at and below the diagonal ----
+    floatx4 gk[4], gq[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+        gk[nt] = gq[nt] = floatx4{0, 0, 0, 0};
+        if (nt <= int(wave)) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                const int ao = (16 * wave + n) * KROW + 32 * ks + 8 * j, bo = (16 * nt + n) * KROW + 32 * ks + 8 * j;
+                const half8 bh = *reinterpret_cast<const half8 *>(kh + bo), bl = *reinterpret_cast<const half8 *>(kl + bo);
+                gk[nt] = mma3(*reinterpret_cast<const half8 *>(kh + ao), *reinterpret_cast<const half8 *>(kl + ao), bh, bl, gk[nt]);
+                gq[nt] = mma3(*reinterpret_cast<const half8 *>(qh + ao), *reinterpret_cast<const half8 *>(ql + ao), bh, bl, gq[nt]);
+            }
+        }
+    }
+    // ---- the keys once more by key dim: [128][72] hi | lo, what the state's update contracts over tokens ----
+    if (writer) {
+        const uint32_t dk = tid >> 1, half = tid & 1;
+        _Float16 *g = reinterpret_cast<_Float16 *>(ws_k + 4 * K_IMG) + dk * KTROW + 32 * half;
+#pragma unroll
+        for (int part = 0; part < 4; part++) {
+            half8 vh, vl;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const int at = (32 * half + 8 * part + e) * KROW + dk;
+                vh[e] = kh[at], vl[e] = kl[at];
+            }
+            *reinterpret_cast<half8 *>(g + 8 * part) = vh;
+            *reinterpret_cast<half8 *>(g + K_DIM * KTROW + 8 * part) = vl;
+        }
+    }
+    __syncthreads();  // the images are read: A and M go over them
+
+    // C layout: lane (n, j) holds column s = 16 nt + n of rows t = 16 wave + 4j + i
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+        const uint32_t s = 16 * nt + n;
+        const float cs = cum_lds[s];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t t = 16 * wave + 4 * j + i;
+            const float decay = s <= t ? __expf(cum_lds[t] - cs) : 0.0f;
+            a_lds[t * AROW + (s & 3) * 16 + (s >> 2)] = s < t ? beta_lds[t] * decay * gk[nt][i] : 0.0f;
+            _Float16 hi, lo;
+            split2(decay * gq[nt][i], hi, lo);
+            m_lds[t * TROW + s] = hi, m_lds[C * TROW + t * TROW + s] = lo;
+        }
+    }
+    __syncthreads();
+    // M leaves (whole 16-byte pieces; the padding columns go along)
+    {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(m_lds);
+        u32x4 *dst = reinterpret_cast<u32x4 *>(ws_v + 2 * T_IMG);
+        for (uint32_t i = tid; i < 2 * T_IMG / 16; i += 256) dst[i] = src[i];
+    }
+
+    // ---- T = (I + A)^-1 diag(beta): column c = 16 wave + n by forward substitution, x_t = beta_t [t = c] -
+    // sum_{s < t} A_ts x_s; lane group q keeps x_s of s = 4m + q in slot m and adds up those s ----
+    {
+        const uint32_t c = 16 * wave + n, q = j;
+        float x[16];
+#pragma unroll
+        for (int m = 0; m < 16; m++) x[m] = 0.0f;
+#pragma unroll
+        for (int t = 0; t < C; t++) {
+            if (t < int(16 * wave)) continue;  // (the column is zero above its diagonal: uniform per wave)
+            floatx4 part4 = {0, 0, 0, 0};  // (four chains of sums instead of one of up to 16)
+            const float *arow = a_lds + t * AROW + q * 16;
+#pragma unroll
+            for (int m4 = 0; 16 * m4 < t; m4++) {  // s = 4m + q < t needs m <= (t - 1) / 4
+                const floatx4 av = *reinterpret_cast<const floatx4 *>(arow + 4 * m4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) part4[e] += av[e] * x[4 * m4 + e];
+            }
+            const float total = across_rows<16, 64>((part4[0] + part4[1]) + (part4[2] + part4[3]), SumOp());
+            const float xt = (uint32_t(t) == c ? beta_lds[t] : 0.0f) - total;
+            if (q == uint32_t(t & 3)) x[t >> 2] = xt;
+        }
+#pragma unroll
+        for (int m = 0; m < 16; m++) {
+            _Float16 hi, lo;
+            split2(x[m], hi, lo);
+            t_lds[(4 * m + q) * TROW + c] = hi, t_lds[C * TROW + (4 * m + q) * TROW + c] = lo;
+        }
+    }
+    __syncthreads();
+    {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(t_lds);
+        u32x4 *dst = reinterpret_cast<u32x4 *>(ws_v);
+        for (uint32_t i = tid; i < 2 * T_IMG / 16; i += 256) dst[i] = src[i];
+    }
+}
+
+// ---- the chain over the blocks --------------------------------------------------------------------
+// Per block, with S0 [dv][128] the state's slice: P = K S0^T and Q S0^T (rows: tokens); R = V - e^c P;
+// U = T R; O = (e^c (Q S0^T) + M U) / sqrt(128); S1 = e^{c_last} S0 + (e^{c_last - c} U)^T K.
+// The images of the next block are requested as soon as their place is free: k and q (rows: tokens)
+// once every wave has R, the keys by key dim once every wave has the new state; T and M, which a
+// wave needs 16 rows of, come a block ahead straight into registers.  The loads of the loop are inline
+// assembly and waited for by hand.
+struct ChainLds {
+    static constexpr int KH = 0, KL = KH + K_IMG, QH = KL + K_IMG, QL = QH + K_IMG;
+    static constexpr int XH = QL + K_IMG, XL = XH + X_IMG;  // the keys by key dim: [128][KTROW] f16
+    static constexpr int GAM = XL + X_IMG;                 // e^{c_t}, e^{c_last - c_t}: 128 f32
+    static constexpr int V = GAM + 2 * C * 4;              // [token][DV] f32
+    static constexpr int SROW = K_DIM + 8;                 // f16 per row of the state's operand image [dv][128]
+    static constexpr int SH = V + C * DV * 4, SL = SH + DV * SROW * 2;
+    static constexpr int RH = SL + DV * SROW * 2;          // [dv][64 tokens] images, rows of TROW f16: R, U, U scaled
+    static constexpr int RL = RH + DV * TROW * 2, UH = RL + DV * TROW * 2, UL = UH + DV * TROW * 2;
+    static constexpr int WH = UL + DV * TROW * 2, WL = WH + DV * TROW * 2;
+    static constexpr int BYTES = WL + DV * TROW * 2;
+    static_assert(BYTES <= 160 * 1024, "LDS of a CU");
+};
+
+__global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) {
+    using L = ChainLds;
+    constexpr int NT = DV / 16;  // 16-wide tiles of value dims
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const uint32_t slice = blockIdx.x, h = blockIdx.y, group = a.v_heads / a.k_heads, khd = h / group;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), n = lane & 15, j = lane >> 4;
+    const uint32_t nblocks = (a.tokens + C - 1) / C;
+    const size_t per_block = block_bytes(a.k_heads, a.v_heads);
+    const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(lds));
+    auto img = [&](int off) { return reinterpret_cast<const _Float16 *>(lds + off); };
+    auto img_w = [&](int off) { return reinterpret_cast<_Float16 *>(lds + off); };
+    const float *gam = reinterpret_cast<const float *>(lds + L::GAM);
+    float *v_lds = reinterpret_cast<float *>(lds + L::V);
+
+    // `pieces` KB from global memory straight into LDS, the waves taking 1 KB pieces in turn
+    auto copy_in = [&](int lds_off, const unsigned char *src, int pieces) {
+        for (int i = wave; i < pieces; i += 4) {
+            asm volatile("s_mov_b32 m0, %0\n"
+                         "s_nop 0\n"
+                         "global_load_lds_dwordx4 %1, %2\n"
+                         :
+                         : "s"(lds0 + lds_off + i * 1024), "v"(uint32_t(i * 1024 + lane * 16)), "s"(src)
+                         : "memory", "m0");
+        }
+    };
+    auto load16 = [&](const void *p) {
+        u32x4 v;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+        return v;
+    };
+    auto ws_k_of = [&](uint32_t blk) { return a.ws + size_t(blk) * per_block + khd * KHEAD_BYTES; };
+    auto ws_v_of = [&](uint32_t blk) { return a.ws + size_t(blk) * per_block + a.k_heads * KHEAD_BYTES + h * VHEAD_BYTES; };
+    constexpr int KQ_PIECES = 4 * K_IMG / 1024, X_PIECES = 2 * X_IMG / 1024;
+    static_assert(KQ_PIECES % 4 == 0 && X_PIECES == 36, "pieces per wave");
+    constexpr int V_LOADS = C * DV * 4 / 16 / 256;  // 16-byte loads per thread of the block's values
+
+    // T and M: this wave's rows 16 wave + n, columns 32 ks + 8j .. + 7, hi and lo: operands as they are.
+    // (The registers an assembly load fills are handed on only behind the wait that names them, in the
+    // same straight piece of code: the compiler takes them for ready from the load on.)
+    u32x4 tm[8];
+    auto request_ahead = [&](uint32_t blk, u32x4 (&tm_next)[8], u32x4 (&v_next)[V_LOADS], u32x4 &gam_next) {
+        copy_in(L::KH, ws_k_of(blk), KQ_PIECES);
+        const unsigned char *wv = ws_v_of(blk);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            // i: matrix (T | M) * 4 + part (hi | lo) * 2 + k-step
+            tm_next[i] = load16(wv + (i >> 1) * T_IMG + ((16 * wave + n) * TROW + 32 * (i & 1) + 8 * j) * 2);
+        }
+#pragma unroll
+        for (int i = 0; i < V_LOADS; i++) {
+            // piece p of the block's [token][DV] values: token p / (DV / 4), four dims
+            const uint32_t p = tid + 256 * i, tok = min(blk * C + p / (DV / 4), a.tokens - 1);  // (a token past the end: unused, see below)
+            v_next[i] = load16(a.mixed + size_t(tok) * a.channels + 2 * a.k_heads * K_DIM + h * a.v_dim + DV * slice + 4 * (p % (DV / 4)));
+        }
+        gam_next = load16(wv + 4 * T_IMG + 16 * (tid & 31));
+    };
+    auto place_ahead = [&](uint32_t blk, u32x4 (&tm_next)[8], u32x4 (&v_next)[V_LOADS], u32x4 &gam_next) {
+        // (nothing else is in flight: loads into registers and loads into LDS do not return in one order,
+        // so a count that leaves some of one kind in flight says nothing about the other kind)
+        if constexpr (V_LOADS == 1) {
+            asm volatile("s_waitcnt vmcnt(0)" : "+v"(tm_next[0]), "+v"(tm_next[1]), "+v"(tm_next[2]), "+v"(tm_next[3]), "+v"(tm_next[4]),
+                         "+v"(tm_next[5]), "+v"(tm_next[6]), "+v"(tm_next[7]), "+v"(v_next[0]), "+v"(gam_next)::"memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" : "+v"(tm_next[0]), "+v"(tm_next[1]), "+v"(tm_next[2]), "+v"(tm_next[3]), "+v"(tm_next[4]),
+                         "+v"(tm_next[5]), "+v"(tm_next[6]), "+v"(tm_next[7]), "+v"(v_next[0]), "+v"(v_next[V_LOADS - 1]), "+v"(gam_next)::"memory");
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) tm[i] = tm_next[i];
+#pragma unroll
+        for (int i = 0; i < V_LOADS; i++) {
+            const uint32_t p = tid + 256 * i;
+            const bool real = blk * C + p / (DV / 4) < a.tokens;
+            reinterpret_cast<u32x4 *>(v_lds)[p] = real ? v_next[i] : u32x4{0, 0, 0, 0};
+        }
+        if (tid < 32) reinterpret_cast<u32x4 *>(lds + L::GAM)[tid] = gam_next;
+    };
+
+    // ---- the state's slice: S [dv][128]; wave w keeps columns 32 w .. + 31: lane (n, j) the four rows
+    // dv = 16 mt + 4j + i of columns 32 w + 16 nt + n.  Its image for the products lies in LDS as hi and lo parts. ----
+    float *state = a.state + (size_t(h) * a.v_dim + DV * slice) * K_DIM;
+    floatx4 s_reg[NT][2];
+    auto publish_state = [&]() {
+#pragma unroll
+        for (int mt = 0; mt < NT; mt++) {
+#pragma unroll
+            for (int nt = 0; nt < 2; nt++) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    _Float16 hi, lo;
+                    split2(s_reg[mt][nt][i], hi, lo);
+                    const int at = (16 * mt + 4 * j + i) * L::SROW + 32 * wave + 16 * nt + n;
+                    img_w(L::SH)[at] = hi, img_w(L::SL)[at] = lo;
+                }
+            }
+        }
+    };
+#pragma unroll
+    for (int mt = 0; mt < NT; mt++) {
+#pragma unroll
+        for (int nt = 0; nt < 2; nt++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) s_reg[mt][nt][i] = state[(16 * mt + 4 * j + i) * K_DIM + 32 * wave + 16 * nt + n];
+        }
+    }
+    publish_state();
+    {
+        u32x4 tm_next[8], v_next[V_LOADS], gam_next;
+        request_ahead(0, tm_next, v_next, gam_next);
+        place_ahead(0, tm_next, v_next, gam_next);
+        copy_in(L::XH, ws_k_of(0) + 4 * K_IMG, X_PIECES);
+    }
+
+    for (uint32_t blk = 0; blk < nblocks; blk++) {
+        const bool more = blk + 1 < nblocks;
+        __syncthreads();  // the block's k and q images, its values and factors and the state's image are in LDS
+
+        // ---- K S0^T and Q S0^T: rows t = 16 wave + n, columns dv = 16 vt + n' ----
+        floatx4 pk[NT], pq[NT];
+#pragma unroll
+        for (int vt = 0; vt < NT; vt++) pk[vt] = pq[vt] = floatx4{0, 0, 0, 0};
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            const int ao = (16 * wave + n) * KROW + 32 * ks + 8 * j;
+            const half8 akh = *reinterpret_cast<const half8 *>(img(L::KH) + ao), akl = *reinterpret_cast<const half8 *>(img(L::KL) + ao);
+            const half8 aqh = *reinterpret_cast<const half8 *>(img(L::QH) + ao), aql = *reinterpret_cast<const half8 *>(img(L::QL) + ao);
+#pragma unroll
+            for (int vt = 0; vt < NT; vt++) {
+                const int bo = (16 * vt + n) * L::SROW + 32 * ks + 8 * j;
+                const half8 bh = *reinterpret_cast<const half8 *>(img(L::SH) + bo), bl = *reinterpret_cast<const half8 *>(img(L::SL) + bo);
+                pk[vt] = mma3(akh, akl, bh, bl, pk[vt]);
+                pq[vt] = mma3(aqh, aql, bh, bl, pq[vt]);
+            }
+        }
+        // C layout: lane (n, j) holds dv = 16 vt + n of tokens t = 16 wave + 4j + i
+        const floatx4 gam4 = *reinterpret_cast<const floatx4 *>(gam + 16 * wave + 4 * j);
+        const floatx4 gk4 = *reinterpret_cast<const floatx4 *>(gam + C + 16 * wave + 4 * j);
+        const float glast = gam[C - 1];
+#pragma unroll
+        for (int vt = 0; vt < NT; vt++) {
+            // R = V - e^c (K S0^T), as the [dv][token] image
+            half4 rh, rl;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                _Float16 hi, lo;
+                split2(v_lds[(16 * wave + 4 * j + i) * DV + 16 * vt + n] - gam4[i] * pk[vt][i], hi, lo);
+                rh[i] = hi, rl[i] = lo;
+            }
+            const int at = (16 * vt + n) * TROW + 16 * wave + 4 * j;
+            *reinterpret_cast<half4 *>(img_w(L::RH) + at) = rh, *reinterpret_cast<half4 *>(img_w(L::RL) + at) = rl;
+        }
+        __syncthreads();  // R is whole; the k and q images, the values and the factors are read
+        // the next block's (after the last block: the last block's again, unused)
+        const uint32_t nxt = more ? blk + 1 : blk;
+        u32x4 tm_next[8], v_next[V_LOADS], gam_next;
+        request_ahead(nxt, tm_next, v_next, gam_next);
+
+        // ---- U = T R (T is lower triangular: k-steps up to the row tile's own) ----
+        floatx4 u[NT];
+#pragma unroll
+        for (int vt = 0; vt < NT; vt++) {
+            u[vt] = floatx4{0, 0, 0, 0};
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                if (ks > int(wave) / 2) continue;
+                const int bo = (16 * vt + n) * TROW + 32 * ks + 8 * j;
+                u[vt] = mma3(__builtin_bit_cast(half8, tm[0 + ks]), __builtin_bit_cast(half8, tm[2 + ks]),
+                             *reinterpret_cast<const half8 *>(img(L::RH) + bo), *reinterpret_cast<const half8 *>(img(L::RL) + bo), u[vt]);
+            }
+            half4 uh, ul, wh, wl;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                _Float16 hi, lo;
+                split2(u[vt][i], hi, lo);
+                uh[i] = hi, ul[i] = lo;
+                split2(u[vt][i] * gk4[i], hi, lo);  // scaled by e^{c_last - c_t} for the state
+                wh[i] = hi, wl[i] = lo;
+            }
+            const int at = (16 * vt + n) * TROW + 16 * wave + 4 * j;
+            *reinterpret_cast<half4 *>(img_w(L::UH) + at) = uh, *reinterpret_cast<half4 *>(img_w(L::UL) + at) = ul;
+            *reinterpret_cast<half4 *>(img_w(L::WH) + at) = wh, *reinterpret_cast<half4 *>(img_w(L::WL) + at) = wl;
+        }
+        // the keys by key dim are here when at most the images requested after them (loads into LDS return
+        // in order) are in flight
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(KQ_PIECES / 4) : "memory");
+        __syncthreads();  // U is whole, and so are the keys by key dim
+
+        // ---- S1 = e^{c_last} S0 + (U scaled)^T K: rows dv, columns 32 wave + 16 nt + n, over the 64 tokens ----
+#pragma unroll
+        for (int nt = 0; nt < 2; nt++) {
+            floatx4 acc[NT];
+#pragma unroll
+            for (int mt = 0; mt < NT; mt++) acc[mt] = floatx4{0, 0, 0, 0};
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                const int bo = (32 * wave + 16 * nt + n) * KTROW + 32 * ks + 8 * j;
+                const half8 bh = *reinterpret_cast<const half8 *>(img(L::XH) + bo), bl = *reinterpret_cast<const half8 *>(img(L::XL) + bo);
+#pragma unroll
+                for (int mt = 0; mt < NT; mt++) {
+                    const int ao = (16 * mt + n) * TROW + 32 * ks + 8 * j;
+                    acc[mt] = mma3(*reinterpret_cast<const half8 *>(img(L::WH) + ao), *reinterpret_cast<const half8 *>(img(L::WL) + ao), bh, bl, acc[mt]);
+                }
+            }
+#pragma unroll
+            for (int mt = 0; mt < NT; mt++) s_reg[mt][nt] = s_reg[mt][nt] * glast + acc[mt];
+        }
+        // ---- O = (e^c (Q S0^T) + M U) / sqrt(128) ----
+#pragma unroll
+        for (int vt = 0; vt < NT; vt++) {
+            floatx4 mu = {0, 0, 0, 0};
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                if (ks > int(wave) / 2) continue;
+                const int bo = (16 * vt + n) * TROW + 32 * ks + 8 * j;
+                mu = mma3(__builtin_bit_cast(half8, tm[4 + ks]), __builtin_bit_cast(half8, tm[6 + ks]),
+                          *reinterpret_cast<const half8 *>(img(L::UH) + bo), *reinterpret_cast<const half8 *>(img(L::UL) + bo), mu);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t tok = blk * C + 16 * wave + 4 * j + i;
+                if (tok < a.tokens) a.o[(size_t(tok) * a.v_heads + h) * a.v_dim + DV * slice + 16 * vt + n] = Q_SCALE * (gam4[i] * pq[vt][i] + mu[i]);
+            }
+        }
+        __syncthreads();  // every wave is through with the keys by key dim, U and the state's image
+        publish_state();
+        place_ahead(nxt, tm_next, v_next, gam_next);
+        copy_in(L::XH, ws_k_of(nxt) + 4 * K_IMG, X_PIECES);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (nothing may land in LDS after the workgroup has ended)
+#pragma unroll
+    for (int mt = 0; mt < NT; mt++) {
+#pragma unroll
+        for (int nt = 0; nt < 2; nt++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) state[(16 * mt + 4 * j + i) * K_DIM + 32 * wave + 16 * nt + n] = s_reg[mt][nt][i];
+        }
+    }
+}
+
+// The workspace is the library's own, per device, grown on demand.
+struct OwnedWorkspace {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+};
+constexpr int OWNED_DEVICES = 64;
+OwnedWorkspace g_owned[OWNED_DEVICES];
+std::mutex g_owned_mutex;
+
+}  // namespace
+
+int setup_deltanet_chunk() {
+    if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(deltanet_chunk_prepare_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, PREP_LDS))) {
+        return rc;
+    }
+    return int(hipFuncSetAttribute(reinterpret_cast<const void *>(deltanet_chunk_chain_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, ChainLds::BYTES));
+}
+
+size_t deltanet_chunk_workspace_bytes(const saetta_rows_step_params &p) {
+    if (p.snapshots || p.tokens < DELTANET_CHUNK_FROM || p.v_dim % DV != 0 || p.k_heads == 0 || p.v_heads % p.k_heads != 0) return 0;
+    return size_t((p.tokens + C - 1) / C) * block_bytes(p.k_heads, p.v_heads);
+}
+
+int run_deltanet_chunk(hipStream_t stream, const float *mixed, const float *a, const float *b, const float *a_log,
+                       const float *dt_bias, float *state, float *o, const saetta_rows_step_params &p, uint32_t channels,
+                       void *workspace) {
+    const uint32_t nblocks = (p.tokens + C - 1) / C;
+    ChunkArgs args{mixed, a, b, a_log, dt_bias, state, o, static_cast<unsigned char *>(workspace), p.k_heads, p.v_heads, p.v_dim, p.tokens, channels, p.eps};
+    deltanet_chunk_prepare_kernel<<<dim3(nblocks, p.v_heads), 256, PREP_LDS, stream>>>(args);
+    deltanet_chunk_chain_kernel<<<dim3(p.v_dim / DV, p.v_heads), 256, ChainLds::BYTES, stream>>>(args);
+    return SAETTA_OK;
+}
+
+int run_deltanet_chunk_owned(hipStream_t stream, const float *mixed, const float *a, const float *b, const float *a_log,
+                             const float *dt_bias, float *state, float *o, const saetta_rows_step_params &p, uint32_t channels) {
+    const size_t need = deltanet_chunk_workspace_bytes(p);
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev)) return fail(int(e), "deltanet_rows: %s", hipGetErrorString(e));
+    SAETTA_REQUIRE(dev >= 0 && dev < OWNED_DEVICES, SAETTA_E_DEVICE, "deltanet_rows: device index %d (up to %d)", dev, OWNED_DEVICES - 1);
+    // held until the launches that use the workspace are queued (as for the prefill workspace)
+    std::lock_guard<std::mutex> lock(g_owned_mutex);
+    OwnedWorkspace &w = g_owned[dev];
+    if (w.bytes < need) {
+        if (w.ptr) {
+            (void)hipDeviceSynchronize();
+            (void)hipFree(w.ptr);
+        }
+        w.ptr = nullptr;
+        w.bytes = 0;
+        hipError_t e = hipMalloc(&w.ptr, need);
+        if (e != hipSuccess) return fail(int(e), "deltanet_rows: workspace of %zu bytes: %s", need, hipGetErrorString(e));
+        w.bytes = need;
+    }
+    return run_deltanet_chunk(stream, mixed, a, b, a_log, dt_bias, state, o, p, channels, w.ptr);
+}
+
+}  // namespace saetta

@@ -7,7 +7,7 @@ LIB_PATH = os.environ.get("SAETTA_HIP_LIB") or os.path.join(_HERE, "lib", "libsa
 
 # Every symbol include/saetta_hip.h declares; tests check the library exports each.
 SYMBOLS = [
-    "saetta_init", "saetta_last_error", "saetta_kv_quantize", "saetta_kv_dequantize", "saetta_kv_dequantize_f32", "saetta_to_half", "saetta_attn_prep_store", "saetta_deltanet_conv", "saetta_deltanet_step", "saetta_deltanet_conv_rows", "saetta_deltanet_rows", "saetta_deltanet_token", "saetta_deltanet_rows_fused",
+    "saetta_init", "saetta_last_error", "saetta_kv_quantize", "saetta_kv_dequantize", "saetta_kv_dequantize_f32", "saetta_to_half", "saetta_attn_prep_store", "saetta_deltanet_conv", "saetta_deltanet_step", "saetta_deltanet_conv_rows", "saetta_deltanet_rows", "saetta_deltanet_rows_ws", "saetta_deltanet_rows_workspace_bytes", "saetta_deltanet_token", "saetta_deltanet_rows_fused",
     "saetta_part_o_bytes", "saetta_part_ml_bytes", "saetta_attn_decode", "saetta_attn_decode_quant",
     "saetta_attn_rows", "saetta_attn_rows_quant", "saetta_static_scratch_bytes", "saetta_attn_decode_quant_static", "saetta_prefill_workspace_bytes", "saetta_attn_prefill", "saetta_attn_prefill_quant",
 ]
@@ -79,6 +79,10 @@ def lib():
         l.saetta_deltanet_conv_rows.argtypes = [vp] * 6 + [ConvRowsParamsC]
         l.saetta_deltanet_rows.restype = i32
         l.saetta_deltanet_rows.argtypes = [vp] * 11 + [RowsStepParamsC]
+        l.saetta_deltanet_rows_ws.restype = i32
+        l.saetta_deltanet_rows_ws.argtypes = [vp] * 11 + [RowsStepParamsC, vp, ctypes.c_size_t]
+        l.saetta_deltanet_rows_workspace_bytes.restype = ctypes.c_size_t
+        l.saetta_deltanet_rows_workspace_bytes.argtypes = [RowsStepParamsC]
         l.saetta_attn_prep_store.restype = i32
         l.saetta_attn_prep_store.argtypes = [vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, QuantRowsC, QuantRowsC, vp,
                                              PrepParamsC, u32, u32, vp]

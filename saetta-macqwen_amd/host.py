@@ -467,8 +467,13 @@ def deltanet_rows(plan, mixed, a, b, a_log, dt_bias, state, z, norm_w, y, k_head
         if snaps.numel() < tokens * v_heads * v_dim * 128:
             raise ValueError("deltanet_rows: snapshots too small")
     p = ffi.RowsStepParamsC(k_heads, v_heads, v_dim, tokens, eps, int(snaps is not None))
+    # a prefill chunk runs in blocks of 64 tokens and keeps per-block matrices in a workspace, which the
+    # recorded op owns (the reference's prefill works in buffers of its own, src/prefill.rs:1433-1578)
+    need = ffi.lib().saetta_deltanet_rows_workspace_bytes(p)
+    ws = torch.empty(need, dtype=torch.uint8, device=mixed.device) if need else None
     plan.op("deltanet_rows", lambda s: ffi.check(
-        ffi.lib().saetta_deltanet_rows(s, *[_ptr(t) for t in ts], _ptr(snaps) if snaps is not None else None, p),
+        ffi.lib().saetta_deltanet_rows_ws(s, *[_ptr(t) for t in ts], _ptr(snaps) if snaps is not None else None, p,
+                                          _ptr(ws) if ws is not None else None, need),
         "deltanet_rows"))
 
 

@@ -483,10 +483,14 @@ inline void rows(plan::Plan &plan, const View &mixed, const View &a, const View 
     const saetta_rows_step_params p{uint32_t(k_heads), uint32_t(v_heads), uint32_t(v_dim), uint32_t(tokens), eps, snaps ? 1u : 0u};
     const View sn = snaps ? *snaps : View{};
     const bool has = snaps != nullptr;
+    // a prefill chunk runs in blocks of 64 tokens and keeps per-block matrices in a workspace, which the
+    // recorded op owns (the reference's prefill works in buffers of its own, src/prefill.rs:1433-1578)
+    const size_t need = saetta_deltanet_rows_workspace_bytes(p);
+    const gpu::Buffer ws = need ? gpu::Buffer(need) : gpu::Buffer();
     plan.op("deltanet_rows", [=](hipStream_t s) {
-        check(saetta_deltanet_rows(s, mixed.ptr<float>(), a.ptr<float>(), b.ptr<float>(), a_log.ptr<float>(),
-                                   dt_bias.ptr<float>(), state.ptr<float>(), z.ptr<float>(), norm_w.ptr<float>(),
-                                   y.ptr<float>(), has ? sn.ptr<float>() : nullptr, p),
+        check(saetta_deltanet_rows_ws(s, mixed.ptr<float>(), a.ptr<float>(), b.ptr<float>(), a_log.ptr<float>(),
+                                      dt_bias.ptr<float>(), state.ptr<float>(), z.ptr<float>(), norm_w.ptr<float>(),
+                                      y.ptr<float>(), has ? sn.ptr<float>() : nullptr, p, need ? ws.get() : nullptr, need),
               "deltanet_rows");
     });
 }

@@ -80,7 +80,7 @@ def close(got, want, rel):
     return np.abs(got - want).max() <= rel * max(1.0, np.abs(want).max())
 
 
-def check_against_oracle(layer, tokens, pieces, snapshots):
+def check_against_oracle(layer, tokens, pieces, snapshots, tol=2e-5):
     x, z, a, b = layer.inputs(tokens)
     conv_cpu = np.zeros((layer.kernel - 1, layer.channels), np.float32)
     state_cpu = np.zeros(layer.v_heads * layer.v_dim * K_DIM, np.float32)
@@ -91,10 +91,10 @@ def check_against_oracle(layer, tokens, pieces, snapshots):
         s = slice(at, at + n)
         mixed, y, snaps = layer.gpu_rows(x[s], z[s], a[s], b[s], conv, state, snapshots)
         assert close(host(mixed), want_mixed[s], 2e-6), (at, n)
-        assert close(host(y), want_y[s], 2e-5), (at, n)
+        assert close(host(y), want_y[s], tol), (at, n)
         if n:
             assert np.array_equal(host(conv), want_conv[at + n - 1]), (at, n)
-            assert close(host(state), want_state[at + n - 1], 2e-5), (at, n)
+            assert close(host(state), want_state[at + n - 1], tol), (at, n)
         if snapshots and n:
             assert np.array_equal(host(snaps[0]), want_conv[s])
             assert close(host(snaps[1]), want_state[s], 2e-5)
@@ -114,6 +114,29 @@ def test_real_shape_chunk_crosses_token_blocks():
     # 37 tokens: two full staged blocks of 16 and a ragged one
     layer = Layer(16, 32, 128, 4, seed=12)
     check_against_oracle(layer, 37, [37], snapshots=False)
+
+
+def test_real_shape_longer_chunk_against_oracle():
+    # From 128 tokens on a call without snapshots runs the delta rule in blocks of 64 tokens on the
+    # matrix cores (products of f16 hi and lo parts: about 2^-21 relative per product, against the
+    # oracle's f32 chain).  200 tokens at the real shape: three blocks and a ragged one, every
+    # token's output and the last state against the oracle's token-by-token run; then a piece that
+    # takes the token-by-token kernels (100) followed by one that takes the blocks (150), the state
+    # carried from one to the other.
+    layer = Layer(16, 32, 128, 4, seed=13)
+    # (the memory the workspace and the outputs are taken from holds NaN patterns: whatever is read
+    # before it is written shows)
+    junk = [torch.full((32 << 20,), float("nan"), device="cuda") for _ in range(8)]
+    del junk
+    check_against_oracle(layer, 200, [200], snapshots=False, tol=1e-4)
+    check_against_oracle(layer, 250, [100, 150], snapshots=False, tol=1e-4)
+
+
+def test_blocks_of_tokens_other_value_dims():
+    # value dims that are multiples of 16 take the blocks too; 24 keeps to the token-by-token kernels
+    for v_dim, tokens in ((16, 130), (64, 192), (256, 129), (24, 140)):
+        layer = Layer(2, 4, v_dim, 4, seed=v_dim)
+        check_against_oracle(layer, tokens, [tokens], snapshots=False, tol=1e-4)
 
 
 @pytest.mark.parametrize("v_dim,kernel,tokens", [(4, 2, 5), (24, 4, 17), (100, 7, 33), (256, 4, 16), (16, 16, 3)])
@@ -148,9 +171,12 @@ def test_first_row_equals_the_single_token_kernels():
     assert close(host(y[0]), host(y1), 2e-5) and close(host(state), host(state1), 2e-5)
 
 
-def test_full_chunk_equals_uneven_pieces_bit_for_bit():
-    # 4096 tokens at the real shape: what a prefill chunk is.  The arithmetic of a token does not
-    # depend on where the launch or the staged block starts, so any split gives the same bits.
+def test_full_chunk_equals_uneven_pieces():
+    # 4096 tokens at the real shape: what a prefill chunk is.  One call (64 blocks of 64 tokens on the
+    # matrix cores) against the same tokens in uneven pieces: the short ones run token by token, the
+    # long ones in blocks that start elsewhere.  The two ways differ by rounding only (f16 hi/lo
+    # products against the f32 chain): the normalised outputs agree to 2e-4, the states to 1e-4 of
+    # the largest entry.  Short pieces alone (token by token throughout) agree bit for bit.
     layer = Layer(16, 32, 128, 4, seed=31)
     tokens = 4096
     x, z, a, b = layer.inputs(tokens)
@@ -163,11 +189,22 @@ def test_full_chunk_equals_uneven_pieces_bit_for_bit():
         ys.append(layer.gpu_rows(x[s], z[s], a[s], b[s], conv2, state2)[1])
         at += n
     assert at == tokens
-    assert torch.equal(torch.cat(ys), y)
-    assert torch.equal(conv, conv2) and torch.equal(state, state2)
+    assert torch.equal(conv, conv2)
+    assert float((torch.cat(ys) - y).abs().max()) <= 2e-4 * max(1.0, float(y.abs().max()))
+    assert float((state - state2).abs().max()) <= 1e-4 * max(1.0, float(state.abs().max()))
     assert torch.isfinite(y).all() and float(y.abs().max()) > 0.1
     # decay keeps the state bounded: |g| < 1 and beta in (0, 1) with unit keys
     assert float(state.abs().max()) < 1e3
+    # token by token throughout: any split gives the same bits
+    conv3, state3 = layer.zero_state()
+    conv4, state4 = layer.zero_state()
+    whole = layer.gpu_rows(x[:100], z[:100], a[:100], b[:100], conv3, state3)[1]
+    parts, at = [], 0
+    for n in (1, 15, 16, 17, 51):
+        s = slice(at, at + n)
+        parts.append(layer.gpu_rows(x[s], z[s], a[s], b[s], conv4, state4)[1])
+        at += n
+    assert torch.equal(torch.cat(parts), whole) and torch.equal(state3, state4)
 
 
 def test_rejections():
