@@ -1616,9 +1616,7 @@ __global__ __launch_bounds__((KeysFirst<BITS>::LOADERS + KeysFirst<BITS>::WAVES)
     }
 }
 
-// Merges the splits of one (q head, row) and a 64-dim quarter of the head:
-// weights 2^(m_c - M), then the gate.  256 threads: first one thread per split
-// for the weights, then (16 dim quads) x (16 slices of splits) for the sums.
+// Merges the splits of one (q head, row): weights 2^(m_c - M), then the gate
 // (reference: attention_reduce / attention_reduce_rows,
 // kernels/attention.metal:367-409, kernels/attention_rows.metal:296-342).
 struct ReduceArgs {
@@ -1646,63 +1644,78 @@ static __device__ __align__(256) float scratch[STATIC_PART_O_FLOATS + STATIC_PAR
 constexpr int STATIC_MAX_DEVICES = 64;
 float *g_static_scratch[STATIC_MAX_DEVICES] = {};
 
+// One workgroup per (q head, row, 16 dims of the head): wave w takes a quarter of the splits, lane
+// (slot = lane / 4, quad = lane % 4) up to four of them and four dims.  Every load is requested before
+// anything is waited for; a wave sums its splits relative to its own maximum, so that the four waves
+// meet once, through LDS.
+constexpr int REDUCE_DIMS = 16;
 __global__ __launch_bounds__(256) void attention_reduce_kernel(ReduceArgs a) {
-    __shared__ float w_lds[MAX_SPLITS];
-    __shared__ float red[8];
-    __shared__ floatx4 o_lds[16][16];
-    const uint32_t h = blockIdx.x, row = blockIdx.y, quarter = blockIdx.z;
-    const uint32_t tid = threadIdx.x;
+    __shared__ float wave_m[4], wave_l[4];
+    __shared__ floatx4 wave_o[4][4];
+    const uint32_t h = blockIdx.x, row = blockIdx.y, slice = blockIdx.z;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, slot = lane >> 2, quad = lane & 3;
     const float *ml = a.part_ml + size_t(2) * row * a.nsplits * a.heads;
     const float *po = a.part_o + size_t(row) * a.nsplits * a.heads * DIM;
-    // Everything the kernel reads is requested before anything is waited for: (m, l) of every split
-    // slot, the partial sums (thread = quad d4 of the quarter's 64 dims, slice s of the splits) and
-    // the gate do not need TokenParams for their addresses, only for which of them count.  Slots
-    // past the splits at work hold old values: they are dropped by select, never multiplied.
-    floatx2 mlv = {NO_SCORE, 0.0f};
-    if (tid < a.nsplits) mlv = *reinterpret_cast<const floatx2 *>(ml + 2 * (size_t(tid) * a.heads + h));
-    const uint32_t d4 = tid & 15, s = tid >> 4;
-    floatx4 pv[MAX_SPLITS / 16];
+    // splits of this wave: per_wave (a multiple of 16) from per_wave * wave on; of this lane: slot + 16 i
+    const uint32_t per_wave = (a.nsplits + 63) / 64 * 16;
+    constexpr int PER_LANE = MAX_SPLITS / 64;
+    // Slots past the splits at work hold old values: they are dropped by select, never multiplied.
+    floatx2 mlv[PER_LANE];
+    floatx4 pv[PER_LANE];
 #pragma unroll
-    for (uint32_t i = 0; i < MAX_SPLITS / 16; i++) {
-        const uint32_t c = s + 16 * i;
+    for (int i = 0; i < PER_LANE; i++) {
+        const uint32_t c = per_wave * wave + slot + 16 * i;
+        mlv[i] = floatx2{NO_SCORE, 0.0f};
         pv[i] = floatx4{0, 0, 0, 0};
-        if (c < a.nsplits) {
-            pv[i] = *reinterpret_cast<const floatx4 *>(po + (size_t(c) * a.heads + h) * DIM + 64 * quarter + 4 * d4);
+        if (16 * uint32_t(i) < per_wave && c < a.nsplits) {
+            mlv[i] = *reinterpret_cast<const floatx2 *>(ml + 2 * (size_t(c) * a.heads + h));
+            pv[i] = *reinterpret_cast<const floatx4 *>(po + (size_t(c) * a.heads + h) * DIM + REDUCE_DIMS * slice + 4 * quad);
         }
     }
     const size_t qh = size_t(row) * a.heads + h;
-    const float g = tid < 64 ? a.q_and_gate[qh * 2 * DIM + DIM + 64 * quarter + tid] : 0.0f;
+    const float g = tid < REDUCE_DIMS ? a.q_and_gate[qh * 2 * DIM + DIM + REDUCE_DIMS * slice + tid] : 0.0f;
     const uint32_t max_len = min(a.decode_len ? a.tp->kv_len : a.tp->position + a.rows, a.capacity);
     const uint32_t nblocks = (max_len + BLOCK - 1) / BLOCK;
     const uint32_t parts = min(a.nsplits, nblocks);
-    // weights
-    const float m = tid < parts ? mlv[0] : NO_SCORE, l = tid < parts ? mlv[1] : 0.0f;
-    float mx = m;
-    mx = group_reduce<64>(mx, MaxOp());
-    if ((tid & 63) == 0) red[tid >> 6] = mx;
-    __syncthreads();
-    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    const float w = tid < parts ? exp2f(m - mx) : 0.0f;
-    w_lds[tid] = w;
-    float wl = w * l;
-    wl = group_reduce<64>(wl, SumOp());
-    if ((tid & 63) == 0) red[4 + (tid >> 6)] = wl;
-    __syncthreads();
-    const float total = red[4] + red[5] + red[6] + red[7];
-    floatx4 acc = {0, 0, 0, 0};
+    float m[PER_LANE], mx = NO_SCORE;
 #pragma unroll
-    for (uint32_t i = 0; i < MAX_SPLITS / 16; i++) {
-        const uint32_t c = s + 16 * i;
-        if (c < parts) acc += pv[i] * w_lds[c];
+    for (int i = 0; i < PER_LANE; i++) {
+        const bool live = 16 * uint32_t(i) < per_wave && per_wave * wave + slot + 16 * i < parts;
+        m[i] = live ? mlv[i][0] : NO_SCORE;
+        if (!live) mlv[i][1] = 0.0f, pv[i] = floatx4{0, 0, 0, 0};
+        mx = fmaxf(mx, m[i]);
     }
-    o_lds[s][d4] = acc;
-    __syncthreads();
-    if (tid < 64) {
-        const uint32_t d = tid;  // dim inside the quarter
-        float o = 0.0f;
+    mx = group_reduce<64>(mx, MaxOp());  // the wave's maximum
+    float l = 0.0f;
+    floatx4 o = {0, 0, 0, 0};
 #pragma unroll
-        for (int i = 0; i < 16; i++) o += o_lds[i][d >> 2][d & 3];
-        a.out[qh * DIM + 64 * quarter + d] = o * __builtin_amdgcn_rcpf(total) * __builtin_amdgcn_rcpf(1.0f + __expf(-g));
+    for (int i = 0; i < PER_LANE; i++) {
+        const float w = m[i] > 0.5f * NO_SCORE ? __builtin_amdgcn_exp2f(m[i] - mx) : 0.0f;
+        l += w * mlv[i][1];
+        o += pv[i] * w;
+    }
+    // over the 16 slots (lanes 4 apart: two steps inside a row of 16 lanes, two across rows); l is the same in the four quads
+    l += dpp<0x124>(l), l += dpp<0x128>(l);  // row_ror 4, row_ror 8
+    l = across_rows<16, 64>(l, SumOp());
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        float x = o[e];
+        x += dpp<0x124>(x), x += dpp<0x128>(x);
+        o[e] = across_rows<16, 64>(x, SumOp());
+    }
+    if (lane == 0) wave_m[wave] = mx, wave_l[wave] = l;
+    if (lane < 4) wave_o[wave][lane] = o;  // (lane = quad)
+    __syncthreads();
+    if (tid < REDUCE_DIMS) {
+        const float M = fmaxf(fmaxf(wave_m[0], wave_m[1]), fmaxf(wave_m[2], wave_m[3]));
+        float total = 0.0f, sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float f = wave_m[w] > 0.5f * NO_SCORE ? __builtin_amdgcn_exp2f(wave_m[w] - M) : 0.0f;
+            total += f * wave_l[w];
+            sum += f * wave_o[w][tid >> 2][tid & 3];
+        }
+        a.out[qh * DIM + REDUCE_DIMS * slice + tid] = sum * __builtin_amdgcn_rcpf(total) * __builtin_amdgcn_rcpf(1.0f + __expf(-g));
     }
 }
 
@@ -1832,7 +1845,7 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
     }
     if (stages & SAETTA_STAGE_REDUCE) {
         ReduceArgs r{part_o, part_ml, q_and_gate, out, heads, capacity, nsplits, rows, d_tp, decode_len ? 1u : 0u};
-        attention_reduce_kernel<<<dim3(heads, rows, 4), 256, 0, stream>>>(r);
+        attention_reduce_kernel<<<dim3(heads, rows, DIM / REDUCE_DIMS), 256, 0, stream>>>(r);
     }
     return launch_status(what);
 }
