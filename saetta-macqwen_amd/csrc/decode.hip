@@ -1021,7 +1021,7 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel_p(PartialArg
     attention_partial_body<BITS, 1, true, ITB_ONE_PER_CU, true>(a);
 }
 
-// ---- one query row over codes, keys first ---------------------------------------------------------
+// ---- one to four query rows over codes, keys first ------------------------------------------------
 // attention_partial_kernel_s: the workgroup's share is taken in rounds of up to 17 blocks of 16
 // tokens whose codes all lie in LDS at once (17: a context of 128 x 256 tokens and a few more still
 // is one round).  The KEYS of a round are requested before its values, so they are there when half
@@ -1045,8 +1045,14 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel_p(PartialArg
 // instructions in order, so data written before a counter is raised is there when the counter is
 // seen.  Every wait on a counter is bounded (SPIN_LIMIT polls), so every wave ends whatever happens.
 // Longer shares take further rounds with an online softmax between the rounds.
-template <int BITS>
+// M query rows (a verify step, 2..4): every row is a tile of its own (its 8 heads' hi parts in operand
+// rows 0-7, the lo parts in rows 8-15), and the codes in LDS serve all of them.  The scores are taken
+// row by row, the row's query operands staged through the one place in LDS while the scores of the
+// row before are computed; the probability operands and O += P V go two rows at a time (the
+// registers hold two rows' operands), the byte permutes of a value operand serving both.
+template <int BITS, int M>
 struct KeysFirst {
+    static constexpr int PAIRS = (M + 1) / 2;               // tiles of two query rows (one row: its own tile)
     static constexpr int LOADERS = 4, WAVES = 8;            // loader waves (keys: 0, 1; values: 2, 3), then the computing waves
     static constexpr int K_LOADERS = 2, V_LOADERS = 2;
     static constexpr int RB_ = BITS * 32;                   // bytes of a (token, kv head) row of codes
@@ -1057,46 +1063,55 @@ struct KeysFirst {
     static constexpr int PER_BLOCK = PIECES / 4;            // load instructions per block of keys, and of values: 4 | 2
     static constexpr int V_GROUP_TOKENS = 64 / PIECES;      // token rows one load instruction brings: 4 | 8
     static constexpr int K_BLOCK_BYTES = BLOCK * RB_;       // [64-byte piece][token]: what one load instruction brings
-    static constexpr int V_GROUP_BYTES = 1024 + 32;         // whole token rows; 8 banks between the groups of the four lane groups
+    // Values: whole token rows, each rotated by a quarter row per 8 tokens ((token / 8) % 4 quarters),
+    // so that the four lane groups of a value read, which are 8 tokens apart, fall on different banks.
+    static constexpr int V_ROT = RB_ / 4;
     static constexpr int K_LOADS = 8 * PER_BLOCK;           // per key-loader wave: blocks 0-15, half of them before the other
     static constexpr int V_LOADS = 8 * PER_BLOCK;           // per value-loader wave: slots 0-3
     static constexpr int SC_LOADS = 16;                     // scales and biases of a key loader's 128 tokens: 4 arrays x 2 planes x 2
     static constexpr int X_LOADS = 8 + PER_BLOCK;           // block 16: its scales and biases (4 arrays x 2 planes) and its keys
     static_assert(SC_LOADS + K_LOADS + X_LOADS < 64, "vmcnt is 6 bits");
     // LDS map, in bytes.  The scores of a block (its probabilities relative to the block's maximum,
-    // [head][token] f32, 512 bytes) lie over the block's own keys, which only the wave that writes
-    // them has read.
-    static constexpr int Q_OFF = 0;                                // [k-step][lane] half8
+    // [row][head][token] f32, 512 bytes a row) lie over the block's own keys, which only the wave that
+    // writes them has read.
+    static constexpr int Q_OFF = 0;                                // [k-step][lane] half8: one row's operands at a time
     static constexpr int QZ_OFF = Q_OFF + 8 * 64 * 16;             // [hi, lo][lane][k-step] f16
     // scales and biases: per array two planes of one dword per token, the f16 of groups (0, 1) and of (2, 3)
     static constexpr int SB_OFF = QZ_OFF + 2 * 64 * 16;            // [ks | kz | vs | vz][plane][token] u32
     static constexpr int SB_ARRAY = 2 * ROUND_TOKENS * 4;
-    static constexpr int BSTRIDE = 20;                             // blocks 17-19 never exist: maximum "none", sum 0
-    static constexpr int BMAX_OFF = SB_OFF + 4 * SB_ARRAY;         // [head][block] f32: the block's maximum score
-    static constexpr int BSUM_OFF = BMAX_OFF + 8 * BSTRIDE * 4;    // [head][block] f32: sum of 2^(score - maximum)
-    static constexpr int ZS_OFF = BSUM_OFF + 8 * BSTRIDE * 4;      // [wave][head] f32
-    static constexpr int SYNC_OFF = ZS_OFF + WAVES * 8 * 4;        // 32 counters, u32
+    static constexpr int BROW = 8 * ROUND_BLOCKS;                  // floats of a row's [head][block]
+    static constexpr int BMAX_OFF = SB_OFF + 4 * SB_ARRAY;         // [row][head][block] f32: the block's maximum score
+    static constexpr int BSUM_OFF = BMAX_OFF + M * BROW * 4;       // [row][head][block] f32: sum of 2^(score - maximum)
+    static constexpr int ZS_OFF = BSUM_OFF + M * BROW * 4;         // [wave][pair][column] f32 (one row: [wave][head])
+    static constexpr int SYNC_OFF = ZS_OFF + WAVES * PAIRS * 16 * 4;  // 32 counters, u32
     static constexpr int K_OFF = (SYNC_OFF + 32 * 4 + 255) / 256 * 256;
     static constexpr int V_OFF = K_OFF + ROUND_BLOCKS * K_BLOCK_BYTES;
-    static constexpr int LDS_BYTES = V_OFF + ROUND_BLOCKS * PER_BLOCK * V_GROUP_BYTES;
-    static constexpr int X_OFF = K_OFF;                            // the pairs' merge lies over the keys
+    static constexpr int LDS_BYTES = V_OFF + ROUND_BLOCKS * K_BLOCK_BYTES;
+    // one row: the merge of two waves, [group][lane < 32][4 rows] of 16 bytes, lies over the query operands,
+    // which nobody reads after the last scores
+    static constexpr int X_OFF = Q_OFF;
     static_assert(LDS_BYTES <= 160 * 1024, "LDS of a CU");
+    static_assert(M * 512 <= K_BLOCK_BYTES, "the scores fit over the keys");
+    static_assert(4 * 32 * 64 <= QZ_OFF - Q_OFF, "the merge fits over the query operands");
     // the counters
     static constexpr int C_KEYS = 0;    // key loaders that have requested the first round's keys
-    static constexpr int C_QUERY = 1;   // computing waves that have written their query operands
+    static constexpr int C_QUERY = 1;   // computing waves that have written a row's query operands (8 per row)
     static constexpr int C_SCORES = 2;  // ... written their scores (8 per round)
     static constexpr int C_BUILT = 3;   // ... built their probability operands (8 per round)
     static constexpr int C_DONE = 4;    // ... are through with the round's values (8 per round)
     static constexpr int C_LENGTH = 5;  // (not a counter: the context length, for every wave)
+    static constexpr int C_POSITION = 6;  // (not a counter: the position)
+    static constexpr int C_QREAD = 7;   // computing waves that have a row's query operands in registers (several rows)
     static constexpr int C_KPART = 8;   // [3]: key loaders whose blocks 0-7 and scales | blocks 8-15 | block 16 have landed (2 per round)
     static constexpr int C_SLOT = 12;   // [5]: value loaders whose values of slot s have landed (2 per round)
-    static constexpr int C_MERGE = 20;  // [4]: wave 2g + 1 has written its sums for wave 2g
+    static constexpr int C_MERGE = 20;  // [4]: one row: wave 2g + 1 has written its sums for wave 2g | two pairs of rows: blocks
+                                        // whose keys the two waves of scores w % 4 have in registers; then [4] as with one row
     static constexpr uint32_t SPIN_LIMIT = 1u << 20;
 };
 
-template <int BITS>
-__global__ __launch_bounds__((KeysFirst<BITS>::LOADERS + KeysFirst<BITS>::WAVES) * 64) void attention_partial_kernel_s(PartialArgs a) {
-    using W = KeysFirst<BITS>;
+template <int BITS, int M>
+__global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::WAVES) * 64) void attention_partial_kernel_s(PartialArgs a) {
+    using W = KeysFirst<BITS, M>;
     constexpr int RB = W::RB_, RT = W::ROUND_TOKENS, RBK = W::ROUND_BLOCKS;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const int lane = threadIdx.x & 63;
@@ -1108,23 +1123,36 @@ __global__ __launch_bounds__((KeysFirst<BITS>::LOADERS + KeysFirst<BITS>::WAVES)
     uint32_t *sync_lds = reinterpret_cast<uint32_t *>(lds_raw + W::SYNC_OFF);
     const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(lds_raw));
 
-    // ---- query values: requested first (computing waves: thread = (k-step, lane) item) ----------
-    float qv[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (!loader) {
+    // ---- query values: requested first (computing waves: thread = (k-step, lane) item of every row) ----
+    auto load_query = [&](int r, float (&v)[8]) {
         const int step = wave, g = step >> 1, ab = step & 1;
-        const float *src = a.q + (size_t(kv) * 8 + (n & 7)) * DIM + 64 * g + 16 * j + 8 * ab;
+        const float *src = a.q + (size_t(r) * a.heads + kv * 8 + (n & 7)) * DIM + 64 * g + 16 * j + 8 * ab;
         const float4 f0 = *reinterpret_cast<const float4 *>(src);
         const float4 f1 = *reinterpret_cast<const float4 *>(src + 4);
-        qv[0] = f0.x, qv[1] = f0.y, qv[2] = f0.z, qv[3] = f0.w, qv[4] = f1.x, qv[5] = f1.y, qv[6] = f1.z, qv[7] = f1.w;
+        v[0] = f0.x, v[1] = f0.y, v[2] = f0.z, v[3] = f0.w, v[4] = f1.x, v[5] = f1.y, v[6] = f1.z, v[7] = f1.w;
+    };
+    // (several rows: per pair of rows, the row that the lane's column of the pair's tile belongs to)
+    float qv[W::PAIRS][8];
+#pragma unroll
+    for (int p = 0; p < W::PAIRS; p++) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) qv[p][e] = 0.0f;
+        if (!loader) load_query(M == 1 ? 0 : min(2 * p + (n >> 3), M - 1), qv[p]);
     }
 
     // ---- the context and this workgroup's share of it -----------------------------
-    // One wave of the workgroup reads the context length and hands it on through LDS.  The counters
-    // start at zero behind the same barrier, the only s_barrier of the kernel, before anybody
-    // requests anything of the cache.
-    if (threadIdx.x < 32) sync_lds[threadIdx.x] = threadIdx.x == W::C_LENGTH ? a.tp->kv_len : 0u;
+    // One wave of the workgroup reads the token's parameters and hands them on through LDS.  The
+    // counters start at zero behind the same barrier, the only s_barrier of the kernel, before
+    // anybody requests anything of the cache.
+    if (threadIdx.x < 32) {
+        sync_lds[threadIdx.x] = threadIdx.x == W::C_LENGTH ? a.tp->kv_len : threadIdx.x == W::C_POSITION ? a.tp->position : 0u;
+    }
     __syncthreads();
-    const uint32_t max_len = min(uint32_t(__builtin_amdgcn_readfirstlane(sync_lds[W::C_LENGTH])), a.capacity);
+    const uint32_t kv_len = __builtin_amdgcn_readfirstlane(sync_lds[W::C_LENGTH]);
+    const uint32_t position = __builtin_amdgcn_readfirstlane(sync_lds[W::C_POSITION]);
+    // tokens row r sees; the last row's are the launch's
+    auto len_of = [&](int r) -> uint32_t { return min<uint32_t>(a.decode_len ? kv_len : position + uint32_t(r) + 1, a.capacity); };
+    const uint32_t max_len = len_of(M - 1);
     const uint32_t nblocks = (max_len + BLOCK - 1) / BLOCK;
     uint32_t blk_begin, blk_end;
     if (nblocks <= a.nsplits) {
@@ -1139,7 +1167,8 @@ __global__ __launch_bounds__((KeysFirst<BITS>::LOADERS + KeysFirst<BITS>::WAVES)
     const uint32_t last_tok = limit - 1;                   // rows past it are never read: loads are clamped to it
     const uint32_t range = blk_end - blk_begin;
     // rounds of equal size (to within a block), none longer than 17 blocks
-    const uint32_t n_rounds = (range + RBK - 1) / RBK;
+    // (several rows: the launch has made sure that no share is longer)
+    const uint32_t n_rounds = M > 1 ? 1 : (range + RBK - 1) / RBK;
     const uint32_t per_round = (range + n_rounds - 1) / n_rounds;
     auto blocks_of = [&](uint32_t round) { return min(range - round * per_round, per_round); };
 
@@ -1262,9 +1291,11 @@ __global__ __launch_bounds__((KeysFirst<BITS>::LOADERS + KeysFirst<BITS>::WAVES)
             auto request_block = [&](uint32_t blk) {
 #pragma unroll
                 for (int i = 0; i < W::PER_BLOCK; i++) {
-                    // lane -> (token lane / PIECES of the instruction's group, piece lane % PIECES)
-                    const uint32_t tok = min(base + BLOCK * blk + W::V_GROUP_TOKENS * i + lane / W::PIECES, last_tok);
-                    dma(lds0 + W::V_OFF + (W::PER_BLOCK * blk + i) * W::V_GROUP_BYTES, (tok * kvh + kv) * RB + (lane % W::PIECES) * 16, a.vdata);
+                    // lane -> (token lane / PIECES of the instruction's group, the piece that goes to place lane % PIECES
+                    // of the row, which is rotated by (token / 8) % 4 quarters: the same for the group's tokens)
+                    const uint32_t t = BLOCK * blk + W::V_GROUP_TOKENS * i + lane / W::PIECES;  // token of the round
+                    const uint32_t piece = (lane % W::PIECES + W::PIECES - ((t >> 3) & 3) * (W::PIECES / 4)) % W::PIECES;
+                    dma(lds0 + W::V_OFF + (W::PER_BLOCK * blk + i) * 1024, (min(base + t, last_tok) * kvh + kv) * RB + piece * 16, a.vdata);
                 }
             };
 #pragma unroll
@@ -1312,19 +1343,19 @@ __global__ __launch_bounds__((KeysFirst<BITS>::LOADERS + KeysFirst<BITS>::WAVES)
     float *bmax_lds = reinterpret_cast<float *>(lds_raw + W::BMAX_OFF);
     float *bsum_lds = reinterpret_cast<float *>(lds_raw + W::BSUM_OFF);
     float *zs_lds = reinterpret_cast<float *>(lds_raw + W::ZS_OFF);
-    // the scores of block b: [head][token] f32 over the block's keys
-    auto s_block = [&](int b) { return reinterpret_cast<float *>(lds_raw + W::K_OFF + b * W::K_BLOCK_BYTES); };
+    // the scores of block b, row r: [head][token] f32 over the block's keys
+    auto s_block = [&](int b, int r) { return reinterpret_cast<float *>(lds_raw + W::K_OFF + b * W::K_BLOCK_BYTES + r * 512); };
 
-    // ---- prologue: the query row to f16 hi/lo operands in LDS (operand row n: head n & 7, hi part in
-    // rows 0-7 and lo part in rows 8-15 of the one tile) ---------------------------------------------
-    {
+    // A row's query operands to LDS: f16 hi/lo parts (operand row n: head n & 7, hi part in rows 0-7 and
+    // lo part in rows 8-15 of the row's tile); this thread's item is k-step `wave`, lane `lane`.
+    auto stage_query = [&](const float (&v)[8]) {
         const float qmul = a.scale * 1.4426950408889634f * Q_UP;
         half8 op;
         float sum = 0.0f;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             _Float16 h, lw;
-            split_hi_lo(qv[key_slot_dim<BITS>(e)] * qmul, h, lw);
+            split_hi_lo(v[key_slot_dim<BITS>(e)] * qmul, h, lw);
             const _Float16 x = n < 8 ? h : lw;
             op[e] = x;
             sum += (float)x;
@@ -1335,94 +1366,288 @@ __global__ __launch_bounds__((KeysFirst<BITS>::LOADERS + KeysFirst<BITS>::WAVES)
         split_hi_lo(sum * (1.0f / Q_UP), h, lw);
         qz_lds[(0 * 64 + lane) * 8 + wave] = h;
         qz_lds[(1 * 64 + lane) * 8 + wave] = lw;
-        // blocks that never exist
-        if (wave == 0 && lane < 8 * (W::BSTRIDE - RBK)) {
-            const int idx = (lane / (W::BSTRIDE - RBK)) * W::BSTRIDE + RBK + lane % (W::BSTRIDE - RBK);
-            bmax_lds[idx] = NO_SCORE, bsum_lds[idx] = 0.0f;
+    };
+    // The scores of one block of 16 tokens for R query rows whose operands are in registers: the key
+    // operands are made once and serve every row.  Returns in s[ri] the lane's probabilities relative to
+    // the block's maximum (tokens 4j .. 4j + 3 of the block, head n & 7) and stores the block's maximum and sum.
+    auto block_scores = [&](auto rows_c, int blk, uint32_t base, const half8 (*q_reg)[8], const half8 (*qz_reg)[2], const int *row_of,
+                            const uint32_t *row_limit, int rows_here, floatx4 *s) {
+        constexpr int R = decltype(rows_c)::value;
+        const unsigned char *kb = lds_raw + W::K_OFF + blk * W::K_BLOCK_BYTES;
+        KeyRegs<BITS> kreg[4];
+#pragma unroll
+        for (int gg = 0; gg < 4; gg++) {
+            if constexpr (BITS == 8) {
+                // the group's 64 bytes of token n are piece gg: 16 bytes j of them
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(kb + gg * 1024 + n * 64 + j * 16);
+                kreg[gg].w[0] = v.x, kreg[gg].w[1] = v.y, kreg[gg].w[2] = v.z, kreg[gg].w[3] = v.w;
+            } else {
+                // the group's 32 bytes of token n are half gg % 2 of piece gg / 2: 8 bytes j of them
+                const u32x2 v = *reinterpret_cast<const u32x2 *>(kb + (gg >> 1) * 1024 + n * 64 + (gg & 1) * 32 + j * 8);
+                kreg[gg].w[0] = v.x, kreg[gg].w[1] = v.y;
+            }
         }
-    }
-    raise(W::C_QUERY);
-
-    // ---- running state -------------------------------------------------------------
-    const int g = wave >> 1, b2 = wave & 1;  // phase C: the wave's group and which k-steps of a slot
-    float m_run = NO_SCORE;
-    float l_run = 0.0f;    // sum of P of head n & 7 (wave 0 keeps it)
-    float zacc = 0.0f;     // sum of P * P_UP * value bias of group g over this lane's tokens
-    floatx4 acc[4];        // [tile of 16 dims 4n' + e]: rows 4j .. 4j+3 (operand rows), column n'
+        const int tok0 = BLOCK * blk + 4 * j;  // this lane's 4 tokens of the round in C layout
+        const uint32_t *sb_w = sb_lds + BLOCK * blk;  // the block's dwords of groups (0, 1); + RT: groups (2, 3)
+        // bias term: slot e of every lane group belongs to group e / 2 of token n
+        const u32x2 zr = {sb_w[W::SB_ARRAY / 4 + n], sb_w[W::SB_ARRAY / 4 + RT + n]};
+        const half8 zop = as_half8(perm(0, zr.x, 0x01000100u), perm(0, zr.x, 0x03020302u), perm(0, zr.y, 0x01000100u), perm(0, zr.y, 0x03020302u));
+        // scales of the lane's tokens 4j .. 4j+3 of the block: groups (0, 1) and groups (2, 3)
+        const u32x4 s01 = *reinterpret_cast<const u32x4 *>(sb_w + 4 * j);
+        const u32x4 s23 = *reinterpret_cast<const u32x4 *>(sb_w + RT + 4 * j);
+        const uint32_t sw[8] = {s01.x, s23.x, s01.y, s23.y, s01.z, s23.z, s01.w, s23.w};
+        floatx4 rr[R][4];
 #pragma unroll
-    for (int e = 0; e < 4; e++) acc[e] = floatx4{0, 0, 0, 0};
-    await(W::C_QUERY, W::WAVES);
+        for (int ri = 0; ri < R; ri++) {
+            s[ri] = floatx4{0, 0, 0, 0};
+            s[ri] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz_reg[ri][0], s[ri], 0, 0, 0);
+            s[ri] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz_reg[ri][1], s[ri], 0, 0, 0);
+#pragma unroll
+            for (int gg = 0; gg < 4; gg++) rr[ri][gg] = floatx4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int gg = 0; gg < 4; gg++) {
+#pragma unroll
+            for (int ab = 0; ab < 2; ab++) {
+                const half8 kop = key_operand<BITS>(kreg[gg], ab);
+#pragma unroll
+                for (int ri = 0; ri < R; ri++) rr[ri][gg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop, q_reg[ri][gg * 2 + ab], rr[ri][gg], 0, 0, 0);
+            }
+        }
+        constexpr float C1 = code_up<BITS>() / Q_UP;
+        float scl[4][4];
+#pragma unroll
+        for (int tk = 0; tk < 4; tk++) {
+#pragma unroll
+            for (int gg = 0; gg < 4; gg++) scl[tk][gg] = half_bits_to_float(sw[2 * tk + (gg >> 1)] >> (16 * (gg & 1))) * C1;
+        }
+#pragma unroll
+        for (int ri = 0; ri < R; ri++) {
+            if (ri >= rows_here) continue;
+#pragma unroll
+            for (int tk = 0; tk < 4; tk++) {
+                float d = 0.0f;
+#pragma unroll
+                for (int gg = 0; gg < 4; gg++) d += scl[tk][gg] * rr[ri][gg][tk];
+                float v = s[ri][tk] + d;
+                v += dpp<0x128>(v);  // row_ror 8: the other part (hi | lo) of the same head
+                s[ri][tk] = base + tok0 + tk < row_limit[ri] ? v : NO_SCORE;  // (also whatever a block past the round left in LDS)
+            }
+            // the block's softmax relative to its own maximum, per head
+            float cm = fmaxf(fmaxf(s[ri][0], s[ri][1]), fmaxf(s[ri][2], s[ri][3]));
+            cm = across_rows<16, 64>(cm, MaxOp());
+            float sum = 0.0f;
+#pragma unroll
+            for (int tk = 0; tk < 4; tk++) {
+                s[ri][tk] = s[ri][tk] > 0.5f * NO_SCORE ? __builtin_amdgcn_exp2f(s[ri][tk] - cm) : 0.0f;
+                sum += s[ri][tk];
+            }
+            sum = across_rows<16, 64>(sum, SumOp());
+            if (j == 0 && n < 8) bmax_lds[row_of[ri] * W::BROW + n * RBK + blk] = cm, bsum_lds[row_of[ri] * W::BROW + n * RBK + blk] = sum;
+        }
+    };
+    // The probability operands of k-step ks (tokens 32 ks .. 32 ks + 31 of the round) for R rows: P * value
+    // scale of group g, hi part in operand rows 0-7 and lo part in rows 8-15.  The two lanes of a head (n and
+    // n + 8) make four of the lane group's eight tokens each, both parts, and exchange what the other one
+    // feeds.  K-step 8 is block 16 alone: lane groups 0 and 1; the others repeat them with factor 0.
+    auto build_operands = [&](auto rows_c, int ks, int g, const int *row_of, const float *nm, int rows_here, float *zacc, half8 *out) {
+        constexpr int R = decltype(rows_c)::value;
+        const int hh = n >> 3;  // this lane makes tokens 8j + 4 hh .. + 3 of the k-step
+        const int sh = 16 * (g & 1);
+        const int jj = ks == 8 ? (j & 1) : j;
+        const int blk = 2 * ks + (jj >> 1);
+        // value scales and biases of group g: half g % 2 of the tokens' dwords of groups (g, g ^ 1).
+        // (Tokens past the share have probability 0 and the scales of the share's last token:
+        // every load is clamped to it, so nothing but cache rows in use is ever read.)
+        const uint32_t *vsp = sb_lds + 2 * (W::SB_ARRAY / 4) + (g >> 1) * RT + 32 * ks + 8 * jj + 4 * hh;
+        const u32x4 sv = *reinterpret_cast<const u32x4 *>(vsp);
+        const u32x4 zv = *reinterpret_cast<const u32x4 *>(vsp + W::SB_ARRAY / 4);
+        const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w}, zw[4] = {zv.x, zv.y, zv.z, zv.w};
+        float vscale[4], vbias[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) vscale[e] = half_bits_to_float(sw[e] >> sh), vbias[e] = half_bits_to_float(zw[e] >> sh);
+        const int fb = 2 * ks + (j >> 1);  // block 17 does not exist: factor 0
+#pragma unroll
+        for (int ri = 0; ri < R; ri++) {
+            if (ri >= rows_here) {
+                out[ri] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+                continue;
+            }
+            const int r = row_of[ri];
+            const floatx4 pt = *reinterpret_cast<const floatx4 *>(s_block(blk, r) + (n & 7) * BLOCK + 8 * (jj & 1) + 4 * hh);
+            // 2^(block maximum - round maximum) * P_UP (2^8, so that the lo part stays a normal f16)
+            const float f = fb < RBK ? __builtin_amdgcn_exp2f(bmax_lds[r * W::BROW + (n & 7) * RBK + (fb < RBK ? fb : 0)] - nm[ri] + 8.0f) : 0.0f;
+            float x[4], lo[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float p = pt[e] * f;
+                zacc[ri] += p * vbias[e];
+                x[e] = p * vscale[e];
+                lo[e] = x[e] - __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x[e]) & 0xffffe000u);
+            }
+            // round toward zero: exact truncation to the hi part
+            const uint32_t hi0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x[0], x[1]));
+            const uint32_t hi1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x[2], x[3]));
+            const uint32_t lo0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo[0], lo[1]));
+            const uint32_t lo1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo[2], lo[3]));
+            // the hi lane (n < 8) feeds hi parts and wants the other lane's hi parts of tokens 4-7; the lo
+            // lane feeds lo parts and wants the other lane's lo parts of tokens 0-3
+            const uint32_t send0 = hh ? hi0 : lo0, send1 = hh ? hi1 : lo1;
+            const uint32_t recv0 = uint32_t(__builtin_amdgcn_update_dpp(0, int(send0), 0x128, 0xf, 0xf, false));  // row_ror 8
+            const uint32_t recv1 = uint32_t(__builtin_amdgcn_update_dpp(0, int(send1), 0x128, 0xf, 0xf, false));
+            uint32_t o[4] = {hh ? recv0 : hi0, hh ? recv1 : hi1, hh ? lo0 : recv0, hh ? lo1 : recv1};
+            // (pinned: left alone, the compiler moves an operand's arithmetic down to its use, behind the wait for the values)
+            asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]));
+            out[ri] = as_half8(o[0], o[1], o[2], o[3]);
+        }
+    };
+    // the value codes of k-step ks for group g: the lane's dword of tokens 32 ks + 8j .. + 7
+    auto read_values = [&](int ks, int g, ValRegs<BITS> &vreg) {
+        const int v_lane = val_lane_offset<BITS>(g, n);
+        const int jj = ks == 8 ? (j & 1) : j;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int tk = 32 * ks + 8 * jj + e;
+            // (the token's row is rotated by (tk / 8) % 4 quarters)
+            vreg.w[e] = *reinterpret_cast<const uint32_t *>(lds_raw + W::V_OFF + tk * RB + ((v_lane + ((tk >> 3) & 3) * W::V_ROT) & (RB - 1)));
+        }
+    };
+    // a row's maximum per head over the round's blocks
+    auto round_max = [&](int r, float start) {
+        const float *bmx = bmax_lds + r * W::BROW + (n & 7) * RBK;
+        float v = start;
+#pragma unroll
+        for (int i = 0; i < RBK; i++) v = fmaxf(v, bmx[i]);
+        return v;
+    };
+    // a row's sum of P of head n & 7 over the round's blocks, relative to the maximum nm: lane group j adds blocks j, j + 4, ...
+    auto round_sum = [&](int r, float nm) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < (RBK + 3) / 4; i++) {
+            const int b = j + 4 * i;
+            if (b < RBK) sum += bsum_lds[r * W::BROW + (n & 7) * RBK + b] * __builtin_amdgcn_exp2f(bmax_lds[r * W::BROW + (n & 7) * RBK + b] - nm);  // (a block that is not there: sum 0)
+        }
+        return across_rows<16, 64>(sum, SumOp());
+    };
+    constexpr float unscale = code_up<BITS>() / P_UP;
+    const int g = wave >> 1, b2 = wave & 1;
 
-    for (uint32_t round = 0; round < n_rounds; round++) {
-        const uint32_t base = (blk_begin + round * per_round) * BLOCK, nb = blocks_of(round);
-        const bool more = round + 1 < n_rounds;
-        const bool extra = nb == uint32_t(RBK);  // the round has block 16
-        const uint32_t round_limit = min(limit, base + nb * BLOCK);  // tokens of this round end here
+    if constexpr (M > 1) {
+        // ---- several rows ------------------------------------------------------------------------
+        // Two rows share a tile: its 16 columns are (row of the pair, head), and the hi and the lo parts of
+        // an operand go through two MFMAs into one accumulator, so that every lane of a result holds a
+        // whole score (or output) of its own column.  Three rows: the second pair's upper columns repeat
+        // row 2 and are not written out.
+        // Scores: with one pair every wave takes its blocks (wave, wave + 8; wave 0 also 16); with two
+        // pairs waves 0-3 take the first and waves 4-7 the second, blocks w % 4 + 4 i.  The pair's query
+        // operands stay in registers: they go through the one place in LDS, the hi parts and then the lo
+        // parts of a pair, while the first keys are on their way.
+        // O += P V: as with one row, waves 2g and 2g + 1 share group g and take alternate k-steps, for
+        // every pair, the byte permutes of a value operand serving both pairs.
+        constexpr int PAIRS = W::PAIRS, WT = W::WAVES / PAIRS;
+        const int at = wave / WT, wt = wave % WT;
+        const int col_row = n >> 3;  // the row of the pair that this lane's column belongs to
+        auto row_of = [&](int pair, int half) { return min(2 * pair + half, M - 1); };
+        const uint32_t base = blk_begin * BLOCK;
+        const bool extra = range >= uint32_t(RBK);  // the round has block 16
 
-        // ---- phase A: scores of blocks wave, wave + 8 (and wave 0: 16) --------------------------
-        // (the query operands are read again in every round: they are not needed between the scores
-        // of one round and the next, and the registers are)
+        half8 q_hi[8], q_lo[8], qz_reg[2];
         {
-            half8 q_reg[8], qz_reg[2];
+            const float qmul = a.scale * 1.4426950408889634f * Q_UP;
 #pragma unroll
-            for (int i = 0; i < 8; i++) q_reg[i] = q_lds[i * 64 + lane];
-            qz_reg[0] = *reinterpret_cast<const half8 *>(qz_lds + lane * 8);
-            qz_reg[1] = *reinterpret_cast<const half8 *>(qz_lds + (64 + lane) * 8);
-            const int parts = (wave == 0 && extra) ? 3 : 2;
+            for (int pass = 0; pass < 2 * PAIRS; pass++) {
+                const int pair = pass >> 1, lo_part = pass & 1;
+                // this thread's item: k-step `wave`, lane `lane`: column n = (row n / 8 of the pair, head n % 8)
+                half8 op;
+                float sum = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    _Float16 h, lw;
+                    split_hi_lo(qv[pair][key_slot_dim<BITS>(e)] * qmul, h, lw);
+                    op[e] = lo_part ? lw : h;
+                    sum += (float)h + (float)lw;
+                }
+                // the place is free when the readers of the pass before (the waves of its pair) have it in registers
+                if (pass > 0) await(W::C_QREAD, WT * pass);
+                q_lds[wave * 64 + lane] = op;
+                if (!lo_part) {
+                    // key bias term: slot `k-step` of this lane in the B operand of one more MFMA, as hi and lo halves
+                    _Float16 h, lw;
+                    split_hi_lo(sum * (1.0f / Q_UP), h, lw);
+                    qz_lds[(0 * 64 + lane) * 8 + wave] = h;
+                    qz_lds[(1 * 64 + lane) * 8 + wave] = lw;
+                }
+                raise(W::C_QUERY);
+                if (pair == at) {
+                    await(W::C_QUERY, W::WAVES * (pass + 1));
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const half8 v = q_lds[i * 64 + lane];
+                        if (lo_part) q_lo[i] = v; else q_hi[i] = v;
+                    }
+                    if (!lo_part) {
+                        qz_reg[0] = *reinterpret_cast<const half8 *>(qz_lds + lane * 8);
+                        qz_reg[1] = *reinterpret_cast<const half8 *>(qz_lds + (64 + lane) * 8);
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    raise(W::C_QREAD);
+                }
+            }
+        }
+
+        // ---- phase A: the scores of this wave's blocks for its pair of rows ----
+        {
+            const int my_row = row_of(at, col_row);
+            const uint32_t my_limit = min<uint32_t>(limit, len_of(my_row));
+            constexpr int A_BLOCKS = (RBK + WT - 1) / WT;
 #pragma unroll 1
-            for (int part = 0; part < parts; part++) {
-                await(W::C_KPART + part, W::K_LOADERS * (round + 1));  // this part of the keys is in LDS (first: and the scales)
-                const int blk = wave + 8 * part;
+            for (int i = 0; i < A_BLOCKS; i++) {
+                const int blk = wt + WT * i;
+                if (blk >= (extra ? RBK : RBK - 1)) break;
+                await(W::C_KPART + (blk >> 3), W::K_LOADERS);  // this part of the keys is in LDS (first: and the scales)
                 const unsigned char *kb = lds_raw + W::K_OFF + blk * W::K_BLOCK_BYTES;
                 KeyRegs<BITS> kreg[4];
 #pragma unroll
                 for (int gg = 0; gg < 4; gg++) {
                     if constexpr (BITS == 8) {
-                        // the group's 64 bytes of token n are piece gg: 16 bytes j of them
                         const u32x4 v = *reinterpret_cast<const u32x4 *>(kb + gg * 1024 + n * 64 + j * 16);
                         kreg[gg].w[0] = v.x, kreg[gg].w[1] = v.y, kreg[gg].w[2] = v.z, kreg[gg].w[3] = v.w;
                     } else {
-                        // the group's 32 bytes of token n are half gg % 2 of piece gg / 2: 8 bytes j of them
                         const u32x2 v = *reinterpret_cast<const u32x2 *>(kb + (gg >> 1) * 1024 + n * 64 + (gg & 1) * 32 + j * 8);
                         kreg[gg].w[0] = v.x, kreg[gg].w[1] = v.y;
                     }
                 }
                 const int tok0 = BLOCK * blk + 4 * j;  // this lane's 4 tokens of the round in C layout
-                const uint32_t *sb_w = sb_lds + BLOCK * blk;  // the block's dwords of groups (0, 1); + RT: groups (2, 3)
-                floatx4 s;
-                {
-                    // bias term: slot e of every lane group belongs to group e / 2 of token n
-                    const u32x2 zr = {sb_w[W::SB_ARRAY / 4 + n], sb_w[W::SB_ARRAY / 4 + RT + n]};
-                    const half8 zop = as_half8(perm(0, zr.x, 0x01000100u), perm(0, zr.x, 0x03020302u), perm(0, zr.y, 0x01000100u),
-                                               perm(0, zr.y, 0x03020302u));
-                    s = floatx4{0, 0, 0, 0};
-                    s = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz_reg[0], s, 0, 0, 0);
-                    s = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz_reg[1], s, 0, 0, 0);
-                }
-                floatx4 r[4];
-#pragma unroll
-                for (int gg = 0; gg < 4; gg++) {
-                    r[gg] = floatx4{0, 0, 0, 0};
-#pragma unroll
-                    for (int ab = 0; ab < 2; ab++) {
-                        r[gg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(key_operand<BITS>(kreg[gg], ab), q_reg[gg * 2 + ab], r[gg], 0, 0, 0);
-                    }
-                }
-                // scales of the lane's tokens 4j .. 4j+3 of the block: groups (0, 1) and groups (2, 3)
+                const uint32_t *sb_w = sb_lds + BLOCK * blk;
+                const u32x2 zr = {sb_w[W::SB_ARRAY / 4 + n], sb_w[W::SB_ARRAY / 4 + RT + n]};
+                const half8 zop = as_half8(perm(0, zr.x, 0x01000100u), perm(0, zr.x, 0x03020302u), perm(0, zr.y, 0x01000100u), perm(0, zr.y, 0x03020302u));
                 const u32x4 s01 = *reinterpret_cast<const u32x4 *>(sb_w + 4 * j);
                 const u32x4 s23 = *reinterpret_cast<const u32x4 *>(sb_w + RT + 4 * j);
                 const uint32_t sw[8] = {s01.x, s23.x, s01.y, s23.y, s01.z, s23.z, s01.w, s23.w};
+                floatx4 s = {0, 0, 0, 0}, rr[4];
+                s = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz_reg[0], s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz_reg[1], s, 0, 0, 0);
+#pragma unroll
+                for (int gg = 0; gg < 4; gg++) {
+                    rr[gg] = floatx4{0, 0, 0, 0};
+#pragma unroll
+                    for (int ab = 0; ab < 2; ab++) {
+                        const half8 kop = key_operand<BITS>(kreg[gg], ab);
+                        rr[gg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop, q_hi[gg * 2 + ab], rr[gg], 0, 0, 0);
+                        rr[gg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop, q_lo[gg * 2 + ab], rr[gg], 0, 0, 0);
+                    }
+                }
                 constexpr float C1 = code_up<BITS>() / Q_UP;
 #pragma unroll
                 for (int tk = 0; tk < 4; tk++) {
                     float d = 0.0f;
 #pragma unroll
-                    for (int gg = 0; gg < 4; gg++) d += half_bits_to_float(sw[2 * tk + (gg >> 1)] >> (16 * (gg & 1))) * r[gg][tk];
-                    float v = s[tk] + d * C1;
-                    v += dpp<0x128>(v);  // row_ror 8: the other part (hi | lo) of the same head
-                    s[tk] = base + tok0 + tk < round_limit ? v : NO_SCORE;  // (also whatever a block past the round left in LDS)
+                    for (int gg = 0; gg < 4; gg++) d += half_bits_to_float(sw[2 * tk + (gg >> 1)] >> (16 * (gg & 1))) * rr[gg][tk];
+                    const float v = s[tk] + d * C1;
+                    s[tk] = base + tok0 + tk < my_limit ? v : NO_SCORE;  // (also whatever a block past the round left in LDS)
                 }
-                // the block's softmax relative to its own maximum, per head
+                // the block's softmax relative to its own maximum, per column
                 float cm = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
                 cm = across_rows<16, 64>(cm, MaxOp());
                 float sum = 0.0f;
@@ -1432,186 +1657,310 @@ __global__ __launch_bounds__((KeysFirst<BITS>::LOADERS + KeysFirst<BITS>::WAVES)
                     sum += s[tk];
                 }
                 sum = across_rows<16, 64>(sum, SumOp());
-                // over the block's own keys (every lane of the wave has its key registers by now)
+                if (j == 0) bmax_lds[my_row * W::BROW + (n & 7) * RBK + blk] = cm, bsum_lds[my_row * W::BROW + (n & 7) * RBK + blk] = sum;
+                // the scores go over the block's own keys: when this wave has them in registers, and with
+                // two pairs the other pair's wave of the same blocks, which takes them in the same order
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                if (n < 8) *reinterpret_cast<floatx4 *>(s_block(blk) + n * BLOCK + 4 * j) = s;
-                if (j == 0 && n < 8) bmax_lds[n * W::BSTRIDE + blk] = cm, bsum_lds[n * W::BSTRIDE + blk] = sum;
+                if constexpr (PAIRS > 1) {
+                    raise(W::C_MERGE + wt);
+                    await(W::C_MERGE + wt, PAIRS * (i + 1));
+                }
+                *reinterpret_cast<floatx4 *>(s_block(blk, my_row) + (n & 7) * BLOCK + 4 * j) = s;
             }
-            if (wave == 0 && !extra && j == 0 && n < 8) bmax_lds[n * W::BSTRIDE + 16] = NO_SCORE, bsum_lds[n * W::BSTRIDE + 16] = 0.0f;
+            if (wt == 0 && !extra && j == 0) bmax_lds[my_row * W::BROW + (n & 7) * RBK + 16] = NO_SCORE, bsum_lds[my_row * W::BROW + (n & 7) * RBK + 16] = 0.0f;
         }
         raise(W::C_SCORES);
-        await(W::C_SCORES, W::WAVES * (round + 1));
+        await(W::C_SCORES, W::WAVES);
 
-        // ---- the round's maximum per head, and what was summed so far brought to it -------------
-        float nm = m_run;
-        {
-            const floatx4 *bmx = reinterpret_cast<const floatx4 *>(bmax_lds + (n & 7) * W::BSTRIDE);
+        // ---- the columns' maxima, the probability operands of this wave's k-steps ----
+        // A operand: lane (n, j) holds tokens 8j .. 8j + 7 of the k-step for column n, as hi and as lo parts.
+        float nm[PAIRS], zacc[PAIRS];
 #pragma unroll
-            for (int i = 0; i < W::BSTRIDE / 4; i++) {
-                const floatx4 w = bmx[i];
-                nm = fmaxf(nm, fmaxf(fmaxf(w[0], w[1]), fmaxf(w[2], w[3])));
+        for (int p = 0; p < PAIRS; p++) nm[p] = round_max(row_of(p, col_row), NO_SCORE), zacc[p] = 0.0f;
+        const bool fifth = extra && b2 == 0;  // k-step 8: block 16 (lane groups 0 and 1; the others repeat them with factor 0)
+        half8 p_hi[PAIRS][W::SLOTS], p_lo[PAIRS][W::SLOTS];
+#pragma unroll
+        for (int sl = 0; sl < W::SLOTS; sl++) {
+            if (sl == 4 && !fifth) {
+#pragma unroll
+                for (int p = 0; p < PAIRS; p++) p_hi[p][sl] = p_lo[p][sl] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+                continue;
+            }
+            const int ks = 2 * sl + b2;  // tokens 32 ks ..: blocks 2 ks and 2 ks + 1
+            const int jj = sl == 4 ? (j & 1) : j;
+            const int blk = 2 * ks + (jj >> 1);
+            const int sh = 16 * (g & 1);
+            // value scales and biases of group g: half g % 2 of the tokens' dwords of groups (g, g ^ 1).
+            // (Tokens past the share have probability 0 and the scales of the share's last token:
+            // every load is clamped to it, so nothing but cache rows in use is ever read.)
+            const uint32_t *vsp = sb_lds + 2 * (W::SB_ARRAY / 4) + (g >> 1) * RT + 32 * ks + 8 * jj;
+            const u32x4 sv0 = *reinterpret_cast<const u32x4 *>(vsp), sv1 = *reinterpret_cast<const u32x4 *>(vsp + 4);
+            const u32x4 zv0 = *reinterpret_cast<const u32x4 *>(vsp + W::SB_ARRAY / 4), zv1 = *reinterpret_cast<const u32x4 *>(vsp + W::SB_ARRAY / 4 + 4);
+            const uint32_t sw[8] = {sv0.x, sv0.y, sv0.z, sv0.w, sv1.x, sv1.y, sv1.z, sv1.w};
+            const uint32_t zw[8] = {zv0.x, zv0.y, zv0.z, zv0.w, zv1.x, zv1.y, zv1.z, zv1.w};
+            float vscale[8], vbias[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) vscale[e] = half_bits_to_float(sw[e] >> sh), vbias[e] = half_bits_to_float(zw[e] >> sh);
+            const int fb = 2 * ks + (j >> 1);  // block 17 does not exist: factor 0
+#pragma unroll
+            for (int p = 0; p < PAIRS; p++) {
+                const int r = row_of(p, col_row);
+                const float *sp = s_block(blk, r) + (n & 7) * BLOCK + 8 * (jj & 1);
+                const floatx4 pt0 = *reinterpret_cast<const floatx4 *>(sp), pt1 = *reinterpret_cast<const floatx4 *>(sp + 4);
+                const float pt[8] = {pt0[0], pt0[1], pt0[2], pt0[3], pt1[0], pt1[1], pt1[2], pt1[3]};
+                // 2^(block maximum - round maximum) * P_UP (2^8, so that the lo part stays a normal f16)
+                const float f = fb < RBK ? __builtin_amdgcn_exp2f(bmax_lds[r * W::BROW + (n & 7) * RBK + (fb < RBK ? fb : 0)] - nm[p] + 8.0f) : 0.0f;
+                float x[8], lo[8], zb = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    zb += pt[e] * vbias[e];
+                    x[e] = pt[e] * f * vscale[e];
+                    lo[e] = x[e] - __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x[e]) & 0xffffe000u);
+                }
+                zacc[p] += zb * f;
+                uint32_t o[8];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    // round toward zero: exact truncation to the hi part
+                    o[e] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x[2 * e], x[2 * e + 1]));
+                    o[4 + e] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo[2 * e], lo[2 * e + 1]));
+                }
+                // (pinned: left alone, the compiler moves an operand's arithmetic down to its use, behind the wait for the values)
+                asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]), "+v"(o[4]), "+v"(o[5]), "+v"(o[6]), "+v"(o[7]));
+                p_hi[p][sl] = as_half8(o[0], o[1], o[2], o[3]);
+                p_lo[p][sl] = as_half8(o[4], o[5], o[6], o[7]);
             }
         }
-        const float al = __builtin_amdgcn_exp2f(m_run - nm);  // (first round: 2^(-1e30 - nm) = 0, and nothing to scale)
-        if (round > 0) {
-            zacc *= al;
-            // accumulator rows 4j + i are heads (4j + i) & 7: lane h (j = 0, n = h) holds head h's factor
-            floatx4 al4;
+        raise(W::C_BUILT);  // this wave is through with the scores
+
+        // ---- phase C: O += P V, one k-step per value slot as the slots land ----
+        floatx4 acc[PAIRS][4];  // [pair][tile of 16 dims 4n' + e]: rows 4j .. 4j+3 (columns of the pair), column n'
+#pragma unroll
+        for (int p = 0; p < PAIRS; p++) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[p][e] = floatx4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int sl = 0; sl < W::SLOTS; sl++) {
+            if (sl == 4 && !fifth) continue;
+            await(W::C_SLOT + sl, W::V_LOADERS);  // value slot sl is in LDS
+            ValRegs<BITS> vreg;
+            read_values(sl == 4 ? 8 : 2 * sl + b2, g, vreg);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const half8 vop = val_operand<BITS>(vreg, e, n);
+#pragma unroll
+                for (int p = 0; p < PAIRS; p++) {
+                    acc[p][e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p_hi[p][sl], vop, acc[p][e], 0, 0, 0);
+                    acc[p][e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p_lo[p][sl], vop, acc[p][e], 0, 0, 0);
+                }
+            }
+        }
+
+        // ---- epilogue: the two waves of a group add up, wave 2g writes the partials ----
+#pragma unroll
+        for (int p = 0; p < PAIRS; p++) {
+            // a column's bias sum: over the four lane groups
+            const float z = across_rows<16, 64>(zacc[p], SumOp());
+            if (j == 0) zs_lds[(wave * PAIRS + p) * 16 + n] = z;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        floatx4 mine[PAIRS][4];  // column 4j + i of the pair, dims 64 g + 4n .. + 3
+#pragma unroll
+        for (int p = 0; p < PAIRS; p++) {
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                al4[i] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(4 * ((4 * j + i) & 7), __builtin_bit_cast(int, al)));
-            }
+                const float zb = zs_lds[(wave * PAIRS + p) * 16 + 4 * j + i] * (1.0f / P_UP);
 #pragma unroll
-            for (int e = 0; e < 4; e++) acc[e] *= al4;
+                for (int e = 0; e < 4; e++) mine[p][i][e] = acc[p][e][i] * unscale + zb;
+            }
         }
-        m_run = nm;
+        // (the merge lies over the keys, which hold the scores until every wave has built its operands)
+        floatx4 *x_o = reinterpret_cast<floatx4 *>(lds_raw + W::K_OFF);  // [pair][group][lane][4 columns]
+        await(W::C_BUILT, W::WAVES);
+        if (b2 == 1) {
+#pragma unroll
+            for (int p = 0; p < PAIRS; p++) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) x_o[((p * 4 + g) * 64 + lane) * 4 + i] = mine[p][i];
+            }
+            raise(W::C_MERGE + 4 + g);
+            return;
+        }
         if (wave == 0) {
-            // the round's sum of P of head n & 7: lane group j adds blocks 5j .. 5j + 4
-            float sum = 0.0f;
 #pragma unroll
-            for (int i = 0; i < W::BSTRIDE / 4; i++) {
-                const int b = (W::BSTRIDE / 4) * j + i;
-                sum += bsum_lds[(n & 7) * W::BSTRIDE + b] * __builtin_amdgcn_exp2f(bmax_lds[(n & 7) * W::BSTRIDE + b] - nm);  // (a block that is not there: sum 0)
+            for (int p = 0; p < PAIRS; p++) {
+                const int r = 2 * p + col_row;
+                const float l = round_sum(row_of(p, col_row), nm[p]);
+                if (j == 0 && r < M) {
+                    const size_t slot = (size_t(r) * a.nsplits + split) * a.heads + kv * 8 + (n & 7);
+                    *reinterpret_cast<floatx2 *>(a.part_ml + 2 * slot) = floatx2{nm[p], l};
+                }
             }
-            l_run = l_run * al + across_rows<16, 64>(sum, SumOp());
         }
+        await(W::C_MERGE + 4 + g, 1);
+#pragma unroll
+        for (int p = 0; p < PAIRS; p++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int c = 4 * j + i, r = 2 * p + (c >> 3);
+                if (r < M) {
+                    const size_t slot = (size_t(r) * a.nsplits + split) * a.heads + kv * 8 + (c & 7);
+                    // (nobody on this CU reads the partials again: past the caches)
+                    __builtin_nontemporal_store(mine[p][i] + x_o[((p * 4 + g) * 64 + lane) * 4 + i], reinterpret_cast<floatx4 *>(a.part_o + slot * DIM + 64 * g + 4 * n));
+                }
+            }
+        }
+    } else {
+        // ---- one row -----------------------------------------------------------------------------
+        // Scores: wave w takes the blocks w and w + 8 (wave 0 also 16).  O += P V: waves 2g and 2g + 1 share
+        // group g and take alternate k-steps, so that each value slot gives every wave one k-step.
+        stage_query(qv[0]);
+        raise(W::C_QUERY);
+        float m_run = NO_SCORE;
+        float l_run = 0.0f;  // sum of P of head n & 7 (wave 0 keeps it)
+        float zacc[1] = {0.0f};  // sum of P * P_UP * value bias of group g over this lane's tokens
+        floatx4 acc[4];      // [tile of 16 dims 4n' + e]: rows 4j .. 4j+3 (operand rows), column n'
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[e] = floatx4{0, 0, 0, 0};
+        await(W::C_QUERY, W::WAVES);
+        const int row0[1] = {0};
 
-        // ---- probability operands of this wave's k-steps: P * value scale of group g, hi part in
-        // operand rows 0-7 and lo part in rows 8-15.  The two lanes of a head (n and n + 8) make four of
-        // the lane group's eight tokens each, both parts, and exchange what the other one feeds. ----
-        half8 p_op[W::SLOTS];
-        {
-            const int hh = n >> 3;  // this lane makes tokens 8j + 4 hh .. + 3 of a k-step
-            const int sh = 16 * (g & 1);
-            const bool fifth = extra && b2 == 0;  // k-step 8: block 16 (lane groups 0 and 1; the others repeat them with factor 0)
+        for (uint32_t round = 0; round < n_rounds; round++) {
+            const uint32_t base = (blk_begin + round * per_round) * BLOCK, nb = blocks_of(round);
+            const bool more = round + 1 < n_rounds;
+            const bool extra = nb == uint32_t(RBK);  // the round has block 16
+            const uint32_t round_limit[1] = {min(limit, base + nb * BLOCK)};  // tokens of this round end here
+
+            // ---- phase A: scores of blocks wave, wave + 8 (and wave 0: 16) --------------------------
+            // (the query operands are read again in every round: they are not needed between the scores
+            // of one round and the next, and the registers are)
+            {
+                half8 q_reg[1][8], qz_reg[1][2];
+#pragma unroll
+                for (int i = 0; i < 8; i++) q_reg[0][i] = q_lds[i * 64 + lane];
+                qz_reg[0][0] = *reinterpret_cast<const half8 *>(qz_lds + lane * 8);
+                qz_reg[0][1] = *reinterpret_cast<const half8 *>(qz_lds + (64 + lane) * 8);
+                const int parts = (wave == 0 && extra) ? 3 : 2;
+#pragma unroll 1
+                for (int part = 0; part < parts; part++) {
+                    await(W::C_KPART + part, W::K_LOADERS * (round + 1));  // this part of the keys is in LDS (first: and the scales)
+                    const int blk = wave + 8 * part;
+                    floatx4 s[1];
+                    block_scores(std::integral_constant<int, 1>(), blk, base, q_reg, qz_reg, row0, round_limit, 1, s);
+                    // over the block's own keys (every lane of the wave has its key registers by now)
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    if (n < 8) *reinterpret_cast<floatx4 *>(s_block(blk, 0) + n * BLOCK + 4 * j) = s[0];
+                }
+                if (wave == 0 && !extra && j == 0 && n < 8) bmax_lds[n * RBK + 16] = NO_SCORE, bsum_lds[n * RBK + 16] = 0.0f;
+            }
+            raise(W::C_SCORES);
+            await(W::C_SCORES, W::WAVES * (round + 1));
+
+            // ---- the round's maximum per head, and what was summed so far brought to it -------------
+            const float nm[1] = {round_max(0, m_run)};
+            const float al = __builtin_amdgcn_exp2f(m_run - nm[0]);  // (first round: 2^(-1e30 - nm) = 0, and nothing to scale)
+            if (round > 0) {
+                zacc[0] *= al;
+                // accumulator rows 4j + i are heads (4j + i) & 7: lane h (j = 0, n = h) holds head h's factor
+                floatx4 al4;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    al4[i] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(4 * ((4 * j + i) & 7), __builtin_bit_cast(int, al)));
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[e] *= al4;
+            }
+            m_run = nm[0];
+            if (wave == 0) l_run = l_run * al + round_sum(0, nm[0]);
+
+            // ---- probability operands of this wave's k-steps ----
+            const bool fifth = extra && b2 == 0;  // k-step 8: block 16
+            half8 p_op[W::SLOTS];
 #pragma unroll
             for (int sl = 0; sl < W::SLOTS; sl++) {
                 if (sl == 4 && !fifth) {
                     p_op[sl] = half8{0, 0, 0, 0, 0, 0, 0, 0};
                     continue;
                 }
-                const int ks = 2 * sl + b2;  // tokens 32 ks ..: blocks 2 ks and 2 ks + 1
-                const int jj = sl == 4 ? (j & 1) : j;
-                const int blk = 2 * ks + (jj >> 1);
-                const floatx4 pt = *reinterpret_cast<const floatx4 *>(s_block(blk) + (n & 7) * BLOCK + 8 * (jj & 1) + 4 * hh);
-                // value scales and biases of group g: half g % 2 of the tokens' dwords of groups (g, g ^ 1).
-                // (Tokens past the share have probability 0 and the scales of the share's last token:
-                // every load is clamped to it, so nothing but cache rows in use is ever read.)
-                const uint32_t *vsp = sb_lds + 2 * (W::SB_ARRAY / 4) + (g >> 1) * RT + 32 * ks + 8 * jj + 4 * hh;
-                const u32x4 sv = *reinterpret_cast<const u32x4 *>(vsp);
-                const u32x4 zv = *reinterpret_cast<const u32x4 *>(vsp + W::SB_ARRAY / 4);
-                // 2^(block maximum - round maximum) * P_UP (2^8, so that the lo part stays a normal f16)
-                const float f = __builtin_amdgcn_exp2f(bmax_lds[(n & 7) * W::BSTRIDE + 2 * ks + (j >> 1)] - nm + 8.0f);
-                const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w}, zw[4] = {zv.x, zv.y, zv.z, zv.w};
-                float x[4], lo[4];
+                build_operands(std::integral_constant<int, 1>(), 2 * sl + b2, g, row0, nm, 1, zacc, &p_op[sl]);
+            }
+            if (more) raise(W::C_BUILT);  // this wave is through with the round's scores, scales and biases
+
+            // ---- phase C: O += P V, one k-step per value slot as the slots land ---------------------
+            auto add_values = [&](int sl, const ValRegs<BITS> &vreg) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const float p = pt[e] * f;
-                    zacc += p * half_bits_to_float(zw[e] >> sh);
-                    x[e] = p * half_bits_to_float(sw[e] >> sh);
-                    lo[e] = x[e] - __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x[e]) & 0xffffe000u);
+                    acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p_op[sl], val_operand<BITS>(vreg, e, n), acc[e], 0, 0, 0);
                 }
-                // round toward zero: exact truncation to the hi part
-                const uint32_t hi0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x[0], x[1]));
-                const uint32_t hi1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x[2], x[3]));
-                const uint32_t lo0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo[0], lo[1]));
-                const uint32_t lo1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo[2], lo[3]));
-                // the hi lane (n < 8) feeds hi parts and wants the other lane's hi parts of tokens 4-7; the lo
-                // lane feeds lo parts and wants the other lane's lo parts of tokens 0-3
-                const uint32_t send0 = hh ? hi0 : lo0, send1 = hh ? hi1 : lo1;
-                const uint32_t recv0 = uint32_t(__builtin_amdgcn_update_dpp(0, int(send0), 0x128, 0xf, 0xf, false));  // row_ror 8
-                const uint32_t recv1 = uint32_t(__builtin_amdgcn_update_dpp(0, int(send1), 0x128, 0xf, 0xf, false));
-                uint32_t o[4] = {hh ? recv0 : hi0, hh ? recv1 : hi1, hh ? lo0 : recv0, hh ? lo1 : recv1};
-                // (pinned: left alone, the compiler moves an operand's arithmetic down to its use, behind the wait for the values)
-                asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]));
-                p_op[sl] = as_half8(o[0], o[1], o[2], o[3]);
+            };
+            if (peek(W::C_SLOT + 3) >= W::V_LOADERS * (round + 1)) {
+                // slots 0-3 are there already (the slots land in order): every read at once
+                ValRegs<BITS> vreg[4];
+#pragma unroll
+                for (int sl = 0; sl < 4; sl++) read_values(2 * sl + b2, g, vreg[sl]);
+#pragma unroll
+                for (int sl = 0; sl < 4; sl++) add_values(sl, vreg[sl]);
+            } else {
+#pragma unroll
+                for (int sl = 0; sl < 4; sl++) {
+                    await(W::C_SLOT + sl, W::V_LOADERS * (round + 1));  // value slot sl is in LDS
+                    ValRegs<BITS> vreg;
+                    read_values(2 * sl + b2, g, vreg);
+                    add_values(sl, vreg);
+                }
             }
-        }
-        if (more) raise(W::C_BUILT);  // this wave is through with the round's scores, scales and biases
-
-        // ---- phase C: O += P V, one k-step per value slot as the slots land ---------------------
-        const unsigned char *vb = lds_raw + W::V_OFF + val_lane_offset<BITS>(g, n);
-        auto read_values = [&](int sl, ValRegs<BITS> &vreg) {
-            const int jj = sl == 4 ? (j & 1) : j;
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const int tk = 32 * (2 * sl + b2) + 8 * jj + e;
-                vreg.w[e] = *reinterpret_cast<const uint32_t *>(vb + (tk / W::V_GROUP_TOKENS) * W::V_GROUP_BYTES + (tk % W::V_GROUP_TOKENS) * RB);
-            }
-        };
-        auto add_values = [&](int sl, const ValRegs<BITS> &vreg) {
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p_op[sl], val_operand<BITS>(vreg, e, n), acc[e], 0, 0, 0);
-            }
-        };
-        const bool fifth = extra && b2 == 0;
-        if (peek(W::C_SLOT + 3) >= W::V_LOADERS * (round + 1)) {
-            // slots 0-3 are there already (the slots land in order): every read at once
-            ValRegs<BITS> vreg[4];
-#pragma unroll
-            for (int sl = 0; sl < 4; sl++) read_values(sl, vreg[sl]);
-#pragma unroll
-            for (int sl = 0; sl < 4; sl++) add_values(sl, vreg[sl]);
-        } else {
-#pragma unroll
-            for (int sl = 0; sl < 4; sl++) {
-                await(W::C_SLOT + sl, W::V_LOADERS * (round + 1));  // value slot sl is in LDS
+            if (fifth) {
+                await(W::C_SLOT + 4, W::V_LOADERS * (round + 1));
                 ValRegs<BITS> vreg;
-                read_values(sl, vreg);
-                add_values(sl, vreg);
+                read_values(8, g, vreg);
+                add_values(4, vreg);
+            }
+            if (more) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the value codes are in registers
+                raise(W::C_DONE);
             }
         }
-        if (fifth) {
-            await(W::C_SLOT + 4, W::V_LOADERS * (round + 1));
-            ValRegs<BITS> vreg;
-            read_values(4, vreg);
-            add_values(4, vreg);
-        }
-        if (more) {
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the value codes are in registers
-            raise(W::C_DONE);
-        }
-    }
 
-    // ---- epilogue: the two waves of a group add up, wave 2g writes the partial ---------------------
-    {
-        // the head's bias sum: over the four lane groups and the two lanes of the head
-        float z = across_rows<16, 64>(zacc, SumOp());
-        z += dpp<0x128>(z);
-        if (j == 0 && n < 8) zs_lds[wave * 8 + n] = z;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-    }
-    constexpr float unscale = code_up<BITS>() / P_UP;
-    floatx4 mine[4];  // head 4j + i (j < 2), dims 64 g + 4n .. + 3
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const float zb = zs_lds[wave * 8 + ((4 * j + i) & 7)] * (1.0f / P_UP);
-#pragma unroll
-        for (int e = 0; e < 4; e++) mine[i][e] = across_rows<32, 64>(acc[e][i], SumOp()) * unscale + zb;
-    }
-    // (the key area is free: the key loaders request nothing after the last round, and every wave is
-    // past the last round's scores, having built its operands from them)
-    floatx4 *x_o = reinterpret_cast<floatx4 *>(lds_raw + W::X_OFF);  // [group][lane < 32][4 rows]
-    if (b2 == 1) {
-        if (j < 2) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) x_o[(g * 32 + lane) * 4 + i] = mine[i];
+        // ---- epilogue: the two waves of a group add up, wave 2g writes the partial ---------------------
+        {
+            // the head's bias sum: over the four lane groups and the two lanes of the head
+            float z = across_rows<16, 64>(zacc[0], SumOp());
+            z += dpp<0x128>(z);
+            if (j == 0 && n < 8) zs_lds[wave * 8 + n] = z;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
         }
-        raise(W::C_MERGE + g);
-        return;
-    }
-    await(W::C_MERGE + g, 1);
-    if (wave == 0 && j == 0 && n < 8) {
-        const size_t slot = size_t(split) * a.heads + kv * 8 + n;
-        *reinterpret_cast<floatx2 *>(a.part_ml + 2 * slot) = floatx2{m_run, l_run};
-    }
-    if (j < 2) {
+        floatx4 mine[4];  // head 4j + i (j < 2), dims 64 g + 4n .. + 3
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const size_t slot = size_t(split) * a.heads + kv * 8 + 4 * j + i;
-            *reinterpret_cast<floatx4 *>(a.part_o + slot * DIM + 64 * g + 4 * n) = mine[i] + x_o[(g * 32 + lane) * 4 + i];
+            const float zb = zs_lds[wave * 8 + ((4 * j + i) & 7)] * (1.0f / P_UP);
+#pragma unroll
+            for (int e = 0; e < 4; e++) mine[i][e] = across_rows<32, 64>(acc[e][i], SumOp()) * unscale + zb;
+        }
+        // (the merge lies over the query operands, which nobody reads after the last round's scores)
+        floatx4 *x_o = reinterpret_cast<floatx4 *>(lds_raw + W::X_OFF);  // [group][lane < 32][4 rows]
+        if (b2 == 1) {
+            if (j < 2) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) x_o[(g * 32 + lane) * 4 + i] = mine[i];
+            }
+            raise(W::C_MERGE + g);
+            return;
+        }
+        await(W::C_MERGE + g, 1);
+        if (wave == 0 && j == 0 && n < 8) {
+            const size_t slot = size_t(split) * a.heads + kv * 8 + n;
+            *reinterpret_cast<floatx2 *>(a.part_ml + 2 * slot) = floatx2{m_run, l_run};
+        }
+        if (j < 2) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const size_t slot = size_t(split) * a.heads + kv * 8 + 4 * j + i;
+                // (nobody on this CU reads the partials again: past the caches)
+                __builtin_nontemporal_store(mine[i] + x_o[(g * 32 + lane) * 4 + i], reinterpret_cast<floatx4 *>(a.part_o + slot * DIM + 64 * g + 4 * n));
+            }
         }
     }
 }
@@ -1743,12 +2092,21 @@ template <int BITS, int TILES, bool PACKED>
 void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu, bool loaders, bool keys_first) {
     void (*kernel)(PartialArgs);
     int lds_bytes;
-    if constexpr (TILES == 1 && BITS != 16 && PACKED) {
-        if (loaders && keys_first) {
-            using W = KeysFirst<BITS>;
-            attention_partial_kernel_s<BITS><<<dim3(a.nsplits, a.kv_heads), (W::LOADERS + W::WAVES) * 64, W::LDS_BYTES, stream>>>(a);
+    if constexpr (BITS != 16) {
+        if (keys_first) {
+            auto launch = [&](auto rows_c) {
+                constexpr int MR = decltype(rows_c)::value;
+                using W = KeysFirst<BITS, MR>;
+                attention_partial_kernel_s<BITS, MR><<<dim3(a.nsplits, a.kv_heads), (W::LOADERS + W::WAVES) * 64, W::LDS_BYTES, stream>>>(a);
+            };
+            if (a.rows == 1) launch(std::integral_constant<int, 1>());
+            else if (a.rows == 2) launch(std::integral_constant<int, 2>());
+            else if (a.rows == 3) launch(std::integral_constant<int, 3>());
+            else launch(std::integral_constant<int, 4>());
             return;
         }
+    }
+    if constexpr (TILES == 1 && BITS != 16 && PACKED) {
         if (loaders) {
             attention_partial_kernel_d<BITS><<<dim3(a.nsplits, a.kv_heads), (TEAMS_DMA + 1) * THREADS,
                                                Shape<BITS, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA), stream>>>(a);
@@ -1829,8 +2187,14 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
     // 10.2 against 11.7, 4-bit) and again from about four rounds on (17.1 against 18.6 us at 64k, 29.7
     // against 31.1 at 131k, 8-bit); with two or three short rounds the ring of slots is ahead (14.1
     // against 15.6 us at 40k), and so it is for 4-bit codes above 100k tokens (28.0 against 29.3 at 131k).
-    const bool keys_first = loaders && (capacity <= KEYS_FIRST_ONE_ROUND || (capacity >= KEYS_FIRST_AGAIN_FROM &&
-                                                                               (bits == 8 || capacity <= KEYS_FIRST_4BIT_UP_TO)));
+    // Two to four rows over codes (a verify step) run the same kernel, the codes in LDS serving every
+    // row, where no share can be longer than the one round that kernel takes with several rows.
+    const uint32_t splits_one_per_cu = nsplits > MAX_SPLITS / 2 ? MAX_SPLITS / 2 : nsplits;
+    const uint32_t longest_share = (capacity / BLOCK + splits_one_per_cu - 1) / splits_one_per_cu;  // in blocks
+    const bool rows_keys_first = rows >= 2 && rows <= 4 && bits != 16 && capacity >= LOADERS_FROM && longest_share <= 17 &&
+                                 !(stages & SAETTA_STAGE_NO_LOADERS);
+    const bool keys_first = rows_keys_first || (loaders && (capacity <= KEYS_FIRST_ONE_ROUND || (capacity >= KEYS_FIRST_AGAIN_FROM &&
+                                                                               (bits == 8 || capacity <= KEYS_FIRST_4BIT_UP_TO))));
     if (one_per_cu && nsplits > MAX_SPLITS / 2) nsplits = MAX_SPLITS / 2;
     if (stages & SAETTA_STAGE_PARTIAL) {
         PartialArgs a{q,     kdata,    vdata,    ks,    kz,   vs,      vz,   part_o, part_ml,
@@ -1859,6 +2223,11 @@ int raise_lds(void (*kernel)(PartialArgs)) {
     if (Shape<BITS, TILES, PACKED, ITB>::LDS_BYTES <= 48 * 1024) return 0;
     return int(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    Shape<BITS, TILES, PACKED, ITB>::LDS_BYTES));
+}
+template <int BITS, int M>
+int raise_lds_keys_first() {
+    return int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_partial_kernel_s<BITS, M>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, KeysFirst<BITS, M>::LDS_BYTES));
 }
 template <int BITS>
 int raise_lds_of_bits() {
@@ -1891,14 +2260,14 @@ int setup_decode() {
                                          Shape<4, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA)))) {
         return rc;
     }
-    if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_partial_kernel_s<8>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, KeysFirst<8>::LDS_BYTES))) {
-        return rc;
-    }
-    if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_partial_kernel_s<4>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, KeysFirst<4>::LDS_BYTES))) {
-        return rc;
-    }
+    if (int rc = raise_lds_keys_first<8, 1>()) return rc;
+    if (int rc = raise_lds_keys_first<8, 2>()) return rc;
+    if (int rc = raise_lds_keys_first<8, 3>()) return rc;
+    if (int rc = raise_lds_keys_first<8, 4>()) return rc;
+    if (int rc = raise_lds_keys_first<4, 1>()) return rc;
+    if (int rc = raise_lds_keys_first<4, 2>()) return rc;
+    if (int rc = raise_lds_keys_first<4, 3>()) return rc;
+    if (int rc = raise_lds_keys_first<4, 4>()) return rc;
     if (int rc = raise_lds_of_bits<8>()) return rc;
     if (int rc = raise_lds_of_bits<4>()) return rc;
     if (int rc = raise_lds_of_bits<16>()) return rc;
