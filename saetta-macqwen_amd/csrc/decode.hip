@@ -1958,8 +1958,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const size_t slot = size_t(split) * a.heads + kv * 8 + 4 * j + i;
-                // (nobody on this CU reads the partials again: past the caches)
-                __builtin_nontemporal_store(mine[i] + x_o[(g * 32 + lane) * 4 + i], reinterpret_cast<floatx4 *>(a.part_o + slot * DIM + 64 * g + 4 * n));
+                *reinterpret_cast<floatx4 *>(a.part_o + slot * DIM + 64 * g + 4 * n) = mine[i] + x_o[(g * 32 + lane) * 4 + i];
             }
         }
     }

@@ -256,6 +256,41 @@ def test_capacity_must_be_whole_blocks():
         plan.build().run()
 
 
+@pytest.mark.parametrize("m", [2, 3, 4])
+@pytest.mark.parametrize("kind", [saetta.KvBits.Eight, saetta.KvBits.Four])
+def test_large_cache_of_codes_several_rows(kind, m):
+    # Two to four rows over codes in a cache of 24k tokens and more whose longest share is one round of
+    # 17 blocks (capacities up to 34816) run the keys-first kernel with two rows to a tile; three
+    # rows: the second tile's upper half repeats row 2.  Capacity 35072: a share can be 18 blocks, and
+    # the register kernels take over.  Positions: the first tokens of a cache (row r sees r + 1
+    # tokens: whole shares are empty for the earlier rows); one block per share; shares of a few
+    # blocks; shares of 16 and of 17 blocks side by side; the whole capacity.  The rows past the last
+    # token are poisoned.
+    rng = np.random.default_rng(770 + m)
+    q = rng.standard_normal((m, H, D)).astype(np.float32)
+    qg = rng.standard_normal((m, H, 2 * D)).astype(np.float32)
+    for capacity in (34816, 24576, 35072):
+        k = (rng.standard_normal((capacity, VALUES)) * 2.0).astype(np.float32)
+        v = rng.standard_normal((capacity, VALUES)).astype(np.float32)
+        rows = saetta.AttentionRows(H, KV, capacity, m)
+        for tokens in [m, 2049, 16400, 33000, capacity]:
+            if tokens > capacity:
+                continue
+            pos = tokens - m
+            kc, vc, kf, vf = cache_pair(k[:tokens], v[:tokens], kind, capacity, poison=True)
+            out = torch.full((m, H, D), float("nan"), device="cuda")
+            params = [saetta.TokenParams(0, pos + r).as_tensor("cuda") for r in range(m)]
+            plan = saetta.Plan()
+            rows.record_quant(plan, m, dev(q), kc, vc, dev(qg), out, params)
+            plan.build().run()
+            got = host(out)
+            assert np.isfinite(got).all(), (capacity, tokens)
+            want64 = oracle.rows(q, kf, vf, pos, m, q_and_gate=qg, threads=8, f64=True)
+            worst = np.abs(got - want64).max()
+            assert worst < MAX_ABS_F64, (capacity, tokens, worst)
+            del kc, vc
+
+
 @pytest.mark.parametrize("capacity", [81920, 49152, 34816])
 @pytest.mark.parametrize("kind", [saetta.KvBits.Eight, saetta.KvBits.Four])
 def test_large_cache_of_codes_one_row(kind, capacity):
