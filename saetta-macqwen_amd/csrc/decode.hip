@@ -1079,7 +1079,10 @@ struct KeysFirst {
     // scales and biases: per array two planes of one dword per token, the f16 of groups (0, 1) and of (2, 3)
     static constexpr int SB_OFF = QZ_OFF + 2 * 64 * 16;            // [ks | kz | vs | vz][plane][token] u32
     static constexpr int SB_ARRAY = 2 * ROUND_TOKENS * 4;
-    static constexpr int BROW = 8 * ROUND_BLOCKS;                  // floats of a row's [head][block]
+    // the blocks' maxima and sums, [row][head][block]: one row has room for a stride of 20 (16-byte reads; blocks 17-19
+    // never exist: maximum "none", sum 0), several rows have not
+    static constexpr int BSTRIDE = M == 1 ? 20 : ROUND_BLOCKS;
+    static constexpr int BROW = 8 * BSTRIDE;                       // floats of a row's table
     static constexpr int BMAX_OFF = SB_OFF + 4 * SB_ARRAY;         // [row][head][block] f32: the block's maximum score
     static constexpr int BSUM_OFF = BMAX_OFF + M * BROW * 4;       // [row][head][block] f32: sum of 2^(score - maximum)
     static constexpr int ZS_OFF = BSUM_OFF + M * BROW * 4;         // [wave][pair][column] f32 (one row: [wave][head])
@@ -1099,8 +1102,7 @@ struct KeysFirst {
     static constexpr int C_SCORES = 2;  // ... written their scores (8 per round)
     static constexpr int C_BUILT = 3;   // ... built their probability operands (8 per round)
     static constexpr int C_DONE = 4;    // ... are through with the round's values (8 per round)
-    static constexpr int C_LENGTH = 5;  // (not a counter: the context length, for every wave)
-    static constexpr int C_POSITION = 6;  // (not a counter: the position)
+    static constexpr int C_LENGTH = 5;  // (not a counter: the context length or the position, for every wave)
     static constexpr int C_QREAD = 7;   // computing waves that have a row's query operands in registers (several rows)
     static constexpr int C_KPART = 8;   // [3]: key loaders whose blocks 0-7 and scales | blocks 8-15 | block 16 have landed (2 per round)
     static constexpr int C_SLOT = 12;   // [5]: value loaders whose values of slot s have landed (2 per round)
@@ -1144,14 +1146,13 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
     // One wave of the workgroup reads the token's parameters and hands them on through LDS.  The
     // counters start at zero behind the same barrier, the only s_barrier of the kernel, before
     // anybody requests anything of the cache.
-    if (threadIdx.x < 32) {
-        sync_lds[threadIdx.x] = threadIdx.x == W::C_LENGTH ? a.tp->kv_len : threadIdx.x == W::C_POSITION ? a.tp->position : 0u;
-    }
+    // (the context length of a decode step | the position of the first of a verify step's rows: one scalar load)
+    static_assert(offsetof(saetta_token_params, position) == 4 && offsetof(saetta_token_params, kv_len) == 8, "dwords 1 and 2");
+    if (threadIdx.x < 32) sync_lds[threadIdx.x] = threadIdx.x == W::C_LENGTH ? reinterpret_cast<const uint32_t *>(a.tp)[a.decode_len ? 2 : 1] : 0u;
     __syncthreads();
-    const uint32_t kv_len = __builtin_amdgcn_readfirstlane(sync_lds[W::C_LENGTH]);
-    const uint32_t position = __builtin_amdgcn_readfirstlane(sync_lds[W::C_POSITION]);
+    const uint32_t tp_first = __builtin_amdgcn_readfirstlane(sync_lds[W::C_LENGTH]);
     // tokens row r sees; the last row's are the launch's
-    auto len_of = [&](int r) -> uint32_t { return min<uint32_t>(a.decode_len ? kv_len : position + uint32_t(r) + 1, a.capacity); };
+    auto len_of = [&](int r) -> uint32_t { return min<uint32_t>(a.decode_len ? tp_first : tp_first + uint32_t(r) + 1, a.capacity); };
     const uint32_t max_len = len_of(M - 1);
     const uint32_t nblocks = (max_len + BLOCK - 1) / BLOCK;
     uint32_t blk_begin, blk_end;
@@ -1346,192 +1347,51 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
     // the scores of block b, row r: [head][token] f32 over the block's keys
     auto s_block = [&](int b, int r) { return reinterpret_cast<float *>(lds_raw + W::K_OFF + b * W::K_BLOCK_BYTES + r * 512); };
 
-    // A row's query operands to LDS: f16 hi/lo parts (operand row n: head n & 7, hi part in rows 0-7 and
-    // lo part in rows 8-15 of the row's tile); this thread's item is k-step `wave`, lane `lane`.
-    auto stage_query = [&](const float (&v)[8]) {
-        const float qmul = a.scale * 1.4426950408889634f * Q_UP;
-        half8 op;
-        float sum = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            _Float16 h, lw;
-            split_hi_lo(v[key_slot_dim<BITS>(e)] * qmul, h, lw);
-            const _Float16 x = n < 8 ? h : lw;
-            op[e] = x;
-            sum += (float)x;
-        }
-        q_lds[wave * 64 + lane] = op;
-        // key bias term: slot `k-step` of this lane in the B operand of one more MFMA, as hi and lo halves
-        _Float16 h, lw;
-        split_hi_lo(sum * (1.0f / Q_UP), h, lw);
-        qz_lds[(0 * 64 + lane) * 8 + wave] = h;
-        qz_lds[(1 * 64 + lane) * 8 + wave] = lw;
-    };
-    // The scores of one block of 16 tokens for R query rows whose operands are in registers: the key
-    // operands are made once and serve every row.  Returns in s[ri] the lane's probabilities relative to
-    // the block's maximum (tokens 4j .. 4j + 3 of the block, head n & 7) and stores the block's maximum and sum.
-    auto block_scores = [&](auto rows_c, int blk, uint32_t base, const half8 (*q_reg)[8], const half8 (*qz_reg)[2], const int *row_of,
-                            const uint32_t *row_limit, int rows_here, floatx4 *s) {
-        constexpr int R = decltype(rows_c)::value;
-        const unsigned char *kb = lds_raw + W::K_OFF + blk * W::K_BLOCK_BYTES;
-        KeyRegs<BITS> kreg[4];
-#pragma unroll
-        for (int gg = 0; gg < 4; gg++) {
-            if constexpr (BITS == 8) {
-                // the group's 64 bytes of token n are piece gg: 16 bytes j of them
-                const u32x4 v = *reinterpret_cast<const u32x4 *>(kb + gg * 1024 + n * 64 + j * 16);
-                kreg[gg].w[0] = v.x, kreg[gg].w[1] = v.y, kreg[gg].w[2] = v.z, kreg[gg].w[3] = v.w;
-            } else {
-                // the group's 32 bytes of token n are half gg % 2 of piece gg / 2: 8 bytes j of them
-                const u32x2 v = *reinterpret_cast<const u32x2 *>(kb + (gg >> 1) * 1024 + n * 64 + (gg & 1) * 32 + j * 8);
-                kreg[gg].w[0] = v.x, kreg[gg].w[1] = v.y;
-            }
-        }
-        const int tok0 = BLOCK * blk + 4 * j;  // this lane's 4 tokens of the round in C layout
-        const uint32_t *sb_w = sb_lds + BLOCK * blk;  // the block's dwords of groups (0, 1); + RT: groups (2, 3)
-        // bias term: slot e of every lane group belongs to group e / 2 of token n
-        const u32x2 zr = {sb_w[W::SB_ARRAY / 4 + n], sb_w[W::SB_ARRAY / 4 + RT + n]};
-        const half8 zop = as_half8(perm(0, zr.x, 0x01000100u), perm(0, zr.x, 0x03020302u), perm(0, zr.y, 0x01000100u), perm(0, zr.y, 0x03020302u));
-        // scales of the lane's tokens 4j .. 4j+3 of the block: groups (0, 1) and groups (2, 3)
-        const u32x4 s01 = *reinterpret_cast<const u32x4 *>(sb_w + 4 * j);
-        const u32x4 s23 = *reinterpret_cast<const u32x4 *>(sb_w + RT + 4 * j);
-        const uint32_t sw[8] = {s01.x, s23.x, s01.y, s23.y, s01.z, s23.z, s01.w, s23.w};
-        floatx4 rr[R][4];
-#pragma unroll
-        for (int ri = 0; ri < R; ri++) {
-            s[ri] = floatx4{0, 0, 0, 0};
-            s[ri] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz_reg[ri][0], s[ri], 0, 0, 0);
-            s[ri] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz_reg[ri][1], s[ri], 0, 0, 0);
-#pragma unroll
-            for (int gg = 0; gg < 4; gg++) rr[ri][gg] = floatx4{0, 0, 0, 0};
-        }
-#pragma unroll
-        for (int gg = 0; gg < 4; gg++) {
-#pragma unroll
-            for (int ab = 0; ab < 2; ab++) {
-                const half8 kop = key_operand<BITS>(kreg[gg], ab);
-#pragma unroll
-                for (int ri = 0; ri < R; ri++) rr[ri][gg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop, q_reg[ri][gg * 2 + ab], rr[ri][gg], 0, 0, 0);
-            }
-        }
-        constexpr float C1 = code_up<BITS>() / Q_UP;
-        float scl[4][4];
-#pragma unroll
-        for (int tk = 0; tk < 4; tk++) {
-#pragma unroll
-            for (int gg = 0; gg < 4; gg++) scl[tk][gg] = half_bits_to_float(sw[2 * tk + (gg >> 1)] >> (16 * (gg & 1))) * C1;
-        }
-#pragma unroll
-        for (int ri = 0; ri < R; ri++) {
-            if (ri >= rows_here) continue;
-#pragma unroll
-            for (int tk = 0; tk < 4; tk++) {
-                float d = 0.0f;
-#pragma unroll
-                for (int gg = 0; gg < 4; gg++) d += scl[tk][gg] * rr[ri][gg][tk];
-                float v = s[ri][tk] + d;
-                v += dpp<0x128>(v);  // row_ror 8: the other part (hi | lo) of the same head
-                s[ri][tk] = base + tok0 + tk < row_limit[ri] ? v : NO_SCORE;  // (also whatever a block past the round left in LDS)
-            }
-            // the block's softmax relative to its own maximum, per head
-            float cm = fmaxf(fmaxf(s[ri][0], s[ri][1]), fmaxf(s[ri][2], s[ri][3]));
-            cm = across_rows<16, 64>(cm, MaxOp());
-            float sum = 0.0f;
-#pragma unroll
-            for (int tk = 0; tk < 4; tk++) {
-                s[ri][tk] = s[ri][tk] > 0.5f * NO_SCORE ? __builtin_amdgcn_exp2f(s[ri][tk] - cm) : 0.0f;
-                sum += s[ri][tk];
-            }
-            sum = across_rows<16, 64>(sum, SumOp());
-            if (j == 0 && n < 8) bmax_lds[row_of[ri] * W::BROW + n * RBK + blk] = cm, bsum_lds[row_of[ri] * W::BROW + n * RBK + blk] = sum;
-        }
-    };
-    // The probability operands of k-step ks (tokens 32 ks .. 32 ks + 31 of the round) for R rows: P * value
-    // scale of group g, hi part in operand rows 0-7 and lo part in rows 8-15.  The two lanes of a head (n and
-    // n + 8) make four of the lane group's eight tokens each, both parts, and exchange what the other one
-    // feeds.  K-step 8 is block 16 alone: lane groups 0 and 1; the others repeat them with factor 0.
-    auto build_operands = [&](auto rows_c, int ks, int g, const int *row_of, const float *nm, int rows_here, float *zacc, half8 *out) {
-        constexpr int R = decltype(rows_c)::value;
-        const int hh = n >> 3;  // this lane makes tokens 8j + 4 hh .. + 3 of the k-step
-        const int sh = 16 * (g & 1);
-        const int jj = ks == 8 ? (j & 1) : j;
-        const int blk = 2 * ks + (jj >> 1);
-        // value scales and biases of group g: half g % 2 of the tokens' dwords of groups (g, g ^ 1).
-        // (Tokens past the share have probability 0 and the scales of the share's last token:
-        // every load is clamped to it, so nothing but cache rows in use is ever read.)
-        const uint32_t *vsp = sb_lds + 2 * (W::SB_ARRAY / 4) + (g >> 1) * RT + 32 * ks + 8 * jj + 4 * hh;
-        const u32x4 sv = *reinterpret_cast<const u32x4 *>(vsp);
-        const u32x4 zv = *reinterpret_cast<const u32x4 *>(vsp + W::SB_ARRAY / 4);
-        const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w}, zw[4] = {zv.x, zv.y, zv.z, zv.w};
-        float vscale[4], vbias[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) vscale[e] = half_bits_to_float(sw[e] >> sh), vbias[e] = half_bits_to_float(zw[e] >> sh);
-        const int fb = 2 * ks + (j >> 1);  // block 17 does not exist: factor 0
-#pragma unroll
-        for (int ri = 0; ri < R; ri++) {
-            if (ri >= rows_here) {
-                out[ri] = half8{0, 0, 0, 0, 0, 0, 0, 0};
-                continue;
-            }
-            const int r = row_of[ri];
-            const floatx4 pt = *reinterpret_cast<const floatx4 *>(s_block(blk, r) + (n & 7) * BLOCK + 8 * (jj & 1) + 4 * hh);
-            // 2^(block maximum - round maximum) * P_UP (2^8, so that the lo part stays a normal f16)
-            const float f = fb < RBK ? __builtin_amdgcn_exp2f(bmax_lds[r * W::BROW + (n & 7) * RBK + (fb < RBK ? fb : 0)] - nm[ri] + 8.0f) : 0.0f;
-            float x[4], lo[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const float p = pt[e] * f;
-                zacc[ri] += p * vbias[e];
-                x[e] = p * vscale[e];
-                lo[e] = x[e] - __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x[e]) & 0xffffe000u);
-            }
-            // round toward zero: exact truncation to the hi part
-            const uint32_t hi0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x[0], x[1]));
-            const uint32_t hi1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x[2], x[3]));
-            const uint32_t lo0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo[0], lo[1]));
-            const uint32_t lo1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo[2], lo[3]));
-            // the hi lane (n < 8) feeds hi parts and wants the other lane's hi parts of tokens 4-7; the lo
-            // lane feeds lo parts and wants the other lane's lo parts of tokens 0-3
-            const uint32_t send0 = hh ? hi0 : lo0, send1 = hh ? hi1 : lo1;
-            const uint32_t recv0 = uint32_t(__builtin_amdgcn_update_dpp(0, int(send0), 0x128, 0xf, 0xf, false));  // row_ror 8
-            const uint32_t recv1 = uint32_t(__builtin_amdgcn_update_dpp(0, int(send1), 0x128, 0xf, 0xf, false));
-            uint32_t o[4] = {hh ? recv0 : hi0, hh ? recv1 : hi1, hh ? lo0 : recv0, hh ? lo1 : recv1};
-            // (pinned: left alone, the compiler moves an operand's arithmetic down to its use, behind the wait for the values)
-            asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]));
-            out[ri] = as_half8(o[0], o[1], o[2], o[3]);
-        }
-    };
     // the value codes of k-step ks for group g: the lane's dword of tokens 32 ks + 8j .. + 7
     auto read_values = [&](int ks, int g, ValRegs<BITS> &vreg) {
-        const int v_lane = val_lane_offset<BITS>(g, n);
         const int jj = ks == 8 ? (j & 1) : j;
+        // (tokens 8 jj .. 8 jj + 7 of a k-step: their rows are rotated by jj quarters)
+        const unsigned char *vb = lds_raw + W::V_OFF + 8 * jj * RB + ((val_lane_offset<BITS>(g, n) + jj * W::V_ROT) & (RB - 1));
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const int tk = 32 * ks + 8 * jj + e;
-            // (the token's row is rotated by (tk / 8) % 4 quarters)
-            vreg.w[e] = *reinterpret_cast<const uint32_t *>(lds_raw + W::V_OFF + tk * RB + ((v_lane + ((tk >> 3) & 3) * W::V_ROT) & (RB - 1)));
-        }
+        for (int e = 0; e < 8; e++) vreg.w[e] = *reinterpret_cast<const uint32_t *>(vb + (32 * ks + e) * RB);
     };
     // a row's maximum per head over the round's blocks
     auto round_max = [&](int r, float start) {
-        const float *bmx = bmax_lds + r * W::BROW + (n & 7) * RBK;
+        const float *bmx = bmax_lds + r * W::BROW + (n & 7) * W::BSTRIDE;
         float v = start;
+        if constexpr (W::BSTRIDE % 4 == 0) {
 #pragma unroll
-        for (int i = 0; i < RBK; i++) v = fmaxf(v, bmx[i]);
+            for (int i = 0; i < W::BSTRIDE / 4; i++) {
+                const floatx4 w = reinterpret_cast<const floatx4 *>(bmx)[i];
+                v = fmaxf(v, fmaxf(fmaxf(w[0], w[1]), fmaxf(w[2], w[3])));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < RBK; i++) v = fmaxf(v, bmx[i]);
+        }
         return v;
     };
     // a row's sum of P of head n & 7 over the round's blocks, relative to the maximum nm: lane group j adds blocks j, j + 4, ...
     auto round_sum = [&](int r, float nm) {
         float sum = 0.0f;
+        if constexpr (W::BSTRIDE % 4 == 0) {
+            // lane group j adds blocks 5j .. 5j + 4
+#pragma unroll
+            for (int i = 0; i < W::BSTRIDE / 4; i++) {
+                const int b = (W::BSTRIDE / 4) * j + i;
+                sum += bsum_lds[r * W::BROW + (n & 7) * W::BSTRIDE + b] * __builtin_amdgcn_exp2f(bmax_lds[r * W::BROW + (n & 7) * W::BSTRIDE + b] - nm);
+            }
+            return across_rows<16, 64>(sum, SumOp());
+        }
 #pragma unroll
         for (int i = 0; i < (RBK + 3) / 4; i++) {
             const int b = j + 4 * i;
-            if (b < RBK) sum += bsum_lds[r * W::BROW + (n & 7) * RBK + b] * __builtin_amdgcn_exp2f(bmax_lds[r * W::BROW + (n & 7) * RBK + b] - nm);  // (a block that is not there: sum 0)
+            if (b < RBK) sum += bsum_lds[r * W::BROW + (n & 7) * W::BSTRIDE + b] * __builtin_amdgcn_exp2f(bmax_lds[r * W::BROW + (n & 7) * W::BSTRIDE + b] - nm);  // (a block that is not there: sum 0)
         }
         return across_rows<16, 64>(sum, SumOp());
     };
     constexpr float unscale = code_up<BITS>() / P_UP;
-    const int g = wave >> 1, b2 = wave & 1;
+    const int g = wave >> 1, b2 = wave & 1;  // O += P V: the wave's group and which k-steps of a slot
 
     if constexpr (M > 1) {
         // ---- several rows ------------------------------------------------------------------------
@@ -1657,7 +1517,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
                     sum += s[tk];
                 }
                 sum = across_rows<16, 64>(sum, SumOp());
-                if (j == 0) bmax_lds[my_row * W::BROW + (n & 7) * RBK + blk] = cm, bsum_lds[my_row * W::BROW + (n & 7) * RBK + blk] = sum;
+                if (j == 0) bmax_lds[my_row * W::BROW + (n & 7) * W::BSTRIDE + blk] = cm, bsum_lds[my_row * W::BROW + (n & 7) * W::BSTRIDE + blk] = sum;
                 // the scores go over the block's own keys: when this wave has them in registers, and with
                 // two pairs the other pair's wave of the same blocks, which takes them in the same order
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -1667,7 +1527,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
                 }
                 *reinterpret_cast<floatx4 *>(s_block(blk, my_row) + (n & 7) * BLOCK + 4 * j) = s;
             }
-            if (wt == 0 && !extra && j == 0) bmax_lds[my_row * W::BROW + (n & 7) * RBK + 16] = NO_SCORE, bsum_lds[my_row * W::BROW + (n & 7) * RBK + 16] = 0.0f;
+            if (wt == 0 && !extra && j == 0) bmax_lds[my_row * W::BROW + (n & 7) * W::BSTRIDE + 16] = NO_SCORE, bsum_lds[my_row * W::BROW + (n & 7) * W::BSTRIDE + 16] = 0.0f;
         }
         raise(W::C_SCORES);
         await(W::C_SCORES, W::WAVES);
@@ -1709,7 +1569,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
                 const floatx4 pt0 = *reinterpret_cast<const floatx4 *>(sp), pt1 = *reinterpret_cast<const floatx4 *>(sp + 4);
                 const float pt[8] = {pt0[0], pt0[1], pt0[2], pt0[3], pt1[0], pt1[1], pt1[2], pt1[3]};
                 // 2^(block maximum - round maximum) * P_UP (2^8, so that the lo part stays a normal f16)
-                const float f = fb < RBK ? __builtin_amdgcn_exp2f(bmax_lds[r * W::BROW + (n & 7) * RBK + (fb < RBK ? fb : 0)] - nm[p] + 8.0f) : 0.0f;
+                const float f = fb < RBK ? __builtin_amdgcn_exp2f(bmax_lds[r * W::BROW + (n & 7) * W::BSTRIDE + (fb < RBK ? fb : 0)] - nm[p] + 8.0f) : 0.0f;
                 float x[8], lo[8], zb = 0.0f;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
@@ -1816,53 +1676,145 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
         // ---- one row -----------------------------------------------------------------------------
         // Scores: wave w takes the blocks w and w + 8 (wave 0 also 16).  O += P V: waves 2g and 2g + 1 share
         // group g and take alternate k-steps, so that each value slot gives every wave one k-step.
-        stage_query(qv[0]);
+        // ---- prologue: the query row to f16 hi/lo operands in LDS (operand row n: head n & 7, hi part in
+        // rows 0-7 and lo part in rows 8-15 of the one tile) ---------------------------------------------
+        {
+            const float qmul = a.scale * 1.4426950408889634f * Q_UP;
+            half8 op;
+            float sum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                _Float16 h, lw;
+                split_hi_lo(qv[0][key_slot_dim<BITS>(e)] * qmul, h, lw);
+                const _Float16 x = n < 8 ? h : lw;
+                op[e] = x;
+                sum += (float)x;
+            }
+            q_lds[wave * 64 + lane] = op;
+            // key bias term: slot `k-step` of this lane in the B operand of one more MFMA, as hi and lo halves
+            _Float16 h, lw;
+            split_hi_lo(sum * (1.0f / Q_UP), h, lw);
+            qz_lds[(0 * 64 + lane) * 8 + wave] = h;
+            qz_lds[(1 * 64 + lane) * 8 + wave] = lw;
+            // blocks that never exist
+            if (wave == 0 && lane < 8 * (W::BSTRIDE - RBK)) {
+                const int idx = (lane / (W::BSTRIDE - RBK)) * W::BSTRIDE + RBK + lane % (W::BSTRIDE - RBK);
+                bmax_lds[idx] = NO_SCORE, bsum_lds[idx] = 0.0f;
+            }
+        }
         raise(W::C_QUERY);
+
+        // ---- running state -------------------------------------------------------------
         float m_run = NO_SCORE;
-        float l_run = 0.0f;  // sum of P of head n & 7 (wave 0 keeps it)
-        float zacc[1] = {0.0f};  // sum of P * P_UP * value bias of group g over this lane's tokens
-        floatx4 acc[4];      // [tile of 16 dims 4n' + e]: rows 4j .. 4j+3 (operand rows), column n'
+        float l_run = 0.0f;    // sum of P of head n & 7 (wave 0 keeps it)
+        float zacc = 0.0f;     // sum of P * P_UP * value bias of group g over this lane's tokens
+        floatx4 acc[4];        // [tile of 16 dims 4n' + e]: rows 4j .. 4j+3 (operand rows), column n'
 #pragma unroll
         for (int e = 0; e < 4; e++) acc[e] = floatx4{0, 0, 0, 0};
         await(W::C_QUERY, W::WAVES);
-        const int row0[1] = {0};
 
         for (uint32_t round = 0; round < n_rounds; round++) {
             const uint32_t base = (blk_begin + round * per_round) * BLOCK, nb = blocks_of(round);
             const bool more = round + 1 < n_rounds;
             const bool extra = nb == uint32_t(RBK);  // the round has block 16
-            const uint32_t round_limit[1] = {min(limit, base + nb * BLOCK)};  // tokens of this round end here
+            const uint32_t round_limit = min(limit, base + nb * BLOCK);  // tokens of this round end here
 
             // ---- phase A: scores of blocks wave, wave + 8 (and wave 0: 16) --------------------------
             // (the query operands are read again in every round: they are not needed between the scores
             // of one round and the next, and the registers are)
             {
-                half8 q_reg[1][8], qz_reg[1][2];
+                half8 q_reg[8], qz_reg[2];
 #pragma unroll
-                for (int i = 0; i < 8; i++) q_reg[0][i] = q_lds[i * 64 + lane];
-                qz_reg[0][0] = *reinterpret_cast<const half8 *>(qz_lds + lane * 8);
-                qz_reg[0][1] = *reinterpret_cast<const half8 *>(qz_lds + (64 + lane) * 8);
+                for (int i = 0; i < 8; i++) q_reg[i] = q_lds[i * 64 + lane];
+                qz_reg[0] = *reinterpret_cast<const half8 *>(qz_lds + lane * 8);
+                qz_reg[1] = *reinterpret_cast<const half8 *>(qz_lds + (64 + lane) * 8);
                 const int parts = (wave == 0 && extra) ? 3 : 2;
 #pragma unroll 1
                 for (int part = 0; part < parts; part++) {
                     await(W::C_KPART + part, W::K_LOADERS * (round + 1));  // this part of the keys is in LDS (first: and the scales)
                     const int blk = wave + 8 * part;
-                    floatx4 s[1];
-                    block_scores(std::integral_constant<int, 1>(), blk, base, q_reg, qz_reg, row0, round_limit, 1, s);
+                    const unsigned char *kb = lds_raw + W::K_OFF + blk * W::K_BLOCK_BYTES;
+                    KeyRegs<BITS> kreg[4];
+#pragma unroll
+                    for (int gg = 0; gg < 4; gg++) {
+                        if constexpr (BITS == 8) {
+                            // the group's 64 bytes of token n are piece gg: 16 bytes j of them
+                            const u32x4 v = *reinterpret_cast<const u32x4 *>(kb + gg * 1024 + n * 64 + j * 16);
+                            kreg[gg].w[0] = v.x, kreg[gg].w[1] = v.y, kreg[gg].w[2] = v.z, kreg[gg].w[3] = v.w;
+                        } else {
+                            // the group's 32 bytes of token n are half gg % 2 of piece gg / 2: 8 bytes j of them
+                            const u32x2 v = *reinterpret_cast<const u32x2 *>(kb + (gg >> 1) * 1024 + n * 64 + (gg & 1) * 32 + j * 8);
+                            kreg[gg].w[0] = v.x, kreg[gg].w[1] = v.y;
+                        }
+                    }
+                    const int tok0 = BLOCK * blk + 4 * j;  // this lane's 4 tokens of the round in C layout
+                    const uint32_t *sb_w = sb_lds + BLOCK * blk;  // the block's dwords of groups (0, 1); + RT: groups (2, 3)
+                    floatx4 s;
+                    {
+                        // bias term: slot e of every lane group belongs to group e / 2 of token n
+                        const u32x2 zr = {sb_w[W::SB_ARRAY / 4 + n], sb_w[W::SB_ARRAY / 4 + RT + n]};
+                        const half8 zop = as_half8(perm(0, zr.x, 0x01000100u), perm(0, zr.x, 0x03020302u), perm(0, zr.y, 0x01000100u),
+                                                   perm(0, zr.y, 0x03020302u));
+                        s = floatx4{0, 0, 0, 0};
+                        s = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz_reg[0], s, 0, 0, 0);
+                        s = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz_reg[1], s, 0, 0, 0);
+                    }
+                    floatx4 r[4];
+#pragma unroll
+                    for (int gg = 0; gg < 4; gg++) {
+                        r[gg] = floatx4{0, 0, 0, 0};
+#pragma unroll
+                        for (int ab = 0; ab < 2; ab++) {
+                            r[gg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(key_operand<BITS>(kreg[gg], ab), q_reg[gg * 2 + ab], r[gg], 0, 0, 0);
+                        }
+                    }
+                    // scales of the lane's tokens 4j .. 4j+3 of the block: groups (0, 1) and groups (2, 3)
+                    const u32x4 s01 = *reinterpret_cast<const u32x4 *>(sb_w + 4 * j);
+                    const u32x4 s23 = *reinterpret_cast<const u32x4 *>(sb_w + RT + 4 * j);
+                    const uint32_t sw[8] = {s01.x, s23.x, s01.y, s23.y, s01.z, s23.z, s01.w, s23.w};
+                    constexpr float C1 = code_up<BITS>() / Q_UP;
+#pragma unroll
+                    for (int tk = 0; tk < 4; tk++) {
+                        float d = 0.0f;
+#pragma unroll
+                        for (int gg = 0; gg < 4; gg++) d += half_bits_to_float(sw[2 * tk + (gg >> 1)] >> (16 * (gg & 1))) * r[gg][tk];
+                        float v = s[tk] + d * C1;
+                        v += dpp<0x128>(v);  // row_ror 8: the other part (hi | lo) of the same head
+                        s[tk] = base + tok0 + tk < round_limit ? v : NO_SCORE;  // (also whatever a block past the round left in LDS)
+                    }
+                    // the block's softmax relative to its own maximum, per head
+                    float cm = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+                    cm = across_rows<16, 64>(cm, MaxOp());
+                    float sum = 0.0f;
+#pragma unroll
+                    for (int tk = 0; tk < 4; tk++) {
+                        s[tk] = s[tk] > 0.5f * NO_SCORE ? __builtin_amdgcn_exp2f(s[tk] - cm) : 0.0f;
+                        sum += s[tk];
+                    }
+                    sum = across_rows<16, 64>(sum, SumOp());
                     // over the block's own keys (every lane of the wave has its key registers by now)
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                    if (n < 8) *reinterpret_cast<floatx4 *>(s_block(blk, 0) + n * BLOCK + 4 * j) = s[0];
+                    if (n < 8) *reinterpret_cast<floatx4 *>(s_block(blk, 0) + n * BLOCK + 4 * j) = s;
+                    if (j == 0 && n < 8) bmax_lds[n * W::BSTRIDE + blk] = cm, bsum_lds[n * W::BSTRIDE + blk] = sum;
                 }
-                if (wave == 0 && !extra && j == 0 && n < 8) bmax_lds[n * RBK + 16] = NO_SCORE, bsum_lds[n * RBK + 16] = 0.0f;
+                if (wave == 0 && !extra && j == 0 && n < 8) bmax_lds[n * W::BSTRIDE + 16] = NO_SCORE, bsum_lds[n * W::BSTRIDE + 16] = 0.0f;
             }
             raise(W::C_SCORES);
             await(W::C_SCORES, W::WAVES * (round + 1));
 
             // ---- the round's maximum per head, and what was summed so far brought to it -------------
-            const float nm[1] = {round_max(0, m_run)};
-            const float al = __builtin_amdgcn_exp2f(m_run - nm[0]);  // (first round: 2^(-1e30 - nm) = 0, and nothing to scale)
+            float nm = m_run;
+            {
+                const floatx4 *bmx = reinterpret_cast<const floatx4 *>(bmax_lds + (n & 7) * W::BSTRIDE);
+#pragma unroll
+                for (int i = 0; i < W::BSTRIDE / 4; i++) {
+                    const floatx4 w = bmx[i];
+                    nm = fmaxf(nm, fmaxf(fmaxf(w[0], w[1]), fmaxf(w[2], w[3])));
+                }
+            }
+            const float al = __builtin_amdgcn_exp2f(m_run - nm);  // (first round: 2^(-1e30 - nm) = 0, and nothing to scale)
             if (round > 0) {
-                zacc[0] *= al;
+                zacc *= al;
                 // accumulator rows 4j + i are heads (4j + i) & 7: lane h (j = 0, n = h) holds head h's factor
                 floatx4 al4;
 #pragma unroll
@@ -1872,34 +1824,93 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
 #pragma unroll
                 for (int e = 0; e < 4; e++) acc[e] *= al4;
             }
-            m_run = nm[0];
-            if (wave == 0) l_run = l_run * al + round_sum(0, nm[0]);
-
-            // ---- probability operands of this wave's k-steps ----
-            const bool fifth = extra && b2 == 0;  // k-step 8: block 16
-            half8 p_op[W::SLOTS];
+            m_run = nm;
+            if (wave == 0) {
+                // the round's sum of P of head n & 7: lane group j adds blocks 5j .. 5j + 4
+                float sum = 0.0f;
 #pragma unroll
-            for (int sl = 0; sl < W::SLOTS; sl++) {
-                if (sl == 4 && !fifth) {
-                    p_op[sl] = half8{0, 0, 0, 0, 0, 0, 0, 0};
-                    continue;
+                for (int i = 0; i < W::BSTRIDE / 4; i++) {
+                    const int b = (W::BSTRIDE / 4) * j + i;
+                    sum += bsum_lds[(n & 7) * W::BSTRIDE + b] * __builtin_amdgcn_exp2f(bmax_lds[(n & 7) * W::BSTRIDE + b] - nm);  // (a block that is not there: sum 0)
                 }
-                build_operands(std::integral_constant<int, 1>(), 2 * sl + b2, g, row0, nm, 1, zacc, &p_op[sl]);
+                l_run = l_run * al + across_rows<16, 64>(sum, SumOp());
+            }
+
+            // ---- probability operands of this wave's k-steps: P * value scale of group g, hi part in
+            // operand rows 0-7 and lo part in rows 8-15.  The two lanes of a head (n and n + 8) make four of
+            // the lane group's eight tokens each, both parts, and exchange what the other one feeds. ----
+            half8 p_op[W::SLOTS];
+            {
+                const int hh = n >> 3;  // this lane makes tokens 8j + 4 hh .. + 3 of a k-step
+                const int sh = 16 * (g & 1);
+                const bool fifth = extra && b2 == 0;  // k-step 8: block 16 (lane groups 0 and 1; the others repeat them with factor 0)
+#pragma unroll
+                for (int sl = 0; sl < W::SLOTS; sl++) {
+                    if (sl == 4 && !fifth) {
+                        p_op[sl] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+                        continue;
+                    }
+                    const int ks = 2 * sl + b2;  // tokens 32 ks ..: blocks 2 ks and 2 ks + 1
+                    const int jj = sl == 4 ? (j & 1) : j;
+                    const int blk = 2 * ks + (jj >> 1);
+                    const floatx4 pt = *reinterpret_cast<const floatx4 *>(s_block(blk, 0) + (n & 7) * BLOCK + 8 * (jj & 1) + 4 * hh);
+                    // value scales and biases of group g: half g % 2 of the tokens' dwords of groups (g, g ^ 1).
+                    // (Tokens past the share have probability 0 and the scales of the share's last token:
+                    // every load is clamped to it, so nothing but cache rows in use is ever read.)
+                    const uint32_t *vsp = sb_lds + 2 * (W::SB_ARRAY / 4) + (g >> 1) * RT + 32 * ks + 8 * jj + 4 * hh;
+                    const u32x4 sv = *reinterpret_cast<const u32x4 *>(vsp);
+                    const u32x4 zv = *reinterpret_cast<const u32x4 *>(vsp + W::SB_ARRAY / 4);
+                    // 2^(block maximum - round maximum) * P_UP (2^8, so that the lo part stays a normal f16)
+                    const float f = __builtin_amdgcn_exp2f(bmax_lds[(n & 7) * W::BSTRIDE + 2 * ks + (j >> 1)] - nm + 8.0f);
+                    const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w}, zw[4] = {zv.x, zv.y, zv.z, zv.w};
+                    float x[4], lo[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const float p = pt[e] * f;
+                        zacc += p * half_bits_to_float(zw[e] >> sh);
+                        x[e] = p * half_bits_to_float(sw[e] >> sh);
+                        lo[e] = x[e] - __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x[e]) & 0xffffe000u);
+                    }
+                    // round toward zero: exact truncation to the hi part
+                    const uint32_t hi0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x[0], x[1]));
+                    const uint32_t hi1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x[2], x[3]));
+                    const uint32_t lo0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo[0], lo[1]));
+                    const uint32_t lo1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo[2], lo[3]));
+                    // the hi lane (n < 8) feeds hi parts and wants the other lane's hi parts of tokens 4-7; the lo
+                    // lane feeds lo parts and wants the other lane's lo parts of tokens 0-3
+                    const uint32_t send0 = hh ? hi0 : lo0, send1 = hh ? hi1 : lo1;
+                    const uint32_t recv0 = uint32_t(__builtin_amdgcn_update_dpp(0, int(send0), 0x128, 0xf, 0xf, false));  // row_ror 8
+                    const uint32_t recv1 = uint32_t(__builtin_amdgcn_update_dpp(0, int(send1), 0x128, 0xf, 0xf, false));
+                    uint32_t o[4] = {hh ? recv0 : hi0, hh ? recv1 : hi1, hh ? lo0 : recv0, hh ? lo1 : recv1};
+                    // (pinned: left alone, the compiler moves an operand's arithmetic down to its use, behind the wait for the values)
+                    asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]));
+                    p_op[sl] = as_half8(o[0], o[1], o[2], o[3]);
+                }
             }
             if (more) raise(W::C_BUILT);  // this wave is through with the round's scores, scales and biases
 
             // ---- phase C: O += P V, one k-step per value slot as the slots land ---------------------
+            const unsigned char *vb = lds_raw + W::V_OFF;
+            auto read_values = [&](int sl, ValRegs<BITS> &vreg) {
+                const int jj = sl == 4 ? (j & 1) : j;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int tk = 32 * (2 * sl + b2) + 8 * jj + e;
+                    vreg.w[e] = *reinterpret_cast<const uint32_t *>(vb + tk * RB + ((val_lane_offset<BITS>(g, n) + jj * (RB / 4)) & (RB - 1)));
+                }
+            };
             auto add_values = [&](int sl, const ValRegs<BITS> &vreg) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p_op[sl], val_operand<BITS>(vreg, e, n), acc[e], 0, 0, 0);
                 }
             };
+            const bool fifth = extra && b2 == 0;
             if (peek(W::C_SLOT + 3) >= W::V_LOADERS * (round + 1)) {
                 // slots 0-3 are there already (the slots land in order): every read at once
                 ValRegs<BITS> vreg[4];
 #pragma unroll
-                for (int sl = 0; sl < 4; sl++) read_values(2 * sl + b2, g, vreg[sl]);
+                for (int sl = 0; sl < 4; sl++) read_values(sl, vreg[sl]);
 #pragma unroll
                 for (int sl = 0; sl < 4; sl++) add_values(sl, vreg[sl]);
             } else {
@@ -1907,14 +1918,14 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
                 for (int sl = 0; sl < 4; sl++) {
                     await(W::C_SLOT + sl, W::V_LOADERS * (round + 1));  // value slot sl is in LDS
                     ValRegs<BITS> vreg;
-                    read_values(2 * sl + b2, g, vreg);
+                    read_values(sl, vreg);
                     add_values(sl, vreg);
                 }
             }
             if (fifth) {
                 await(W::C_SLOT + 4, W::V_LOADERS * (round + 1));
                 ValRegs<BITS> vreg;
-                read_values(8, g, vreg);
+                read_values(4, vreg);
                 add_values(4, vreg);
             }
             if (more) {
@@ -1926,7 +1937,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
         // ---- epilogue: the two waves of a group add up, wave 2g writes the partial ---------------------
         {
             // the head's bias sum: over the four lane groups and the two lanes of the head
-            float z = across_rows<16, 64>(zacc[0], SumOp());
+            float z = across_rows<16, 64>(zacc, SumOp());
             z += dpp<0x128>(z);
             if (j == 0 && n < 8) zs_lds[wave * 8 + n] = z;
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -1939,7 +1950,8 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
 #pragma unroll
             for (int e = 0; e < 4; e++) mine[i][e] = across_rows<32, 64>(acc[e][i], SumOp()) * unscale + zb;
         }
-        // (the merge lies over the query operands, which nobody reads after the last round's scores)
+        // (the key area is free: the key loaders request nothing after the last round, and every wave is
+        // past the last round's scores, having built its operands from them)
         floatx4 *x_o = reinterpret_cast<floatx4 *>(lds_raw + W::X_OFF);  // [group][lane < 32][4 rows]
         if (b2 == 1) {
             if (j < 2) {
