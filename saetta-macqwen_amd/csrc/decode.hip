@@ -1133,13 +1133,14 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
         const float4 f1 = *reinterpret_cast<const float4 *>(src + 4);
         v[0] = f0.x, v[1] = f0.y, v[2] = f0.z, v[3] = f0.w, v[4] = f1.x, v[5] = f1.y, v[6] = f1.z, v[7] = f1.w;
     };
-    // (several rows: per pair of rows, the row that the lane's column of the pair's tile belongs to)
+    // (several rows: per pair of rows, the row that the lane's column of the pair's tile belongs to.  The
+    // loader waves leave the registers as they are: a value set for them would have to be merged with the
+    // loaded one, and that copy would wait for the load in front of the barrier, where the loader waves
+    // stand until every wave has arrived.)
     float qv[W::PAIRS][8];
+    if (!loader) {
 #pragma unroll
-    for (int p = 0; p < W::PAIRS; p++) {
-#pragma unroll
-        for (int e = 0; e < 8; e++) qv[p][e] = 0.0f;
-        if (!loader) load_query(M == 1 ? 0 : min(2 * p + (n >> 3), M - 1), qv[p]);
+        for (int p = 0; p < W::PAIRS; p++) load_query(M == 1 ? 0 : min(2 * p + (n >> 3), M - 1), qv[p]);
     }
 
     // ---- the context and this workgroup's share of it -----------------------------
