@@ -52,6 +52,9 @@
 //   attention_partial_kernel_d   one query row over codes in large caches: four more waves
 //                                move the codes into LDS (global_load_lds), two teams of four
 //                                computing waves take alternate 64-token iterations
+//   attention_partial_kernel_s   one to four query rows over codes in large caches: loader waves
+//                                again, a whole share in LDS with the keys requested first, the
+//                                waves meeting through counters in LDS
 //   attention_reduce_kernel      the merge of the splits and the gate
 // Which one runs is decided in run_attention from the launch arguments alone, so that the partial
 // and the reduce stage of a step agree on the number of splits.
@@ -1045,11 +1048,8 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel_p(PartialArg
 // instructions in order, so data written before a counter is raised is there when the counter is
 // seen.  Every wait on a counter is bounded (SPIN_LIMIT polls), so every wave ends whatever happens.
 // Longer shares take further rounds with an online softmax between the rounds.
-// M query rows (a verify step, 2..4): every row is a tile of its own (its 8 heads' hi parts in operand
-// rows 0-7, the lo parts in rows 8-15), and the codes in LDS serve all of them.  The scores are taken
-// row by row, the row's query operands staged through the one place in LDS while the scores of the
-// row before are computed; the probability operands and O += P V go two rows at a time (the
-// registers hold two rows' operands), the byte permutes of a value operand serving both.
+// M query rows (a verify step, 2..4) take one round over codes that serve every row; two rows share a
+// tile (see the rows' part of the kernel).
 template <int BITS, int M>
 struct KeysFirst {
     static constexpr int PAIRS = (M + 1) / 2;               // tiles of two query rows (one row: its own tile)
