@@ -12,7 +12,8 @@
 //     O = diag(e^c) Q S0^T + M U,                       M_ts = e^{c_t - c_s} (q_t . k_s)         (s <= t)
 //     S1^T = e^{c_last} S0^T + K^T diag(e^{c_last - c}) U
 // (U, V, O: [C][v_dim]; K, Q: [C][128], normalised as the reference does).  Two kernels:
-//   deltanet_chunk_prepare_kernel   one workgroup per (block, value head), all blocks at once: the
+//   deltanet_chunk_prepare_kernel   one workgroup per (block, key head) with its two value heads (or per
+//       value head, for another ratio), all blocks at once: the
 //       normalised q and k, A and M (64 x 64 x 128 products), T = (I + A)^-1 diag(beta) by forward
 //       substitution, and the decay factors, to a workspace;
 //   deltanet_chunk_chain_kernel     one workgroup per (16 value dims, value head) walks the blocks in
@@ -77,27 +78,42 @@ __device__ __forceinline__ floatx4 mma3(half8 ah, half8 al, half8 bh, half8 bl, 
 }
 
 // ---- prepare: everything of a block that does not depend on the state ------------------------------
-// LDS: the four q / k images; once the products are taken, A (f32, over kh), the M images (over kl) and
-// later the T images (over qh) are staged over them, so that they leave as whole 16-byte stores.
-constexpr int PREP_LDS = 4 * K_IMG + 2 * C * 4;
-constexpr int AROW = C + 4;  // f32 per row of A in LDS: [t][q * 16 + m] holds A_t,s of s = 4m + q
-static_assert(C * AROW * 4 <= K_IMG && 2 * T_IMG <= K_IMG + K_IMG, "the staged matrices fit over the images");
+// One workgroup takes G value heads of one key head: the q / k images and the k . k and q . k products
+// belong to the key head, the gates, A, M and T to a value head.  (G = 2, the model's two value heads
+// per key head: the two triangular solves, each a chain of 64 dependent steps, run side by side in the
+// same lanes; G = 1: any other ratio, one workgroup per value head, the first of a key head's writing
+// the key head's images.)
+// LDS: the four q / k images; once the products are taken, the heads' A (f32) go over kh | kl, their M
+// images and later their T images over qh | ql (and 2 KB more), so that they leave as whole 16-byte stores.
+template <int G>
+struct PrepLds {
+    static constexpr int AROW = C + 4;  // f32 per row of A in LDS: [t][q * 16 + m] holds A_t,s of s = 4m + q
+    static constexpr int A_OFF = 0, A_BYTES = C * AROW * 4;
+    static constexpr int M_OFF = 2 * K_IMG, M_BYTES = 2 * T_IMG;  // mh | ml (then th | tl) of a head
+    static constexpr int GATES = M_OFF + G * M_BYTES > 4 * K_IMG ? M_OFF + G * M_BYTES : 4 * K_IMG;  // [head][cum | beta][C] f32
+    static constexpr int BYTES = GATES + G * 2 * C * 4;
+    static_assert(G * A_BYTES <= M_OFF, "the heads' A fit over kh | kl");
+    static_assert(2 * BYTES <= 160 * 1024, "two workgroups per CU");
+};
 
+template <int G>
 __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a) {
+    using L = PrepLds<G>;
+    constexpr int AROW = L::AROW;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     _Float16 *kh = reinterpret_cast<_Float16 *>(lds), *kl = kh + C * KROW, *qh = kl + C * KROW, *ql = qh + C * KROW;
-    float *a_lds = reinterpret_cast<float *>(lds);                        // over kh
-    _Float16 *m_lds = reinterpret_cast<_Float16 *>(lds + K_IMG);           // mh | ml over kl (and the start of qh)
-    _Float16 *t_lds = reinterpret_cast<_Float16 *>(lds + 2 * K_IMG + T_IMG);  // th | tl over the rest of qh and ql
-    float *cum_lds = reinterpret_cast<float *>(lds + 4 * K_IMG), *beta_lds = cum_lds + C;
-    static_assert(K_IMG + 2 * T_IMG <= 2 * K_IMG + T_IMG && 2 * K_IMG + 3 * T_IMG <= 4 * K_IMG, "M and T do not overlap");
-    const uint32_t blk = blockIdx.x, h = blockIdx.y, group = a.v_heads / a.k_heads, khd = h / group;
+    auto a_lds = [&](int hh) { return reinterpret_cast<float *>(lds + L::A_OFF + hh * L::A_BYTES); };
+    auto m_lds = [&](int hh) { return reinterpret_cast<_Float16 *>(lds + L::M_OFF + hh * L::M_BYTES); };
+    auto cum_lds = [&](int hh) { return reinterpret_cast<float *>(lds + L::GATES) + hh * 2 * C; };
+    auto beta_lds = [&](int hh) { return reinterpret_cast<float *>(lds + L::GATES) + hh * 2 * C + C; };
+    const uint32_t blk = blockIdx.x, group = a.v_heads / a.k_heads;
+    const uint32_t h0 = blockIdx.y * G, khd = h0 / group;  // the workgroup's first value head, its key head
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), n = lane & 15, j = lane >> 4;
     const uint32_t key_size = a.k_heads * K_DIM;
     unsigned char *ws_blk = a.ws + size_t(blk) * block_bytes(a.k_heads, a.v_heads);
     unsigned char *ws_k = ws_blk + khd * KHEAD_BYTES;
-    unsigned char *ws_v = ws_blk + a.k_heads * KHEAD_BYTES + h * VHEAD_BYTES;
-    const bool writer = h % group == 0;  // one value head of the key head's group keeps the q / k images
+    auto ws_v = [&](int hh) { return ws_blk + a.k_heads * KHEAD_BYTES + (h0 + hh) * VHEAD_BYTES; };
+    const bool writer = h0 % group == 0;  // one workgroup of the key head's keeps the q / k images
 
     // ---- q and k of the block's tokens, normalised (src/cpu/deltanet.rs:133-146), as hi and lo parts ----
     {
@@ -145,9 +161,9 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
             }
         }
     }
-    // ---- the gates: c_t = sum of log g up to t, beta_t (tokens past the end: g = 1, beta = 0) ----
-    if (tid < C) {
-        const uint32_t tok = blk * C + tid;
+    // ---- the gates of head h0 + wave: c_t = sum of log g up to t, beta_t (tokens past the end: g = 1, beta = 0) ----
+    if (wave < G) {
+        const uint32_t tok = blk * C + lane, h = h0 + wave;
         float lg = 0.0f, beta = 0.0f;
         if (tok < a.tokens) {
             float g;
@@ -160,10 +176,10 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
             const float up = __shfl_up(c, d, 64);
             if (int(lane) >= d) c += up;
         }
-        cum_lds[tid] = c, beta_lds[tid] = beta;
+        cum_lds(wave)[lane] = c, beta_lds(wave)[lane] = beta;
         const float last = __shfl(c, 63, 64);
-        float *gam = reinterpret_cast<float *>(ws_v + 4 * T_IMG);
-        gam[tid] = __expf(c), gam[C + tid] = __expf(last - c);
+        float *gam = reinterpret_cast<float *>(ws_v(wave) + 4 * T_IMG);
+        gam[lane] = __expf(c), gam[C + lane] = __expf(last - c);
     }
     __syncthreads();
 
@@ -202,60 +218,81 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
 
     // C layout: lane (n, j) holds column s = 16 nt + n of rows t = 16 wave + 4j + i
 #pragma unroll
-    for (int nt = 0; nt < 4; nt++) {
-        const uint32_t s = 16 * nt + n;
-        const float cs = cum_lds[s];
+    for (int hh = 0; hh < G; hh++) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t t = 16 * wave + 4 * j + i;
-            const float decay = s <= t ? __expf(cum_lds[t] - cs) : 0.0f;
-            a_lds[t * AROW + (s & 3) * 16 + (s >> 2)] = s < t ? beta_lds[t] * decay * gk[nt][i] : 0.0f;
-            _Float16 hi, lo;
-            split2(decay * gq[nt][i], hi, lo);
-            m_lds[t * TROW + s] = hi, m_lds[C * TROW + t * TROW + s] = lo;
+        for (int nt = 0; nt < 4; nt++) {
+            const uint32_t s = 16 * nt + n;
+            const float cs = cum_lds(hh)[s];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t t = 16 * wave + 4 * j + i;
+                const float decay = s <= t ? __expf(cum_lds(hh)[t] - cs) : 0.0f;
+                a_lds(hh)[t * AROW + (s & 3) * 16 + (s >> 2)] = s < t ? beta_lds(hh)[t] * decay * gk[nt][i] : 0.0f;
+                _Float16 hi, lo;
+                split2(decay * gq[nt][i], hi, lo);
+                m_lds(hh)[t * TROW + s] = hi, m_lds(hh)[C * TROW + t * TROW + s] = lo;
+            }
         }
     }
     __syncthreads();
     // M leaves (whole 16-byte pieces; the padding columns go along)
-    {
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(m_lds);
-        u32x4 *dst = reinterpret_cast<u32x4 *>(ws_v + 2 * T_IMG);
+#pragma unroll
+    for (int hh = 0; hh < G; hh++) {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(m_lds(hh));
+        u32x4 *dst = reinterpret_cast<u32x4 *>(ws_v(hh) + 2 * T_IMG);
         for (uint32_t i = tid; i < 2 * T_IMG / 16; i += 256) dst[i] = src[i];
     }
 
     // ---- T = (I + A)^-1 diag(beta): column c = 16 wave + n by forward substitution, x_t = beta_t [t = c] -
-    // sum_{s < t} A_ts x_s; lane group q keeps x_s of s = 4m + q in slot m and adds up those s ----
+    // sum_{s < t} A_ts x_s; lane group q keeps x_s of s = 4m + q in slot m and adds up those s.  The heads'
+    // columns are solved side by side: their chains do not depend on each other. ----
     {
         const uint32_t c = 16 * wave + n, q = j;
-        float x[16];
+        float x[G][16];
 #pragma unroll
-        for (int m = 0; m < 16; m++) x[m] = 0.0f;
+        for (int hh = 0; hh < G; hh++) {
+#pragma unroll
+            for (int m = 0; m < 16; m++) x[hh][m] = 0.0f;
+        }
 #pragma unroll
         for (int t = 0; t < C; t++) {
             if (t < int(16 * wave)) continue;  // (the column is zero above its diagonal: uniform per wave)
-            floatx4 part4 = {0, 0, 0, 0};  // (four chains of sums instead of one of up to 16)
-            const float *arow = a_lds + t * AROW + q * 16;
+            float total[G];
 #pragma unroll
-            for (int m4 = 0; 16 * m4 < t; m4++) {  // s = 4m + q < t needs m <= (t - 1) / 4
-                const floatx4 av = *reinterpret_cast<const floatx4 *>(arow + 4 * m4);
+            for (int hh = 0; hh < G; hh++) {
+                floatx4 part4 = {0, 0, 0, 0};  // (four chains of sums instead of one of up to 16)
+                const float *arow = a_lds(hh) + t * AROW + q * 16;
 #pragma unroll
-                for (int e = 0; e < 4; e++) part4[e] += av[e] * x[4 * m4 + e];
+                for (int m4 = 0; 16 * m4 < t; m4++) {  // s = 4m + q < t needs m <= (t - 1) / 4
+                    const floatx4 av = *reinterpret_cast<const floatx4 *>(arow + 4 * m4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) part4[e] += av[e] * x[hh][4 * m4 + e];
+                }
+                total[hh] = (part4[0] + part4[1]) + (part4[2] + part4[3]);
             }
-            const float total = across_rows<16, 64>((part4[0] + part4[1]) + (part4[2] + part4[3]), SumOp());
-            const float xt = (uint32_t(t) == c ? beta_lds[t] : 0.0f) - total;
-            if (q == uint32_t(t & 3)) x[t >> 2] = xt;
-        }
 #pragma unroll
-        for (int m = 0; m < 16; m++) {
-            _Float16 hi, lo;
-            split2(x[m], hi, lo);
-            t_lds[(4 * m + q) * TROW + c] = hi, t_lds[C * TROW + (4 * m + q) * TROW + c] = lo;
+            for (int hh = 0; hh < G; hh++) {
+                const float sum = across_rows<16, 64>(total[hh], SumOp());
+                const float xt = (uint32_t(t) == c ? beta_lds(hh)[t] : 0.0f) - sum;
+                if (q == uint32_t(t & 3)) x[hh][t >> 2] = xt;
+            }
+        }
+        __syncthreads();  // M has left: T goes over it
+#pragma unroll
+        for (int hh = 0; hh < G; hh++) {
+#pragma unroll
+            for (int m = 0; m < 16; m++) {
+                _Float16 hi, lo;
+                split2(x[hh][m], hi, lo);
+                m_lds(hh)[(4 * m + q) * TROW + c] = hi, m_lds(hh)[C * TROW + (4 * m + q) * TROW + c] = lo;
+            }
         }
     }
     __syncthreads();
-    {
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(t_lds);
-        u32x4 *dst = reinterpret_cast<u32x4 *>(ws_v);
+#pragma unroll
+    for (int hh = 0; hh < G; hh++) {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(m_lds(hh));
+        u32x4 *dst = reinterpret_cast<u32x4 *>(ws_v(hh));
         for (uint32_t i = tid; i < 2 * T_IMG / 16; i += 256) dst[i] = src[i];
     }
 }
@@ -531,8 +568,12 @@ std::mutex g_owned_mutex;
 }  // namespace
 
 int setup_deltanet_chunk() {
-    if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(deltanet_chunk_prepare_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, PREP_LDS))) {
+    if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(deltanet_chunk_prepare_kernel<1>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, PrepLds<1>::BYTES))) {
+        return rc;
+    }
+    if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(deltanet_chunk_prepare_kernel<2>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, PrepLds<2>::BYTES))) {
         return rc;
     }
     return int(hipFuncSetAttribute(reinterpret_cast<const void *>(deltanet_chunk_chain_kernel),
@@ -549,7 +590,11 @@ int run_deltanet_chunk(hipStream_t stream, const float *mixed, const float *a, c
                        void *workspace) {
     const uint32_t nblocks = (p.tokens + C - 1) / C;
     ChunkArgs args{mixed, a, b, a_log, dt_bias, state, o, static_cast<unsigned char *>(workspace), p.k_heads, p.v_heads, p.v_dim, p.tokens, channels, p.eps};
-    deltanet_chunk_prepare_kernel<<<dim3(nblocks, p.v_heads), 256, PREP_LDS, stream>>>(args);
+    if (p.v_heads == 2 * p.k_heads) {
+        deltanet_chunk_prepare_kernel<2><<<dim3(nblocks, p.k_heads), 256, PrepLds<2>::BYTES, stream>>>(args);
+    } else {
+        deltanet_chunk_prepare_kernel<1><<<dim3(nblocks, p.v_heads), 256, PrepLds<1>::BYTES, stream>>>(args);
+    }
     deltanet_chunk_chain_kernel<<<dim3(p.v_dim / DV, p.v_heads), 256, ChainLds::BYTES, stream>>>(args);
     return SAETTA_OK;
 }
