@@ -1412,6 +1412,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
         auto row_of = [&](int pair, int half) { return min(2 * pair + half, M - 1); };
         const uint32_t base = blk_begin * BLOCK;
         const bool extra = range >= uint32_t(RBK);  // the round has block 16
+        const uint32_t live_blocks = (range + 1) & ~1u;  // k-steps are two blocks: the blocks of the k-steps that have tokens
 
         half8 q_hi[8], q_lo[8], qz_reg[2];
         {
@@ -1466,6 +1467,12 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
             for (int i = 0; i < A_BLOCKS; i++) {
                 const int blk = wt + WT * i;
                 if (blk >= (extra ? RBK : RBK - 1)) break;
+                if (uint32_t(blk) >= live_blocks) {
+                    // (a short share: no scores to take, and no operands will be made of this block; the other
+                    // pair's wave of the same blocks leaves it out as well)
+                    if (j == 0) bmax_lds[my_row * W::BROW + (n & 7) * W::BSTRIDE + blk] = NO_SCORE, bsum_lds[my_row * W::BROW + (n & 7) * W::BSTRIDE + blk] = 0.0f;
+                    continue;
+                }
                 await(W::C_KPART + (blk >> 3), W::K_LOADERS);  // this part of the keys is in LDS (first: and the scales)
                 const unsigned char *kb = lds_raw + W::K_OFF + blk * W::K_BLOCK_BYTES;
                 KeyRegs<BITS> kreg[4];
@@ -1523,6 +1530,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
                 // two pairs the other pair's wave of the same blocks, which takes them in the same order
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 if constexpr (PAIRS > 1) {
+                    // (the blocks a wave leaves out are its last ones: i counts the ones it takes)
                     raise(W::C_MERGE + wt);
                     await(W::C_MERGE + wt, PAIRS * (i + 1));
                 }
@@ -1542,7 +1550,8 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
         half8 p_hi[PAIRS][W::SLOTS], p_lo[PAIRS][W::SLOTS];
 #pragma unroll
         for (int sl = 0; sl < W::SLOTS; sl++) {
-            if (sl == 4 && !fifth) {
+            // (no block 16 | a short share: the k-step has no tokens)
+            if ((sl == 4 && !fifth) || uint32_t(2 * (2 * sl + b2)) >= range) {
 #pragma unroll
                 for (int p = 0; p < PAIRS; p++) p_hi[p][sl] = p_lo[p][sl] = half8{0, 0, 0, 0, 0, 0, 0, 0};
                 continue;
@@ -1603,7 +1612,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
         }
 #pragma unroll
         for (int sl = 0; sl < W::SLOTS; sl++) {
-            if (sl == 4 && !fifth) continue;
+            if ((sl == 4 && !fifth) || uint32_t(2 * (2 * sl + b2)) >= range) continue;
             await(W::C_SLOT + sl, W::V_LOADERS);  // value slot sl is in LDS
             ValRegs<BITS> vreg;
             read_values(sl == 4 ? 8 : 2 * sl + b2, g, vreg);
@@ -1719,6 +1728,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
             const bool more = round + 1 < n_rounds;
             const bool extra = nb == uint32_t(RBK);  // the round has block 16
             const uint32_t round_limit = min(limit, base + nb * BLOCK);  // tokens of this round end here
+            const uint32_t live_blocks = (nb + 1) & ~1u;  // k-steps are two blocks: the blocks of the k-steps that have tokens
 
             // ---- phase A: scores of blocks wave, wave + 8 (and wave 0: 16) --------------------------
             // (the query operands are read again in every round: they are not needed between the scores
@@ -1732,8 +1742,13 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
                 const int parts = (wave == 0 && extra) ? 3 : 2;
 #pragma unroll 1
                 for (int part = 0; part < parts; part++) {
-                    await(W::C_KPART + part, W::K_LOADERS * (round + 1));  // this part of the keys is in LDS (first: and the scales)
                     const int blk = wave + 8 * part;
+                    if (uint32_t(blk) >= live_blocks) {
+                        // (a short round: no scores to take, and no operands will be made of this block)
+                        if (j == 0 && n < 8) bmax_lds[n * W::BSTRIDE + blk] = NO_SCORE, bsum_lds[n * W::BSTRIDE + blk] = 0.0f;
+                        continue;
+                    }
+                    await(W::C_KPART + part, W::K_LOADERS * (round + 1));  // this part of the keys is in LDS (first: and the scales)
                     const unsigned char *kb = lds_raw + W::K_OFF + blk * W::K_BLOCK_BYTES;
                     KeyRegs<BITS> kreg[4];
 #pragma unroll
@@ -1847,7 +1862,8 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
                 const bool fifth = extra && b2 == 0;  // k-step 8: block 16 (lane groups 0 and 1; the others repeat them with factor 0)
 #pragma unroll
                 for (int sl = 0; sl < W::SLOTS; sl++) {
-                    if (sl == 4 && !fifth) {
+                    // (no block 16 | a short round: the k-step has no tokens)
+                    if ((sl == 4 && !fifth) || uint32_t(2 * (2 * sl + b2)) >= nb) {
                         p_op[sl] = half8{0, 0, 0, 0, 0, 0, 0, 0};
                         continue;
                     }
@@ -1907,7 +1923,9 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
                 }
             };
             const bool fifth = extra && b2 == 0;
-            if (peek(W::C_SLOT + 3) >= W::V_LOADERS * (round + 1)) {
+            // (a short round: not every k-step of this wave has tokens)
+            auto has_tokens = [&](int sl) { return uint32_t(2 * (2 * sl + b2)) < nb; };
+            if (nb >= 16 && peek(W::C_SLOT + 3) >= W::V_LOADERS * (round + 1)) {
                 // slots 0-3 are there already (the slots land in order): every read at once
                 ValRegs<BITS> vreg[4];
 #pragma unroll
@@ -1917,6 +1935,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
             } else {
 #pragma unroll
                 for (int sl = 0; sl < 4; sl++) {
+                    if (!has_tokens(sl)) continue;
                     await(W::C_SLOT + sl, W::V_LOADERS * (round + 1));  // value slot sl is in LDS
                     ValRegs<BITS> vreg;
                     read_values(sl, vreg);
