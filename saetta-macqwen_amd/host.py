@@ -156,6 +156,9 @@ class Built:
         waiting: the stream orders what follows, as for any torch op.  Built::commit
         (src/plan.rs:254-256) without the Pending; `run_timed` is the reference's waiting `run`."""
         if self.graph is not None:
+            # a captured graph replays on torch's current stream: another stream is the caller's to make current
+            if stream is not None and stream.cuda_stream != torch.cuda.current_stream().cuda_stream:
+                raise ValueError("Built.run: a captured plan replays on the current stream; make the stream current instead of passing it")
             self.graph.replay()
             return
         s = _stream(stream)
@@ -669,6 +672,7 @@ class AttentionRows:
         if m > self.rows or len(params) < m:
             raise ValueError("AttentionRows.record: too many rows")
         _need(q, torch.float32, "q"), _need(keys, torch.float16, "keys"), _need(values, torch.float16, "values")
+        _need(q_and_gate, torch.float32, "q_and_gate"), _need(out, torch.float32, "out")
         p, tp, po, pml = self._params(m), params[0], self.part_o, self.part_ml
 
         def launch(stage):
@@ -685,6 +689,7 @@ class AttentionRows:
             raise ValueError("AttentionRows.record_quant: too many rows")
         if keys.bits is KvBits.Half:
             raise ValueError("a half cache goes through record")
+        _need(q, torch.float32, "q"), _need(q_and_gate, torch.float32, "q_and_gate"), _need(out, torch.float32, "out")
         p, tp, po, pml, bits = self._params(m), params[0], self.part_o, self.part_ml, keys.bits.value
         kc, vc = keys.c(), values.c()
 

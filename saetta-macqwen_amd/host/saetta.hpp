@@ -130,7 +130,14 @@ class Built {
         gpu.sync();
         hipGraph_t g = nullptr;
         hip_check(hipStreamBeginCapture(gpu.stream(), hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
-        for (auto &op : ops_) op.second(gpu.stream());
+        try {
+            for (auto &op : ops_) op.second(gpu.stream());
+        } catch (...) {
+            // an op that refuses its arguments must not leave the stream capturing
+            (void)hipStreamEndCapture(gpu.stream(), &g);
+            if (g) (void)hipGraphDestroy(g);
+            throw;
+        }
         hip_check(hipStreamEndCapture(gpu.stream(), &g), "hipStreamEndCapture");
         hipGraphExec_t e = nullptr;
         hip_check(hipGraphInstantiate(&e, g, nullptr, nullptr, 0), "hipGraphInstantiate");
@@ -188,12 +195,29 @@ class Built {
 // TokenParams buffer, which the kernels read when they run.
 class Plan {
   public:
-    explicit Plan(const gpu::Gpu &gpu) : params(gpu.buffer(sizeof(TokenParams))), gpu_(gpu) {}
+    explicit Plan(const gpu::Gpu &gpu) : params(gpu.buffer(sizeof(TokenParams))), gpu_(gpu) {
+        // set_params copies from pinned memory, so that the copy is ordered by the stream and needs no wait:
+        // a ring of slots, each guarded by the event of the copy that last read it
+        TokenParams *ring = nullptr;
+        hip_check(hipHostMalloc(reinterpret_cast<void **>(&ring), RING * sizeof(TokenParams), hipHostMallocDefault), "hipHostMalloc");
+        ring_ = std::shared_ptr<TokenParams>(ring, [](TokenParams *x) { (void)hipHostFree(x); });
+        for (int i = 0; i < RING; i++) {
+            hipEvent_t e = nullptr;
+            hip_check(hipEventCreateWithFlags(&e, hipEventDisableTiming), "hipEventCreate");
+            read_[i] = std::shared_ptr<ihipEvent_t>(e, [](hipEvent_t x) { (void)hipEventDestroy(x); });
+        }
+    }
     View params;
     void op(std::string kernel, std::function<void(hipStream_t)> launch) { ops_.emplace_back(std::move(kernel), std::move(launch)); }
+    // Plan::set_params (src/plan.rs:144-146): a small copy on the stream, in order with the runs around it.
     void set_params(TokenParams tp) {
-        hip_check(hipMemcpyAsync(params.ptr<void>(), &tp, sizeof tp, hipMemcpyHostToDevice, gpu_.stream()), "set_params");
-        gpu_.sync();
+        const int slot = next_;
+        next_ = (next_ + 1) % RING;
+        if (used_[slot]) hip_check(hipEventSynchronize(read_[slot].get()), "hipEventSynchronize");  // (RING copies ago: long done)
+        ring_.get()[slot] = tp;
+        hip_check(hipMemcpyAsync(params.ptr<void>(), ring_.get() + slot, sizeof tp, hipMemcpyHostToDevice, gpu_.stream()), "set_params");
+        hip_check(hipEventRecord(read_[slot].get(), gpu_.stream()), "hipEventRecord");
+        used_[slot] = true;
     }
     const gpu::Gpu &gpu() const { return gpu_; }
     size_t len() const { return ops_.size(); }
@@ -237,6 +261,11 @@ class Plan {
   private:
     std::vector<std::pair<std::string, std::function<void(hipStream_t)>>> ops_;
     const gpu::Gpu &gpu_;
+    static constexpr int RING = 8;
+    std::shared_ptr<TokenParams> ring_;
+    std::shared_ptr<ihipEvent_t> read_[RING];
+    bool used_[RING] = {};
+    int next_ = 0;
 };
 
 }  // namespace plan

@@ -94,6 +94,27 @@ int main() {
             compare(second, x, 60, bits);
             const View c = plan.constant(std::vector<float>{1.5f, 2.5f});
             EXPECT(gpu::contents<float>(c.buffer, 2) == (std::vector<float>{1.5f, 2.5f}), "Plan::constant");
+            // set_params is ordered by the stream without a wait: many positions back to back, the last one counts
+            for (uint32_t pos = 0; pos < 40; pos++) {
+                plan.set_params(plan::token_params(0, pos % 60));
+                graph.commit(gpu);
+            }
+            gpu.sync();
+            compare(second, x, 39, bits);
+            // an op that throws while the plan is captured leaves the stream usable
+            plan::Plan bad(gpu);
+            second.record(bad, xb);
+            bad.op("throws", [](hipStream_t) { throw std::runtime_error("refused"); });
+            bool thrown = false;
+            try {
+                bad.build(true);
+            } catch (const std::runtime_error &) {
+                thrown = true;
+            }
+            EXPECT(thrown, "an op's exception comes out of Plan::build");
+            plan.set_params(plan::token_params(0, 33));
+            graph.run(gpu);
+            compare(second, x, 33, bits);
         }
         {  // dequantize_matches_cpu
             const size_t tokens = 9;

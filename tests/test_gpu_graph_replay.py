@@ -110,3 +110,10 @@ def test_serial_and_replay_agree_on_a_chain():
     assert bool((data == 3307.0).all())
     two = plan.constant([1.5, 2.5])
     assert two.is_cuda and two.tolist() == [1.5, 2.5]
+    # a captured plan replays on the current stream: naming another one is refused, not ignored
+    other = torch.cuda.Stream()
+    with pytest.raises(ValueError, match="current stream"):
+        built.run(other)
+    built.run(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    assert bool((data == 4307.0 + 100.0).all())
