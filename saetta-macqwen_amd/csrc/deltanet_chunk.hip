@@ -322,7 +322,17 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
     using L = ChainLds;
     constexpr int NT = DV / 16;  // 16-wide tiles of value dims
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    const uint32_t slice = blockIdx.x, h = blockIdx.y, group = a.v_heads / a.k_heads, khd = h / group;
+    // Workgroups go to the 8 XCDs in turn, and each XCD has its own L2: workgroup w of the launch runs on
+    // XCD w % 8.  The slices of a value head, and the value heads of a key head, read the same images, so
+    // they are given to one XCD (v_heads / 8 value heads each, where that divides): five times less
+    // traffic between the L2s and memory than with a head's slices dealt over all of them.
+    const uint32_t slices = a.v_dim / DV;
+    uint32_t slice = blockIdx.x % slices, h = blockIdx.x / slices;
+    if (a.v_heads % 8 == 0) {
+        const uint32_t xcd = blockIdx.x % 8, at = blockIdx.x / 8;  // at: the XCD's workgroups in order
+        h = xcd * (a.v_heads / 8) + at / slices, slice = at % slices;
+    }
+    const uint32_t group = a.v_heads / a.k_heads, khd = h / group;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), n = lane & 15, j = lane >> 4;
     const uint32_t nblocks = (a.tokens + C - 1) / C;
     const size_t per_block = block_bytes(a.k_heads, a.v_heads);
@@ -595,7 +605,7 @@ int run_deltanet_chunk(hipStream_t stream, const float *mixed, const float *a, c
     } else {
         deltanet_chunk_prepare_kernel<1><<<dim3(nblocks, p.v_heads), 256, PrepLds<1>::BYTES, stream>>>(args);
     }
-    deltanet_chunk_chain_kernel<<<dim3(p.v_dim / DV, p.v_heads), 256, ChainLds::BYTES, stream>>>(args);
+    deltanet_chunk_chain_kernel<<<dim3(p.v_dim / DV * p.v_heads), 256, ChainLds::BYTES, stream>>>(args);
     return SAETTA_OK;
 }
 
