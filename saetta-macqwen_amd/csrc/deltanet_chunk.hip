@@ -39,21 +39,26 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int K_DIM = 128;
 constexpr int C = 64;                 // tokens per block
-constexpr int KROW = K_DIM + 8;       // f16 per row of a q / k image: 272 bytes, so that 16 rows' 16-byte reads fall on all banks
-constexpr int TROW = C + 8;           // f16 per row of a T / M image: 144 bytes, likewise
-constexpr int K_IMG = C * KROW * 2;   // bytes: 17408 = 17 load instructions of 1 KB
-constexpr int T_IMG = C * TROW * 2;   // bytes: 9216 = 9 load instructions
-constexpr int KTROW = C + 8;          // f16 per row of the keys' image by key dim, [128][72]
-constexpr int X_IMG = K_DIM * KTROW * 2;  // bytes: 18432 = 18 load instructions
 constexpr int DV = 16;                // value dims per workgroup of the chain kernel (32: 317 against 253 us per 4096 tokens)
 constexpr float Q_SCALE = 0.08838834764831845f;  // 1 / sqrt(128), the reference's factor on q
-static_assert(K_IMG % 1024 == 0 && T_IMG % 1024 == 0, "images are whole load instructions");
+// LDS images of the prepare kernel: rows padded so that 16 rows' 16-byte reads fall on all banks
+constexpr int KROW = K_DIM + 8;       // f16 per row of a q / k image: 272 bytes
+constexpr int TROW = C + 8;           // f16 per row of a T / M image (and of the chain's [dv][token] images): 144 bytes
+constexpr int K_IMG = C * KROW * 2;   // bytes: 17408
+constexpr int T_IMG = C * TROW * 2;   // bytes: 9216
 
-// Workspace, per block: per key head the images kh | kl | qh | ql and the keys by key dim xh | xl, then
-// per value head th | tl | mh | ml and 128 floats: e^{c_t} and e^{c_last - c_t}.
-static_assert(X_IMG % 1024 == 0, "images are whole load instructions");
-constexpr size_t KHEAD_BYTES = 4 * size_t(K_IMG) + 2 * size_t(X_IMG);
-constexpr size_t VHEAD_BYTES = 4 * size_t(T_IMG) + 2 * C * sizeof(float);
+// Workspace, per block.  Everything the chain kernel reads lies in the order its waves take it as MFMA
+// operands: an operand of a wave is 64 lanes x 16 bytes = 1 KB (lane (n, j): row or column n, 8 values of
+// the k index from 8j), so a load instruction of a wave reads one contiguous kilobyte.
+//   per key head:   K hi | K lo | Q hi | Q lo   [wave 4][k-step 4][lane]: row 16 wave + n, key dims 32 ks + 8j ..
+//                   X hi | X lo                 [wave 4][nt 2][k-step 2][lane]: the keys by key dim, column
+//                                               32 wave + 16 nt + n, tokens 32 ks + 8j ..
+//   per value head: T hi | T lo | M hi | M lo   [wave 4][k-step 2][lane]: row 16 wave + n, columns 32 ks + 8j ..
+//                   128 floats: e^{c_t} and e^{c_last - c_t}
+constexpr int OPERAND = 1024;
+constexpr int K_GL = 4 * 4 * OPERAND, X_GL = 4 * 2 * 2 * OPERAND, T_GL = 4 * 2 * OPERAND;
+constexpr size_t KHEAD_BYTES = 4 * size_t(K_GL) + 2 * size_t(X_GL);
+constexpr size_t VHEAD_BYTES = 4 * size_t(T_GL) + 2 * C * sizeof(float);
 __host__ __device__ inline size_t block_bytes(uint32_t k_heads, uint32_t v_heads) { return k_heads * KHEAD_BYTES + v_heads * VHEAD_BYTES; }
 
 struct ChunkArgs {
@@ -155,9 +160,10 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
             *reinterpret_cast<half8 *>(kh + at) = a_kh, *reinterpret_cast<half8 *>(kl + at) = a_kl;
             *reinterpret_cast<half8 *>(qh + at) = a_qh, *reinterpret_cast<half8 *>(ql + at) = a_ql;
             if (writer) {
-                _Float16 *g = reinterpret_cast<_Float16 *>(ws_k) + at;
-                *reinterpret_cast<half8 *>(g) = a_kh, *reinterpret_cast<half8 *>(g + C * KROW) = a_kl;
-                *reinterpret_cast<half8 *>(g + 2 * C * KROW) = a_qh, *reinterpret_cast<half8 *>(g + 3 * C * KROW) = a_ql;
+                // operand (wave t / 16, k-step part), lane (n = t % 16, j = i / 2)
+                unsigned char *g = ws_k + ((((t >> 4) * 4 + part) * 64 + (i >> 1) * 16 + (t & 15)) * 16);
+                *reinterpret_cast<half8 *>(g) = a_kh, *reinterpret_cast<half8 *>(g + K_GL) = a_kl;
+                *reinterpret_cast<half8 *>(g + 2 * K_GL) = a_qh, *reinterpret_cast<half8 *>(g + 3 * K_GL) = a_ql;
             }
         }
     }
@@ -178,7 +184,7 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
         }
         cum_lds(wave)[lane] = c, beta_lds(wave)[lane] = beta;
         const float last = __shfl(c, 63, 64);
-        float *gam = reinterpret_cast<float *>(ws_v(wave) + 4 * T_IMG);
+        float *gam = reinterpret_cast<float *>(ws_v(wave) + 4 * T_GL);
         gam[lane] = __expf(c), gam[C + lane] = __expf(last - c);
     }
     __syncthreads();
@@ -200,8 +206,9 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
     }
     // ---- the keys once more by key dim: [128][72] hi | lo, what the state's update contracts over tokens ----
     if (writer) {
+        // thread: key dim dk, tokens 32 half ..: operand (wave dk / 32, nt (dk / 16) % 2, k-step half), lanes (n = dk % 16, j = part)
         const uint32_t dk = tid >> 1, half = tid & 1;
-        _Float16 *g = reinterpret_cast<_Float16 *>(ws_k + 4 * K_IMG) + dk * KTROW + 32 * half;
+        unsigned char *g = ws_k + 4 * K_GL + ((((dk >> 5) * 2 + ((dk >> 4) & 1)) * 2 + half) * 64 + (dk & 15)) * 16;
 #pragma unroll
         for (int part = 0; part < 4; part++) {
             half8 vh, vl;
@@ -210,8 +217,8 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
                 const int at = (32 * half + 8 * part + e) * KROW + dk;
                 vh[e] = kh[at], vl[e] = kl[at];
             }
-            *reinterpret_cast<half8 *>(g + 8 * part) = vh;
-            *reinterpret_cast<half8 *>(g + K_DIM * KTROW + 8 * part) = vl;
+            *reinterpret_cast<half8 *>(g + part * 256) = vh;
+            *reinterpret_cast<half8 *>(g + X_GL + part * 256) = vl;
         }
     }
     __syncthreads();  // the images are read: A and M go over them
@@ -235,13 +242,16 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
         }
     }
     __syncthreads();
-    // M leaves (whole 16-byte pieces; the padding columns go along)
+    // A staged matrix leaves in operand order, 16 bytes per piece: piece (part hi | lo, wave w, k-step ks, lane (n, j))
+    // is row 16 w + n, columns 32 ks + 8j .. of the part's image
+    auto leave = [&](int hh, unsigned char *dst) {
+        for (uint32_t i = tid; i < 2 * T_GL / 16; i += 256) {
+            const uint32_t part = i >> 9, w = (i >> 7) & 3, ks = (i >> 6) & 1, nn = i & 15, jj = (i >> 4) & 3;
+            reinterpret_cast<u32x4 *>(dst)[i] = *reinterpret_cast<const u32x4 *>(m_lds(hh) + part * C * TROW + (16 * w + nn) * TROW + 32 * ks + 8 * jj);
+        }
+    };
 #pragma unroll
-    for (int hh = 0; hh < G; hh++) {
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(m_lds(hh));
-        u32x4 *dst = reinterpret_cast<u32x4 *>(ws_v(hh) + 2 * T_IMG);
-        for (uint32_t i = tid; i < 2 * T_IMG / 16; i += 256) dst[i] = src[i];
-    }
+    for (int hh = 0; hh < G; hh++) leave(hh, ws_v(hh) + 2 * T_GL);
 
     // ---- T = (I + A)^-1 diag(beta): column c = 16 wave + n by forward substitution, x_t = beta_t [t = c] -
     // sum_{s < t} A_ts x_s; lane group q keeps x_s of s = 4m + q in slot m and adds up those s.  The heads'
@@ -290,24 +300,18 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
     }
     __syncthreads();
 #pragma unroll
-    for (int hh = 0; hh < G; hh++) {
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(m_lds(hh));
-        u32x4 *dst = reinterpret_cast<u32x4 *>(ws_v(hh));
-        for (uint32_t i = tid; i < 2 * T_IMG / 16; i += 256) dst[i] = src[i];
-    }
+    for (int hh = 0; hh < G; hh++) leave(hh, ws_v(hh));
 }
 
 // ---- the chain over the blocks --------------------------------------------------------------------
 // Per block, with S0 [dv][128] the state's slice: P = K S0^T and Q S0^T (rows: tokens); R = V - e^c P;
 // U = T R; O = (e^c (Q S0^T) + M U) / sqrt(128); S1 = e^{c_last} S0 + (e^{c_last - c} U)^T K.
-// The images of the next block are requested as soon as their place is free: k and q (rows: tokens)
-// once every wave has R, the keys by key dim once every wave has the new state; T and M, which a
-// wave needs 16 rows of, come a block ahead straight into registers.  The loads of the loop are inline
-// assembly and waited for by hand.
+// A wave takes 16 tokens' rows of K, Q, T and M and 32 key dims' columns of the keys by key dim, and nobody
+// else reads those: they come from the workspace straight into its registers, a whole block ahead, as
+// the MFMA operands they are.  LDS holds what the waves hand to each other: the state's image, R, U and
+// the scaled U, and the block's values and decay factors.
 struct ChainLds {
-    static constexpr int KH = 0, KL = KH + K_IMG, QH = KL + K_IMG, QL = QH + K_IMG;
-    static constexpr int XH = QL + K_IMG, XL = XH + X_IMG;  // the keys by key dim: [128][KTROW] f16
-    static constexpr int GAM = XL + X_IMG;                 // e^{c_t}, e^{c_last - c_t}: 128 f32
+    static constexpr int GAM = 0;                          // e^{c_t}, e^{c_last - c_t}: 128 f32
     static constexpr int V = GAM + 2 * C * 4;              // [token][DV] f32
     static constexpr int SROW = K_DIM + 8;                 // f16 per row of the state's operand image [dv][128]
     static constexpr int SH = V + C * DV * 4, SL = SH + DV * SROW * 2;
@@ -315,17 +319,26 @@ struct ChainLds {
     static constexpr int RL = RH + DV * TROW * 2, UH = RL + DV * TROW * 2, UL = UH + DV * TROW * 2;
     static constexpr int WH = UL + DV * TROW * 2, WL = WH + DV * TROW * 2;
     static constexpr int BYTES = WL + DV * TROW * 2;
-    static_assert(BYTES <= 160 * 1024, "LDS of a CU");
+};
+
+// What a wave reads of a block: 32 operands and, for the workgroup, its share of the block's values and factors.
+struct ChainBlock {
+    u32x4 k[2][4], q[2][4];  // [hi | lo][k-step]: rows 16 wave + n of K and Q
+    u32x4 x[2][2][2];        // [hi | lo][nt][k-step]: columns 32 wave + 16 nt + n of the keys by key dim
+    u32x4 tm[2][2][2];       // [T | M][hi | lo][k-step]: rows 16 wave + n
+    static constexpr int V_LOADS = C * DV * 4 / 16 / 256;  // 16-byte pieces per thread of the block's [token][DV] values
+    u32x4 v[V_LOADS], gam;   // ...; 16 bytes of the 128 factors (threads 0-31)
 };
 
 __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) {
     using L = ChainLds;
     constexpr int NT = DV / 16;  // 16-wide tiles of value dims
+    constexpr int V_LOADS = ChainBlock::V_LOADS;
+    static_assert(V_LOADS >= 1 && V_LOADS * 256 * 16 == C * DV * 4, "whole 16-byte pieces of the block's values per thread");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     // Workgroups go to the 8 XCDs in turn, and each XCD has its own L2: workgroup w of the launch runs on
-    // XCD w % 8.  The slices of a value head, and the value heads of a key head, read the same images, so
-    // they are given to one XCD (v_heads / 8 value heads each, where that divides): five times less
-    // traffic between the L2s and memory than with a head's slices dealt over all of them.
+    // XCD w % 8.  The slices of a value head, and the value heads of a key head, read the same operands, so
+    // they are given to one XCD (v_heads / 8 value heads each, where that divides).
     const uint32_t slices = a.v_dim / DV;
     uint32_t slice = blockIdx.x % slices, h = blockIdx.x / slices;
     if (a.v_heads % 8 == 0) {
@@ -336,73 +349,52 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), n = lane & 15, j = lane >> 4;
     const uint32_t nblocks = (a.tokens + C - 1) / C;
     const size_t per_block = block_bytes(a.k_heads, a.v_heads);
-    const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(lds));
     auto img = [&](int off) { return reinterpret_cast<const _Float16 *>(lds + off); };
     auto img_w = [&](int off) { return reinterpret_cast<_Float16 *>(lds + off); };
     const float *gam = reinterpret_cast<const float *>(lds + L::GAM);
     float *v_lds = reinterpret_cast<float *>(lds + L::V);
 
-    // `pieces` KB from global memory straight into LDS, the waves taking 1 KB pieces in turn
-    auto copy_in = [&](int lds_off, const unsigned char *src, int pieces) {
-        for (int i = wave; i < pieces; i += 4) {
-            asm volatile("s_mov_b32 m0, %0\n"
-                         "s_nop 0\n"
-                         "global_load_lds_dwordx4 %1, %2\n"
-                         :
-                         : "s"(lds0 + lds_off + i * 1024), "v"(uint32_t(i * 1024 + lane * 16)), "s"(src)
-                         : "memory", "m0");
-        }
-    };
-    auto load16 = [&](const void *p) {
-        u32x4 v;
-        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
-        return v;
-    };
-    auto ws_k_of = [&](uint32_t blk) { return a.ws + size_t(blk) * per_block + khd * KHEAD_BYTES; };
-    auto ws_v_of = [&](uint32_t blk) { return a.ws + size_t(blk) * per_block + a.k_heads * KHEAD_BYTES + h * VHEAD_BYTES; };
-    constexpr int KQ_PIECES = 4 * K_IMG / 1024, X_PIECES = 2 * X_IMG / 1024;
-    static_assert(KQ_PIECES % 4 == 0 && X_PIECES == 36, "pieces per wave");
-    constexpr int V_LOADS = C * DV * 4 / 16 / 256;  // 16-byte loads per thread of the block's values
-
-    // T and M: this wave's rows 16 wave + n, columns 32 ks + 8j .. + 7, hi and lo: operands as they are.
-    // (The registers an assembly load fills are handed on only behind the wait that names them, in the
-    // same straight piece of code: the compiler takes them for ready from the load on.)
-    u32x4 tm[8];
-    auto request_ahead = [&](uint32_t blk, u32x4 (&tm_next)[8], u32x4 (&v_next)[V_LOADS], u32x4 &gam_next) {
-        copy_in(L::KH, ws_k_of(blk), KQ_PIECES);
-        const unsigned char *wv = ws_v_of(blk);
+    auto request = [&](uint32_t blk, ChainBlock &b) {
+        const u32x4 *wk = reinterpret_cast<const u32x4 *>(a.ws + size_t(blk) * per_block + khd * KHEAD_BYTES);
+        const u32x4 *wv = reinterpret_cast<const u32x4 *>(a.ws + size_t(blk) * per_block + a.k_heads * KHEAD_BYTES + h * VHEAD_BYTES);
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            // i: matrix (T | M) * 4 + part (hi | lo) * 2 + k-step
-            tm_next[i] = load16(wv + (i >> 1) * T_IMG + ((16 * wave + n) * TROW + 32 * (i & 1) + 8 * j) * 2);
+        for (int part = 0; part < 2; part++) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                b.k[part][ks] = wk[(part * K_GL) / 16 + (wave * 4 + ks) * 64 + lane];
+                b.q[part][ks] = wk[((2 + part) * K_GL) / 16 + (wave * 4 + ks) * 64 + lane];
+            }
+#pragma unroll
+            for (int nt = 0; nt < 2; nt++) {
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) b.x[part][nt][ks] = wk[(4 * K_GL + part * X_GL) / 16 + ((wave * 2 + nt) * 2 + ks) * 64 + lane];
+            }
+#pragma unroll
+            for (int m = 0; m < 2; m++) {
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) {
+                    // (T and M are lower triangular: rows 16 wave .. have nothing in columns 32 ks .. beyond their own)
+                    if (ks <= int(wave) / 2) b.tm[m][part][ks] = wv[((2 * m + part) * T_GL) / 16 + (wave * 2 + ks) * 64 + lane];
+                }
+            }
         }
 #pragma unroll
         for (int i = 0; i < V_LOADS; i++) {
-            // piece p of the block's [token][DV] values: token p / (DV / 4), four dims
-            const uint32_t p = tid + 256 * i, tok = min(blk * C + p / (DV / 4), a.tokens - 1);  // (a token past the end: unused, see below)
-            v_next[i] = load16(a.mixed + size_t(tok) * a.channels + 2 * a.k_heads * K_DIM + h * a.v_dim + DV * slice + 4 * (p % (DV / 4)));
+            // piece p of the block's [token][DV] values: token p / (DV / 4), four dims (a token past the end: unused, see `place`)
+            const uint32_t p = tid + 256 * i, tok = min(blk * C + p / (DV / 4), a.tokens - 1);
+            b.v[i] = *reinterpret_cast<const u32x4 *>(a.mixed + size_t(tok) * a.channels + 2 * a.k_heads * K_DIM + h * a.v_dim + DV * slice + 4 * (p % (DV / 4)));
         }
-        gam_next = load16(wv + 4 * T_IMG + 16 * (tid & 31));
+        b.gam = wv[(4 * T_GL) / 16 + (tid & 31)];
     };
-    auto place_ahead = [&](uint32_t blk, u32x4 (&tm_next)[8], u32x4 (&v_next)[V_LOADS], u32x4 &gam_next) {
-        // (nothing else is in flight: loads into registers and loads into LDS do not return in one order,
-        // so a count that leaves some of one kind in flight says nothing about the other kind)
-        if constexpr (V_LOADS == 1) {
-            asm volatile("s_waitcnt vmcnt(0)" : "+v"(tm_next[0]), "+v"(tm_next[1]), "+v"(tm_next[2]), "+v"(tm_next[3]), "+v"(tm_next[4]),
-                         "+v"(tm_next[5]), "+v"(tm_next[6]), "+v"(tm_next[7]), "+v"(v_next[0]), "+v"(gam_next)::"memory");
-        } else {
-            asm volatile("s_waitcnt vmcnt(0)" : "+v"(tm_next[0]), "+v"(tm_next[1]), "+v"(tm_next[2]), "+v"(tm_next[3]), "+v"(tm_next[4]),
-                         "+v"(tm_next[5]), "+v"(tm_next[6]), "+v"(tm_next[7]), "+v"(v_next[0]), "+v"(v_next[V_LOADS - 1]), "+v"(gam_next)::"memory");
-        }
-#pragma unroll
-        for (int i = 0; i < 8; i++) tm[i] = tm_next[i];
+    // the block's values (tokens past the end: zeros) and factors to LDS
+    auto place = [&](uint32_t blk, const ChainBlock &b) {
 #pragma unroll
         for (int i = 0; i < V_LOADS; i++) {
             const uint32_t p = tid + 256 * i;
             const bool real = blk * C + p / (DV / 4) < a.tokens;
-            reinterpret_cast<u32x4 *>(v_lds)[p] = real ? v_next[i] : u32x4{0, 0, 0, 0};
+            reinterpret_cast<u32x4 *>(v_lds)[p] = real ? b.v[i] : u32x4{0, 0, 0, 0};
         }
-        if (tid < 32) reinterpret_cast<u32x4 *>(lds + L::GAM)[tid] = gam_next;
+        if (tid < 32) reinterpret_cast<u32x4 *>(lds + L::GAM)[tid] = b.gam;
     };
 
     // ---- the state's slice: S [dv][128]; wave w keeps columns 32 w .. + 31: lane (n, j) the four rows
@@ -432,17 +424,12 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
             for (int i = 0; i < 4; i++) s_reg[mt][nt][i] = state[(16 * mt + 4 * j + i) * K_DIM + 32 * wave + 16 * nt + n];
         }
     }
-    publish_state();
-    {
-        u32x4 tm_next[8], v_next[V_LOADS], gam_next;
-        request_ahead(0, tm_next, v_next, gam_next);
-        place_ahead(0, tm_next, v_next, gam_next);
-        copy_in(L::XH, ws_k_of(0) + 4 * K_IMG, X_PIECES);
-    }
-
-    for (uint32_t blk = 0; blk < nblocks; blk++) {
-        const bool more = blk + 1 < nblocks;
-        __syncthreads();  // the block's k and q images, its values and factors and the state's image are in LDS
+    // One block: `cur` holds its operands; the next block's are asked for now, into `next`, and used a block
+    // later (after the last block: the last block's again, unused).
+    auto step = [&](uint32_t blk, const ChainBlock &cur, ChainBlock &next) {
+        const uint32_t nxt = blk + 1 < nblocks ? blk + 1 : blk;
+        request(nxt, next);
+        __syncthreads();  // the block's values and factors and the state's image are in LDS
 
         // ---- K S0^T and Q S0^T: rows t = 16 wave + n, columns dv = 16 vt + n' ----
         floatx4 pk[NT], pq[NT];
@@ -450,15 +437,12 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
         for (int vt = 0; vt < NT; vt++) pk[vt] = pq[vt] = floatx4{0, 0, 0, 0};
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-            const int ao = (16 * wave + n) * KROW + 32 * ks + 8 * j;
-            const half8 akh = *reinterpret_cast<const half8 *>(img(L::KH) + ao), akl = *reinterpret_cast<const half8 *>(img(L::KL) + ao);
-            const half8 aqh = *reinterpret_cast<const half8 *>(img(L::QH) + ao), aql = *reinterpret_cast<const half8 *>(img(L::QL) + ao);
 #pragma unroll
             for (int vt = 0; vt < NT; vt++) {
                 const int bo = (16 * vt + n) * L::SROW + 32 * ks + 8 * j;
                 const half8 bh = *reinterpret_cast<const half8 *>(img(L::SH) + bo), bl = *reinterpret_cast<const half8 *>(img(L::SL) + bo);
-                pk[vt] = mma3(akh, akl, bh, bl, pk[vt]);
-                pq[vt] = mma3(aqh, aql, bh, bl, pq[vt]);
+                pk[vt] = mma3(__builtin_bit_cast(half8, cur.k[0][ks]), __builtin_bit_cast(half8, cur.k[1][ks]), bh, bl, pk[vt]);
+                pq[vt] = mma3(__builtin_bit_cast(half8, cur.q[0][ks]), __builtin_bit_cast(half8, cur.q[1][ks]), bh, bl, pq[vt]);
             }
         }
         // C layout: lane (n, j) holds dv = 16 vt + n of tokens t = 16 wave + 4j + i
@@ -478,11 +462,7 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
             const int at = (16 * vt + n) * TROW + 16 * wave + 4 * j;
             *reinterpret_cast<half4 *>(img_w(L::RH) + at) = rh, *reinterpret_cast<half4 *>(img_w(L::RL) + at) = rl;
         }
-        __syncthreads();  // R is whole; the k and q images, the values and the factors are read
-        // the next block's (after the last block: the last block's again, unused)
-        const uint32_t nxt = more ? blk + 1 : blk;
-        u32x4 tm_next[8], v_next[V_LOADS], gam_next;
-        request_ahead(nxt, tm_next, v_next, gam_next);
+        __syncthreads();  // R is whole
 
         // ---- U = T R (T is lower triangular: k-steps up to the row tile's own) ----
         floatx4 u[NT];
@@ -493,7 +473,7 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
             for (int ks = 0; ks < 2; ks++) {
                 if (ks > int(wave) / 2) continue;
                 const int bo = (16 * vt + n) * TROW + 32 * ks + 8 * j;
-                u[vt] = mma3(__builtin_bit_cast(half8, tm[0 + ks]), __builtin_bit_cast(half8, tm[2 + ks]),
+                u[vt] = mma3(__builtin_bit_cast(half8, cur.tm[0][0][ks]), __builtin_bit_cast(half8, cur.tm[0][1][ks]),
                              *reinterpret_cast<const half8 *>(img(L::RH) + bo), *reinterpret_cast<const half8 *>(img(L::RL) + bo), u[vt]);
             }
             half4 uh, ul, wh, wl;
@@ -509,10 +489,7 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
             *reinterpret_cast<half4 *>(img_w(L::UH) + at) = uh, *reinterpret_cast<half4 *>(img_w(L::UL) + at) = ul;
             *reinterpret_cast<half4 *>(img_w(L::WH) + at) = wh, *reinterpret_cast<half4 *>(img_w(L::WL) + at) = wl;
         }
-        // the keys by key dim are here when at most the images requested after them (loads into LDS return
-        // in order) are in flight
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(KQ_PIECES / 4) : "memory");
-        __syncthreads();  // U is whole, and so are the keys by key dim
+        __syncthreads();  // U is whole; every wave is through with the state's image, the values and the factors
 
         // ---- S1 = e^{c_last} S0 + (U scaled)^T K: rows dv, columns 32 wave + 16 nt + n, over the 64 tokens ----
 #pragma unroll
@@ -522,17 +499,19 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
             for (int mt = 0; mt < NT; mt++) acc[mt] = floatx4{0, 0, 0, 0};
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
-                const int bo = (32 * wave + 16 * nt + n) * KTROW + 32 * ks + 8 * j;
-                const half8 bh = *reinterpret_cast<const half8 *>(img(L::XH) + bo), bl = *reinterpret_cast<const half8 *>(img(L::XL) + bo);
 #pragma unroll
                 for (int mt = 0; mt < NT; mt++) {
                     const int ao = (16 * mt + n) * TROW + 32 * ks + 8 * j;
-                    acc[mt] = mma3(*reinterpret_cast<const half8 *>(img(L::WH) + ao), *reinterpret_cast<const half8 *>(img(L::WL) + ao), bh, bl, acc[mt]);
+                    acc[mt] = mma3(*reinterpret_cast<const half8 *>(img(L::WH) + ao), *reinterpret_cast<const half8 *>(img(L::WL) + ao),
+                                   __builtin_bit_cast(half8, cur.x[0][nt][ks]), __builtin_bit_cast(half8, cur.x[1][nt][ks]), acc[mt]);
                 }
             }
 #pragma unroll
             for (int mt = 0; mt < NT; mt++) s_reg[mt][nt] = s_reg[mt][nt] * glast + acc[mt];
         }
+        // the next block's state image, values and factors: their places were last read before the barrier above
+        publish_state();
+        place(nxt, next);
         // ---- O = (e^c (Q S0^T) + M U) / sqrt(128) ----
 #pragma unroll
         for (int vt = 0; vt < NT; vt++) {
@@ -541,7 +520,7 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
             for (int ks = 0; ks < 2; ks++) {
                 if (ks > int(wave) / 2) continue;
                 const int bo = (16 * vt + n) * TROW + 32 * ks + 8 * j;
-                mu = mma3(__builtin_bit_cast(half8, tm[4 + ks]), __builtin_bit_cast(half8, tm[6 + ks]),
+                mu = mma3(__builtin_bit_cast(half8, cur.tm[1][0][ks]), __builtin_bit_cast(half8, cur.tm[1][1][ks]),
                           *reinterpret_cast<const half8 *>(img(L::UH) + bo), *reinterpret_cast<const half8 *>(img(L::UL) + bo), mu);
             }
 #pragma unroll
@@ -550,12 +529,16 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
                 if (tok < a.tokens) a.o[(size_t(tok) * a.v_heads + h) * a.v_dim + DV * slice + 16 * vt + n] = Q_SCALE * (gam4[i] * pq[vt][i] + mu[i]);
             }
         }
-        __syncthreads();  // every wave is through with the keys by key dim, U and the state's image
-        publish_state();
-        place_ahead(nxt, tm_next, v_next, gam_next);
-        copy_in(L::XH, ws_k_of(nxt) + 4 * K_IMG, X_PIECES);
+    };
+    // (two sets of operand registers that change roles, so that nothing is copied from one to the other)
+    ChainBlock even, odd;
+    request(0, even);
+    publish_state();
+    place(0, even);
+    for (uint32_t blk = 0; blk < nblocks; blk += 2) {
+        step(blk, even, odd);
+        if (blk + 1 < nblocks) step(blk + 1, odd, even);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (nothing may land in LDS after the workgroup has ended)
 #pragma unroll
     for (int mt = 0; mt < NT; mt++) {
 #pragma unroll
