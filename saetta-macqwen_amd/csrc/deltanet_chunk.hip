@@ -36,6 +36,7 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int K_DIM = 128;
 constexpr int C = 64;                 // tokens per block
@@ -51,13 +52,11 @@ constexpr int T_IMG = C * TROW * 2;   // bytes: 9216
 // operands: an operand of a wave is 64 lanes x 16 bytes = 1 KB (lane (n, j): row or column n, 8 values of
 // the k index from 8j), so a load instruction of a wave reads one contiguous kilobyte.
 //   per key head:   K hi | K lo | Q hi | Q lo   [wave 4][k-step 4][lane]: row 16 wave + n, key dims 32 ks + 8j ..
-//                   X hi | X lo                 [wave 4][nt 2][k-step 2][lane]: the keys by key dim, column
-//                                               32 wave + 16 nt + n, tokens 32 ks + 8j ..
 //   per value head: T hi | T lo | M hi | M lo   [wave 4][k-step 2][lane]: row 16 wave + n, columns 32 ks + 8j ..
 //                   128 floats: e^{c_t} and e^{c_last - c_t}
 constexpr int OPERAND = 1024;
-constexpr int K_GL = 4 * 4 * OPERAND, X_GL = 4 * 2 * 2 * OPERAND, T_GL = 4 * 2 * OPERAND;
-constexpr size_t KHEAD_BYTES = 4 * size_t(K_GL) + 2 * size_t(X_GL);
+constexpr int K_GL = 4 * 4 * OPERAND, T_GL = 4 * 2 * OPERAND;
+constexpr size_t KHEAD_BYTES = 4 * size_t(K_GL);
 constexpr size_t VHEAD_BYTES = 4 * size_t(T_GL) + 2 * C * sizeof(float);
 __host__ __device__ inline size_t block_bytes(uint32_t k_heads, uint32_t v_heads) { return k_heads * KHEAD_BYTES + v_heads * VHEAD_BYTES; }
 
@@ -204,23 +203,6 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
             }
         }
     }
-    // ---- the keys once more by key dim: [128][72] hi | lo, what the state's update contracts over tokens ----
-    if (writer) {
-        // thread: key dim dk, tokens 32 half ..: operand (wave dk / 32, nt (dk / 16) % 2, k-step half), lanes (n = dk % 16, j = part)
-        const uint32_t dk = tid >> 1, half = tid & 1;
-        unsigned char *g = ws_k + 4 * K_GL + ((((dk >> 5) * 2 + ((dk >> 4) & 1)) * 2 + half) * 64 + (dk & 15)) * 16;
-#pragma unroll
-        for (int part = 0; part < 4; part++) {
-            half8 vh, vl;
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const int at = (32 * half + 8 * part + e) * KROW + dk;
-                vh[e] = kh[at], vl[e] = kl[at];
-            }
-            *reinterpret_cast<half8 *>(g + part * 256) = vh;
-            *reinterpret_cast<half8 *>(g + X_GL + part * 256) = vl;
-        }
-    }
     __syncthreads();  // the images are read: A and M go over them
 
     // C layout: lane (n, j) holds column s = 16 nt + n of rows t = 16 wave + 4j + i
@@ -306,10 +288,11 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
 // ---- the chain over the blocks --------------------------------------------------------------------
 // Per block, with S0 [dv][128] the state's slice: P = K S0^T and Q S0^T (rows: tokens); R = V - e^c P;
 // U = T R; O = (e^c (Q S0^T) + M U) / sqrt(128); S1 = e^{c_last} S0 + (e^{c_last - c} U)^T K.
-// A wave takes 16 tokens' rows of K, Q, T and M and 32 key dims' columns of the keys by key dim, and nobody
-// else reads those: they come from the workspace straight into its registers, a whole block ahead, as
-// the MFMA operands they are.  LDS holds what the waves hand to each other: the state's image, R, U and
-// the scaled U, and the block's values and decay factors.
+// A wave takes 16 tokens' rows of K, Q, T and M, and nobody else reads those: they come from the workspace
+// straight into its registers, a whole block ahead, as the MFMA operands they are.  LDS holds what the
+// waves hand to each other: the state's image, R, U and the scaled U, the block's values and decay
+// factors, and the block's keys, which the state's update contracts over the tokens: every wave puts
+// its rows there, and ds_read_b64_tr_b16 hands them out by key dim.
 struct ChainLds {
     static constexpr int GAM = 0;                          // e^{c_t}, e^{c_last - c_t}: 128 f32
     static constexpr int V = GAM + 2 * C * 4;              // [token][DV] f32
@@ -318,13 +301,15 @@ struct ChainLds {
     static constexpr int RH = SL + DV * SROW * 2;          // [dv][64 tokens] images, rows of TROW f16: R, U, U scaled
     static constexpr int RL = RH + DV * TROW * 2, UH = RL + DV * TROW * 2, UL = UH + DV * TROW * 2;
     static constexpr int WH = UL + DV * TROW * 2, WL = WH + DV * TROW * 2;
-    static constexpr int BYTES = WL + DV * TROW * 2;
+    // the block's keys [token][128] as hi and lo images, two sets for alternate blocks: every wave puts its 16
+    // rows there, and the state's update reads them by key dim (transposing reads)
+    static constexpr int KIMG = (WL + DV * TROW * 2 + 15) / 16 * 16;
+    static constexpr int BYTES = KIMG + 4 * K_IMG;
 };
 
-// What a wave reads of a block: 32 operands and, for the workgroup, its share of the block's values and factors.
+// What a wave reads of a block: 24 operands and, for the workgroup, its share of the block's values and factors.
 struct ChainBlock {
     u32x4 k[2][4], q[2][4];  // [hi | lo][k-step]: rows 16 wave + n of K and Q
-    u32x4 x[2][2][2];        // [hi | lo][nt][k-step]: columns 32 wave + 16 nt + n of the keys by key dim
     u32x4 tm[2][2][2];       // [T | M][hi | lo][k-step]: rows 16 wave + n
     static constexpr int V_LOADS = C * DV * 4 / 16 / 256;  // 16-byte pieces per thread of the block's [token][DV] values
     u32x4 v[V_LOADS], gam;   // ...; 16 bytes of the 128 factors (threads 0-31)
@@ -363,11 +348,6 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
             for (int ks = 0; ks < 4; ks++) {
                 b.k[part][ks] = wk[(part * K_GL) / 16 + (wave * 4 + ks) * 64 + lane];
                 b.q[part][ks] = wk[((2 + part) * K_GL) / 16 + (wave * 4 + ks) * 64 + lane];
-            }
-#pragma unroll
-            for (int nt = 0; nt < 2; nt++) {
-#pragma unroll
-                for (int ks = 0; ks < 2; ks++) b.x[part][nt][ks] = wk[(4 * K_GL + part * X_GL) / 16 + ((wave * 2 + nt) * 2 + ks) * 64 + lane];
             }
 #pragma unroll
             for (int m = 0; m < 2; m++) {
@@ -429,7 +409,17 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
     auto step = [&](uint32_t blk, const ChainBlock &cur, ChainBlock &next) {
         const uint32_t nxt = blk + 1 < nblocks ? blk + 1 : blk;
         request(nxt, next);
-        __syncthreads();  // the block's values and factors and the state's image are in LDS
+        // this wave's rows of the block's keys, for the state's update (the set of two blocks ago is read no more:
+        // every wave has been through the three barriers of the block between)
+        _Float16 *kimg = img_w(L::KIMG + int(blk & 1) * 2 * K_IMG);
+#pragma unroll
+        for (int part = 0; part < 2; part++) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                *reinterpret_cast<u32x4 *>(kimg + part * C * KROW + (16 * wave + n) * KROW + 32 * ks + 8 * j) = cur.k[part][ks];
+            }
+        }
+        __syncthreads();  // the block's values and factors, the state's image and the keys are in LDS
 
         // ---- K S0^T and Q S0^T: rows t = 16 wave + n, columns dv = 16 vt + n' ----
         floatx4 pk[NT], pq[NT];
@@ -492,6 +482,39 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
         __syncthreads();  // U is whole; every wave is through with the state's image, the values and the factors
 
         // ---- S1 = e^{c_last} S0 + (U scaled)^T K: rows dv, columns 32 wave + 16 nt + n, over the 64 tokens ----
+        // The B operands, K by key dim: lane (n, j) wants column 32 wave + 16 nt + n, tokens 32 ks + 8j .. + 7.
+        // ds_read_b64_tr_b16 works on 16 lanes: lane a + 4e of them names 8 bytes (4 values of a row), and lane
+        // 4a + c receives value c of the lanes a, a + 4, a + 8, a + 12.  So lane a + 4e names token .. + e, key
+        // dims .. + 4a .. + 3, and lane n = 4a + c receives key dim .. + n of four tokens in a row; two reads an operand.
+        u32x2 xr[2][2][2][2];  // [hi | lo][nt][k-step][tokens + 0 | + 4]
+        {
+            const uint32_t kbase = uint32_t(reinterpret_cast<uintptr_t>(lds)) + L::KIMG + (blk & 1) * 2 * K_IMG;
+            const uint32_t la = lane & 3, le = (lane >> 2) & 3;
+#pragma unroll
+            for (int part = 0; part < 2; part++) {
+#pragma unroll
+                for (int nt = 0; nt < 2; nt++) {
+#pragma unroll
+                    for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+                        for (int hf = 0; hf < 2; hf++) {
+                            const uint32_t at = kbase + part * K_IMG + ((32 * ks + 8 * j + 4 * hf + le) * KROW + 32 * wave + 16 * nt + 4 * la) * 2;
+                            asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(xr[part][nt][ks][hf]) : "v"(at) : "memory");
+                        }
+                    }
+                }
+            }
+            // (the registers are handed on only behind the wait, in the same straight piece of code)
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(xr[0][0][0][0]), "+v"(xr[0][0][0][1]), "+v"(xr[0][0][1][0]), "+v"(xr[0][0][1][1]), "+v"(xr[0][1][0][0]),
+                           "+v"(xr[0][1][0][1]), "+v"(xr[0][1][1][0]), "+v"(xr[0][1][1][1]), "+v"(xr[1][0][0][0]), "+v"(xr[1][0][0][1]),
+                           "+v"(xr[1][0][1][0]), "+v"(xr[1][0][1][1]), "+v"(xr[1][1][0][0]), "+v"(xr[1][1][0][1]), "+v"(xr[1][1][1][0]),
+                           "+v"(xr[1][1][1][1])::"memory");
+        }
+        auto x_operand = [&](int part, int nt, int ks) {
+            const u32x4 v = {xr[part][nt][ks][0].x, xr[part][nt][ks][0].y, xr[part][nt][ks][1].x, xr[part][nt][ks][1].y};
+            return __builtin_bit_cast(half8, v);
+        };
 #pragma unroll
         for (int nt = 0; nt < 2; nt++) {
             floatx4 acc[NT];
@@ -503,7 +526,7 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
                 for (int mt = 0; mt < NT; mt++) {
                     const int ao = (16 * mt + n) * TROW + 32 * ks + 8 * j;
                     acc[mt] = mma3(*reinterpret_cast<const half8 *>(img(L::WH) + ao), *reinterpret_cast<const half8 *>(img(L::WL) + ao),
-                                   __builtin_bit_cast(half8, cur.x[0][nt][ks]), __builtin_bit_cast(half8, cur.x[1][nt][ks]), acc[mt]);
+                                   x_operand(0, nt, ks), x_operand(1, nt, ks), acc[mt]);
                 }
             }
 #pragma unroll
