@@ -291,6 +291,33 @@ def test_large_cache_of_codes_several_rows(kind, m):
             del kc, vc
 
 
+@pytest.mark.parametrize("splits", [100, 64, 7])
+def test_several_rows_with_fewer_splits(splits):
+    # RowsAttentionParams.splits is an upper bound the caller may lower (src/rows.rs:344-367).  In a
+    # cache of 24576 tokens: 100 splits are shares of 15 and 16 blocks, still one round of the
+    # keys-first kernel; 64 splits are shares of 24 blocks and 7 of 220, which the register kernels take.
+    rng = np.random.default_rng(4100 + splits)
+    capacity, m, kind = 24576, 3, saetta.KvBits.Eight
+    k = rng.standard_normal((capacity, VALUES)).astype(np.float32)
+    v = rng.standard_normal((capacity, VALUES)).astype(np.float32)
+    q = rng.standard_normal((m, H, D)).astype(np.float32)
+    qg = rng.standard_normal((m, H, 2 * D)).astype(np.float32)
+    rows = saetta.AttentionRows(H, KV, capacity, m)
+    rows.splits = splits
+    for tokens in [capacity, 5000]:
+        pos = tokens - m
+        kc, vc, kf, vf = cache_pair(k[:tokens], v[:tokens], kind, capacity, poison=True)
+        out = torch.full((m, H, D), float("nan"), device="cuda")
+        plan = saetta.Plan()
+        rows.record_quant(plan, m, dev(q), kc, vc, dev(qg), out, [saetta.TokenParams(0, pos + r).as_tensor("cuda") for r in range(m)])
+        plan.build().run()
+        got = host(out)
+        assert np.isfinite(got).all(), tokens
+        worst = np.abs(got - oracle.rows(q, kf, vf, pos, m, q_and_gate=qg, threads=8, f64=True)).max()
+        assert worst < MAX_ABS_F64, (tokens, worst)
+        del kc, vc
+
+
 @pytest.mark.parametrize("capacity", [81920, 49152, 34816])
 @pytest.mark.parametrize("kind", [saetta.KvBits.Eight, saetta.KvBits.Four])
 def test_large_cache_of_codes_one_row(kind, capacity):
