@@ -307,15 +307,19 @@ struct ChainLds {
     static constexpr int BYTES = KIMG + 4 * K_IMG;
 };
 
-// What a wave reads of a block: 24 operands and, for the workgroup, its share of the block's values and factors.
+// Eight waves in two teams.  Waves 0-3 carry the state: K S0^T, R, U and the state's update, each for 16 of
+// the block's tokens (the update: for 32 key dims).  Waves 4-7 make the outputs, which nothing in the chain
+// waits for: Q S0^T beside the first team's K S0^T, M U beside its update of the state, and the stores.
+// What a wave reads of a block: its 16 rows of K (or Q) and of T (or M), 12 operands at most, and, in the
+// first team, its share of the block's values and factors.
 struct ChainBlock {
-    u32x4 k[2][4], q[2][4];  // [hi | lo][k-step]: rows 16 wave + n of K and Q
-    u32x4 tm[2][2][2];       // [T | M][hi | lo][k-step]: rows 16 wave + n
+    u32x4 kq[2][4];  // [hi | lo][k-step]: rows 16 w + n of K | Q
+    u32x4 tm[2][2];  // [hi | lo][k-step]: rows 16 w + n of T | M
     static constexpr int V_LOADS = C * DV * 4 / 16 / 256;  // 16-byte pieces per thread of the block's [token][DV] values
     u32x4 v[V_LOADS], gam;   // ...; 16 bytes of the 128 factors (threads 0-31)
 };
 
-__global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) {
+__global__ __launch_bounds__(512) void deltanet_chunk_chain_kernel(ChunkArgs a) {
     using L = ChainLds;
     constexpr int NT = DV / 16;  // 16-wide tiles of value dims
     constexpr int V_LOADS = ChainBlock::V_LOADS;
@@ -331,7 +335,9 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
         h = xcd * (a.v_heads / 8) + at / slices, slice = at % slices;
     }
     const uint32_t group = a.v_heads / a.k_heads, khd = h / group;
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), n = lane & 15, j = lane >> 4;
+    const uint32_t lane = threadIdx.x & 63, wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n = lane & 15, j = lane >> 4;
+    const bool state_team = wave_all < 4;
+    const uint32_t wave = wave_all & 3, tid = threadIdx.x & 255;  // the wave and the thread inside the team
     const uint32_t nblocks = (a.tokens + C - 1) / C;
     const size_t per_block = block_bytes(a.k_heads, a.v_heads);
     auto img = [&](int off) { return reinterpret_cast<const _Float16 *>(lds + off); };
@@ -340,33 +346,31 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
     float *v_lds = reinterpret_cast<float *>(lds + L::V);
 
     auto request = [&](uint32_t blk, ChainBlock &b) {
-        const u32x4 *wk = reinterpret_cast<const u32x4 *>(a.ws + size_t(blk) * per_block + khd * KHEAD_BYTES);
+        // (the second team's operands lie two parts on: Q behind K, M behind T)
+        const u32x4 *wk = reinterpret_cast<const u32x4 *>(a.ws + size_t(blk) * per_block + khd * KHEAD_BYTES + (state_team ? 0 : 2 * K_GL));
         const u32x4 *wv = reinterpret_cast<const u32x4 *>(a.ws + size_t(blk) * per_block + a.k_heads * KHEAD_BYTES + h * VHEAD_BYTES);
+        const u32x4 *wt = wv + (state_team ? 0 : 2 * T_GL) / 16;
 #pragma unroll
         for (int part = 0; part < 2; part++) {
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++) {
-                b.k[part][ks] = wk[(part * K_GL) / 16 + (wave * 4 + ks) * 64 + lane];
-                b.q[part][ks] = wk[((2 + part) * K_GL) / 16 + (wave * 4 + ks) * 64 + lane];
-            }
+            for (int ks = 0; ks < 4; ks++) b.kq[part][ks] = wk[(part * K_GL) / 16 + (wave * 4 + ks) * 64 + lane];
 #pragma unroll
-            for (int m = 0; m < 2; m++) {
-#pragma unroll
-                for (int ks = 0; ks < 2; ks++) {
-                    // (T and M are lower triangular: rows 16 wave .. have nothing in columns 32 ks .. beyond their own)
-                    if (ks <= int(wave) / 2) b.tm[m][part][ks] = wv[((2 * m + part) * T_GL) / 16 + (wave * 2 + ks) * 64 + lane];
-                }
+            for (int ks = 0; ks < 2; ks++) {
+                // (T and M are lower triangular: rows 16 wave .. have nothing in columns 32 ks .. beyond their own)
+                if (ks <= int(wave) / 2) b.tm[part][ks] = wt[(part * T_GL) / 16 + (wave * 2 + ks) * 64 + lane];
             }
         }
+        if (state_team) {
 #pragma unroll
-        for (int i = 0; i < V_LOADS; i++) {
-            // piece p of the block's [token][DV] values: token p / (DV / 4), four dims (a token past the end: unused, see `place`)
-            const uint32_t p = tid + 256 * i, tok = min(blk * C + p / (DV / 4), a.tokens - 1);
-            b.v[i] = *reinterpret_cast<const u32x4 *>(a.mixed + size_t(tok) * a.channels + 2 * a.k_heads * K_DIM + h * a.v_dim + DV * slice + 4 * (p % (DV / 4)));
+            for (int i = 0; i < V_LOADS; i++) {
+                // piece p of the block's [token][DV] values: token p / (DV / 4), four dims (a token past the end: unused, see `place`)
+                const uint32_t p = tid + 256 * i, tok = min(blk * C + p / (DV / 4), a.tokens - 1);
+                b.v[i] = *reinterpret_cast<const u32x4 *>(a.mixed + size_t(tok) * a.channels + 2 * a.k_heads * K_DIM + h * a.v_dim + DV * slice + 4 * (p % (DV / 4)));
+            }
+            b.gam = wv[(4 * T_GL) / 16 + (tid & 31)];
         }
-        b.gam = wv[(4 * T_GL) / 16 + (tid & 31)];
     };
-    // the block's values (tokens past the end: zeros) and factors to LDS
+    // the block's values (tokens past the end: zeros) and factors to LDS (the first team)
     auto place = [&](uint32_t blk, const ChainBlock &b) {
 #pragma unroll
         for (int i = 0; i < V_LOADS; i++) {
@@ -377,8 +381,8 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
         if (tid < 32) reinterpret_cast<u32x4 *>(lds + L::GAM)[tid] = b.gam;
     };
 
-    // ---- the state's slice: S [dv][128]; wave w keeps columns 32 w .. + 31: lane (n, j) the four rows
-    // dv = 16 mt + 4j + i of columns 32 w + 16 nt + n.  Its image for the products lies in LDS as hi and lo parts. ----
+    // ---- the state's slice: S [dv][128]; wave w of the first team keeps columns 32 w .. + 31: lane (n, j) the four
+    // rows dv = 16 mt + 4j + i of columns 32 w + 16 nt + n.  Its image for the products lies in LDS as hi and lo parts. ----
     float *state = a.state + (size_t(h) * a.v_dim + DV * slice) * K_DIM;
     floatx4 s_reg[NT][2];
     auto publish_state = [&]() {
@@ -401,173 +405,185 @@ __global__ __launch_bounds__(256) void deltanet_chunk_chain_kernel(ChunkArgs a) 
 #pragma unroll
         for (int nt = 0; nt < 2; nt++) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) s_reg[mt][nt][i] = state[(16 * mt + 4 * j + i) * K_DIM + 32 * wave + 16 * nt + n];
+            for (int i = 0; i < 4; i++) s_reg[mt][nt][i] = state_team ? state[(16 * mt + 4 * j + i) * K_DIM + 32 * wave + 16 * nt + n] : 0.0f;
         }
     }
+
     // One block: `cur` holds its operands; the next block's are asked for now, into `next`, and used a block
     // later (after the last block: the last block's again, unused).
     auto step = [&](uint32_t blk, const ChainBlock &cur, ChainBlock &next) {
         const uint32_t nxt = blk + 1 < nblocks ? blk + 1 : blk;
         request(nxt, next);
-        // this wave's rows of the block's keys, for the state's update (the set of two blocks ago is read no more:
-        // every wave has been through the three barriers of the block between)
-        _Float16 *kimg = img_w(L::KIMG + int(blk & 1) * 2 * K_IMG);
+        if (state_team) {
+            // this wave's rows of the block's keys, for the state's update (the set of two blocks ago is read no more:
+            // every wave has been through the three barriers of the block between)
+            _Float16 *kimg = img_w(L::KIMG + int(blk & 1) * 2 * K_IMG);
 #pragma unroll
-        for (int part = 0; part < 2; part++) {
+            for (int part = 0; part < 2; part++) {
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++) {
-                *reinterpret_cast<u32x4 *>(kimg + part * C * KROW + (16 * wave + n) * KROW + 32 * ks + 8 * j) = cur.k[part][ks];
+                for (int ks = 0; ks < 4; ks++) {
+                    *reinterpret_cast<u32x4 *>(kimg + part * C * KROW + (16 * wave + n) * KROW + 32 * ks + 8 * j) = cur.kq[part][ks];
+                }
             }
         }
         __syncthreads();  // the block's values and factors, the state's image and the keys are in LDS
 
-        // ---- K S0^T and Q S0^T: rows t = 16 wave + n, columns dv = 16 vt + n' ----
-        floatx4 pk[NT], pq[NT];
+        // ---- K S0^T (first team) | Q S0^T (second team): rows t = 16 wave + n, columns dv = 16 vt + n' ----
+        floatx4 pkq[NT];
 #pragma unroll
-        for (int vt = 0; vt < NT; vt++) pk[vt] = pq[vt] = floatx4{0, 0, 0, 0};
+        for (int vt = 0; vt < NT; vt++) pkq[vt] = floatx4{0, 0, 0, 0};
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
 #pragma unroll
             for (int vt = 0; vt < NT; vt++) {
                 const int bo = (16 * vt + n) * L::SROW + 32 * ks + 8 * j;
                 const half8 bh = *reinterpret_cast<const half8 *>(img(L::SH) + bo), bl = *reinterpret_cast<const half8 *>(img(L::SL) + bo);
-                pk[vt] = mma3(__builtin_bit_cast(half8, cur.k[0][ks]), __builtin_bit_cast(half8, cur.k[1][ks]), bh, bl, pk[vt]);
-                pq[vt] = mma3(__builtin_bit_cast(half8, cur.q[0][ks]), __builtin_bit_cast(half8, cur.q[1][ks]), bh, bl, pq[vt]);
+                pkq[vt] = mma3(__builtin_bit_cast(half8, cur.kq[0][ks]), __builtin_bit_cast(half8, cur.kq[1][ks]), bh, bl, pkq[vt]);
             }
         }
         // C layout: lane (n, j) holds dv = 16 vt + n of tokens t = 16 wave + 4j + i
         const floatx4 gam4 = *reinterpret_cast<const floatx4 *>(gam + 16 * wave + 4 * j);
         const floatx4 gk4 = *reinterpret_cast<const floatx4 *>(gam + C + 16 * wave + 4 * j);
         const float glast = gam[C - 1];
+        if (state_team) {
 #pragma unroll
-        for (int vt = 0; vt < NT; vt++) {
-            // R = V - e^c (K S0^T), as the [dv][token] image
-            half4 rh, rl;
+            for (int vt = 0; vt < NT; vt++) {
+                // R = V - e^c (K S0^T), as the [dv][token] image
+                half4 rh, rl;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                _Float16 hi, lo;
-                split2(v_lds[(16 * wave + 4 * j + i) * DV + 16 * vt + n] - gam4[i] * pk[vt][i], hi, lo);
-                rh[i] = hi, rl[i] = lo;
+                for (int i = 0; i < 4; i++) {
+                    _Float16 hi, lo;
+                    split2(v_lds[(16 * wave + 4 * j + i) * DV + 16 * vt + n] - gam4[i] * pkq[vt][i], hi, lo);
+                    rh[i] = hi, rl[i] = lo;
+                }
+                const int at = (16 * vt + n) * TROW + 16 * wave + 4 * j;
+                *reinterpret_cast<half4 *>(img_w(L::RH) + at) = rh, *reinterpret_cast<half4 *>(img_w(L::RL) + at) = rl;
             }
-            const int at = (16 * vt + n) * TROW + 16 * wave + 4 * j;
-            *reinterpret_cast<half4 *>(img_w(L::RH) + at) = rh, *reinterpret_cast<half4 *>(img_w(L::RL) + at) = rl;
         }
         __syncthreads();  // R is whole
 
-        // ---- U = T R (T is lower triangular: k-steps up to the row tile's own) ----
-        floatx4 u[NT];
+        if (state_team) {
+            // ---- U = T R (T is lower triangular: k-steps up to the row tile's own) ----
 #pragma unroll
-        for (int vt = 0; vt < NT; vt++) {
-            u[vt] = floatx4{0, 0, 0, 0};
+            for (int vt = 0; vt < NT; vt++) {
+                floatx4 u = {0, 0, 0, 0};
 #pragma unroll
-            for (int ks = 0; ks < 2; ks++) {
-                if (ks > int(wave) / 2) continue;
-                const int bo = (16 * vt + n) * TROW + 32 * ks + 8 * j;
-                u[vt] = mma3(__builtin_bit_cast(half8, cur.tm[0][0][ks]), __builtin_bit_cast(half8, cur.tm[0][1][ks]),
-                             *reinterpret_cast<const half8 *>(img(L::RH) + bo), *reinterpret_cast<const half8 *>(img(L::RL) + bo), u[vt]);
+                for (int ks = 0; ks < 2; ks++) {
+                    if (ks > int(wave) / 2) continue;
+                    const int bo = (16 * vt + n) * TROW + 32 * ks + 8 * j;
+                    u = mma3(__builtin_bit_cast(half8, cur.tm[0][ks]), __builtin_bit_cast(half8, cur.tm[1][ks]),
+                             *reinterpret_cast<const half8 *>(img(L::RH) + bo), *reinterpret_cast<const half8 *>(img(L::RL) + bo), u);
+                }
+                half4 uh, ul, wh, wl;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    _Float16 hi, lo;
+                    split2(u[i], hi, lo);
+                    uh[i] = hi, ul[i] = lo;
+                    split2(u[i] * gk4[i], hi, lo);  // scaled by e^{c_last - c_t} for the state
+                    wh[i] = hi, wl[i] = lo;
+                }
+                const int at = (16 * vt + n) * TROW + 16 * wave + 4 * j;
+                *reinterpret_cast<half4 *>(img_w(L::UH) + at) = uh, *reinterpret_cast<half4 *>(img_w(L::UL) + at) = ul;
+                *reinterpret_cast<half4 *>(img_w(L::WH) + at) = wh, *reinterpret_cast<half4 *>(img_w(L::WL) + at) = wl;
             }
-            half4 uh, ul, wh, wl;
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                _Float16 hi, lo;
-                split2(u[vt][i], hi, lo);
-                uh[i] = hi, ul[i] = lo;
-                split2(u[vt][i] * gk4[i], hi, lo);  // scaled by e^{c_last - c_t} for the state
-                wh[i] = hi, wl[i] = lo;
-            }
-            const int at = (16 * vt + n) * TROW + 16 * wave + 4 * j;
-            *reinterpret_cast<half4 *>(img_w(L::UH) + at) = uh, *reinterpret_cast<half4 *>(img_w(L::UL) + at) = ul;
-            *reinterpret_cast<half4 *>(img_w(L::WH) + at) = wh, *reinterpret_cast<half4 *>(img_w(L::WL) + at) = wl;
         }
         __syncthreads();  // U is whole; every wave is through with the state's image, the values and the factors
 
-        // ---- S1 = e^{c_last} S0 + (U scaled)^T K: rows dv, columns 32 wave + 16 nt + n, over the 64 tokens ----
-        // The B operands, K by key dim: lane (n, j) wants column 32 wave + 16 nt + n, tokens 32 ks + 8j .. + 7.
-        // ds_read_b64_tr_b16 works on 16 lanes: lane a + 4e of them names 8 bytes (4 values of a row), and lane
-        // 4a + c receives value c of the lanes a, a + 4, a + 8, a + 12.  So lane a + 4e names token .. + e, key
-        // dims .. + 4a .. + 3, and lane n = 4a + c receives key dim .. + n of four tokens in a row; two reads an operand.
-        u32x2 xr[2][2][2][2];  // [hi | lo][nt][k-step][tokens + 0 | + 4]
-        {
-            const uint32_t kbase = uint32_t(reinterpret_cast<uintptr_t>(lds)) + L::KIMG + (blk & 1) * 2 * K_IMG;
-            const uint32_t la = lane & 3, le = (lane >> 2) & 3;
+        if (state_team) {
+            // ---- S1 = e^{c_last} S0 + (U scaled)^T K: rows dv, columns 32 wave + 16 nt + n, over the 64 tokens ----
+            // The B operands, K by key dim: lane (n, j) wants column 32 wave + 16 nt + n, tokens 32 ks + 8j .. + 7.
+            // ds_read_b64_tr_b16 works on 16 lanes: lane a + 4e of them names 8 bytes (4 values of a row), and lane
+            // 4a + c receives value c of the lanes a, a + 4, a + 8, a + 12.  So lane a + 4e names token .. + e, key
+            // dims .. + 4a .. + 3, and lane n = 4a + c receives key dim .. + n of four tokens in a row; two reads an operand.
+            u32x2 xr[2][2][2][2];  // [hi | lo][nt][k-step][tokens + 0 | + 4]
+            {
+                const uint32_t kbase = uint32_t(reinterpret_cast<uintptr_t>(lds)) + L::KIMG + (blk & 1) * 2 * K_IMG;
+                const uint32_t la = lane & 3, le = (lane >> 2) & 3;
 #pragma unroll
-            for (int part = 0; part < 2; part++) {
+                for (int part = 0; part < 2; part++) {
 #pragma unroll
-                for (int nt = 0; nt < 2; nt++) {
+                    for (int nt = 0; nt < 2; nt++) {
 #pragma unroll
-                    for (int ks = 0; ks < 2; ks++) {
+                        for (int ks = 0; ks < 2; ks++) {
 #pragma unroll
-                        for (int hf = 0; hf < 2; hf++) {
-                            const uint32_t at = kbase + part * K_IMG + ((32 * ks + 8 * j + 4 * hf + le) * KROW + 32 * wave + 16 * nt + 4 * la) * 2;
-                            asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(xr[part][nt][ks][hf]) : "v"(at) : "memory");
+                            for (int hf = 0; hf < 2; hf++) {
+                                const uint32_t at = kbase + part * K_IMG + ((32 * ks + 8 * j + 4 * hf + le) * KROW + 32 * wave + 16 * nt + 4 * la) * 2;
+                                asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(xr[part][nt][ks][hf]) : "v"(at) : "memory");
+                            }
                         }
                     }
                 }
+                // (the registers are handed on only behind the wait, in the same straight piece of code)
+                asm volatile("s_waitcnt lgkmcnt(0)"
+                             : "+v"(xr[0][0][0][0]), "+v"(xr[0][0][0][1]), "+v"(xr[0][0][1][0]), "+v"(xr[0][0][1][1]), "+v"(xr[0][1][0][0]),
+                               "+v"(xr[0][1][0][1]), "+v"(xr[0][1][1][0]), "+v"(xr[0][1][1][1]), "+v"(xr[1][0][0][0]), "+v"(xr[1][0][0][1]),
+                               "+v"(xr[1][0][1][0]), "+v"(xr[1][0][1][1]), "+v"(xr[1][1][0][0]), "+v"(xr[1][1][0][1]), "+v"(xr[1][1][1][0]),
+                               "+v"(xr[1][1][1][1])::"memory");
             }
-            // (the registers are handed on only behind the wait, in the same straight piece of code)
-            asm volatile("s_waitcnt lgkmcnt(0)"
-                         : "+v"(xr[0][0][0][0]), "+v"(xr[0][0][0][1]), "+v"(xr[0][0][1][0]), "+v"(xr[0][0][1][1]), "+v"(xr[0][1][0][0]),
-                           "+v"(xr[0][1][0][1]), "+v"(xr[0][1][1][0]), "+v"(xr[0][1][1][1]), "+v"(xr[1][0][0][0]), "+v"(xr[1][0][0][1]),
-                           "+v"(xr[1][0][1][0]), "+v"(xr[1][0][1][1]), "+v"(xr[1][1][0][0]), "+v"(xr[1][1][0][1]), "+v"(xr[1][1][1][0]),
-                           "+v"(xr[1][1][1][1])::"memory");
-        }
-        auto x_operand = [&](int part, int nt, int ks) {
-            const u32x4 v = {xr[part][nt][ks][0].x, xr[part][nt][ks][0].y, xr[part][nt][ks][1].x, xr[part][nt][ks][1].y};
-            return __builtin_bit_cast(half8, v);
-        };
+            auto x_operand = [&](int part, int nt, int ks) {
+                const u32x4 v = {xr[part][nt][ks][0].x, xr[part][nt][ks][0].y, xr[part][nt][ks][1].x, xr[part][nt][ks][1].y};
+                return __builtin_bit_cast(half8, v);
+            };
 #pragma unroll
-        for (int nt = 0; nt < 2; nt++) {
-            floatx4 acc[NT];
+            for (int nt = 0; nt < 2; nt++) {
+                floatx4 acc[NT];
 #pragma unroll
-            for (int mt = 0; mt < NT; mt++) acc[mt] = floatx4{0, 0, 0, 0};
+                for (int mt = 0; mt < NT; mt++) acc[mt] = floatx4{0, 0, 0, 0};
 #pragma unroll
-            for (int ks = 0; ks < 2; ks++) {
+                for (int ks = 0; ks < 2; ks++) {
 #pragma unroll
-                for (int mt = 0; mt < NT; mt++) {
-                    const int ao = (16 * mt + n) * TROW + 32 * ks + 8 * j;
-                    acc[mt] = mma3(*reinterpret_cast<const half8 *>(img(L::WH) + ao), *reinterpret_cast<const half8 *>(img(L::WL) + ao),
-                                   x_operand(0, nt, ks), x_operand(1, nt, ks), acc[mt]);
+                    for (int mt = 0; mt < NT; mt++) {
+                        const int ao = (16 * mt + n) * TROW + 32 * ks + 8 * j;
+                        acc[mt] = mma3(*reinterpret_cast<const half8 *>(img(L::WH) + ao), *reinterpret_cast<const half8 *>(img(L::WL) + ao),
+                                       x_operand(0, nt, ks), x_operand(1, nt, ks), acc[mt]);
+                    }
                 }
+#pragma unroll
+                for (int mt = 0; mt < NT; mt++) s_reg[mt][nt] = s_reg[mt][nt] * glast + acc[mt];
             }
+            // the next block's state image, values and factors: their places were last read before the barrier above
+            publish_state();
+            place(nxt, next);
+        } else {
+            // ---- O = (e^c (Q S0^T) + M U) / sqrt(128) ----
 #pragma unroll
-            for (int mt = 0; mt < NT; mt++) s_reg[mt][nt] = s_reg[mt][nt] * glast + acc[mt];
-        }
-        // the next block's state image, values and factors: their places were last read before the barrier above
-        publish_state();
-        place(nxt, next);
-        // ---- O = (e^c (Q S0^T) + M U) / sqrt(128) ----
+            for (int vt = 0; vt < NT; vt++) {
+                floatx4 mu = {0, 0, 0, 0};
 #pragma unroll
-        for (int vt = 0; vt < NT; vt++) {
-            floatx4 mu = {0, 0, 0, 0};
+                for (int ks = 0; ks < 2; ks++) {
+                    if (ks > int(wave) / 2) continue;
+                    const int bo = (16 * vt + n) * TROW + 32 * ks + 8 * j;
+                    mu = mma3(__builtin_bit_cast(half8, cur.tm[0][ks]), __builtin_bit_cast(half8, cur.tm[1][ks]),
+                              *reinterpret_cast<const half8 *>(img(L::UH) + bo), *reinterpret_cast<const half8 *>(img(L::UL) + bo), mu);
+                }
 #pragma unroll
-            for (int ks = 0; ks < 2; ks++) {
-                if (ks > int(wave) / 2) continue;
-                const int bo = (16 * vt + n) * TROW + 32 * ks + 8 * j;
-                mu = mma3(__builtin_bit_cast(half8, cur.tm[1][0][ks]), __builtin_bit_cast(half8, cur.tm[1][1][ks]),
-                          *reinterpret_cast<const half8 *>(img(L::UH) + bo), *reinterpret_cast<const half8 *>(img(L::UL) + bo), mu);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const uint32_t tok = blk * C + 16 * wave + 4 * j + i;
-                if (tok < a.tokens) a.o[(size_t(tok) * a.v_heads + h) * a.v_dim + DV * slice + 16 * vt + n] = Q_SCALE * (gam4[i] * pq[vt][i] + mu[i]);
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t tok = blk * C + 16 * wave + 4 * j + i;
+                    if (tok < a.tokens) a.o[(size_t(tok) * a.v_heads + h) * a.v_dim + DV * slice + 16 * vt + n] = Q_SCALE * (gam4[i] * pkq[vt][i] + mu[i]);
+                }
             }
         }
     };
     // (two sets of operand registers that change roles, so that nothing is copied from one to the other)
     ChainBlock even, odd;
     request(0, even);
-    publish_state();
-    place(0, even);
+    if (state_team) {
+        publish_state();
+        place(0, even);
+    }
     for (uint32_t blk = 0; blk < nblocks; blk += 2) {
         step(blk, even, odd);
         if (blk + 1 < nblocks) step(blk + 1, odd, even);
     }
+    if (state_team) {
 #pragma unroll
-    for (int mt = 0; mt < NT; mt++) {
+        for (int mt = 0; mt < NT; mt++) {
 #pragma unroll
-        for (int nt = 0; nt < 2; nt++) {
+            for (int nt = 0; nt < 2; nt++) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) state[(16 * mt + 4 * j + i) * K_DIM + 32 * wave + 16 * nt + n] = s_reg[mt][nt][i];
+                for (int i = 0; i < 4; i++) state[(16 * mt + 4 * j + i) * K_DIM + 32 * wave + 16 * nt + n] = s_reg[mt][nt][i];
+            }
         }
     }
 }
@@ -611,7 +627,7 @@ int run_deltanet_chunk(hipStream_t stream, const float *mixed, const float *a, c
     } else {
         deltanet_chunk_prepare_kernel<1><<<dim3(nblocks, p.v_heads), 256, PrepLds<1>::BYTES, stream>>>(args);
     }
-    deltanet_chunk_chain_kernel<<<dim3(p.v_dim / DV * p.v_heads), 256, ChainLds::BYTES, stream>>>(args);
+    deltanet_chunk_chain_kernel<<<dim3(p.v_dim / DV * p.v_heads), 512, ChainLds::BYTES, stream>>>(args);
     return SAETTA_OK;
 }
 
