@@ -631,7 +631,7 @@ def bench_deltanet_prefill(s, torch, args, tokens=4096):
                    "bytes_rows_launch": rows_bytes, "bytes_conv_launch": conv_bytes},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "deltanet_chunk_prepare_kernel + deltanet_chunk_chain_kernel + deltanet_gated_norm_rows_kernel",
+                     "kernel": "deltanet_chunk_prepare_kernel + deltanet_chunk_chain_kernel + deltanet_gated_norm_wide_kernel",
                      "avg_us": round(rows_us, 1), "token_chain_TFLOPs": round(flops / rows_us / 1e6, 2)},
         "cpu_baseline": {"value": round(1.0 / cpu_s, 1), "unit": "tokens/s", "cores": 1, "kind": "port",
                          "sample": f"the first {n_check} tokens, conv + step each ({cpu_s * 1e3:.2f} ms per token)"},

@@ -406,6 +406,21 @@ __global__ __launch_bounds__(256) void deltanet_rows_kernel(RowsArgs a) {
     }
 }
 
+// The same for the chunks of a prefill, which are held to a tolerance and not to the single-token kernels'
+// bits: LP = v_dim / 4 lanes per pair, four values each (16-byte loads and stores, two pairs per wavefront at
+// the model's 128), the sum of squares over the LP lanes.
+template <int LP>
+__global__ __launch_bounds__(256) void deltanet_gated_norm_wide_kernel(float *y, const float *__restrict__ z,
+                                                                       const float *__restrict__ norm_w, uint32_t pairs, float eps) {
+    const uint32_t at = blockIdx.x * 256 + threadIdx.x, pair = at / LP, part = at % LP;
+    if (pair >= pairs) return;  // (whole groups of LP lanes: 256 is a multiple of LP)
+    float4 *yp = reinterpret_cast<float4 *>(y) + size_t(pair) * LP + part;
+    const float4 o = *yp, g = reinterpret_cast<const float4 *>(z)[size_t(pair) * LP + part], w = reinterpret_cast<const float4 *>(norm_w)[part];
+    const float total = group_reduce<LP>(o.x * o.x + o.y * o.y + o.z * o.z + o.w * o.w, SumOp());
+    const float inv = 1.0f / sqrtf(total / float(4 * LP) + eps);
+    *yp = make_float4(o.x * (inv * w.x) * silu_f(g.x), o.y * (inv * w.y) * silu_f(g.y), o.z * (inv * w.z) * silu_f(g.z), o.w * (inv * w.w) * silu_f(g.w));
+}
+
 // y = o / sqrt(mean(o^2) + eps) * norm_w * silu(z) per (token, value head), in place on y:
 // one wavefront per pair, v_dim up to 256.
 __global__ __launch_bounds__(256) void deltanet_gated_norm_rows_kernel(float *y, const float *__restrict__ z,
@@ -773,7 +788,16 @@ extern "C" int saetta_deltanet_rows_ws(saetta_stream_t stream, const float *mixe
         }
     }
     const uint32_t pairs = p.tokens * p.v_heads;
-    deltanet_gated_norm_rows_kernel<<<(pairs + 3) / 4, 256, 0, as_stream(stream)>>>(y, z, norm_w, pairs, p.v_dim, p.eps);
+    const bool wide = blocks && aligned(y, 16) && aligned(z, 16) && aligned(norm_w, 16);
+    if (wide && p.v_dim == 128) {
+        deltanet_gated_norm_wide_kernel<32><<<(pairs * 32 + 255) / 256, 256, 0, as_stream(stream)>>>(y, z, norm_w, pairs, p.eps);
+    } else if (wide && p.v_dim == 64) {
+        deltanet_gated_norm_wide_kernel<16><<<(pairs * 16 + 255) / 256, 256, 0, as_stream(stream)>>>(y, z, norm_w, pairs, p.eps);
+    } else if (wide && p.v_dim == 256) {
+        deltanet_gated_norm_wide_kernel<64><<<(pairs * 64 + 255) / 256, 256, 0, as_stream(stream)>>>(y, z, norm_w, pairs, p.eps);
+    } else {
+        deltanet_gated_norm_rows_kernel<<<(pairs + 3) / 4, 256, 0, as_stream(stream)>>>(y, z, norm_w, pairs, p.v_dim, p.eps);
+    }
     return launch_status("deltanet_rows");
 }
 
