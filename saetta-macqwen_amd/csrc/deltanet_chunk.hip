@@ -121,6 +121,8 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
 
     // ---- q and k of the block's tokens, normalised (src/cpu/deltanet.rs:133-146), as hi and lo parts ----
     {
+        // thread (token t, part): the 8-value pieces part, part + 4, part + 8, part + 12 of the token's q and k, so
+        // that the four threads of a token read 128 bytes in a row with every pair of loads
         const uint32_t t = tid >> 2, part = tid & 3, tok = blk * C + t;
         float4 qv[8], kv[8];
         float qs = 0.0f, ks = 0.0f;
@@ -128,7 +130,7 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
         for (int i = 0; i < 8; i++) {
             qv[i] = kv[i] = make_float4(0, 0, 0, 0);
             if (tok < a.tokens) {
-                const float *row = a.mixed + size_t(tok) * a.channels + khd * K_DIM + 32 * part + 4 * i;
+                const float *row = a.mixed + size_t(tok) * a.channels + khd * K_DIM + 8 * (part + 4 * (i >> 1)) + 4 * (i & 1);
                 qv[i] = *reinterpret_cast<const float4 *>(row);
                 kv[i] = *reinterpret_cast<const float4 *>(row + key_size);
             }
@@ -155,12 +157,12 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
                 split2(kf, hi, lo);
                 a_kh[e] = hi, a_kl[e] = lo;
             }
-            const int at = t * KROW + 32 * part + 4 * i;
+            const int at = t * KROW + 8 * (part + 2 * i);  // piece part + 4 (i / 2): key dims 32 (i / 2) + 8 part ..
             *reinterpret_cast<half8 *>(kh + at) = a_kh, *reinterpret_cast<half8 *>(kl + at) = a_kl;
             *reinterpret_cast<half8 *>(qh + at) = a_qh, *reinterpret_cast<half8 *>(ql + at) = a_ql;
             if (writer) {
-                // operand (wave t / 16, k-step part), lane (n = t % 16, j = i / 2)
-                unsigned char *g = ws_k + ((((t >> 4) * 4 + part) * 64 + (i >> 1) * 16 + (t & 15)) * 16);
+                // operand (wave t / 16, k-step i / 2), lane (n = t % 16, j = part): a wave's store is one kilobyte in a row
+                unsigned char *g = ws_k + ((((t >> 4) * 4 + (i >> 1)) * 64 + part * 16 + (t & 15)) * 16);
                 *reinterpret_cast<half8 *>(g) = a_kh, *reinterpret_cast<half8 *>(g + K_GL) = a_kl;
                 *reinterpret_cast<half8 *>(g + 2 * K_GL) = a_qh, *reinterpret_cast<half8 *>(g + 3 * K_GL) = a_ql;
             }
