@@ -143,6 +143,60 @@ __device__ __forceinline__ float conv_input(const float *x, const float *state, 
     return i >= 0 ? x[size_t(i) * p.channels + c] : state[size_t(i + int(p.kernel_size) - 1) * p.channels + c];
 }
 
+// The same for four channels a thread (16-byte loads and stores, eight tokens' loads in flight), four taps:
+// every channel's sums are taken in the same order as above, so the results are the same bit for bit.
+constexpr uint32_t CONV4_AHEAD = 8;
+static_assert(CONV_TILE % CONV4_AHEAD == 0, "whole groups of tokens in a tile");
+__global__ __launch_bounds__(256) void deltanet_conv_rows4_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                                  const float *__restrict__ state, float *__restrict__ out,
+                                                                  float *__restrict__ snaps, saetta_conv_rows_params p) {
+    constexpr int KS = 4;
+    const uint32_t c4 = blockIdx.x * 256 + threadIdx.x, quads = p.channels / 4;
+    if (c4 >= quads) return;
+    const float4 *x4 = reinterpret_cast<const float4 *>(x), *s4 = reinterpret_cast<const float4 *>(state);
+    float4 *o4 = reinterpret_cast<float4 *>(out);
+    // taps[j] holds tap j of the four channels (w is [channel][4]: the thread's 16 floats lie in a row)
+    float4 taps[KS];
+    {
+        const float4 *w4 = reinterpret_cast<const float4 *>(w) + size_t(c4) * 4;
+        const float4 a = w4[0], b = w4[1], c = w4[2], d = w4[3];
+        taps[0] = make_float4(a.x, b.x, c.x, d.x), taps[1] = make_float4(a.y, b.y, c.y, d.y);
+        taps[2] = make_float4(a.z, b.z, c.z, d.z), taps[3] = make_float4(a.w, b.w, c.w, d.w);
+    }
+    const uint32_t t_begin = blockIdx.y * CONV_TILE, t_end = min(p.tokens, t_begin + CONV_TILE);
+    float4 win[KS - 1];
+#pragma unroll
+    for (int j = 0; j < KS - 1; j++) {
+        const int i = int(t_begin) - (KS - 1) + j;
+        win[j] = i >= 0 ? x4[size_t(i) * quads + c4] : s4[size_t(i + KS - 1) * quads + c4];
+    }
+    for (uint32_t t0 = t_begin; t0 < t_end; t0 += CONV4_AHEAD) {
+        float4 xt[CONV4_AHEAD];
+#pragma unroll
+        for (uint32_t u = 0; u < CONV4_AHEAD; u++) xt[u] = x4[size_t(min(t0 + u, p.tokens - 1)) * quads + c4];
+#pragma unroll
+        for (uint32_t u = 0; u < CONV4_AHEAD; u++) {
+            const uint32_t t = t0 + u;
+            if (t >= t_end) break;
+            float4 acc = make_float4(0, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < KS - 1; j++) {
+                acc.x += taps[j].x * win[j].x, acc.y += taps[j].y * win[j].y, acc.z += taps[j].z * win[j].z, acc.w += taps[j].w * win[j].w;
+            }
+            o4[size_t(t) * quads + c4] = make_float4(silu_f(acc.x + taps[KS - 1].x * xt[u].x), silu_f(acc.y + taps[KS - 1].y * xt[u].y),
+                                                     silu_f(acc.z + taps[KS - 1].z * xt[u].z), silu_f(acc.w + taps[KS - 1].w * xt[u].w));
+#pragma unroll
+            for (int j = 0; j + 1 < KS - 1; j++) win[j] = win[j + 1];
+            win[KS - 2] = xt[u];
+            if (p.snapshots) {
+                float4 *snap = reinterpret_cast<float4 *>(snaps) + size_t(t) * (KS - 1) * quads;
+#pragma unroll
+                for (int j = 0; j < KS - 1; j++) snap[size_t(j) * quads + c4] = win[j];
+            }
+        }
+    }
+}
+
 template <int KS>  // taps; 0: any number (read from p), the window is re-read from memory
 __global__ __launch_bounds__(256) void deltanet_conv_rows_kernel(const float *__restrict__ x,
                                                                  const float *__restrict__ w,
@@ -724,7 +778,11 @@ extern "C" int saetta_deltanet_conv_rows(saetta_stream_t stream, const float *x,
     if (int rc = ensure_device()) return rc;
     if (p.channels == 0 || p.tokens == 0) return SAETTA_OK;
     const dim3 grid((p.channels + 255) / 256, (p.tokens + CONV_TILE - 1) / CONV_TILE);
-    if (p.kernel_size == 4) {
+    const bool by_four = p.channels % 4 == 0 && aligned(x, 16) && aligned(w, 16) && aligned(state, 16) && aligned(out, 16) &&
+                         (!p.snapshots || aligned(snaps, 16));
+    if (p.kernel_size == 4 && by_four) {
+        deltanet_conv_rows4_kernel<<<dim3((p.channels / 4 + 255) / 256, grid.y), 256, 0, as_stream(stream)>>>(x, w, state, out, snaps, p);
+    } else if (p.kernel_size == 4) {
         deltanet_conv_rows_kernel<4><<<grid, 256, 0, as_stream(stream)>>>(x, w, state, out, snaps, p);
     } else if (p.kernel_size == 2) {
         deltanet_conv_rows_kernel<2><<<grid, 256, 0, as_stream(stream)>>>(x, w, state, out, snaps, p);
