@@ -139,6 +139,15 @@ def test_blocks_of_tokens_other_value_dims():
         check_against_oracle(layer, tokens, [tokens], snapshots=False, tol=1e-4)
 
 
+@pytest.mark.parametrize("k_heads,v_heads,v_dim,tokens", [(2, 2, 32, 130), (1, 4, 16, 200), (8, 8, 16, 128), (1, 3, 48, 150)])
+def test_blocks_of_tokens_other_head_ratios(k_heads, v_heads, v_dim, tokens):
+    # Two value heads per key head (the model's ratio) share a workgroup of the blocks' prepare kernel; any
+    # other ratio takes one workgroup per value head.  Eight value heads and more are dealt to the XCDs by
+    # head, fewer in launch order.
+    layer = Layer(k_heads, v_heads, v_dim, 4, seed=100 * k_heads + v_heads)
+    check_against_oracle(layer, tokens, [tokens], snapshots=False, tol=1e-4)
+
+
 @pytest.mark.parametrize("v_dim,kernel,tokens", [(4, 2, 5), (24, 4, 17), (100, 7, 33), (256, 4, 16), (16, 16, 3)])
 def test_other_shapes(v_dim, kernel, tokens):
     layer = Layer(2, 4, v_dim, kernel, seed=v_dim + kernel)
