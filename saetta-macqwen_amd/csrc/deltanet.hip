@@ -778,7 +778,8 @@ extern "C" int saetta_deltanet_conv_rows(saetta_stream_t stream, const float *x,
     if (int rc = ensure_device()) return rc;
     if (p.channels == 0 || p.tokens == 0) return SAETTA_OK;
     const dim3 grid((p.channels + 255) / 256, (p.tokens + CONV_TILE - 1) / CONV_TILE);
-    const bool by_four = p.channels % 4 == 0 && aligned(x, 16) && aligned(w, 16) && aligned(state, 16) && aligned(out, 16) &&
+    // (four channels a thread pays from a tile of tokens up: a verify step's few rows want the workgroups)
+    const bool by_four = p.tokens >= CONV_TILE && p.channels % 4 == 0 && aligned(x, 16) && aligned(w, 16) && aligned(state, 16) && aligned(out, 16) &&
                          (!p.snapshots || aligned(snaps, 16));
     if (p.kernel_size == 4 && by_four) {
         deltanet_conv_rows4_kernel<<<dim3((p.channels / 4 + 255) / 256, grid.y), 256, 0, as_stream(stream)>>>(x, w, state, out, snaps, p);

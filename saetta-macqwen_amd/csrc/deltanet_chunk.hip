@@ -91,22 +91,43 @@ __device__ __forceinline__ floatx4 mma3(half8 ah, half8 al, half8 bh, half8 bl, 
 // images and later their T images over qh | ql (and 2 KB more), so that they leave as whole 16-byte stores.
 template <int G>
 struct PrepLds {
-    static constexpr int AROW = C + 4;  // f32 per row of A in LDS: [t][q * 16 + m] holds A_t,s of s = 4m + q
-    static constexpr int A_OFF = 0, A_BYTES = C * AROW * 4;
-    static constexpr int M_OFF = 2 * K_IMG, M_BYTES = 2 * T_IMG;  // mh | ml (then th | tl) of a head
+    // per head, over kh | kl once the products are taken: the two diagonal 32 x 32 blocks of A as f32, rows of
+    // DROW ([t][q * 16 + m] holds A_t,s of s = 2m + q; the product of the off-diagonal block goes over them
+    // later), then the block below the diagonal and the inverse of the second diagonal block as f16 images
+    static constexpr int DROW = 32 + 4, D_BYTES = 32 * DROW * 4;
+    static constexpr int HROW = 32 + 8, H_IMG = 32 * HROW * 2;  // f16 per row of a 32 x 32 image; bytes of one part
+    static constexpr int W_OFF = 0, LBA_OFF = 2 * D_BYTES, XBB_OFF = LBA_OFF + 2 * H_IMG, HEAD_BYTES = XBB_OFF + 2 * H_IMG;
+    static_assert(2 * H_IMG <= 2 * D_BYTES, "the product's images fit over the diagonal blocks");
+    static constexpr int M_BYTES = 2 * T_IMG;  // mh | ml (then th | tl) of a head
+    static constexpr int M_OFF = G * HEAD_BYTES > 2 * K_IMG ? G * HEAD_BYTES : 2 * K_IMG;
     static constexpr int GATES = M_OFF + G * M_BYTES > 4 * K_IMG ? M_OFF + G * M_BYTES : 4 * K_IMG;  // [head][cum | beta][C] f32
     static constexpr int BYTES = GATES + G * 2 * C * 4;
-    static_assert(G * A_BYTES <= M_OFF, "the heads' A fit over kh | kl");
     static_assert(2 * BYTES <= 160 * 1024, "two workgroups per CU");
 };
+
+// The B operand of a 16-column tile out of a row-major f16 image in LDS (hi part at `at`, lo part `part_bytes`
+// on; `at`: the byte address of row 8j + e, column 4a of the tile for lane a + 4e of its 16): lane (n, j)
+// gets column n of rows 8j .. 8j + 7.  ds_read_b64_tr_b16 works on 16 lanes: lane a + 4e of them names 8
+// bytes (4 values of a row), and lane 4a + c receives value c of the lanes a, a + 4, a + 8, a + 12.
+__device__ __forceinline__ void read_by_column(uint32_t at, uint32_t part_bytes, uint32_t four_rows_bytes, half8 &hi, half8 &lo) {
+    u32x2 r[2][2];
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(r[0][0]) : "v"(at) : "memory");
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(r[0][1]) : "v"(at + four_rows_bytes) : "memory");
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(r[1][0]) : "v"(at + part_bytes) : "memory");
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(r[1][1]) : "v"(at + part_bytes + four_rows_bytes) : "memory");
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[1][0]), "+v"(r[1][1])::"memory");
+    hi = __builtin_bit_cast(half8, u32x4{r[0][0].x, r[0][0].y, r[0][1].x, r[0][1].y});
+    lo = __builtin_bit_cast(half8, u32x4{r[1][0].x, r[1][0].y, r[1][1].x, r[1][1].y});
+}
 
 template <int G>
 __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a) {
     using L = PrepLds<G>;
-    constexpr int AROW = L::AROW;
+    constexpr int DROW = L::DROW, HROW = L::HROW;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     _Float16 *kh = reinterpret_cast<_Float16 *>(lds), *kl = kh + C * KROW, *qh = kl + C * KROW, *ql = qh + C * KROW;
-    auto a_lds = [&](int hh) { return reinterpret_cast<float *>(lds + L::A_OFF + hh * L::A_BYTES); };
+    auto diag_lds = [&](int hh, int half) { return reinterpret_cast<float *>(lds + hh * L::HEAD_BYTES + half * L::D_BYTES); };
+    auto half_img = [&](int hh, int off) { return reinterpret_cast<_Float16 *>(lds + hh * L::HEAD_BYTES + off); };  // hi part; lo: 32 * HROW on
     auto m_lds = [&](int hh) { return reinterpret_cast<_Float16 *>(lds + L::M_OFF + hh * L::M_BYTES); };
     auto cum_lds = [&](int hh) { return reinterpret_cast<float *>(lds + L::GATES) + hh * 2 * C; };
     auto beta_lds = [&](int hh) { return reinterpret_cast<float *>(lds + L::GATES) + hh * 2 * C + C; };
@@ -218,7 +239,14 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
             for (int i = 0; i < 4; i++) {
                 const uint32_t t = 16 * wave + 4 * j + i;
                 const float decay = s <= t ? __expf(cum_lds(hh)[t] - cs) : 0.0f;
-                a_lds(hh)[t * AROW + (s & 3) * 16 + (s >> 2)] = s < t ? beta_lds(hh)[t] * decay * gk[nt][i] : 0.0f;
+                const float at_s = s < t ? beta_lds(hh)[t] * decay * gk[nt][i] : 0.0f;
+                if ((nt >> 1) == int(wave >> 1)) {  // a diagonal 32 x 32 block, zeros above the diagonal included
+                    diag_lds(hh, nt >> 1)[(t & 31) * DROW + (s & 1) * 16 + ((s & 31) >> 1)] = at_s;
+                } else if (nt < 2) {  // the block below the diagonal, as an MFMA operand
+                    _Float16 hi, lo;
+                    split2(at_s, hi, lo);
+                    half_img(hh, L::LBA_OFF)[(t - 32) * HROW + s] = hi, half_img(hh, L::LBA_OFF)[32 * HROW + (t - 32) * HROW + s] = lo;
+                }
                 _Float16 hi, lo;
                 split2(decay * gq[nt][i], hi, lo);
                 m_lds(hh)[t * TROW + s] = hi, m_lds(hh)[C * TROW + t * TROW + s] = lo;
@@ -237,48 +265,95 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
 #pragma unroll
     for (int hh = 0; hh < G; hh++) leave(hh, ws_v(hh) + 2 * T_GL);
 
-    // ---- T = (I + A)^-1 diag(beta): column c = 16 wave + n by forward substitution, x_t = beta_t [t = c] -
-    // sum_{s < t} A_ts x_s; lane group q keeps x_s of s = 4m + q in slot m and adds up those s.  The heads'
-    // columns are solved side by side: their chains do not depend on each other. ----
+    // ---- T = (I + A)^-1 diag(beta), in 32 x 32 blocks: with L = I + A = [[L_AA, 0], [L_BA, L_BB]],
+    //     T_AA = L_AA^-1 diag(beta_A),  T_BB = L_BB^-1 diag(beta_B),  T_BA = -L_BB^-1 (L_BA T_AA).
+    // The diagonal blocks by forward substitution, one wave per (head, block): lane (column c, q) solves
+    // x_t = [t = c] - sum_{s < t} A_ts x_s, lane group q keeps x_s of s = 2m + q in slot m and adds up those s.
+    // The block below the diagonal: two products on the matrix cores. ----
     {
-        const uint32_t c = 16 * wave + n, q = j;
-        float x[G][16];
+        const uint32_t hs = G == 2 ? wave >> 1 : 0, half = wave & 1;  // the wave's head and diagonal block
+        const bool solver = G == 2 || wave < 2;
+        const uint32_t c = lane & 31, q = lane >> 5;
+        float x[16];
 #pragma unroll
-        for (int hh = 0; hh < G; hh++) {
+        for (int m = 0; m < 16; m++) x[m] = 0.0f;
+        if (solver) {
+            const float *ad = diag_lds(hs, half) + q * 16;
 #pragma unroll
-            for (int m = 0; m < 16; m++) x[hh][m] = 0.0f;
-        }
-#pragma unroll
-        for (int t = 0; t < C; t++) {
-            if (t < int(16 * wave)) continue;  // (the column is zero above its diagonal: uniform per wave)
-            float total[G];
-#pragma unroll
-            for (int hh = 0; hh < G; hh++) {
+            for (int t = 0; t < 32; t++) {
                 floatx4 part4 = {0, 0, 0, 0};  // (four chains of sums instead of one of up to 16)
-                const float *arow = a_lds(hh) + t * AROW + q * 16;
 #pragma unroll
-                for (int m4 = 0; 16 * m4 < t; m4++) {  // s = 4m + q < t needs m <= (t - 1) / 4
-                    const floatx4 av = *reinterpret_cast<const floatx4 *>(arow + 4 * m4);
+                for (int m4 = 0; 8 * m4 < t; m4++) {  // s = 2m + q < t needs m <= (t - 1) / 2
+                    const floatx4 av = *reinterpret_cast<const floatx4 *>(ad + t * DROW + 4 * m4);
 #pragma unroll
-                    for (int e = 0; e < 4; e++) part4[e] += av[e] * x[hh][4 * m4 + e];
+                    for (int e = 0; e < 4; e++) part4[e] += av[e] * x[4 * m4 + e];
                 }
-                total[hh] = (part4[0] + part4[1]) + (part4[2] + part4[3]);
-            }
-#pragma unroll
-            for (int hh = 0; hh < G; hh++) {
-                const float sum = across_rows<16, 64>(total[hh], SumOp());
-                const float xt = (uint32_t(t) == c ? beta_lds(hh)[t] : 0.0f) - sum;
-                if (q == uint32_t(t & 3)) x[hh][t >> 2] = xt;
+                const float sum = across_rows<32, 64>((part4[0] + part4[1]) + (part4[2] + part4[3]), SumOp());
+                const float xt = (uint32_t(t) == c ? 1.0f : 0.0f) - sum;
+                if (q == uint32_t(t & 1)) x[t >> 1] = xt;
             }
         }
         __syncthreads();  // M has left: T goes over it
-#pragma unroll
-        for (int hh = 0; hh < G; hh++) {
+        if (solver) {
+            const float bc = beta_lds(hs)[32 * half + c];
+            _Float16 *th = m_lds(hs), *tl = th + C * TROW;
 #pragma unroll
             for (int m = 0; m < 16; m++) {
+                const uint32_t t = 2 * m + q;
                 _Float16 hi, lo;
-                split2(x[hh][m], hi, lo);
-                m_lds(hh)[(4 * m + q) * TROW + c] = hi, m_lds(hh)[C * TROW + (4 * m + q) * TROW + c] = lo;
+                split2(x[m] * bc, hi, lo);
+                th[(32 * half + t) * TROW + 32 * half + c] = hi, tl[(32 * half + t) * TROW + 32 * half + c] = lo;
+                if (half == 0) {
+                    th[t * TROW + 32 + c] = (_Float16)0.0f, tl[t * TROW + 32 + c] = (_Float16)0.0f;  // nothing above the diagonal
+                } else {
+                    split2(x[m], hi, lo);
+                    half_img(hs, L::XBB_OFF)[t * HROW + c] = hi, half_img(hs, L::XBB_OFF)[32 * HROW + t * HROW + c] = lo;
+                }
+            }
+        }
+        __syncthreads();
+        // W = L_BA T_AA and then T_BA = -L_BB^-1 W: a wave takes 16 rows (two column tiles of its head; with one
+        // head, one tile).  The right operands are read by column out of row-major images.
+        const uint32_t r = wave & 1, la = lane & 3, le = (lane >> 2) & 3;
+        const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(lds));
+        floatx4 w[2];
+#pragma unroll
+        for (int ct = 0; ct < 2; ct++) {
+            if (G == 1 && ct != int(wave >> 1)) continue;
+            const int ao = (16 * r + n) * HROW + 8 * j;
+            half8 bh, bl;
+            read_by_column(lds0 + L::M_OFF + hs * L::M_BYTES + ((8 * j + le) * TROW + 16 * ct + 4 * la) * 2, C * TROW * 2, 4 * TROW * 2, bh, bl);
+            w[ct] = mma3(*reinterpret_cast<const half8 *>(half_img(hs, L::LBA_OFF) + ao),
+                         *reinterpret_cast<const half8 *>(half_img(hs, L::LBA_OFF) + 32 * HROW + ao), bh, bl, floatx4{0, 0, 0, 0});
+        }
+        // (the diagonal blocks were last read before the barrier above)
+#pragma unroll
+        for (int ct = 0; ct < 2; ct++) {
+            if (G == 1 && ct != int(wave >> 1)) continue;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                _Float16 hi, lo;
+                split2(w[ct][i], hi, lo);
+                const int at = (16 * r + 4 * j + i) * HROW + 16 * ct + n;
+                half_img(hs, L::W_OFF)[at] = hi, half_img(hs, L::W_OFF)[32 * HROW + at] = lo;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ct = 0; ct < 2; ct++) {
+            if (G == 1 && ct != int(wave >> 1)) continue;
+            const int ao = (16 * r + n) * HROW + 8 * j;
+            half8 bh, bl;
+            read_by_column(lds0 + hs * L::HEAD_BYTES + L::W_OFF + ((8 * j + le) * HROW + 16 * ct + 4 * la) * 2, 32 * HROW * 2, 4 * HROW * 2, bh, bl);
+            const floatx4 tba = mma3(*reinterpret_cast<const half8 *>(half_img(hs, L::XBB_OFF) + ao),
+                                     *reinterpret_cast<const half8 *>(half_img(hs, L::XBB_OFF) + 32 * HROW + ao), bh, bl, floatx4{0, 0, 0, 0});
+            _Float16 *th = m_lds(hs), *tl = th + C * TROW;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                _Float16 hi, lo;
+                split2(-tba[i], hi, lo);
+                const int at = (32 + 16 * r + 4 * j + i) * TROW + 16 * ct + n;
+                th[at] = hi, tl[at] = lo;
             }
         }
     }
