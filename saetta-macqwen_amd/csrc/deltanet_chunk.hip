@@ -28,6 +28,7 @@
 #include "lanes.hpp"
 
 #include <mutex>
+#include <type_traits>
 
 namespace saetta {
 namespace {
@@ -422,30 +423,42 @@ __global__ __launch_bounds__(512) void deltanet_chunk_chain_kernel(ChunkArgs a) 
     const float *gam = reinterpret_cast<const float *>(lds + L::GAM);
     float *v_lds = reinterpret_cast<float *>(lds + L::V);
 
-    auto request = [&](uint32_t blk, ChainBlock &b) {
+    // A block's operands are asked for in three lots, each as soon as the registers it goes to have been read
+    // for the block two before: the rows of K | Q, the rows of T | M, the block's values and factors.
+    auto clamp_block = [&](uint32_t blk) { return blk < nblocks ? blk : nblocks - 1; };  // (past the last block: its operands again, unused)
+    auto request_kq = [&](uint32_t at, ChainBlock &b) {
+        const uint32_t blk = clamp_block(at);
         // (the second team's operands lie two parts on: Q behind K, M behind T)
         const u32x4 *wk = reinterpret_cast<const u32x4 *>(a.ws + size_t(blk) * per_block + khd * KHEAD_BYTES + (state_team ? 0 : 2 * K_GL));
-        const u32x4 *wv = reinterpret_cast<const u32x4 *>(a.ws + size_t(blk) * per_block + a.k_heads * KHEAD_BYTES + h * VHEAD_BYTES);
-        const u32x4 *wt = wv + (state_team ? 0 : 2 * T_GL) / 16;
 #pragma unroll
         for (int part = 0; part < 2; part++) {
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) b.kq[part][ks] = wk[(part * K_GL) / 16 + (wave * 4 + ks) * 64 + lane];
+        }
+    };
+    auto request_tm = [&](uint32_t at, ChainBlock &b) {
+        const uint32_t blk = clamp_block(at);
+        const u32x4 *wv = reinterpret_cast<const u32x4 *>(a.ws + size_t(blk) * per_block + a.k_heads * KHEAD_BYTES + h * VHEAD_BYTES);
+        const u32x4 *wt = wv + (state_team ? 0 : 2 * T_GL) / 16;
+#pragma unroll
+        for (int part = 0; part < 2; part++) {
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
                 // (T and M are lower triangular: rows 16 wave .. have nothing in columns 32 ks .. beyond their own)
                 if (ks <= int(wave) / 2) b.tm[part][ks] = wt[(part * T_GL) / 16 + (wave * 2 + ks) * 64 + lane];
             }
         }
-        if (state_team) {
+    };
+    auto request_values = [&](uint32_t at, ChainBlock &b) {  // (the first team)
+        const uint32_t blk = clamp_block(at);
+        const u32x4 *wv = reinterpret_cast<const u32x4 *>(a.ws + size_t(blk) * per_block + a.k_heads * KHEAD_BYTES + h * VHEAD_BYTES);
 #pragma unroll
-            for (int i = 0; i < V_LOADS; i++) {
-                // piece p of the block's [token][DV] values: token p / (DV / 4), four dims (a token past the end: unused, see `place`)
-                const uint32_t p = tid + 256 * i, tok = min(blk * C + p / (DV / 4), a.tokens - 1);
-                b.v[i] = *reinterpret_cast<const u32x4 *>(a.mixed + size_t(tok) * a.channels + 2 * a.k_heads * K_DIM + h * a.v_dim + DV * slice + 4 * (p % (DV / 4)));
-            }
-            b.gam = wv[(4 * T_GL) / 16 + (tid & 31)];
+        for (int i = 0; i < V_LOADS; i++) {
+            // piece p of the block's [token][DV] values: token p / (DV / 4), four dims (a token past the end: unused, see `place`)
+            const uint32_t p = tid + 256 * i, tok = min(blk * C + p / (DV / 4), a.tokens - 1);
+            b.v[i] = *reinterpret_cast<const u32x4 *>(a.mixed + size_t(tok) * a.channels + 2 * a.k_heads * K_DIM + h * a.v_dim + DV * slice + 4 * (p % (DV / 4)));
         }
+        b.gam = wv[(4 * T_GL) / 16 + (tid & 31)];
     };
     // the block's values (tokens past the end: zeros) and factors to LDS (the first team)
     auto place = [&](uint32_t blk, const ChainBlock &b) {
@@ -486,12 +499,17 @@ __global__ __launch_bounds__(512) void deltanet_chunk_chain_kernel(ChunkArgs a) 
         }
     }
 
-    // One block: `cur` holds its operands; the next block's are asked for now, into `next`, and used a block
-    // later (after the last block: the last block's again, unused).
-    auto step = [&](uint32_t blk, const ChainBlock &cur, ChainBlock &next) {
+    // One block: `cur` holds its operands, `next` those of the block after it (asked for during the block before
+    // this one).  Each lot of `cur`, once read, is asked for again for the block after next: a load has two
+    // blocks' time to come back (one block's time is less than the 2.9 us a wave's batch takes under this load).
+    // (the team is a type, so that a team's blocks are one piece of code: what one team asks for is not taken to be
+    // in flight where the other team waits)
+    auto step = [&](auto team, uint32_t blk, ChainBlock &cur, const ChainBlock &next) {
+        constexpr bool STATE = decltype(team)::value;
         const uint32_t nxt = blk + 1 < nblocks ? blk + 1 : blk;
-        request(nxt, next);
-        if (state_team) {
+        if constexpr (STATE) {
+            request_values(blk + 2, cur);  // (this block's values went to LDS during the block before)
+            __builtin_amdgcn_sched_barrier(0);
             // this wave's rows of the block's keys, for the state's update (the set of two blocks ago is read no more:
             // every wave has been through the three barriers of the block between)
             _Float16 *kimg = img_w(L::KIMG + int(blk & 1) * 2 * K_IMG);
@@ -518,11 +536,14 @@ __global__ __launch_bounds__(512) void deltanet_chunk_chain_kernel(ChunkArgs a) 
                 pkq[vt] = mma3(__builtin_bit_cast(half8, cur.kq[0][ks]), __builtin_bit_cast(half8, cur.kq[1][ks]), bh, bl, pkq[vt]);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
+        request_kq(blk + 2, cur);
+        __builtin_amdgcn_sched_barrier(0);
         // C layout: lane (n, j) holds dv = 16 vt + n of tokens t = 16 wave + 4j + i
         const floatx4 gam4 = *reinterpret_cast<const floatx4 *>(gam + 16 * wave + 4 * j);
         const floatx4 gk4 = *reinterpret_cast<const floatx4 *>(gam + C + 16 * wave + 4 * j);
         const float glast = gam[C - 1];
-        if (state_team) {
+        if constexpr (STATE) {
 #pragma unroll
             for (int vt = 0; vt < NT; vt++) {
                 // R = V - e^c (K S0^T), as the [dv][token] image
@@ -539,7 +560,7 @@ __global__ __launch_bounds__(512) void deltanet_chunk_chain_kernel(ChunkArgs a) 
         }
         __syncthreads();  // R is whole
 
-        if (state_team) {
+        if constexpr (STATE) {
             // ---- U = T R (T is lower triangular: k-steps up to the row tile's own) ----
 #pragma unroll
             for (int vt = 0; vt < NT; vt++) {
@@ -564,10 +585,13 @@ __global__ __launch_bounds__(512) void deltanet_chunk_chain_kernel(ChunkArgs a) 
                 *reinterpret_cast<half4 *>(img_w(L::UH) + at) = uh, *reinterpret_cast<half4 *>(img_w(L::UL) + at) = ul;
                 *reinterpret_cast<half4 *>(img_w(L::WH) + at) = wh, *reinterpret_cast<half4 *>(img_w(L::WL) + at) = wl;
             }
+            __builtin_amdgcn_sched_barrier(0);
+            request_tm(blk + 2, cur);
+            __builtin_amdgcn_sched_barrier(0);
         }
         __syncthreads();  // U is whole; every wave is through with the state's image, the values and the factors
 
-        if (state_team) {
+        if constexpr (STATE) {
             // ---- S1 = e^{c_last} S0 + (U scaled)^T K: rows dv, columns 32 wave + 16 nt + n, over the 64 tokens ----
             // The B operands, K by key dim: lane (n, j) wants column 32 wave + 16 nt + n, tokens 32 ks + 8j .. + 7.
             // ds_read_b64_tr_b16 works on 16 lanes: lane a + 4e of them names 8 bytes (4 values of a row), and lane
@@ -624,34 +648,56 @@ __global__ __launch_bounds__(512) void deltanet_chunk_chain_kernel(ChunkArgs a) 
             place(nxt, next);
         } else {
             // ---- O = (e^c (Q S0^T) + M U) / sqrt(128) ----
+            floatx4 mu[NT];
 #pragma unroll
             for (int vt = 0; vt < NT; vt++) {
-                floatx4 mu = {0, 0, 0, 0};
+                mu[vt] = floatx4{0, 0, 0, 0};
 #pragma unroll
                 for (int ks = 0; ks < 2; ks++) {
                     if (ks > int(wave) / 2) continue;
                     const int bo = (16 * vt + n) * TROW + 32 * ks + 8 * j;
-                    mu = mma3(__builtin_bit_cast(half8, cur.tm[0][ks]), __builtin_bit_cast(half8, cur.tm[1][ks]),
-                              *reinterpret_cast<const half8 *>(img(L::UH) + bo), *reinterpret_cast<const half8 *>(img(L::UL) + bo), mu);
+                    mu[vt] = mma3(__builtin_bit_cast(half8, cur.tm[0][ks]), __builtin_bit_cast(half8, cur.tm[1][ks]),
+                                  *reinterpret_cast<const half8 *>(img(L::UH) + bo), *reinterpret_cast<const half8 *>(img(L::UL) + bo), mu[vt]);
                 }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            request_tm(blk + 2, cur);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int vt = 0; vt < NT; vt++) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const uint32_t tok = blk * C + 16 * wave + 4 * j + i;
-                    if (tok < a.tokens) a.o[(size_t(tok) * a.v_heads + h) * a.v_dim + DV * slice + 16 * vt + n] = Q_SCALE * (gam4[i] * pkq[vt][i] + mu[i]);
+                    if (tok < a.tokens) a.o[(size_t(tok) * a.v_heads + h) * a.v_dim + DV * slice + 16 * vt + n] = Q_SCALE * (gam4[i] * pkq[vt][i] + mu[vt][i]);
                 }
             }
         }
     };
     // (two sets of operand registers that change roles, so that nothing is copied from one to the other)
-    ChainBlock even, odd;
-    request(0, even);
+    auto walk = [&](auto team) {
+        constexpr bool STATE = decltype(team)::value;
+        ChainBlock even, odd;
+        request_kq(0, even), request_tm(0, even);
+        if constexpr (STATE) request_values(0, even);
+        request_kq(1, odd), request_tm(1, odd);
+        if constexpr (STATE) {
+            request_values(1, odd);
+            publish_state();
+            place(0, even);
+        }
+        // (pairs of blocks without a branch between them, so that the loads asked for in one block are known to be
+        // behind those of the block before wherever a wait is placed)
+        uint32_t blk = 0;
+        for (; blk + 1 < nblocks; blk += 2) {
+            step(team, blk, even, odd);
+            step(team, blk + 1, odd, even);
+        }
+        if (blk < nblocks) step(team, blk, even, odd);
+    };
     if (state_team) {
-        publish_state();
-        place(0, even);
-    }
-    for (uint32_t blk = 0; blk < nblocks; blk += 2) {
-        step(blk, even, odd);
-        if (blk + 1 < nblocks) step(blk + 1, odd, even);
+        walk(std::true_type{});
+    } else {
+        walk(std::false_type{});
     }
     if (state_team) {
 #pragma unroll
