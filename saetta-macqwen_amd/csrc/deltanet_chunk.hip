@@ -677,11 +677,12 @@ __global__ __launch_bounds__(512) void deltanet_chunk_chain_kernel(ChunkArgs a) 
     auto walk = [&](auto team) {
         constexpr bool STATE = decltype(team)::value;
         ChainBlock even, odd;
-        request_kq(0, even), request_tm(0, even);
+        // (in the order the blocks ask in, so that the first blocks' waits are those of every block)
         if constexpr (STATE) request_values(0, even);
+        request_kq(0, even), request_tm(0, even);
+        if constexpr (STATE) request_values(1, odd);
         request_kq(1, odd), request_tm(1, odd);
         if constexpr (STATE) {
-            request_values(1, odd);
             publish_state();
             place(0, even);
         }
