@@ -85,9 +85,8 @@ __device__ __forceinline__ floatx4 mma3(half8 ah, half8 al, half8 bh, half8 bl, 
 // ---- prepare: everything of a block that does not depend on the state ------------------------------
 // One workgroup takes G value heads of one key head: the q / k images and the k . k and q . k products
 // belong to the key head, the gates, A, M and T to a value head.  (G = 2, the model's two value heads
-// per key head: the two triangular solves, each a chain of 64 dependent steps, run side by side in the
-// same lanes; G = 1: any other ratio, one workgroup per value head, the first of a key head's writing
-// the key head's images.)
+// per key head: the four waves take the heads' four diagonal blocks of the triangular solve; G = 1: any
+// other ratio, one workgroup per value head, the first of a key head's writing the key head's images.)
 // LDS: the four q / k images; once the products are taken, the heads' A (f32) go over kh | kl, their M
 // images and later their T images over qh | ql (and 2 KB more), so that they leave as whole 16-byte stores.
 template <int G>
