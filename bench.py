@@ -49,7 +49,8 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # rocprofv3 --pmc, each scaled by what the same counter reads for a 256 MiB copy in the same run;
 # the runs are summarised in profiles/*_hbm_traffic.txt).  Counters cannot be read inside this
 # script, so the figures are carried here for the workloads they were measured on.
-MEASURED_TRAFFIC = {"decode8_32k": 38.2e6, "prefill": 296.2e6, "decode4_150k": 91.7e6, "verify4": 45.1e6}
+MEASURED_TRAFFIC = {"decode8_32k": 38.2e6, "prefill": 296.2e6, "decode4_150k": 91.7e6, "verify4": 45.1e6,
+                    "deltanet_prefill": 664.1e6}  # (the three kernels of the chunk together)
 
 
 def median(xs):
@@ -630,7 +631,8 @@ def bench_deltanet_prefill(s, torch, args, tokens=4096):
                    "k_heads": kh, "v_heads": vh, "k_dim": 128, "v_dim": dv, "conv_kernel": kernel,
                    "bytes_rows_launch": rows_bytes, "bytes_conv_launch": conv_bytes},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC.get("deltanet_prefill") if (tokens, kh, vh, dv) == (4096, 16, 32, 128) else None,
                      "kernel": "deltanet_chunk_prepare_kernel + deltanet_chunk_chain_kernel + deltanet_gated_norm_wide_kernel",
                      "avg_us": round(rows_us, 1), "token_chain_TFLOPs": round(flops / rows_us / 1e6, 2)},
         "cpu_baseline": {"value": round(1.0 / cpu_s, 1), "unit": "tokens/s", "cores": 1, "kind": "port",
