@@ -679,6 +679,16 @@ __device__ __forceinline__ void prefill_tile(const PrefillArgs &a, unsigned char
 
     settle(acc);
 
+    // The gate values of this wave's half of the dims, asked for before the merge below so that they travel while
+    // it runs (scattered 16-byte pieces, one round trip for the lot; a token past the end: the last token's, unused).
+    float4 g[16];
+    {
+        const size_t grow = size_t(min(tok, a.tokens - 1)) * a.heads + head;
+        const float *gate = a.q_and_gate + grow * 2 * DIM + DIM + 128 * parity;
+#pragma unroll
+        for (int i = 0; i < 16; i++) g[i] = *reinterpret_cast<const float4 *>(gate + 32 * (i >> 2) + 8 * (i & 3) + 4 * hf);
+    }
+
     // ---- the two waves of a row group merge their halves of the keys ----------------------
     // Each wave finishes half of the dims: parity 0 the accumulators 0..3 (dims 0..127), parity 1
     // the rest.  It hands the other half, m and l to its partner through LDS (the tiles are done
@@ -715,12 +725,7 @@ __device__ __forceinline__ void prefill_tile(const PrefillArgs &a, unsigned char
     if (tok < a.tokens) {
         const float inv = 1.0f / l;
         const size_t row = size_t(tok) * a.heads + head;
-        const float *gate = a.q_and_gate + row * 2 * DIM + DIM + 128 * parity;
         float *out = a.out + row * DIM + 128 * parity;
-        // all the gate loads first: they are scattered 16-byte pieces, one round trip for the lot
-        float4 g[16];
-#pragma unroll
-        for (int i = 0; i < 16; i++) g[i] = *reinterpret_cast<const float4 *>(gate + 32 * (i >> 2) + 8 * (i & 3) + 4 * hf);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             const int mt = i >> 2, q4 = i & 3;
