@@ -350,7 +350,7 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8):
     kern_us = median(ts)
     achieved = flops / (kern_us * 1e-6) / 1e12
     # CPU baseline on a bounded sample: the last `sample` tokens of the chunk (the longest rows).
-    sample = 512  # about 7 s on one core
+    sample = max(16, 512 * 8192 // (pos + tokens))  # 512 tokens at the headline shape: about 7 s on one core
     groups = (pos + tokens) * 8
 
     def deq(rows_q):
@@ -647,7 +647,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="default",
-                    choices=["decode8_32k", "decode4_150k", "decode16_4k", "verify2", "verify3", "verify4", "prefill", "deltanet",
+                    choices=["decode8_32k", "decode4_150k", "decode16_4k", "verify2", "verify3", "verify4", "prefill", "prefill_131k", "deltanet",
                              "deltanet_prefill", "prep_store", "reader_floor", "default", "all"])
     ap.add_argument("--no-graph", action="store_true", help="launch from Python instead of replaying a HIP graph")
     ap.add_argument("--layers", type=int, default=0, help="layer caches per step (default 32; 12 at 150k)")
@@ -693,6 +693,10 @@ def main():
             return bench_prep_store(s, torch, args)
         if workload == "reader_floor":
             return bench_reader_floor(s, torch, args)
+        if workload == "prefill_131k":
+            # the last 4096-token chunk of a 131072-token context: whether the one flash kernel holds up where
+            # the reference switches to its multi-pass form (src/attention_gemm.rs)
+            return bench_prefill(s, torch, args, tokens=4096, pos=131072 - 4096)
         return bench_prefill(s, torch, args)
 
     if args.workload in ("default", "all"):
@@ -704,7 +708,7 @@ def main():
         res["prefill"] = one("prefill")
     if args.workload == "all":
         res["other_workloads"] = {}
-        for w in ["verify2", "verify3", "verify4", "decode4_150k", "decode16_4k", "deltanet", "deltanet_prefill", "prep_store"]:
+        for w in ["verify2", "verify3", "verify4", "decode4_150k", "decode16_4k", "prefill_131k", "deltanet", "deltanet_prefill", "prep_store"]:
             torch.cuda.empty_cache()
             r = one(w)
             res["other_workloads"][w] = {k: r[k] for k in ("metric", "value", "unit", "ms_per_step", "roofline",
