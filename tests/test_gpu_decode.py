@@ -345,3 +345,49 @@ def test_large_cache_of_codes_one_row(kind, capacity):
         worst = np.abs(got - oracle.attention_f64(q, kf, vf, qg, length, threads=8)).max()
         assert worst < MAX_ABS_F64, (length, worst)
         del kc, vc
+
+
+@pytest.mark.parametrize("kind,ctx,m", [(saetta.KvBits.Eight, 32768, 1), (saetta.KvBits.Eight, 32768, 4),
+                                        (saetta.KvBits.Eight, 131072, 1), (saetta.KvBits.Four, 150000, 1),
+                                        (saetta.KvBits.Four, 32768, 3), (saetta.KvBits.Half, 4096, 2)])
+def test_equal_keys_give_the_mean_of_the_values(kind, ctx, m):
+    # A closed form that holds at any size and needs no attention code to check: when every key in the
+    # cache is the same row, every token's score is the same number whatever q is, so row r's output is
+    # the plain mean of the first pos + r + 1 value rows times sigmoid(gate).  A token counted twice, a
+    # share dropped or a merge weighted wrongly moves the mean.  The mean is taken here in f64 over the
+    # values the cache stands for.
+    rng = np.random.default_rng(9000 + ctx % 1000 + m)
+    tokens = ctx - 1 + m
+    capacity = -(-tokens // 128) * 128
+    k = np.tile((rng.standard_normal(VALUES) * 3.0).astype(np.float32), (tokens, 1))
+    v = rng.standard_normal((tokens, VALUES)).astype(np.float32)
+    v[:, 5] += 3.0  # a channel whose mean is far from zero
+    q = rng.standard_normal((m, H, D)).astype(np.float32)
+    qg = rng.standard_normal((m, H, 2 * D)).astype(np.float32)
+    kc, vc, kf, vf = cache_pair(k, v, kind, capacity, poison=True)
+    out = torch.full((m, H, D), float("nan"), device="cuda")
+    pos = ctx - 1
+    plan = saetta.Plan()
+    if m == 1:
+        att = saetta.DecodeAttention(H, KV, D, capacity)
+        if kind is saetta.KvBits.Half:
+            att.record(plan, dev(q[0]), kc, vc, dev(qg[0]), out[0])
+        else:
+            att.record_quant(plan, dev(q[0]), kc, vc, dev(qg[0]), out[0])
+        plan.set_params(saetta.TokenParams(0, pos))
+    else:
+        rows = saetta.AttentionRows(H, KV, capacity, m)
+        params = [saetta.TokenParams(0, pos + r).as_tensor("cuda") for r in range(m)]
+        if kind is saetta.KvBits.Half:
+            rows.record(plan, m, dev(q), kc, vc, dev(qg), out, params)
+        else:
+            rows.record_quant(plan, m, dev(q), kc, vc, dev(qg), out, params)
+    plan.build().run()
+    got = host(out)
+    sums = np.cumsum(vf[pos:tokens].astype(np.float64), axis=0) + vf[:pos].astype(np.float64).sum(axis=0)
+    for r in range(m):
+        mean = (sums[r] / (pos + r + 1)).reshape(KV, D)
+        gate = 1.0 / (1.0 + np.exp(-qg[r].reshape(H, 2 * D)[:, D:].astype(np.float64)))
+        want = np.repeat(mean, H // KV, axis=0) * gate
+        worst = np.abs(got[r] - want).max()
+        assert worst < MAX_ABS_F64, (kind, ctx, m, r, worst)

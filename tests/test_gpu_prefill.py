@@ -181,3 +181,34 @@ def test_spread_rows2_and_bench_mirror_the_reference():
     for bits in (saetta.KvBits.Half, saetta.KvBits.Eight):
         rows = saetta.bench([256, 1000], 2, 3, bits)
         assert [r["tokens"] for r in rows] == [256, 1000] and all(r["GB/s"] > 0 and r["reduce_ms"] > 0 for r in rows)
+
+
+def test_equal_keys_give_running_means_at_full_size():
+    # A closed form for every one of the 4096 x 16 rows of the headline shape: with the same key in every cache
+    # row all scores of a token are equal, so token i's output is the mean of the first pos + i + 1 value rows
+    # (as the half values the cache is read through) times sigmoid(gate), whatever q is.  A key block skipped,
+    # taken twice or masked at the wrong place, or a wrong merge of the two waves of a row group, moves it.
+    pos = tokens = 4096
+    n = pos + tokens
+    kind = saetta.KvBits.Eight
+    gen = torch.Generator(device="cuda").manual_seed(17)
+    krow = torch.randn(VALUES, generator=gen, device="cuda") * 2.0
+    kx = krow.repeat(n, 1).contiguous()
+    vx = torch.randn(n, VALUES, generator=gen, device="cuda")
+    vx[:, 7] += 2.0
+    q16 = torch.randn(tokens, H, D, generator=gen, device="cuda").to(torch.float16)
+    qg = torch.randn(tokens, H, 2 * D, generator=gen, device="cuda")
+    kc, vc = saetta.QuantRows(kind, VALUES, n), saetta.QuantRows(kind, VALUES, n)
+    kc.encode(kx.view(-1), 0, n), vc.encode(vx.view(-1), 0, n)
+    p = saetta.FlashParams(H, KV, pos, tokens, 1.0 / 16)
+    out = torch.full((tokens, H, D), float("nan"), device="cuda")
+    saetta.attention_prefill.encode_quant(q16, kc, vc, qg, out, p)
+    got = host(out)
+    vf = oracle.dequantize(host(vc.data).view(np.uint32), host(vc.scales).view(np.uint16), host(vc.biases).view(np.uint16), 8)
+    vf = vf.reshape(n, VALUES).astype(np.float16).astype(np.float64)
+    sums = np.cumsum(vf[pos:], axis=0) + vf[:pos].sum(axis=0)          # [tokens, 512]
+    means = (sums / (pos + 1 + np.arange(tokens))[:, None]).reshape(tokens, KV, D)
+    gate = 1.0 / (1.0 + np.exp(-host(qg).reshape(tokens, H, 2 * D)[:, :, D:].astype(np.float64)))
+    want = np.repeat(means, H // KV, axis=1) * gate
+    worst = np.abs(got - want).max()
+    assert worst < 2e-5, worst
