@@ -180,6 +180,29 @@ def test_first_row_equals_the_single_token_kernels():
     assert close(host(y[0]), host(y1), 2e-5) and close(host(state), host(state1), 2e-5)
 
 
+def test_full_chunk_against_oracle():
+    # The whole 4096-token chunk of the real shape, one call (64 blocks of 64 tokens on the matrix cores),
+    # against the oracle's token-by-token run: every token's output and the state after the last one.  The
+    # blocks' f16 hi/lo products against the oracle's f32 chain over 4096 dependent steps: outputs to 2e-4,
+    # the state to 1e-4 of the largest entry (the decay keeps rounding from piling up).
+    layer = Layer(16, 32, 128, 4, seed=77)
+    tokens = 4096
+    x, z, a, b = layer.inputs(tokens)
+    conv_cpu = np.zeros((layer.kernel - 1, layer.channels), np.float32)
+    state_cpu = np.zeros(layer.v_heads * layer.v_dim * K_DIM, np.float32)
+    want_y = np.empty((tokens, layer.v_heads * layer.v_dim), np.float32)
+    for t in range(tokens):
+        m = oracle.deltanet_conv(layer.conv_w, x[t], conv_cpu, layer.kernel)
+        want_y[t] = oracle.deltanet_step(m[:layer.key], m[layer.key:2 * layer.key], m[2 * layer.key:], a[t], b[t],
+                                         layer.a_log, layer.dt_bias, state_cpu, z[t], layer.norm, layer.k_heads,
+                                         layer.v_heads, K_DIM, layer.v_dim, EPS).reshape(-1)
+    conv, state = layer.zero_state()
+    _, y, _ = layer.gpu_rows(x, z, a, b, conv, state)
+    assert close(host(y).reshape(tokens, -1), want_y, 2e-4)
+    assert close(host(state).reshape(-1), state_cpu, 1e-4)
+    assert np.array_equal(host(conv), conv_cpu)
+
+
 def test_full_chunk_equals_uneven_pieces():
     # 4096 tokens at the real shape: what a prefill chunk is.  One call (64 blocks of 64 tokens on the
     # matrix cores) against the same tokens in uneven pieces: the short ones run token by token, the
