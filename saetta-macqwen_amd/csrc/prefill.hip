@@ -563,10 +563,14 @@ __device__ __forceinline__ void prefill_tile(const PrefillArgs &a, unsigned char
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[mt][r] = 0.0f;
     }
-    float m_ref = NO_SCORE, l_sum = 0.0f;
+    // The reference maximum starts above what a block of masked scores gives (NO_SCORE * c), so that a row that sees
+    // none of a wave's first block never takes that for its maximum: with m_ref equal to the rounded NO_SCORE * c the
+    // exponent s * c - m_ref of a masked score is the product's rounding error, 1e21 either way, not minus infinity.
+    // (The second wave of a row group starts at block 1: rows that end inside block 0 have nothing in it.)
+    float m_ref = 0.25f * NO_SCORE * c, l_sum = 0.0f;
 
     // Row maximum of a block's scaled scores (first half of the softmax).  Register r of the
-    // accumulator is key 4 hf + r % 4 + 8 (r / 4) of the block; masked scores become NO_SCORE / c.
+    // accumulator is key 4 hf + r % 4 + 8 (r / 4) of the block; masked scores become NO_SCORE (NO_SCORE * c in the units of the maximum).
     auto mask_max = [&](floatx16 &s, uint32_t key0, bool masked) {
         float bm = NO_SCORE;
         if (masked) {

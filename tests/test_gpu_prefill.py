@@ -212,3 +212,24 @@ def test_equal_keys_give_running_means_at_full_size():
     want = np.repeat(means, H // KV, axis=1) * gate
     worst = np.abs(got - want).max()
     assert worst < 2e-5, worst
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("pos", [1, 2, 3, 5, 17, 30, 31])
+def test_chunk_from_a_position_that_splits_a_row_group(kind, pos):
+    # A chunk that starts at a position that is no multiple of 4, early in the cache: in the row group whose
+    # tokens see 30 .. 33 keys some rows end inside key block 0 and others reach block 1, so the wave that
+    # takes the odd blocks meets rows for which its first block is masked whole.
+    rng = np.random.default_rng(600 + pos)
+    tokens = 70
+    n = pos + tokens
+    k = rng.standard_normal((n, VALUES)).astype(np.float32)
+    v = rng.standard_normal((n, VALUES)).astype(np.float32)
+    q16 = rng.standard_normal((tokens, H, D)).astype(np.float16)
+    qg = rng.standard_normal((tokens, H, 2 * D)).astype(np.float32)
+    kc, vc, kf, vf = make_cache(kind, k, v, n + 9, chunk_from=pos)
+    got = run(kind, q16, kc, vc, qg, pos, tokens)
+    assert np.isfinite(got).all()
+    want = oracle.prefill(q16.astype(np.float32), kf, vf, pos, tokens, q_and_gate=qg, threads=8)
+    assert oracle.rel_rms(got, want) < REL_RMS
+    assert np.abs(got - want).max() < MAX_ABS
