@@ -70,9 +70,17 @@ struct ChunkArgs {
     float eps;
 };
 
+// x as an f16 hi part and an f16 lo part.  The lo part has to complete the hi part that is stored: where x is
+// a product, the compiler may round the exact product to f16 for the one and the f32 product for the other, and
+// next to a midpoint between two f16 numbers the two roundings differ by an ulp of the hi part (one value in
+// some thousands: an error of 2^-11 of it instead of 2^-22).  So x is pinned as the f32 number it is, and the
+// hi part as the number that the lo part is taken against.
 __device__ __forceinline__ void split2(float x, _Float16 &hi, _Float16 &lo) {
-    hi = (_Float16)x;
-    lo = (_Float16)(x - (float)hi);
+    asm volatile("" : "+v"(x));
+    float h = (float)(_Float16)x;
+    asm volatile("" : "+v"(h));
+    hi = (_Float16)h;  // (exact)
+    lo = (_Float16)(x - h);
 }
 
 // acc += A B with both operands in hi and lo parts
@@ -100,8 +108,9 @@ struct PrepLds {
     static_assert(2 * H_IMG <= 2 * D_BYTES, "the product's images fit over the diagonal blocks");
     static constexpr int M_BYTES = 2 * T_IMG;  // mh | ml (then th | tl) of a head
     static constexpr int M_OFF = G * HEAD_BYTES > 2 * K_IMG ? G * HEAD_BYTES : 2 * K_IMG;
-    static constexpr int GATES = M_OFF + G * M_BYTES > 4 * K_IMG ? M_OFF + G * M_BYTES : 4 * K_IMG;  // [head][cum | beta][C] f32
-    static constexpr int BYTES = GATES + G * 2 * C * 4;
+    static constexpr int GATES = M_OFF + G * M_BYTES > 4 * K_IMG ? M_OFF + G * M_BYTES : 4 * K_IMG;  // [head]: cum f64 [C] | beta f32 [C]
+    static constexpr int GATE_BYTES = C * 8 + C * 4;
+    static constexpr int BYTES = GATES + G * GATE_BYTES;
     static_assert(2 * BYTES <= 160 * 1024, "two workgroups per CU");
 };
 
@@ -129,8 +138,11 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
     auto diag_lds = [&](int hh, int half) { return reinterpret_cast<float *>(lds + hh * L::HEAD_BYTES + half * L::D_BYTES); };
     auto half_img = [&](int hh, int off) { return reinterpret_cast<_Float16 *>(lds + hh * L::HEAD_BYTES + off); };  // hi part; lo: 32 * HROW on
     auto m_lds = [&](int hh) { return reinterpret_cast<_Float16 *>(lds + L::M_OFF + hh * L::M_BYTES); };
-    auto cum_lds = [&](int hh) { return reinterpret_cast<float *>(lds + L::GATES) + hh * 2 * C; };
-    auto beta_lds = [&](int hh) { return reinterpret_cast<float *>(lds + L::GATES) + hh * 2 * C + C; };
+    // The running sums of log g are kept in f64: the decay between two tokens is e^(c_t - c_s), the sums reach
+    // -100 and beyond inside a block, and an f32 difference of two of them carries the ulp of the sums (1e-5), which
+    // is then the relative error of every entry of A and M: three orders above the rest of this path's arithmetic.
+    auto cum_lds = [&](int hh) { return reinterpret_cast<double *>(lds + L::GATES + hh * L::GATE_BYTES); };
+    auto beta_lds = [&](int hh) { return reinterpret_cast<float *>(lds + L::GATES + hh * L::GATE_BYTES + C * 8); };
     const uint32_t blk = blockIdx.x, group = a.v_heads / a.k_heads;
     const uint32_t h0 = blockIdx.y * G, khd = h0 / group;  // the workgroup's first value head, its key head
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), n = lane & 15, j = lane >> 4;
@@ -198,16 +210,16 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
             fast_gates(a.a[size_t(tok) * a.v_heads + h] + a.dt_bias[h], __expf(a.a_log[h]), a.b[size_t(tok) * a.v_heads + h], g, beta, &lg);
         }
         // inclusive sum over the 64 lanes
-        float c = lg;
+        double c = lg;
 #pragma unroll
         for (int d = 1; d < 64; d *= 2) {
-            const float up = __shfl_up(c, d, 64);
+            const double up = __shfl_up(c, d, 64);
             if (int(lane) >= d) c += up;
         }
         cum_lds(wave)[lane] = c, beta_lds(wave)[lane] = beta;
-        const float last = __shfl(c, 63, 64);
+        const double last = __shfl(c, 63, 64);
         float *gam = reinterpret_cast<float *>(ws_v(wave) + 4 * T_GL);
-        gam[lane] = __expf(c), gam[C + lane] = __expf(last - c);
+        gam[lane] = __expf(float(c)), gam[C + lane] = __expf(float(last - c));
     }
     __syncthreads();
 
@@ -234,11 +246,11 @@ __global__ __launch_bounds__(256) void deltanet_chunk_prepare_kernel(ChunkArgs a
 #pragma unroll
         for (int nt = 0; nt < 4; nt++) {
             const uint32_t s = 16 * nt + n;
-            const float cs = cum_lds(hh)[s];
+            const double cs = cum_lds(hh)[s];
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const uint32_t t = 16 * wave + 4 * j + i;
-                const float decay = s <= t ? __expf(cum_lds(hh)[t] - cs) : 0.0f;
+                const float decay = s <= t ? __expf(float(cum_lds(hh)[t] - cs)) : 0.0f;
                 const float at_s = s < t ? beta_lds(hh)[t] * decay * gk[nt][i] : 0.0f;
                 if ((nt >> 1) == int(wave >> 1)) {  // a diagonal 32 x 32 block, zeros above the diagonal included
                     diag_lds(hh, nt >> 1)[(t & 31) * DROW + (s & 1) * 16 + ((s & 31) >> 1)] = at_s;

@@ -1,14 +1,16 @@
 """Seeded sweeps over shapes the other tests do not name: decode / verify over capacities, context
 lengths, cache kinds and row counts against the f64 formula (the bar of tests/attention.rs), and
 prefill chunks over positions, chunk lengths and cache kinds against the oracle's f32 CPU path (the
-bar of tests/attention_prefill.rs).  The cases are drawn from fixed seeds, so every run sees the
-same ones; rows past the context hold NaN patterns.
+bar of tests/attention_prefill.rs); Gated DeltaNet chunks in blocks of 64 tokens over head counts,
+value dims, conv taps and chunk lengths against the oracle's token-by-token run.  The cases are
+drawn from fixed seeds, so every run sees the same ones; rows past the context hold NaN patterns.
 """
 import numpy as np
 import pytest
 import torch
 
 from gpu_common import D, H, KV, VALUES, cache_pair, dev, host, oracle, saetta
+from test_gpu_deltanet_rows import K_DIM, Layer
 from test_gpu_prefill import make_cache, run as run_prefill
 
 pytestmark = pytest.mark.gpu
@@ -73,3 +75,49 @@ def test_prefill_sweep(seed):
         want = oracle.prefill(q16.astype(np.float32), kf, vf, pos, tokens, q_and_gate=qg, threads=8)
         assert np.isfinite(got).all(), (seed, done, kind, pos, tokens, capacity)
         assert np.abs(got - want).max() < 2e-3 and oracle.rel_rms(got, want) < 1e-3, (seed, done, kind, pos, tokens, capacity)
+
+
+def deltanet_case(k_heads, v_heads, v_dim, kernel, tokens, layer_seed):
+    layer = Layer(k_heads, v_heads, v_dim, kernel, seed=layer_seed)
+    x, z, a, b = layer.inputs(tokens)
+    conv_cpu = np.zeros((layer.kernel - 1, layer.channels), np.float32)
+    state_cpu = np.zeros(layer.v_heads * layer.v_dim * K_DIM, np.float32)
+    _, want_y, _, want_s = layer.cpu_rows(x, z, a, b, conv_cpu, state_cpu)
+    conv, state = layer.zero_state()
+    _, y, _ = layer.gpu_rows(x, z, a, b, conv, state, False)
+    got_y, got_s = host(y).reshape(tokens, -1), host(state).reshape(-1)
+    assert np.isfinite(got_y).all()
+    err_y = float(np.abs(got_y - want_y.reshape(tokens, -1)).max() / max(1.0, np.abs(want_y).max()))
+    err_s = float(np.abs(got_s - want_s[-1]).max() / max(1.0, np.abs(want_s[-1]).max()))
+    return err_y, err_s
+
+
+def test_deltanet_chunk_with_a_product_at_a_rounding_midpoint():
+    # A split of a PRODUCT into f16 hi and lo parts must round one and the same f32 number for both: with hi
+    # from the exact product and lo from the rounded one, an entry whose product falls next to the midpoint of
+    # two f16 values comes out one f16 step off (2^-11 of the entry).  This layer holds such an entry in the
+    # q operand of token 126 of key head 5: that token's outputs were off by 2.5e-4 of the largest output.
+    err_y, err_s = deltanet_case(8, 24, 128, 4, 129, 990136)
+    assert err_y < 2e-5 and err_s < 1e-5, (err_y, err_s)
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_deltanet_chunk_sweep(seed):
+    # Chunks of 128 tokens and more run in blocks of 64 on the matrix cores (f16 hi/lo products, three per
+    # product) against the oracle's f32 chain: 2e-5 of the largest output, 1e-5 of the largest state entry
+    # (measured worst over 1200 such cases: 4e-6 and 7e-7).
+    rng = np.random.default_rng(seed)
+    done = 0
+    while done < 60:
+        k_heads = int(rng.choice([1, 2, 3, 4, 8, 16]))
+        v_heads = k_heads * int(rng.choice([1, 2, 2, 3, 4]))
+        if v_heads > 32:
+            continue
+        v_dim = int(rng.choice([16, 32, 48, 64, 128, 256]))
+        kernel = int(rng.choice([2, 3, 4, 4, 4]))
+        tokens = int(rng.choice([128, 129, 191, 192, 193, 256, 300, int(rng.integers(128, 420))]))
+        tokens = max(128, min(tokens, 32 * 128 * 300 // (v_heads * v_dim)))
+        layer_seed = int(rng.integers(1 << 20))
+        err_y, err_s = deltanet_case(k_heads, v_heads, v_dim, kernel, tokens, layer_seed)
+        assert err_y < 2e-5 and err_s < 1e-5, (seed, done, k_heads, v_heads, v_dim, kernel, tokens, layer_seed, err_y, err_s)
+        done += 1
