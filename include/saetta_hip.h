@@ -411,6 +411,37 @@ int saetta_attn_prefill_quant(saetta_stream_t stream, int bits, const uint16_t *
                               const float *q_and_gate, float *out, saetta_flash_params p,
                               void *workspace, size_t workspace_bytes);
 
+/* ---- prefill attention as matrix products (src/attention_gemm.rs) ----------- */
+
+/* attention_gemm::KEYS (src/attention_gemm.rs:28): keys per block. */
+#define SAETTA_AG_KEYS 1024
+
+/* Bytes of workspace AttGemm needs for a chunk at (pos, tokens) run in slices
+ * of up to slice_tokens tokens (0: one slice): the key and value tile images
+ * of saetta_prefill_workspace_bytes, then what AttGemm::new allocates for one
+ * slice (src/attention_gemm.rs:118-142): a block's probabilities, the tile
+ * maxima and sums, the output sums and the per-row softmax state; about 3.3 KB
+ * per query row of a slice. */
+size_t saetta_attn_gemm_workspace_bytes(uint32_t pos, uint32_t tokens, uint32_t slice_tokens,
+                                        uint32_t kv_heads);
+
+/* AttGemm::encode (src/attention_gemm.rs:144-188, encode_slice :190-364), the
+ * default (fused) variant: the same chunk and the same buffers as
+ * saetta_attn_prefill / saetta_attn_prefill_quant, computed block by block of
+ * SAETTA_AG_KEYS keys with the block's probabilities written out and read
+ * back.  bits 16: keys.data and values.data are the half caches and the scales
+ * and biases are not read (the reference's quant = None); bits 8 or 4: the
+ * quantized rows, seen through half.  stages (AttGemm::stages,
+ * src/attention_gemm.rs:112-114): 0 runs everything; 1 or 2 only the scores
+ * pass of each block; 3 scores and pv and no outputs.  workspace as for
+ * saetta_attn_prefill, of saetta_attn_gemm_workspace_bytes bytes.  Kernels
+ * replaced: prefill_ag_scores_t{,_q8,_q4}, prefill_ag_pv_t{,_q8,_q4},
+ * prefill_ag_final (kernels/attention_gemm.metal). */
+int saetta_attn_gemm(saetta_stream_t stream, int bits, const uint16_t *q_f16, saetta_quant_rows keys,
+                     saetta_quant_rows values, const float *q_and_gate, float *out,
+                     saetta_flash_params p, uint32_t slice_tokens, uint32_t stages, void *workspace,
+                     size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -11,12 +11,12 @@ be checked), every call needs the library and a gfx950 device.
 from . import ffi
 from .host import (GROUP, KV_ALIGN, MAX_ROWS, AttentionRows, Built, DecodeAttention, FlashParams, GpuKvCache, KvBits,
                    Plan, RowBackup,
-                   PrepParams, QuantRows, TokenParams, attention_prefill, bench, deltanet_conv, deltanet_conv_rows, deltanet_rows, deltanet_rows_fused, deltanet_token,
+                   PrepParams, QuantRows, TokenParams, attention_gemm, attention_prefill, bench, deltanet_conv, deltanet_conv_rows, deltanet_rows, deltanet_rows_fused, deltanet_token,
                    deltanet_step, dequantize, quantize, round_trip,
                    record_store, round_trip_as_half, test_slack, to_half)
 
 __all__ = ["ffi", "GROUP", "KV_ALIGN", "MAX_ROWS", "AttentionRows", "Built", "DecodeAttention", "FlashParams",
            "GpuKvCache", "KvBits", "RowBackup",
-           "Plan", "PrepParams", "QuantRows", "TokenParams", "attention_prefill", "bench", "deltanet_conv", "deltanet_conv_rows",
+           "Plan", "PrepParams", "QuantRows", "TokenParams", "attention_gemm", "attention_prefill", "bench", "deltanet_conv", "deltanet_conv_rows",
            "deltanet_rows", "deltanet_rows_fused", "deltanet_token", "deltanet_step", "dequantize", "quantize",
            "record_store", "round_trip", "round_trip_as_half", "test_slack", "to_half"]

@@ -778,10 +778,10 @@ size_t workspace_bytes(uint32_t pos, uint32_t tokens, uint32_t kv_heads) {
     return blocks * kv_heads * IMG_BYTES;
 }
 
-int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kdata, const void *vdata,
-                const uint16_t *ks, const uint16_t *kz, const uint16_t *vs, const uint16_t *vz,
-                const float *q_and_gate, float *out, saetta_flash_params p, void *workspace, size_t workspace_size,
-                const char *what) {
+// The checks both prefill paths share.
+int check_prefill(int bits, const uint16_t *q, const void *kdata, const void *vdata, const uint16_t *ks,
+                  const uint16_t *kz, const uint16_t *vs, const uint16_t *vz, const float *q_and_gate, const float *out,
+                  saetta_flash_params p, const void *workspace, const char *what) {
     SAETTA_REQUIRE(bits == 16 || bits == 8 || bits == 4, SAETTA_E_BITS, "%s: bits %d", what, bits);
     SAETTA_REQUIRE(p.kv_heads > 0 && p.heads == p.kv_heads * SAETTA_GQA_GROUP, SAETTA_E_SHAPE,
                    "%s needs 8 q heads per kv head (heads %u, kv heads %u)", what, p.heads, p.kv_heads);
@@ -793,45 +793,54 @@ int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kda
     const uint64_t rows = uint64_t(p.pos) + p.tokens;  // the cache holds the chunk's rows too
     SAETTA_REQUIRE(rows * p.kv_heads * 512 < (uint64_t(1) << 31), SAETTA_E_SHAPE, "%s: pos + tokens %llu out of range",
                    what, (unsigned long long)rows);
-    if (int rc = ensure_device()) return rc;
-    if (p.tokens == 0) return SAETTA_OK;
-    const size_t need = workspace_bytes(p.pos, p.tokens, p.kv_heads);
-    // The library's own workspace is held under its lock until the launches that use it are queued:
-    // a second host thread that has to grow it waits for them (hipDeviceSynchronize) before it frees.
-    std::unique_lock<std::mutex> owned_lock(g_owned_mutex, std::defer_lock);
+    return SAETTA_OK;
+}
+
+// The caller's workspace if it gave one of at least `need` bytes, else the library's own, grown to `need`.
+// The library's own is held under its lock until the launches that use it are queued (the caller keeps
+// `owned_lock` until then): a second host thread that has to grow it waits for them (hipDeviceSynchronize)
+// before it frees.
+int acquire_workspace(hipStream_t stream, void *&workspace, size_t workspace_size, size_t need,
+                      std::unique_lock<std::mutex> &owned_lock, const char *what, const char *sizer) {
     if (workspace) {
         SAETTA_REQUIRE(workspace_size >= need, SAETTA_E_SCRATCH, "%s: workspace of %zu bytes, %zu needed", what,
                        workspace_size, need);
-    } else {
-        // No workspace given: use (and grow) the library's own.  This may allocate, which a stream
-        // under capture cannot do; work queued on other streams must not share it.
-        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) (void)hipGetLastError();
-        SAETTA_REQUIRE(capturing == hipStreamCaptureStatusNone, SAETTA_E_SCRATCH,
-                       "%s: a stream under capture needs a workspace of the caller's (%zu bytes, saetta_prefill_workspace_bytes)",
-                       what, need);
-        int dev = 0;
-        if (hipError_t e = hipGetDevice(&dev)) return fail(int(e), "%s: %s", what, hipGetErrorString(e));
-        SAETTA_REQUIRE(dev >= 0 && dev < OWNED_DEVICES, SAETTA_E_DEVICE, "%s: device index %d (up to %d)", what, dev, OWNED_DEVICES - 1);
-        owned_lock.lock();
-        OwnedWorkspace &w = g_owned[dev];
-        if (w.bytes < need) {
-            if (w.ptr) {
-                (void)hipDeviceSynchronize();
-                (void)hipFree(w.ptr);
-            }
-            w.ptr = nullptr;
-            w.bytes = 0;
-            hipError_t e = hipMalloc(&w.ptr, need);
-            if (e != hipSuccess) return fail(int(e), "%s: workspace of %zu bytes: %s", what, need, hipGetErrorString(e));
-            w.bytes = need;
-        }
-        workspace = w.ptr;
+        return SAETTA_OK;
     }
+    // No workspace given: use (and grow) the library's own.  This may allocate, which a stream
+    // under capture cannot do; work queued on other streams must not share it.
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) (void)hipGetLastError();
+    SAETTA_REQUIRE(capturing == hipStreamCaptureStatusNone, SAETTA_E_SCRATCH,
+                   "%s: a stream under capture needs a workspace of the caller's (%zu bytes, %s)", what, need, sizer);
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev)) return fail(int(e), "%s: %s", what, hipGetErrorString(e));
+    SAETTA_REQUIRE(dev >= 0 && dev < OWNED_DEVICES, SAETTA_E_DEVICE, "%s: device index %d (up to %d)", what, dev, OWNED_DEVICES - 1);
+    owned_lock.lock();
+    OwnedWorkspace &w = g_owned[dev];
+    if (w.bytes < need) {
+        if (w.ptr) {
+            (void)hipDeviceSynchronize();
+            (void)hipFree(w.ptr);
+        }
+        w.ptr = nullptr;
+        w.bytes = 0;
+        hipError_t e = hipMalloc(&w.ptr, need);
+        if (e != hipSuccess) return fail(int(e), "%s: workspace of %zu bytes: %s", what, need, hipGetErrorString(e));
+        w.bytes = need;
+    }
+    workspace = w.ptr;
+    return SAETTA_OK;
+}
+
+// The images of rows 0 .. rows - 1 of the cache, at the start of the workspace.
+uint32_t launch_prepare(hipStream_t stream, int bits, const void *kdata, const void *vdata, const uint16_t *ks,
+                        const uint16_t *kz, const uint16_t *vs, const uint16_t *vz, void *workspace, uint32_t kv_heads,
+                        uint64_t rows) {
     const uint32_t nblocks = uint32_t((rows + BK - 1) / BK);
-    PrepareArgs pa{kdata, vdata, ks, kz, vs, vz, static_cast<unsigned char *>(workspace), p.kv_heads, nblocks,
+    PrepareArgs pa{kdata, vdata, ks, kz, vs, vz, static_cast<unsigned char *>(workspace), kv_heads, nblocks,
                    uint32_t(rows)};
-    const dim3 pgrid(nblocks, p.kv_heads);
+    const dim3 pgrid(nblocks, kv_heads);
     if (bits == 8) {
         prefill_prepare_kernel<8><<<pgrid, PREP_THREADS, 0, stream>>>(pa);
     } else if (bits == 4) {
@@ -839,6 +848,21 @@ int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kda
     } else {
         prefill_prepare_kernel<16><<<pgrid, PREP_THREADS, 0, stream>>>(pa);
     }
+    return nblocks;
+}
+
+int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kdata, const void *vdata,
+                const uint16_t *ks, const uint16_t *kz, const uint16_t *vs, const uint16_t *vz,
+                const float *q_and_gate, float *out, saetta_flash_params p, void *workspace, size_t workspace_size,
+                const char *what) {
+    if (int rc = check_prefill(bits, q, kdata, vdata, ks, kz, vs, vz, q_and_gate, out, p, workspace, what)) return rc;
+    const uint64_t rows = uint64_t(p.pos) + p.tokens;
+    if (int rc = ensure_device()) return rc;
+    if (p.tokens == 0) return SAETTA_OK;
+    const size_t need = workspace_bytes(p.pos, p.tokens, p.kv_heads);
+    std::unique_lock<std::mutex> owned_lock(g_owned_mutex, std::defer_lock);
+    if (int rc = acquire_workspace(stream, workspace, workspace_size, need, owned_lock, what, "saetta_prefill_workspace_bytes")) return rc;
+    const uint32_t nblocks = launch_prepare(stream, bits, kdata, vdata, ks, kz, vs, vz, workspace, p.kv_heads, rows);
     PrefillArgs a{q, static_cast<const unsigned char *>(workspace), q_and_gate, out, p.heads, p.kv_heads, p.pos,
                   p.tokens, p.scale, nblocks};
     // one workgroup per CU at most: a workgroup's LDS ring fills a CU, and further tiles are taken in the kernel
@@ -852,10 +876,328 @@ int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kda
     return launch_status(what);
 }
 
+// ---- the same chunk as matrix products over blocks of 1024 keys ---------------------------------
+// (reference: AttGemm, src/attention_gemm.rs:95-364, its default variant: prefill_ag_scores_t,
+// prefill_ag_pv_t and prefill_ag_final of kernels/attention_gemm.metal.)  The reference's other route to
+// the same output: the keys are walked in blocks of 1024; for a block, one launch writes the
+// probabilities of every query row against the block's keys to a scratch, relative to the maximum of
+// each tile of keys, with the tile's maximum and sum beside them, and a second launch folds the block
+// into the running (m, l, O) of every row: O = alpha O + sum over tiles of e^(t - m) (P_tile V_tile).
+// The scratch is for one slice of the chunk's tokens; the slices run one after the other.
+//
+// Here a tile is 32 keys (one key image), a row group is 4 tokens x 8 heads as above, and a workgroup is
+// 4 waves with a row group each (a 16-token tile).  Both kernels take the image parts through LDS (the
+// next tile's part is fetched into registers while the current one is used; one barrier a tile) and run
+// the same transposed products as the flash kernel, so a lane owns a query row in both:
+//   scores   S^T = K Q^T (Q^T in registers), mask, tile maximum and sum per row, P = 2^(s - t) as f16,
+//            stored as the P^T operands of the second product (the accumulator's registers 8 sp .. 8 sp + 7
+//            are the operand of k-step sp: 1 KB per wave and k-step, read back as it was written);
+//   pv       m' = max(m, max_t t), O^T = alpha O^T + sum_t V^T_t (f_t P^T_t) with f_t = 2^(t - m') rounded
+//            to f16 (the row sum takes the same rounded f_t), one workgroup per half of the dims; the
+//            block that holds a tile's last visible key writes out = O / l * sigmoid(gate) instead of O.
+constexpr int AG_KEYS = SAETTA_AG_KEYS;
+constexpr int AG_TILES = AG_KEYS / BK;
+constexpr int AG_WAVES = 4;
+constexpr int AG_THREADS = 64 * AG_WAVES;
+constexpr int AG_TOKENS = 4 * AG_WAVES;   // tokens of a workgroup
+constexpr int AG_SPLIT = 4;               // scores: workgroups that share a block's tiles for one token tile
+constexpr int AG_P_TILE_BYTES = BK * 32 * 2;  // the P^T operands of one row group and tile of keys
+
+struct GemmArgs {
+    const uint16_t *q;
+    const unsigned char *images;
+    const float *q_and_gate;
+    float *out;
+    unsigned char *p;    // f16 [kv head][row group][tile][2 k-steps][64 lanes][8]
+    float *tmax, *tsum;  // [kv head][row group][tile][32 rows], log2 domain
+    float *o;            // [kv head][row group][8 dim tiles][4][64 lanes][4]: the accumulators as they are
+    float *m, *l;        // [dim half][kv head][row group][32 rows]
+    uint32_t heads, kv_heads, pos, tokens;  // of the slice
+    float c;             // scale * log2(e)
+    uint32_t nblocks;    // images per kv head
+    uint32_t row_groups; // per kv head in the scratch
+    uint32_t j0;         // the block's first key
+    uint32_t write_out;  // 0: the outputs are never written (timing the passes apart)
+};
+
+// Key of the last token of the workgroup's token tile, and how many of the block's tiles hold keys that
+// some token of the tile can see.
+__device__ __forceinline__ uint32_t ag_last_key(const GemmArgs &a, uint32_t tok0) {
+    const uint32_t end = tok0 + AG_TOKENS < a.tokens ? tok0 + AG_TOKENS : a.tokens;
+    return a.pos + end - 1;
+}
+__device__ __forceinline__ uint32_t ag_tiles(const GemmArgs &a, uint32_t tok0) {
+    const uint32_t last_key = ag_last_key(a, tok0);
+    if (last_key < a.j0) return 0;
+    const uint32_t n = (last_key - a.j0) / BK + 1;
+    return n < uint32_t(AG_TILES) ? n : uint32_t(AG_TILES);
+}
+
+__global__ __launch_bounds__(AG_THREADS) void attention_gemm_scores_kernel(GemmArgs a) {
+    __shared__ __attribute__((aligned(1024))) unsigned char k_lds[2][PART_BYTES];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 31, hf = lane >> 5;
+    const uint32_t tok0 = blockIdx.y * AG_TOKENS, kv = blockIdx.z;
+    const uint32_t need = ag_tiles(a, tok0);
+    constexpr uint32_t PER = AG_TILES / AG_SPLIT;
+    const uint32_t first = blockIdx.x * PER;
+    if (first >= need) return;  // (the whole workgroup)
+    const uint32_t count = need - first < PER ? need - first : PER;
+    const uint32_t rg = blockIdx.y * AG_WAVES + wave;
+    const uint32_t tok = tok0 + 4 * wave + (col >> 3), head = kv * SAETTA_GQA_GROUP + (col & 7);
+
+    // Q^T operands: lane (col, hf) holds dims 16 f + 8 hf .. + 7 of query row col
+    half8 qf[16];
+    if (tok < a.tokens) {
+        const half8 *qp = reinterpret_cast<const half8 *>(a.q + (size_t(tok) * a.heads + head) * DIM) + hf;
+#pragma unroll
+        for (int f = 0; f < 16; f++) qf[f] = qp[2 * f];
+    } else {
+#pragma unroll
+        for (int f = 0; f < 16; f++) qf[f] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+
+    const unsigned char *img = a.images + (size_t(kv) * a.nblocks + a.j0 / BK + first) * IMG_BYTES;
+    u32x4 pre[4];
+    auto fetch = [&](uint32_t t) {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(img + size_t(t) * IMG_BYTES);
+#pragma unroll
+        for (int i = 0; i < 4; i++) pre[i] = src[tid + AG_THREADS * i];
+    };
+    fetch(0);
+    const uint32_t limit = a.pos + tok;  // the last key the row sees
+    const size_t row_base = (size_t(kv) * a.row_groups + rg) * AG_TILES;
+    for (uint32_t t = 0; t < count; t++) {
+        unsigned char *buf = k_lds[t & 1];
+#pragma unroll
+        for (int i = 0; i < 4; i++) reinterpret_cast<u32x4 *>(buf)[tid + AG_THREADS * i] = pre[i];
+        __syncthreads();
+        if (t + 1 < count) fetch(t + 1);
+        floatx16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[i] = 0.0f;
+#pragma unroll
+        for (int f = 0; f < 16; f++) {
+            const half8 kf = *reinterpret_cast<const half8 *>(buf + f * 1024 + lane * 16);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[f], acc, 0, 0, 0);
+        }
+        // register i is key 8 (i / 4) + 4 hf + i % 4 of the tile
+        const uint32_t key0 = a.j0 + (first + t) * BK + 4 * hf;
+        float s[16], tmax = NO_SCORE;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const uint32_t key = key0 + 8 * (i >> 2) + (i & 3);
+            s[i] = key <= limit ? acc[i] * a.c : NO_SCORE;
+            tmax = fmaxf(tmax, s[i]);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        half8 p0, p1;
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            // (a masked score is never exponentiated: with the whole tile masked s - tmax would be 0)
+            const _Float16 ph = (_Float16)(s[i] > 0.5f * NO_SCORE ? __builtin_amdgcn_exp2f(s[i] - tmax) : 0.0f);
+            sum += (float)ph;  // the sum of what the second product multiplies
+            if (i < 8) p0[i] = ph; else p1[i - 8] = ph;
+        }
+        sum += __shfl_xor(sum, 32);
+        unsigned char *pt = a.p + (row_base + first + t) * AG_P_TILE_BYTES + lane * 16;
+        *reinterpret_cast<half8 *>(pt) = p0;
+        *reinterpret_cast<half8 *>(pt + 1024) = p1;
+        if (hf == 0) {
+            a.tmax[(row_base + first + t) * 32 + col] = tmax;
+            a.tsum[(row_base + first + t) * 32 + col] = sum;
+        }
+    }
+}
+
+__global__ __launch_bounds__(AG_THREADS) void attention_gemm_pv_kernel(GemmArgs a) {
+    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2][PART_BYTES / 2];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 31, hf = lane >> 5;
+    const uint32_t dh = blockIdx.x, tok0 = blockIdx.y * AG_TOKENS, kv = blockIdx.z;
+    const uint32_t need = ag_tiles(a, tok0);
+    if (need == 0) return;  // the tile sees nothing of this block (its outputs were written at an earlier one)
+    const bool last_block = ag_last_key(a, tok0) < a.j0 + AG_KEYS;
+    const uint32_t rg = blockIdx.y * AG_WAVES + wave;
+    const uint32_t tok = tok0 + 4 * wave + (col >> 3), head = kv * SAETTA_GQA_GROUP + (col & 7);
+    const size_t rows = size_t(kv) * a.row_groups + rg;
+    const size_t state = (size_t(dh) * a.kv_heads * a.row_groups + rows) * 32 + col;
+    const bool first_block = a.j0 == 0;
+
+    const float *tm = a.tmax + rows * AG_TILES * 32 + col, *ts = a.tsum + rows * AG_TILES * 32 + col;
+    float mb = NO_SCORE;
+    for (uint32_t t = 0; t < need; t++) mb = fmaxf(mb, tm[t * 32]);
+    // (every row sees key 0, so m is a score from the first block on)
+    const float m_old = first_block ? NO_SCORE : a.m[state], l_old = first_block ? 0.0f : a.l[state];
+    const float m_new = fmaxf(m_old, mb);
+    const float alpha = first_block ? 0.0f : __builtin_amdgcn_exp2f(m_old - m_new);
+
+    floatx16 acc[4];
+    float *op = a.o + (rows * 8 + 4 * dh) * 1024 + lane * 4;
+    if (first_block) {
+#pragma unroll
+        for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[mt][i] = 0.0f;
+    } else {
+#pragma unroll
+        for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) {
+                const floatx4 x = *reinterpret_cast<const floatx4 *>(op + (mt * 4 + q4) * 256);
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[mt][4 * q4 + e] = x[e] * alpha;
+            }
+    }
+
+    // the V^T part of an image, this half of the dims: fragments 8 dh .. 8 dh + 7
+    const unsigned char *img = a.images + (size_t(kv) * a.nblocks + a.j0 / BK) * IMG_BYTES + PART_BYTES + dh * (PART_BYTES / 2);
+    u32x4 pre[2];
+    auto fetch = [&](uint32_t t) {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(img + size_t(t) * IMG_BYTES);
+#pragma unroll
+        for (int i = 0; i < 2; i++) pre[i] = src[tid + AG_THREADS * i];
+    };
+    const unsigned char *pp = a.p + rows * AG_TILES * AG_P_TILE_BYTES + lane * 16;
+    half8 pn0, pn1;
+    float tmn, tsn;
+    auto fetch_p = [&](uint32_t t) {
+        pn0 = *reinterpret_cast<const half8 *>(pp + size_t(t) * AG_P_TILE_BYTES);
+        pn1 = *reinterpret_cast<const half8 *>(pp + size_t(t) * AG_P_TILE_BYTES + 1024);
+        tmn = tm[t * 32], tsn = ts[t * 32];
+    };
+    fetch(0);
+    fetch_p(0);
+    float lsum = 0.0f;
+    for (uint32_t t = 0; t < need; t++) {
+        unsigned char *buf = v_lds[t & 1];
+#pragma unroll
+        for (int i = 0; i < 2; i++) reinterpret_cast<u32x4 *>(buf)[tid + AG_THREADS * i] = pre[i];
+        __syncthreads();
+        half8 pc0 = pn0, pc1 = pn1;
+        const float tmc = tmn, tsc = tsn;
+        if (t + 1 < need) {
+            fetch(t + 1);
+            fetch_p(t + 1);
+        }
+        // a tile the row sees nothing of has t = NO_SCORE: its factor is 0, like its probabilities
+        const _Float16 fh = (_Float16)__builtin_amdgcn_exp2f(tmc - m_new);
+        lsum += (float)fh * tsc;
+        pc0 *= fh, pc1 *= fh;
+#pragma unroll
+        for (int mt = 0; mt < 4; mt++) {
+            const half8 v0 = *reinterpret_cast<const half8 *>(buf + (2 * mt) * 1024 + lane * 16);
+            const half8 v1 = *reinterpret_cast<const half8 *>(buf + (2 * mt + 1) * 1024 + lane * 16);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(v0, pc0, acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(v1, pc1, acc[mt], 0, 0, 0);
+        }
+    }
+    const float l_new = alpha * l_old + lsum;
+
+    if (last_block && a.write_out) {
+        if (tok < a.tokens) {
+            const float inv = 1.0f / l_new;
+            const size_t row = size_t(tok) * a.heads + head;
+            const float *gate = a.q_and_gate + row * 2 * DIM + DIM + 128 * dh + 4 * hf;
+            float *out = a.out + row * DIM + 128 * dh + 4 * hf;
+            floatx4 g[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) g[i] = *reinterpret_cast<const floatx4 *>(gate + 32 * (i >> 2) + 8 * (i & 3));
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int mt = i >> 2, q4 = i & 3;
+                floatx4 w;
+#pragma unroll
+                for (int e = 0; e < 4; e++) w[e] = acc[mt][4 * q4 + e] * inv * __builtin_amdgcn_rcpf(1.0f + __expf(-g[i][e]));
+                *reinterpret_cast<floatx4 *>(out + 32 * mt + 8 * q4) = w;
+            }
+        }
+        return;
+    }
+    if (hf == 0) a.m[state] = m_new, a.l[state] = l_new;
+#pragma unroll
+    for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+            floatx4 x;
+#pragma unroll
+            for (int e = 0; e < 4; e++) x[e] = acc[mt][4 * q4 + e];
+            *reinterpret_cast<floatx4 *>(op + (mt * 4 + q4) * 256) = x;
+        }
+}
+
+size_t align_up(size_t n, size_t a) { return (n + a - 1) / a * a; }
+
+// Row groups of the scratch per kv head for slices of up to `slice` tokens: whole workgroups.
+size_t gemm_row_groups(uint32_t slice) { return size_t((slice + AG_TOKENS - 1) / AG_TOKENS) * AG_WAVES; }
+
+size_t gemm_scratch_bytes(uint32_t slice, uint32_t kv_heads) {
+    const size_t groups = gemm_row_groups(slice) * kv_heads;
+    return groups * (size_t(AG_TILES) * AG_P_TILE_BYTES + 2 * size_t(AG_TILES) * 32 * 4 + 32 * size_t(DIM) * 4 + 2 * 2 * 32 * 4);
+}
+
+uint32_t gemm_slice(uint32_t tokens, uint32_t slice_tokens) {
+    return slice_tokens == 0 || slice_tokens > tokens ? tokens : slice_tokens;
+}
+
+size_t gemm_workspace_bytes(uint32_t pos, uint32_t tokens, uint32_t slice_tokens, uint32_t kv_heads) {
+    return align_up(workspace_bytes(pos, tokens, kv_heads), 256) + gemm_scratch_bytes(gemm_slice(tokens, slice_tokens), kv_heads);
+}
+
+int run_gemm(hipStream_t stream, int bits, const uint16_t *q, const void *kdata, const void *vdata, const uint16_t *ks,
+             const uint16_t *kz, const uint16_t *vs, const uint16_t *vz, const float *q_and_gate, float *out,
+             saetta_flash_params p, uint32_t slice_tokens, uint32_t stages, void *workspace, size_t workspace_size) {
+    const char *what = "attn_gemm";
+    if (int rc = check_prefill(bits, q, kdata, vdata, ks, kz, vs, vz, q_and_gate, out, p, workspace, what)) return rc;
+    SAETTA_REQUIRE(stages <= 3, SAETTA_E_SHAPE, "%s: stages %u (0: all passes; 1, 2: scores only; 3: no outputs)", what, stages);
+    const uint64_t rows = uint64_t(p.pos) + p.tokens;
+    if (int rc = ensure_device()) return rc;
+    if (p.tokens == 0) return SAETTA_OK;
+    const uint32_t slice = gemm_slice(p.tokens, slice_tokens);
+    const size_t need = gemm_workspace_bytes(p.pos, p.tokens, slice, p.kv_heads);
+    std::unique_lock<std::mutex> owned_lock(g_owned_mutex, std::defer_lock);
+    if (int rc = acquire_workspace(stream, workspace, workspace_size, need, owned_lock, what, "saetta_attn_gemm_workspace_bytes")) return rc;
+    const uint32_t nblocks = launch_prepare(stream, bits, kdata, vdata, ks, kz, vs, vz, workspace, p.kv_heads, rows);
+
+    const size_t groups = gemm_row_groups(slice) * p.kv_heads;
+    unsigned char *at = static_cast<unsigned char *>(workspace) + align_up(workspace_bytes(p.pos, p.tokens, p.kv_heads), 256);
+    GemmArgs a{};
+    a.images = static_cast<const unsigned char *>(workspace);
+    a.p = at, at += groups * AG_TILES * AG_P_TILE_BYTES;
+    a.tmax = reinterpret_cast<float *>(at), at += groups * AG_TILES * 32 * 4;
+    a.tsum = reinterpret_cast<float *>(at), at += groups * AG_TILES * 32 * 4;
+    a.o = reinterpret_cast<float *>(at), at += groups * 32 * DIM * 4;
+    a.m = reinterpret_cast<float *>(at), at += 2 * groups * 32 * 4;
+    a.l = reinterpret_cast<float *>(at);
+    a.heads = p.heads, a.kv_heads = p.kv_heads;
+    a.c = p.scale * 1.4426950408889634f;
+    a.nblocks = nblocks;
+    a.row_groups = uint32_t(gemm_row_groups(slice));
+    a.write_out = stages == 0;
+    const size_t width = size_t(p.heads) * DIM;
+    // A slice of tokens is a chunk of its own at pos + t0: its rows of q, q_and_gate and out, the whole
+    // cache (src/attention_gemm.rs:162-188).
+    for (uint32_t t0 = 0; t0 < p.tokens; t0 += slice) {
+        a.tokens = p.tokens - t0 < slice ? p.tokens - t0 : slice;
+        a.pos = p.pos + t0;
+        a.q = q + t0 * width, a.q_and_gate = q_and_gate + t0 * width * 2, a.out = out + t0 * width;
+        const uint32_t tiles = (a.tokens + AG_TOKENS - 1) / AG_TOKENS;
+        const uint64_t end = uint64_t(a.pos) + a.tokens;
+        for (uint64_t j0 = 0; j0 < end; j0 += AG_KEYS) {
+            a.j0 = uint32_t(j0);
+            attention_gemm_scores_kernel<<<dim3(AG_SPLIT, tiles, p.kv_heads), AG_THREADS, 0, stream>>>(a);
+            if (stages == 1 || stages == 2) continue;
+            attention_gemm_pv_kernel<<<dim3(2, tiles, p.kv_heads), AG_THREADS, 0, stream>>>(a);
+        }
+    }
+    return launch_status(what);
+}
+
 }  // namespace
 
 int setup_prefill() {
     if (int rc = load_kernel(reinterpret_cast<const void *>(attention_prefill_kernel))) return rc;
+    if (int rc = load_kernel(reinterpret_cast<const void *>(attention_gemm_scores_kernel))) return rc;
+    if (int rc = load_kernel(reinterpret_cast<const void *>(attention_gemm_pv_kernel))) return rc;
     return int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_prefill_kernel),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
 }
@@ -882,4 +1224,15 @@ extern "C" int saetta_attn_prefill_quant(saetta_stream_t stream, int bits, const
     return run_prefill(as_stream(stream), bits, q_f16, keys.data, values.data, keys.scales, keys.biases,
                        values.scales, values.biases, q_and_gate, out, p, workspace, workspace_bytes,
                        "attn_prefill_quant");
+}
+
+extern "C" size_t saetta_attn_gemm_workspace_bytes(uint32_t pos, uint32_t tokens, uint32_t slice_tokens, uint32_t kv_heads) {
+    return gemm_workspace_bytes(pos, tokens, slice_tokens, kv_heads);
+}
+
+extern "C" int saetta_attn_gemm(saetta_stream_t stream, int bits, const uint16_t *q_f16, saetta_quant_rows keys,
+                                saetta_quant_rows values, const float *q_and_gate, float *out, saetta_flash_params p,
+                                uint32_t slice_tokens, uint32_t stages, void *workspace, size_t workspace_bytes) {
+    return run_gemm(as_stream(stream), bits, q_f16, keys.data, values.data, keys.scales, keys.biases, values.scales,
+                    values.biases, q_and_gate, out, p, slice_tokens, stages, workspace, workspace_bytes);
 }

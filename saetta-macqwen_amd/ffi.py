@@ -10,6 +10,7 @@ SYMBOLS = [
     "saetta_init", "saetta_last_error", "saetta_kv_quantize", "saetta_kv_dequantize", "saetta_kv_dequantize_f32", "saetta_to_half", "saetta_attn_prep_store", "saetta_deltanet_conv", "saetta_deltanet_step", "saetta_deltanet_conv_rows", "saetta_deltanet_rows", "saetta_deltanet_rows_ws", "saetta_deltanet_rows_workspace_bytes", "saetta_deltanet_token", "saetta_deltanet_rows_fused",
     "saetta_part_o_bytes", "saetta_part_ml_bytes", "saetta_attn_decode", "saetta_attn_decode_quant",
     "saetta_attn_rows", "saetta_attn_rows_quant", "saetta_static_scratch_bytes", "saetta_attn_decode_quant_static", "saetta_prefill_workspace_bytes", "saetta_attn_prefill", "saetta_attn_prefill_quant",
+    "saetta_attn_gemm_workspace_bytes", "saetta_attn_gemm",
 ]
 
 STAGE_PARTIAL, STAGE_REDUCE, STAGE_ALL, STAGE_NO_LOADERS = 1, 2, 3, 4
@@ -108,6 +109,11 @@ def lib():
         l.saetta_attn_prefill_quant.restype = i32
         l.saetta_attn_prefill_quant.argtypes = [vp, i32, vp, QuantRowsC, QuantRowsC, vp, vp, FlashParamsC, vp,
                                                 ctypes.c_size_t]
+        l.saetta_attn_gemm_workspace_bytes.restype = ctypes.c_size_t
+        l.saetta_attn_gemm_workspace_bytes.argtypes = [ctypes.c_uint32] * 4
+        l.saetta_attn_gemm.restype = i32
+        l.saetta_attn_gemm.argtypes = [vp, i32, vp, QuantRowsC, QuantRowsC, vp, vp, FlashParamsC, u32, u32, vp,
+                                       ctypes.c_size_t]
         _lib = l
     return _lib
 

@@ -6,6 +6,7 @@
   attention.rs          DecodeAttention (new / record / record_quant, pub kernel)
   rows.rs               MAX_ROWS, AttentionRows (new / record / record_quant)
   attention_prefill.rs  FlashParams, KERNELS, DEFAULT, KEY_BLOCK, encode
+  attention_gemm.rs     KEYS, AttGemm (new / encode, pub fused, texp, stages), bench
 
 A reference `View` (buffer + byte offset) is a torch tensor here (a slice is a
 view with an offset); a Metal encoder is a HIP stream.  Shape violations raise
@@ -818,3 +819,136 @@ class attention_prefill:
         ffi.check(ffi.lib().saetta_attn_prefill_quant(_stream(stream), keys.bits.value, _ptr(q), keys.c(), values.c(),
                                                       _ptr(q_and_gate), _ptr(out), p.c(), *_workspace(workspace)),
                   "attn_prefill_quant")
+
+
+class attention_gemm:
+    """Namespace of src/attention_gemm.rs: prefill attention as matrix products over blocks of keys."""
+    KEYS = 1024    # src/attention_gemm.rs:28
+    SLICES = 2     # src/attention_gemm.rs:63
+
+    @staticmethod
+    def slices():
+        """SAETTA_AG_SLICES, as the reference reads it (src/attention_gemm.rs:83-89)."""
+        import os
+        try:
+            n = int(os.environ.get("SAETTA_AG_SLICES", ""))
+        except ValueError:
+            n = 0
+        return n if n > 0 else attention_gemm.SLICES
+
+    class AttGemm:
+        """AttGemm (src/attention_gemm.rs:95-364): the buffers of one block for slices of up to `slice`
+        tokens of a chunk, and `encode`.  Only the reference's default variant exists here (`fused` and
+        `texp` both true: the scores pass writes the probabilities relative to each tile's maximum and the
+        tiles' sums, the pv pass scales a tile once); SAETTA_AG_FUSED=0 or SAETTA_AG_TEXP=0 raise.
+        `stages` as in the reference's bench: 0 all passes, 1 or 2 scores only, 3 scores and pv and no
+        outputs."""
+
+        def __init__(self, chunk, kv_heads, device="cuda"):
+            import os
+            for name in ("SAETTA_AG_FUSED", "SAETTA_AG_TEXP"):
+                if os.environ.get(name) == "0":
+                    raise ValueError(f"{name}=0: only the fused variant with tile sums is built")
+            self.slice = -(-chunk // attention_gemm.slices())
+            self.rows_pad = -(-self.slice * 8 // 64) * 64
+            self.chunk, self.kv_heads, self.device = chunk, kv_heads, device
+            self.fused = self.texp = True
+            self.stages = 0
+            self._workspace = None
+
+        def workspace_bytes(self, p):
+            return ffi.lib().saetta_attn_gemm_workspace_bytes(p.pos, p.tokens, self.slice, p.kv_heads)
+
+        def encode(self, q, keys, values, quant, q_and_gate, out, f, stream=None):
+            """encode (src/attention_gemm.rs:144-188): the same as attention_prefill.encode on the same
+            buffers; with `quant` = (QuantRows of the keys, QuantRows of the values) the cache is read from
+            those 8- or 4-bit rows and `keys` and `values` are not read."""
+            if f.heads != f.kv_heads * 8:
+                raise ValueError("needs 8 q heads per kv head")
+            if f.tokens > self.chunk or f.kv_heads != self.kv_heads:
+                raise ValueError(f"AttGemm for chunks of {self.chunk} tokens and {self.kv_heads} kv heads")
+            _need(q, torch.float16, "q"), _need(q_and_gate, torch.float32, "q_and_gate"), _need(out, torch.float32, "out")
+            if quant is None:
+                _need(keys, torch.float16, "keys"), _need(values, torch.float16, "values")
+                bits = 16
+                k = ffi.QuantRowsC(_ptr(keys), None, None)
+                v = ffi.QuantRowsC(_ptr(values), None, None)
+            else:
+                if quant[0].bits is KvBits.Half or quant[0].bits is not quant[1].bits:
+                    raise ValueError(f"no gemm attention for {quant[0].bits} rows")
+                bits, k, v = quant[0].bits.value, quant[0].c(), quant[1].c()
+            need = self.workspace_bytes(f)
+            if self._workspace is None or self._workspace.numel() < need:
+                self._workspace = torch.empty(need, dtype=torch.uint8, device=self.device)
+            ffi.check(ffi.lib().saetta_attn_gemm(_stream(stream), bits, _ptr(q), k, v, _ptr(q_and_gate), _ptr(out),
+                                                 f.c(), self.slice, self.stages, *_workspace(self._workspace)),
+                      "attn_gemm")
+
+    @staticmethod
+    def bench(contexts, chunk, layers, device="cuda"):
+        """bench (src/attention_gemm.rs:366-470): for each context the chunk of `chunk` tokens at its end and
+        at its middle through attention_prefill.encode_rows2 and through AttGemm, best of 3 after a warm-up;
+        the gemm passes of the last chunk one by one as differences of runs that stop early; the largest and
+        the rms relative difference of the two outputs.  One dict per context."""
+        heads, kv, dim = 16, 2, DIM
+        gemm = attention_gemm.AttGemm(chunk, kv, device)
+        rows = []
+        for n in contexts:
+            n = -(-n // chunk) * chunk
+            capacity = -(-n // 64) * 64 + 64
+            q = attention_prefill.spread(chunk * heads * dim, 1, device)
+            k = attention_prefill.spread(capacity * kv * dim, 2, device)
+            v = attention_prefill.spread(capacity * kv * dim, 3, device)
+            g = ((torch.arange(chunk * heads * 2 * dim, device=device) % 7) - 3).to(torch.float32)
+            want = torch.empty(chunk * heads * dim, dtype=torch.float32, device=device)
+            got = torch.empty_like(want)
+            chunks = n // chunk
+            mid, last = (chunks // 2) * chunk, n - chunk
+            ws = torch.empty(attention_prefill.workspace_bytes(FlashParams(heads, kv, last, chunk, 1.0)),
+                             dtype=torch.uint8, device=device)
+
+            def flops(pos):
+                return 4.0 * heads * dim * (chunk * pos + chunk * (chunk + 1) / 2)
+
+            def best_ms(gemm_kernel, pos):
+                p = FlashParams(heads, kv, pos, chunk, 1.0 / math.sqrt(dim))
+
+                def run():
+                    if gemm_kernel:
+                        gemm.encode(q, k, v, None, g, got, p)
+                    else:
+                        attention_prefill.encode_rows2(q, k, v, g, want, p, workspace=ws)
+
+                run()
+                best = float("inf")
+                for _ in range(3):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    run()
+                    e1.record()
+                    e1.synchronize()
+                    best = min(best, e0.elapsed_time(e1))
+                return best
+
+            row = {"context": n, "chunk": chunk}
+            for name, gemm_kernel in (("rows2", False), ("gemm", True)):
+                tl, tm = best_ms(gemm_kernel, last), best_ms(gemm_kernel, mid)
+                row[name] = {"last_ms": tl, "last_TFLOP/s": flops(last) / tl / 1e9, "mid_TFLOP/s": flops(mid) / tm / 1e9,
+                             "prefill_attention_s": tm * 1e-3 * chunks * layers}
+            prefix = [0.0] * 4
+            for stage in (1, 2, 3):
+                gemm.stages = stage
+                prefix[stage] = best_ms(True, last)
+            gemm.stages = 0
+            whole = best_ms(True, last)
+            row["stages"] = {"scores_ms": prefix[1], "scores_TFLOP/s": flops(last) / 2 / prefix[1] / 1e9,
+                             "softmax_ms": prefix[2] - prefix[1], "pv_ms": prefix[3] - prefix[2],
+                             "pv_TFLOP/s": flops(last) / 2 / max(prefix[3] - prefix[2], 1e-9) / 1e9,
+                             "final_ms": whole - prefix[3]}
+            # both outputs are now of the last chunk
+            best_ms(False, last)
+            diff = (want - got).double()
+            row["rel_rms"] = float((diff.pow(2).sum() / want.double().pow(2).sum()).sqrt())
+            row["max_abs"] = float(diff.abs().max())
+            rows.append(row)
+        return rows
