@@ -306,7 +306,9 @@ def bench_reader_floor(s, torch, args, ctx=32768, layers=32):
     }
 
 
-def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8):
+def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8, gemm=False):
+    """gemm: the same chunk by AttGemm (src/attention_gemm.rs), block by block of 1024 keys with the block's
+    probabilities written out and read back, instead of the flash kernel."""
     import numpy as np
     import oracle  # CPU-baseline leg only
 
@@ -323,12 +325,19 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8):
     out = torch.empty(tokens, H, D, device="cuda")
     p = s.FlashParams(H, KV, pos, tokens, 1.0 / math.sqrt(D))
     kx, vx = knew[pos:].reshape(-1).contiguous(), vnew[pos:].reshape(-1).contiguous()
+    att_gemm = s.attention_gemm.AttGemm(tokens, KV) if gemm else None
+
+    def attention():
+        if gemm:
+            att_gemm.encode(q, None, None, (keys, values), qg, out, p)
+        else:
+            s.attention_prefill.encode_quant(q, keys, values, qg, out, p)
 
     def step():
         # quantize-on-append of the chunk's K and V, then the attention over codes in place
         keys.encode(kx, pos, tokens)
         values.encode(vx, pos, tokens)
-        s.attention_prefill.encode_quant(q, keys, values, qg, out, p)
+        attention()
 
     flops = 4.0 * H * D * (tokens * pos + tokens * (tokens + 1) / 2)
     for _ in range(args.warmup):
@@ -343,7 +352,7 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8):
     for _ in range(max(3, args.steps)):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        s.attention_prefill.encode_quant(q, keys, values, qg, out, p)
+        attention()
         e1.record()
         e1.synchronize()
         ts.append(e0.elapsed_time(e1) * 1e3)
@@ -374,15 +383,18 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8):
         "ms_per_step": round(ms_per_step, 4),
         "dtype": "f16 MFMA, f32 softmax state",
         "config": {"workload": f"causal prefill chunk of {tokens} tokens at position {pos}, {bits}-bit KV cache "
-                               "read in place, chunk K/V quantized on append inside the step",
+                               "read in place, chunk K/V quantized on append inside the step"
+                               + (", attention as matrix products over blocks of 1024 keys (AttGemm)" if gemm else ""),
                    "heads": H, "kv_heads": KV, "head_dim": D, "flops": flops,
                    "timing": "value: wall time of steps (2 x kv_quantize of the chunk + prepare + attention); "
-                             "roofline: median of event-timed prepare + attention calls",
+                             "roofline: median of event-timed prepare + attention calls"
+                             + (f" ({2 * -(-(pos + tokens) // 1024)} launches: scores and pv per block of 1024 keys)" if gemm else ""),
                    "inputs": "q (through bf16), K, V, gate ~ N(0,1) from torch's device generator (Philox, seed 99)"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC.get("prefill") if (tokens, pos, bits) == (4096, 4096, 8) else None,
-                     "kernel": "attention_prefill_kernel", "avg_us": round(kern_us, 2)},
+                     "traffic": MEASURED_TRAFFIC.get("prefill") if (tokens, pos, bits, gemm) == (4096, 4096, 8, False) else None,
+                     "kernel": "attention_gemm_scores_kernel + attention_gemm_pv_kernel" if gemm else "attention_prefill_kernel",
+                     "avg_us": round(kern_us, 2)},
         "cpu_baseline": {"value": round(cpu_flops / cpu_s / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
                          "sample": f"the last {sample} tokens of the chunk ({cpu_s:.2f} s)"},
         "parity_rel_rms_vs_oracle": float(f"{rel_rms:.3e}"),
@@ -647,7 +659,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="default",
-                    choices=["decode8_32k", "decode4_150k", "decode16_4k", "verify2", "verify3", "verify4", "prefill", "prefill_131k", "deltanet",
+                    choices=["decode8_32k", "decode4_150k", "decode16_4k", "verify2", "verify3", "verify4", "prefill", "prefill_131k", "prefill_gemm", "prefill_gemm_131k", "deltanet",
                              "deltanet_prefill", "prep_store", "reader_floor", "default", "all"])
     ap.add_argument("--no-graph", action="store_true", help="launch from Python instead of replaying a HIP graph")
     ap.add_argument("--layers", type=int, default=0, help="layer caches per step (default 32; 12 at 150k)")
@@ -697,6 +709,10 @@ def main():
             # the last 4096-token chunk of a 131072-token context: whether the one flash kernel holds up where
             # the reference switches to its multi-pass form (src/attention_gemm.rs)
             return bench_prefill(s, torch, args, tokens=4096, pos=131072 - 4096)
+        if workload == "prefill_gemm":
+            return bench_prefill(s, torch, args, gemm=True)
+        if workload == "prefill_gemm_131k":
+            return bench_prefill(s, torch, args, tokens=4096, pos=131072 - 4096, gemm=True)
         return bench_prefill(s, torch, args)
 
     if args.workload in ("default", "all"):
@@ -708,7 +724,7 @@ def main():
         res["prefill"] = one("prefill")
     if args.workload == "all":
         res["other_workloads"] = {}
-        for w in ["verify2", "verify3", "verify4", "decode4_150k", "decode16_4k", "prefill_131k", "deltanet", "deltanet_prefill", "prep_store"]:
+        for w in ["verify2", "verify3", "verify4", "decode4_150k", "decode16_4k", "prefill_131k", "prefill_gemm", "prefill_gemm_131k", "deltanet", "deltanet_prefill", "prep_store"]:
             torch.cuda.empty_cache()
             r = one(w)
             res["other_workloads"][w] = {k: r[k] for k in ("metric", "value", "unit", "ms_per_step", "roofline",

@@ -893,14 +893,14 @@ int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kda
 //            stored as the P^T operands of the second product (the accumulator's registers 8 sp .. 8 sp + 7
 //            are the operand of k-step sp: 1 KB per wave and k-step, read back as it was written);
 //   pv       m' = max(m, max_t t), O^T = alpha O^T + sum_t V^T_t (f_t P^T_t) with f_t = 2^(t - m') rounded
-//            to f16 (the row sum takes the same rounded f_t), one workgroup per half of the dims; the
-//            block that holds a tile's last visible key writes out = O / l * sigmoid(gate) instead of O.
+//            to f16 (the row sum takes the same rounded f_t); the block that holds a tile's last visible
+//            key writes out = O / l * sigmoid(gate) instead of O.
 constexpr int AG_KEYS = SAETTA_AG_KEYS;
 constexpr int AG_TILES = AG_KEYS / BK;
 constexpr int AG_WAVES = 4;
 constexpr int AG_THREADS = 64 * AG_WAVES;
 constexpr int AG_TOKENS = 4 * AG_WAVES;   // tokens of a workgroup
-constexpr int AG_SPLIT = 4;               // scores: workgroups that share a block's tiles for one token tile
+constexpr int AG_SPLIT = 2;               // scores: workgroups that share a block's tiles for one token tile
 constexpr int AG_P_TILE_BYTES = BK * 32 * 2;  // the P^T operands of one row group and tile of keys
 
 struct GemmArgs {
@@ -911,7 +911,7 @@ struct GemmArgs {
     unsigned char *p;    // f16 [kv head][row group][tile][2 k-steps][64 lanes][8]
     float *tmax, *tsum;  // [kv head][row group][tile][32 rows], log2 domain
     float *o;            // [kv head][row group][8 dim tiles][4][64 lanes][4]: the accumulators as they are
-    float *m, *l;        // [dim half][kv head][row group][32 rows]
+    float *m, *l;        // [kv head][row group][32 rows]
     uint32_t heads, kv_heads, pos, tokens;  // of the slice
     float c;             // scale * log2(e)
     uint32_t nblocks;    // images per kv head
@@ -957,21 +957,23 @@ __global__ __launch_bounds__(AG_THREADS) void attention_gemm_scores_kernel(GemmA
     }
 
     const unsigned char *img = a.images + (size_t(kv) * a.nblocks + a.j0 / BK + first) * IMG_BYTES;
-    u32x4 pre[4];
-    auto fetch = [&](uint32_t t) {
+    // a tile's part is fetched into registers two tiles ahead (two register sets, the loop in pairs)
+    u32x4 pre[2][4];
+    auto fetch = [&](u32x4 *set, uint32_t t) {
         const u32x4 *src = reinterpret_cast<const u32x4 *>(img + size_t(t) * IMG_BYTES);
 #pragma unroll
-        for (int i = 0; i < 4; i++) pre[i] = src[tid + AG_THREADS * i];
+        for (int i = 0; i < 4; i++) set[i] = src[tid + AG_THREADS * i];
     };
-    fetch(0);
+    fetch(pre[0], 0);
+    if (count > 1) fetch(pre[1], 1);
     const uint32_t limit = a.pos + tok;  // the last key the row sees
     const size_t row_base = (size_t(kv) * a.row_groups + rg) * AG_TILES;
-    for (uint32_t t = 0; t < count; t++) {
+    auto tile = [&](u32x4 *set, uint32_t t) {
         unsigned char *buf = k_lds[t & 1];
 #pragma unroll
-        for (int i = 0; i < 4; i++) reinterpret_cast<u32x4 *>(buf)[tid + AG_THREADS * i] = pre[i];
+        for (int i = 0; i < 4; i++) reinterpret_cast<u32x4 *>(buf)[tid + AG_THREADS * i] = set[i];
         __syncthreads();
-        if (t + 1 < count) fetch(t + 1);
+        if (t + 2 < count) fetch(set, t + 2);
         floatx16 acc;
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[i] = 0.0f;
@@ -980,47 +982,64 @@ __global__ __launch_bounds__(AG_THREADS) void attention_gemm_scores_kernel(GemmA
             const half8 kf = *reinterpret_cast<const half8 *>(buf + f * 1024 + lane * 16);
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[f], acc, 0, 0, 0);
         }
-        // register i is key 8 (i / 4) + 4 hf + i % 4 of the tile
-        const uint32_t key0 = a.j0 + (first + t) * BK + 4 * hf;
-        float s[16], tmax = NO_SCORE;
+        // register i is key 8 (i / 4) + 4 hf + i % 4 of the tile.  Only a tile that reaches past the first
+        // token of the wave's row group has anything to mask (wave-uniform).
+        const uint32_t key0 = a.j0 + (first + t) * BK;
+        if (key0 + BK - 1 > a.pos + tok0 + 4 * wave) {
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const uint32_t key = key0 + 8 * (i >> 2) + (i & 3);
-            s[i] = key <= limit ? acc[i] * a.c : NO_SCORE;
-            tmax = fmaxf(tmax, s[i]);
+            for (int i = 0; i < 16; i++) {
+                const uint32_t key = key0 + 4 * hf + 8 * (i >> 2) + (i & 3);
+                acc[i] = key <= limit ? acc[i] : NO_SCORE;
+            }
         }
+        float tmax = fmaxf(acc[0], acc[1]);
+#pragma unroll
+        for (int i = 2; i < 16; i += 2) tmax = fmaxf(tmax, fmaxf(acc[i], acc[i + 1]));
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-        half8 p0, p1;
+        // scores in the log2 domain: s = acc * c, the tile's maximum t = tmax * c (c > 0).  A masked score is
+        // NO_SCORE * c - t: far below any exponent, 0; with the whole tile masked t is that too, and the
+        // probabilities are set to 0 outright.
+        const float t_log2 = tmax * a.c;
+        const bool none = tmax <= 0.5f * NO_SCORE;
+        half2_ ph[8];
         float sum = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            // (a masked score is never exponentiated: with the whole tile masked s - tmax would be 0)
-            const _Float16 ph = (_Float16)(s[i] > 0.5f * NO_SCORE ? __builtin_amdgcn_exp2f(s[i] - tmax) : 0.0f);
-            sum += (float)ph;  // the sum of what the second product multiplies
-            if (i < 8) p0[i] = ph; else p1[i - 8] = ph;
+        for (int i = 0; i < 16; i += 2) {
+            const float e0 = none ? 0.0f : __builtin_amdgcn_exp2f(fmaf(acc[i], a.c, -t_log2));
+            const float e1 = none ? 0.0f : __builtin_amdgcn_exp2f(fmaf(acc[i + 1], a.c, -t_log2));
+            ph[i / 2] = half2_{(_Float16)e0, (_Float16)e1};
+            // the sum of what the second product multiplies: the rounded halves, added in f32
+            sum = __builtin_amdgcn_fdot2(ph[i / 2], half2_{(_Float16)1.0f, (_Float16)1.0f}, sum, false);
         }
         sum += __shfl_xor(sum, 32);
+        const half8 p0 = {ph[0][0], ph[0][1], ph[1][0], ph[1][1], ph[2][0], ph[2][1], ph[3][0], ph[3][1]};
+        const half8 p1 = {ph[4][0], ph[4][1], ph[5][0], ph[5][1], ph[6][0], ph[6][1], ph[7][0], ph[7][1]};
+        const float tmax_out = none ? NO_SCORE : t_log2;
         unsigned char *pt = a.p + (row_base + first + t) * AG_P_TILE_BYTES + lane * 16;
         *reinterpret_cast<half8 *>(pt) = p0;
         *reinterpret_cast<half8 *>(pt + 1024) = p1;
         if (hf == 0) {
-            a.tmax[(row_base + first + t) * 32 + col] = tmax;
+            a.tmax[(row_base + first + t) * 32 + col] = tmax_out;
             a.tsum[(row_base + first + t) * 32 + col] = sum;
         }
+    };
+    for (uint32_t t = 0; t < count; t += 2) {
+        tile(pre[0], t);
+        if (t + 1 < count) tile(pre[1], t + 1);
     }
 }
 
-__global__ __launch_bounds__(AG_THREADS) void attention_gemm_pv_kernel(GemmArgs a) {
-    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2][PART_BYTES / 2];
+__global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_pv_kernel(GemmArgs a) {
+    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2][PART_BYTES];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 31, hf = lane >> 5;
-    const uint32_t dh = blockIdx.x, tok0 = blockIdx.y * AG_TOKENS, kv = blockIdx.z;
+    const uint32_t tok0 = blockIdx.y * AG_TOKENS, kv = blockIdx.z;
     const uint32_t need = ag_tiles(a, tok0);
     if (need == 0) return;  // the tile sees nothing of this block (its outputs were written at an earlier one)
     const bool last_block = ag_last_key(a, tok0) < a.j0 + AG_KEYS;
     const uint32_t rg = blockIdx.y * AG_WAVES + wave;
     const uint32_t tok = tok0 + 4 * wave + (col >> 3), head = kv * SAETTA_GQA_GROUP + (col & 7);
     const size_t rows = size_t(kv) * a.row_groups + rg;
-    const size_t state = (size_t(dh) * a.kv_heads * a.row_groups + rows) * 32 + col;
+    const size_t state = rows * 32 + col;
     const bool first_block = a.j0 == 0;
 
     const float *tm = a.tmax + rows * AG_TILES * 32 + col, *ts = a.tsum + rows * AG_TILES * 32 + col;
@@ -1031,16 +1050,16 @@ __global__ __launch_bounds__(AG_THREADS) void attention_gemm_pv_kernel(GemmArgs 
     const float m_new = fmaxf(m_old, mb);
     const float alpha = first_block ? 0.0f : __builtin_amdgcn_exp2f(m_old - m_new);
 
-    floatx16 acc[4];
-    float *op = a.o + (rows * 8 + 4 * dh) * 1024 + lane * 4;
+    floatx16 acc[8];
+    float *op = a.o + rows * 8 * 1024 + lane * 4;
     if (first_block) {
 #pragma unroll
-        for (int mt = 0; mt < 4; mt++)
+        for (int mt = 0; mt < 8; mt++)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[mt][i] = 0.0f;
     } else {
 #pragma unroll
-        for (int mt = 0; mt < 4; mt++)
+        for (int mt = 0; mt < 8; mt++)
 #pragma unroll
             for (int q4 = 0; q4 < 4; q4++) {
                 const floatx4 x = *reinterpret_cast<const floatx4 *>(op + (mt * 4 + q4) * 256);
@@ -1049,47 +1068,49 @@ __global__ __launch_bounds__(AG_THREADS) void attention_gemm_pv_kernel(GemmArgs 
             }
     }
 
-    // the V^T part of an image, this half of the dims: fragments 8 dh .. 8 dh + 7
-    const unsigned char *img = a.images + (size_t(kv) * a.nblocks + a.j0 / BK) * IMG_BYTES + PART_BYTES + dh * (PART_BYTES / 2);
-    u32x4 pre[2];
-    auto fetch = [&](uint32_t t) {
+    // the V^T part of an image
+    const unsigned char *img = a.images + (size_t(kv) * a.nblocks + a.j0 / BK) * IMG_BYTES + PART_BYTES;
+    // a tile's operands are fetched into registers two tiles ahead (two register sets, the loop in pairs)
+    struct Ahead {
+        u32x4 v[4];
+        half8 p0, p1;
+        float tm, ts;
+    } pre[2];
+    const unsigned char *pp = a.p + rows * AG_TILES * AG_P_TILE_BYTES + lane * 16;
+    auto fetch = [&](Ahead &set, uint32_t t) {
         const u32x4 *src = reinterpret_cast<const u32x4 *>(img + size_t(t) * IMG_BYTES);
 #pragma unroll
-        for (int i = 0; i < 2; i++) pre[i] = src[tid + AG_THREADS * i];
+        for (int i = 0; i < 4; i++) set.v[i] = src[tid + AG_THREADS * i];
+        set.p0 = *reinterpret_cast<const half8 *>(pp + size_t(t) * AG_P_TILE_BYTES);
+        set.p1 = *reinterpret_cast<const half8 *>(pp + size_t(t) * AG_P_TILE_BYTES + 1024);
+        set.tm = tm[t * 32], set.ts = ts[t * 32];
     };
-    const unsigned char *pp = a.p + rows * AG_TILES * AG_P_TILE_BYTES + lane * 16;
-    half8 pn0, pn1;
-    float tmn, tsn;
-    auto fetch_p = [&](uint32_t t) {
-        pn0 = *reinterpret_cast<const half8 *>(pp + size_t(t) * AG_P_TILE_BYTES);
-        pn1 = *reinterpret_cast<const half8 *>(pp + size_t(t) * AG_P_TILE_BYTES + 1024);
-        tmn = tm[t * 32], tsn = ts[t * 32];
-    };
-    fetch(0);
-    fetch_p(0);
+    fetch(pre[0], 0);
+    if (need > 1) fetch(pre[1], 1);
     float lsum = 0.0f;
-    for (uint32_t t = 0; t < need; t++) {
+    auto tile = [&](Ahead &set, uint32_t t) {
         unsigned char *buf = v_lds[t & 1];
 #pragma unroll
-        for (int i = 0; i < 2; i++) reinterpret_cast<u32x4 *>(buf)[tid + AG_THREADS * i] = pre[i];
+        for (int i = 0; i < 4; i++) reinterpret_cast<u32x4 *>(buf)[tid + AG_THREADS * i] = set.v[i];
         __syncthreads();
-        half8 pc0 = pn0, pc1 = pn1;
-        const float tmc = tmn, tsc = tsn;
-        if (t + 1 < need) {
-            fetch(t + 1);
-            fetch_p(t + 1);
-        }
+        half8 pc0 = set.p0, pc1 = set.p1;
+        const float tmc = set.tm, tsc = set.ts;
+        if (t + 2 < need) fetch(set, t + 2);
         // a tile the row sees nothing of has t = NO_SCORE: its factor is 0, like its probabilities
         const _Float16 fh = (_Float16)__builtin_amdgcn_exp2f(tmc - m_new);
         lsum += (float)fh * tsc;
         pc0 *= fh, pc1 *= fh;
 #pragma unroll
-        for (int mt = 0; mt < 4; mt++) {
+        for (int mt = 0; mt < 8; mt++) {
             const half8 v0 = *reinterpret_cast<const half8 *>(buf + (2 * mt) * 1024 + lane * 16);
             const half8 v1 = *reinterpret_cast<const half8 *>(buf + (2 * mt + 1) * 1024 + lane * 16);
             acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(v0, pc0, acc[mt], 0, 0, 0);
             acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(v1, pc1, acc[mt], 0, 0, 0);
         }
+    };
+    for (uint32_t t = 0; t < need; t += 2) {
+        tile(pre[0], t);
+        if (t + 1 < need) tile(pre[1], t + 1);
     }
     const float l_new = alpha * l_old + lsum;
 
@@ -1097,25 +1118,29 @@ __global__ __launch_bounds__(AG_THREADS) void attention_gemm_pv_kernel(GemmArgs 
         if (tok < a.tokens) {
             const float inv = 1.0f / l_new;
             const size_t row = size_t(tok) * a.heads + head;
-            const float *gate = a.q_and_gate + row * 2 * DIM + DIM + 128 * dh + 4 * hf;
-            float *out = a.out + row * DIM + 128 * dh + 4 * hf;
-            floatx4 g[16];
 #pragma unroll
-            for (int i = 0; i < 16; i++) g[i] = *reinterpret_cast<const floatx4 *>(gate + 32 * (i >> 2) + 8 * (i & 3));
+            for (int dh = 0; dh < 2; dh++) {  // (half of the dims at a time: 16 gate loads in flight)
+                const float *gate = a.q_and_gate + row * 2 * DIM + DIM + 128 * dh + 4 * hf;
+                float *out = a.out + row * DIM + 128 * dh + 4 * hf;
+                floatx4 g[16];
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int mt = i >> 2, q4 = i & 3;
-                floatx4 w;
+                for (int i = 0; i < 16; i++) g[i] = *reinterpret_cast<const floatx4 *>(gate + 32 * (i >> 2) + 8 * (i & 3));
 #pragma unroll
-                for (int e = 0; e < 4; e++) w[e] = acc[mt][4 * q4 + e] * inv * __builtin_amdgcn_rcpf(1.0f + __expf(-g[i][e]));
-                *reinterpret_cast<floatx4 *>(out + 32 * mt + 8 * q4) = w;
+                for (int i = 0; i < 16; i++) {
+                    const int mt = 4 * dh + (i >> 2), q4 = i & 3;
+                    floatx4 w;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) w[e] = acc[mt][4 * q4 + e] * inv * __builtin_amdgcn_rcpf(1.0f + __expf(-g[i][e]));
+                    *reinterpret_cast<floatx4 *>(out + 32 * (i >> 2) + 8 * q4) = w;
+                }
+                asm volatile("" ::: "memory");
             }
         }
         return;
     }
     if (hf == 0) a.m[state] = m_new, a.l[state] = l_new;
 #pragma unroll
-    for (int mt = 0; mt < 4; mt++)
+    for (int mt = 0; mt < 8; mt++)
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) {
             floatx4 x;
@@ -1132,7 +1157,7 @@ size_t gemm_row_groups(uint32_t slice) { return size_t((slice + AG_TOKENS - 1) /
 
 size_t gemm_scratch_bytes(uint32_t slice, uint32_t kv_heads) {
     const size_t groups = gemm_row_groups(slice) * kv_heads;
-    return groups * (size_t(AG_TILES) * AG_P_TILE_BYTES + 2 * size_t(AG_TILES) * 32 * 4 + 32 * size_t(DIM) * 4 + 2 * 2 * 32 * 4);
+    return groups * (size_t(AG_TILES) * AG_P_TILE_BYTES + 2 * size_t(AG_TILES) * 32 * 4 + 32 * size_t(DIM) * 4 + 2 * 32 * 4);
 }
 
 uint32_t gemm_slice(uint32_t tokens, uint32_t slice_tokens) {
@@ -1166,7 +1191,7 @@ int run_gemm(hipStream_t stream, int bits, const uint16_t *q, const void *kdata,
     a.tmax = reinterpret_cast<float *>(at), at += groups * AG_TILES * 32 * 4;
     a.tsum = reinterpret_cast<float *>(at), at += groups * AG_TILES * 32 * 4;
     a.o = reinterpret_cast<float *>(at), at += groups * 32 * DIM * 4;
-    a.m = reinterpret_cast<float *>(at), at += 2 * groups * 32 * 4;
+    a.m = reinterpret_cast<float *>(at), at += groups * 32 * 4;
     a.l = reinterpret_cast<float *>(at);
     a.heads = p.heads, a.kv_heads = p.kv_heads;
     a.c = p.scale * 1.4426950408889634f;
@@ -1186,7 +1211,7 @@ int run_gemm(hipStream_t stream, int bits, const uint16_t *q, const void *kdata,
             a.j0 = uint32_t(j0);
             attention_gemm_scores_kernel<<<dim3(AG_SPLIT, tiles, p.kv_heads), AG_THREADS, 0, stream>>>(a);
             if (stages == 1 || stages == 2) continue;
-            attention_gemm_pv_kernel<<<dim3(2, tiles, p.kv_heads), AG_THREADS, 0, stream>>>(a);
+            attention_gemm_pv_kernel<<<dim3(1, tiles, p.kv_heads), AG_THREADS, 0, stream>>>(a);
         }
     }
     return launch_status(what);

@@ -12,6 +12,7 @@
 //   rows::MAX_ROWS, AttentionRows      src/rows.rs:8-9, 344-494
 //   attention_prefill::FlashParams, KERNELS, DEFAULT, KEY_BLOCK, encode
 //                                      src/attention_prefill.rs:4-72
+//   attention_gemm::KEYS, AttGemm      src/attention_gemm.rs:28, 95-364
 //
 // Where the reference asserts or panics, these throw std::runtime_error.  Buffers are
 // reference-counted and zero-filled like Metal's (src/gpu.rs:287-290); a Plan keeps every
@@ -23,6 +24,7 @@
 #include <chrono>
 #include <cmath>
 #include <cstdint>
+#include <cstdlib>
 #include <cstring>
 #include <functional>
 #include <memory>
@@ -723,6 +725,66 @@ inline void encode_quant(const gpu::Gpu &gpu, const View &q, const kv_quant::Qua
 }
 
 }  // namespace attention_prefill
+
+namespace attention_gemm {
+
+constexpr size_t KEYS = SAETTA_AG_KEYS;  // src/attention_gemm.rs:28
+// Query slices a chunk runs in unless SAETTA_AG_SLICES says otherwise (src/attention_gemm.rs:59-63, 83-89).
+// The reference takes 2 to halve a scratch that shares the machine's one memory with the model; here 1.
+constexpr size_t SLICES = 1;
+
+inline size_t slices() {
+    const char *v = std::getenv("SAETTA_AG_SLICES");
+    const long n = v ? std::strtol(v, nullptr, 10) : 0;
+    return n > 0 ? size_t(n) : SLICES;
+}
+
+// AttGemm (src/attention_gemm.rs:95-364): the buffers of one block for slices of up to `slice` tokens of
+// a chunk, and encode.  Only the reference's default variant is built (fused, with tile sums).
+struct AttGemm {
+    size_t slice, rows_pad, chunk, kv_heads;
+    bool fused = true, texp = true;
+    // For a bench: only the first `stages` passes of each block (1, 2: scores; 3: scores and pv, no
+    // outputs); 0 runs all (src/attention_gemm.rs:112-114).
+    mutable uint32_t stages = 0;
+
+    AttGemm(const gpu::Gpu &, size_t chunk_, size_t kv_heads_) : chunk(chunk_), kv_heads(kv_heads_) {
+        for (const char *name : {"SAETTA_AG_FUSED", "SAETTA_AG_TEXP"}) {
+            const char *v = std::getenv(name);
+            if (v && std::string(v) == "0") throw std::runtime_error(std::string(name) + "=0: only the fused variant with tile sums is built");
+        }
+        slice = (chunk + slices() - 1) / slices();
+        rows_pad = (slice * 8 + 63) / 64 * 64;
+    }
+
+    // The same as attention_prefill::encode on the same buffers; with `quant` the keys and values are read
+    // from those 8- or 4-bit rows and `keys` and `values` are not read (src/attention_gemm.rs:144-188).
+    void encode(const gpu::Gpu &gpu, const View &q, const View &keys, const View &values,
+                const std::pair<const kv_quant::QuantRows *, const kv_quant::QuantRows *> *quant, const View &q_and_gate,
+                const View &out, attention_prefill::FlashParams f) const {
+        if (f.heads != f.kv_heads * 8) throw std::runtime_error("needs 8 q heads per kv head");
+        if (f.tokens > chunk || f.kv_heads != kv_heads) throw std::runtime_error("AttGemm: made for another chunk or kv head count");
+        int bits = 16;
+        saetta_quant_rows k{const_cast<uint32_t *>(keys.ptr<uint32_t>()), nullptr, nullptr};
+        saetta_quant_rows v{const_cast<uint32_t *>(values.ptr<uint32_t>()), nullptr, nullptr};
+        if (quant) {
+            if (quant->first->bits == kv_quant::KvBits::Half || quant->first->bits != quant->second->bits)
+                throw std::runtime_error("no gemm attention for these rows");
+            bits = int(kv_quant::bits(quant->first->bits));
+            k = quant->first->c(), v = quant->second->c();
+        }
+        const size_t need = saetta_attn_gemm_workspace_bytes(f.pos, f.tokens, uint32_t(slice), f.kv_heads);
+        if (workspace_.length() < need) workspace_ = gpu::Buffer(need);
+        check(saetta_attn_gemm(gpu.stream(), bits, q.ptr<uint16_t>(), k, v, q_and_gate.ptr<float>(), out.ptr<float>(), f,
+                               uint32_t(slice), stages, workspace_.get(), workspace_.length()),
+              "attn_gemm");
+    }
+
+  private:
+    mutable gpu::Buffer workspace_;
+};
+
+}  // namespace attention_gemm
 
 namespace gpu_layers {
 

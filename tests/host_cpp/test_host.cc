@@ -2,6 +2,7 @@
 // (saetta-macqwen_amd/host/saetta.hpp) with the CPU oracle as the other side:
 //   tests/kv_quant.rs   prefill_rows_match_cpu, decode_row_matches_cpu, dequantize_matches_cpu
 //   tests/attention.rs  quantized_matches_cpu
+//   tests/attention_prefill.rs  (one shape) for attention_prefill::encode and attention_gemm::AttGemm::encode
 // Exit code 0 = all passed.  Run by tests/test_gpu_host_cpp.py on a GPU box.
 #include <cstdio>
 #include <cstdlib>
@@ -16,6 +17,8 @@ void orc_noise(float *out, size_t n, uint64_t seed);
 void orc_quant_rows(float *out, size_t tokens, size_t values);
 int orc_attention_f64(const float *q, const float *k, const float *v, const float *q_and_gate, size_t len, size_t heads,
                       size_t kv_heads, size_t dim, double *out, int threads);
+int orc_prefill(const float *q, const float *keys, const float *values, size_t pos, size_t tokens, size_t heads,
+                size_t kv_heads, size_t dim, const float *q_and_gate, float *out, int threads);
 }
 
 using namespace saetta;
@@ -349,6 +352,44 @@ int main() {
         EXPECT(cache.capacity == 128, "shrink");
         std::vector<float> first(x.begin(), x.begin() + 128 * VALUES);
         compare(cache.quant->first, first, 0, KvBits::Eight);
+    }
+    {   // a prefill chunk over a half cache of spread data (tests/attention_prefill.rs:14-60, shape (1000, 64)) by
+        // the flash kernel and by AttGemm in two slices, against the CPU token by token
+        const size_t pos = 1000, tokens = 64, n = pos + tokens, capacity = 1088;
+        const auto qh = attention_prefill::spread(tokens * HEADS * DIM, 1);
+        const auto kh = attention_prefill::spread(capacity * VALUES, 2), vh = attention_prefill::spread(capacity * VALUES, 3);
+        std::vector<float> gate(tokens * HEADS * 2 * DIM);
+        for (size_t i = 0; i < gate.size(); i++) gate[i] = float(i % 7) - 3.0f;
+        auto widen = [](const std::vector<uint16_t> &h, size_t count) {
+            std::vector<float> f(count);
+            for (size_t i = 0; i < count; i++) {
+                _Float16 x;
+                std::memcpy(&x, &h[i], 2);
+                f[i] = float(x);
+            }
+            return f;
+        };
+        std::vector<float> want(tokens * HEADS * DIM);
+        const auto qf = widen(qh, qh.size()), kf = widen(kh, n * VALUES), vf = widen(vh, n * VALUES);
+        orc_prefill(qf.data(), kf.data(), vf.data(), pos, tokens, HEADS, KV, DIM, gate.data(), want.data(), 8);
+        View q(gpu.buffer_from(qh)), k(gpu.buffer_from(kh)), v(gpu.buffer_from(vh)), g(gpu.buffer_from(gate));
+        View flash(gpu.buffer(want.size() * 4)), gemm(gpu.buffer(want.size() * 4));
+        const attention_prefill::FlashParams f{uint32_t(HEADS), uint32_t(KV), uint32_t(pos), uint32_t(tokens), 1.0f / 16.0f};
+        attention_prefill::encode(gpu, attention_prefill::DEFAULT, q, k, v, g, flash, f);
+        setenv("SAETTA_AG_SLICES", "2", 1);
+        const attention_gemm::AttGemm att(gpu, tokens, KV);
+        unsetenv("SAETTA_AG_SLICES");
+        EXPECT(att.slice == 32 && att.rows_pad == 256 && attention_gemm::KEYS == 1024, "AttGemm::new: slice %zu", att.slice);
+        att.encode(gpu, q, k, v, nullptr, g, gemm, f);
+        gpu.sync();
+        const auto a = gpu::contents<float>(flash.buffer, want.size()), b = gpu::contents<float>(gemm.buffer, want.size());
+        float worst_a = 0.0f, worst_b = 0.0f;
+        for (size_t i = 0; i < want.size(); i++) {
+            worst_a = std::max(worst_a, std::fabs(a[i] - want[i]));
+            worst_b = std::max(worst_b, std::fabs(b[i] - want[i]));
+        }
+        std::printf("prefill (1000, 64): flash worst %.2e, gemm worst %.2e\n", worst_a, worst_b);
+        EXPECT(worst_a < 2e-3f && worst_b < 2e-3f, "prefill chunk: flash %g gemm %g", worst_a, worst_b);
     }
     // shape checks panic (throw) as the reference asserts
     bool threw = false;
