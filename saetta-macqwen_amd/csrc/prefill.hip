@@ -39,6 +39,7 @@
 // more than 2^8 (lazy rescale), so O is rarely rescaled.  Tiles are issued heaviest first and
 // there are two per CU, which evens out the causal imbalance.
 #include "common.hpp"
+#include "lanes.hpp"
 
 #include <mutex>
 
@@ -908,8 +909,8 @@ struct GemmArgs {
     const unsigned char *images;
     const float *q_and_gate;
     float *out;
-    unsigned char *p;    // f16 [kv head][row group][tile][2 k-steps][64 lanes][8]
-    float *tmax, *tsum;  // [kv head][row group][tile][32 rows], log2 domain
+    unsigned char *p;    // f16 [kv head][token tile][tile of keys][row group of the token tile][2 k-steps][64 lanes][8]
+    float *tmax, *tsum;  // [kv head][token tile][tile of keys][row group of the token tile][32 rows], log2 domain
     float *o;            // [kv head][row group][8 dim tiles][4][64 lanes][4]: the accumulators as they are
     float *m, *l;        // [kv head][row group][32 rows]
     uint32_t heads, kv_heads, pos, tokens;  // of the slice
@@ -933,8 +934,8 @@ __device__ __forceinline__ uint32_t ag_tiles(const GemmArgs &a, uint32_t tok0) {
     return n < uint32_t(AG_TILES) ? n : uint32_t(AG_TILES);
 }
 
-__global__ __launch_bounds__(AG_THREADS) void attention_gemm_scores_kernel(GemmArgs a) {
-    __shared__ __attribute__((aligned(1024))) unsigned char k_lds[2][PART_BYTES];
+__global__ __launch_bounds__(AG_THREADS, 3) void attention_gemm_scores_kernel(GemmArgs a) {
+    __shared__ __attribute__((aligned(1024))) unsigned char k_lds[3][PART_BYTES];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 31, hf = lane >> 5;
     const uint32_t tok0 = blockIdx.y * AG_TOKENS, kv = blockIdx.z;
     const uint32_t need = ag_tiles(a, tok0);
@@ -944,6 +945,27 @@ __global__ __launch_bounds__(AG_THREADS) void attention_gemm_scores_kernel(GemmA
     const uint32_t count = need - first < PER ? need - first : PER;
     const uint32_t rg = blockIdx.y * AG_WAVES + wave;
     const uint32_t tok = tok0 + 4 * wave + (col >> 3), head = kv * SAETTA_GQA_GROUP + (col & 7);
+
+    // A tile's K part goes global -> registers (two register sets, four and three tiles ahead) -> LDS (three
+    // buffers, two and one tile ahead) -> MFMA operands; the products of tile t + 1 are issued before the
+    // softmax of tile t, so that they run under it.  One barrier a tile.
+    const unsigned char *img = a.images + (size_t(kv) * a.nblocks + a.j0 / BK + first) * IMG_BYTES;
+    u32x4 pre[2][4];
+    // (Fetches and LDS writes past the last tile are made all the same, of the last tile again and into a
+    // buffer nobody reads any more: with no branch around a load or a store the compiler knows how many are in
+    // flight at each wait, and waits for the oldest only.)
+    auto fetch = [&](u32x4 *set, uint32_t t) {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(img + size_t(t < count ? t : count - 1) * IMG_BYTES);
+#pragma unroll
+        for (int i = 0; i < 4; i++) set[i] = src[tid + AG_THREADS * i];
+    };
+    auto put = [&](const u32x4 *set, uint32_t t) {
+        u32x4 *dst = reinterpret_cast<u32x4 *>(k_lds[t % 3]);
+#pragma unroll
+        for (int i = 0; i < 4; i++) dst[tid + AG_THREADS * i] = set[i];
+    };
+    fetch(pre[0], 0);
+    fetch(pre[1], 1);
 
     // Q^T operands: lane (col, hf) holds dims 16 f + 8 hf .. + 7 of query row col
     half8 qf[16];
@@ -956,24 +978,8 @@ __global__ __launch_bounds__(AG_THREADS) void attention_gemm_scores_kernel(GemmA
         for (int f = 0; f < 16; f++) qf[f] = half8{0, 0, 0, 0, 0, 0, 0, 0};
     }
 
-    const unsigned char *img = a.images + (size_t(kv) * a.nblocks + a.j0 / BK + first) * IMG_BYTES;
-    // a tile's part is fetched into registers two tiles ahead (two register sets, the loop in pairs)
-    u32x4 pre[2][4];
-    auto fetch = [&](u32x4 *set, uint32_t t) {
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(img + size_t(t) * IMG_BYTES);
-#pragma unroll
-        for (int i = 0; i < 4; i++) set[i] = src[tid + AG_THREADS * i];
-    };
-    fetch(pre[0], 0);
-    if (count > 1) fetch(pre[1], 1);
-    const uint32_t limit = a.pos + tok;  // the last key the row sees
-    const size_t row_base = (size_t(kv) * a.row_groups + rg) * AG_TILES;
-    auto tile = [&](u32x4 *set, uint32_t t) {
-        unsigned char *buf = k_lds[t & 1];
-#pragma unroll
-        for (int i = 0; i < 4; i++) reinterpret_cast<u32x4 *>(buf)[tid + AG_THREADS * i] = set[i];
-        __syncthreads();
-        if (t + 2 < count) fetch(set, t + 2);
+    auto products = [&](uint32_t t) {
+        const unsigned char *buf = k_lds[t % 3];
         floatx16 acc;
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[i] = 0.0f;
@@ -982,6 +988,14 @@ __global__ __launch_bounds__(AG_THREADS) void attention_gemm_scores_kernel(GemmA
             const half8 kf = *reinterpret_cast<const half8 *>(buf + f * 1024 + lane * 16);
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[f], acc, 0, 0, 0);
         }
+        return acc;
+    };
+
+    const uint32_t limit = a.pos + tok;  // the last key the row sees
+    // slot of (row group, tile) in the scratch: the four row groups of a workgroup side by side, tile after
+    // tile, so that what a workgroup writes at a step (8 KB of P) and over its tiles is one run of memory
+    const size_t slot0 = ((size_t(kv) * a.row_groups + rg) / AG_WAVES * AG_TILES + first) * AG_WAVES + wave;
+    auto softmax = [&](floatx16 acc, uint32_t t) {
         // register i is key 8 (i / 4) + 4 hf + i % 4 of the tile.  Only a tile that reaches past the first
         // token of the wave's row group has anything to mask (wave-uniform).
         const uint32_t key0 = a.j0 + (first + t) * BK;
@@ -995,7 +1009,7 @@ __global__ __launch_bounds__(AG_THREADS) void attention_gemm_scores_kernel(GemmA
         float tmax = fmaxf(acc[0], acc[1]);
 #pragma unroll
         for (int i = 2; i < 16; i += 2) tmax = fmaxf(tmax, fmaxf(acc[i], acc[i + 1]));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        tmax = across_rows<32, 64>(tmax, MaxOp{});
         // scores in the log2 domain: s = acc * c, the tile's maximum t = tmax * c (c > 0).  A masked score is
         // NO_SCORE * c - t: far below any exponent, 0; with the whole tile masked t is that too, and the
         // probabilities are set to 0 outright.
@@ -1011,22 +1025,47 @@ __global__ __launch_bounds__(AG_THREADS) void attention_gemm_scores_kernel(GemmA
             // the sum of what the second product multiplies: the rounded halves, added in f32
             sum = __builtin_amdgcn_fdot2(ph[i / 2], half2_{(_Float16)1.0f, (_Float16)1.0f}, sum, false);
         }
-        sum += __shfl_xor(sum, 32);
+        sum = across_rows<32, 64>(sum, SumOp{});
         const half8 p0 = {ph[0][0], ph[0][1], ph[1][0], ph[1][1], ph[2][0], ph[2][1], ph[3][0], ph[3][1]};
         const half8 p1 = {ph[4][0], ph[4][1], ph[5][0], ph[5][1], ph[6][0], ph[6][1], ph[7][0], ph[7][1]};
         const float tmax_out = none ? NO_SCORE : t_log2;
-        unsigned char *pt = a.p + (row_base + first + t) * AG_P_TILE_BYTES + lane * 16;
+        const size_t slot = slot0 + size_t(t) * AG_WAVES;
+        unsigned char *pt = a.p + slot * AG_P_TILE_BYTES + lane * 16;
         *reinterpret_cast<half8 *>(pt) = p0;
         *reinterpret_cast<half8 *>(pt + 1024) = p1;
-        if (hf == 0) {
-            a.tmax[(row_base + first + t) * 32 + col] = tmax_out;
-            a.tsum[(row_base + first + t) * 32 + col] = sum;
-        }
+        // (both lanes of a row hold the same two values: one stores the maximum, the other the sum)
+        float *stat = (hf ? a.tsum : a.tmax) + slot * 32 + col;
+        *stat = hf ? sum : tmax_out;
     };
-    for (uint32_t t = 0; t < count; t += 2) {
-        tile(pre[0], t);
-        if (t + 1 < count) tile(pre[1], t + 1);
+
+    put(pre[0], 0);
+    fetch(pre[0], 2);
+    put(pre[1], 1);
+    fetch(pre[1], 3);
+    __syncthreads();
+    floatx16 cur = products(0);
+    // iteration t: the set holds tile t + 2 and goes to the buffer tile t - 1 was read from (every wave has
+    // passed the barrier of iteration t - 1 after those reads); tile t + 1 is in LDS since iteration t - 1.
+    auto step = [&](u32x4 *set, uint32_t t) {
+        put(set, t + 2);
+        fetch(set, t + 4);
+        __syncthreads();
+        const floatx16 next = products(t + 1);  // (past the last tile: of a buffer's leftovers, never used)
+        softmax(cur, t);
+        cur = next;
+    };
+    // (The first pair stands in front of the loop: the loads and stores in flight where the loop is entered
+    // are then the ones in flight where it repeats, and the waits inside it are exact.)
+    uint32_t t = 0;
+    if (count >= 2) {
+        step(pre[0], 0);
+        step(pre[1], 1);
+        for (t = 2; t + 1 < count; t += 2) {
+            step(pre[0], t);
+            step(pre[1], t + 1);
+        }
     }
+    if (t < count) step(pre[0], t);
 }
 
 __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_pv_kernel(GemmArgs a) {
@@ -1042,9 +1081,11 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_pv_kernel(GemmAr
     const size_t state = rows * 32 + col;
     const bool first_block = a.j0 == 0;
 
-    const float *tm = a.tmax + rows * AG_TILES * 32 + col, *ts = a.tsum + rows * AG_TILES * 32 + col;
+    // slot of (row group, tile): as the scores kernel wrote them
+    const size_t slot0 = rows / AG_WAVES * AG_TILES * AG_WAVES + wave;
+    const float *tm = a.tmax + slot0 * 32 + col, *ts = a.tsum + slot0 * 32 + col;
     float mb = NO_SCORE;
-    for (uint32_t t = 0; t < need; t++) mb = fmaxf(mb, tm[t * 32]);
+    for (uint32_t t = 0; t < need; t++) mb = fmaxf(mb, tm[t * AG_WAVES * 32]);
     // (every row sees key 0, so m is a score from the first block on)
     const float m_old = first_block ? NO_SCORE : a.m[state], l_old = first_block ? 0.0f : a.l[state];
     const float m_new = fmaxf(m_old, mb);
@@ -1076,17 +1117,18 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_pv_kernel(GemmAr
         half8 p0, p1;
         float tm, ts;
     } pre[2];
-    const unsigned char *pp = a.p + rows * AG_TILES * AG_P_TILE_BYTES + lane * 16;
-    auto fetch = [&](Ahead &set, uint32_t t) {
+    const unsigned char *pp = a.p + slot0 * AG_P_TILE_BYTES + lane * 16;
+    auto fetch = [&](Ahead &set, uint32_t t) {  // (past the last tile: the last tile again, never used)
+        t = t < need ? t : need - 1;
         const u32x4 *src = reinterpret_cast<const u32x4 *>(img + size_t(t) * IMG_BYTES);
 #pragma unroll
         for (int i = 0; i < 4; i++) set.v[i] = src[tid + AG_THREADS * i];
-        set.p0 = *reinterpret_cast<const half8 *>(pp + size_t(t) * AG_P_TILE_BYTES);
-        set.p1 = *reinterpret_cast<const half8 *>(pp + size_t(t) * AG_P_TILE_BYTES + 1024);
-        set.tm = tm[t * 32], set.ts = ts[t * 32];
+        set.p0 = *reinterpret_cast<const half8 *>(pp + size_t(t) * AG_WAVES * AG_P_TILE_BYTES);
+        set.p1 = *reinterpret_cast<const half8 *>(pp + size_t(t) * AG_WAVES * AG_P_TILE_BYTES + 1024);
+        set.tm = tm[t * AG_WAVES * 32], set.ts = ts[t * AG_WAVES * 32];
     };
     fetch(pre[0], 0);
-    if (need > 1) fetch(pre[1], 1);
+    fetch(pre[1], 1);
     float lsum = 0.0f;
     auto tile = [&](Ahead &set, uint32_t t) {
         unsigned char *buf = v_lds[t & 1];
@@ -1095,7 +1137,7 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_pv_kernel(GemmAr
         __syncthreads();
         half8 pc0 = set.p0, pc1 = set.p1;
         const float tmc = set.tm, tsc = set.ts;
-        if (t + 2 < need) fetch(set, t + 2);
+        fetch(set, t + 2);
         // a tile the row sees nothing of has t = NO_SCORE: its factor is 0, like its probabilities
         const _Float16 fh = (_Float16)__builtin_amdgcn_exp2f(tmc - m_new);
         lsum += (float)fh * tsc;
@@ -1108,10 +1150,16 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_pv_kernel(GemmAr
             acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(v1, pc1, acc[mt], 0, 0, 0);
         }
     };
-    for (uint32_t t = 0; t < need; t += 2) {
-        tile(pre[0], t);
-        if (t + 1 < need) tile(pre[1], t + 1);
+    uint32_t t = 0;
+    if (need >= 2) {  // (the first pair in front of the loop, as in the scores kernel)
+        tile(pre[0], 0);
+        tile(pre[1], 1);
+        for (t = 2; t + 1 < need; t += 2) {
+            tile(pre[0], t);
+            tile(pre[1], t + 1);
+        }
     }
+    if (t < need) tile(pre[0], t);
     const float l_new = alpha * l_old + lsum;
 
     if (last_block && a.write_out) {
