@@ -48,6 +48,7 @@ namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2_ __attribute__((ext_vector_type(2)));
+typedef float float2_ __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -978,14 +979,19 @@ __global__ __launch_bounds__(AG_THREADS, 3) void attention_gemm_scores_kernel(Ge
         for (int f = 0; f < 16; f++) qf[f] = half8{0, 0, 0, 0, 0, 0, 0, 0};
     }
 
+    typedef __attribute__((address_space(3))) half8 lds_half8;
+    const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(&k_lds[0][0]));
     auto products = [&](uint32_t t) {
-        const unsigned char *buf = k_lds[t % 3];
+        // One address per tile, the fragments by the instruction's offset field (the address is hidden from
+        // the loop optimizer, which otherwise keeps sixteen running addresses and two additions a read).
+        uint32_t frag = lds0 + (t % 3) * PART_BYTES + lane * 16;
+        asm volatile("" : "+v"(frag));
         floatx16 acc;
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[i] = 0.0f;
 #pragma unroll
         for (int f = 0; f < 16; f++) {
-            const half8 kf = *reinterpret_cast<const half8 *>(buf + f * 1024 + lane * 16);
+            const half8 kf = *reinterpret_cast<const lds_half8 *>(uintptr_t(frag + f * 1024));
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[f], acc, 0, 0, 0);
         }
         return acc;
@@ -1006,22 +1012,25 @@ __global__ __launch_bounds__(AG_THREADS, 3) void attention_gemm_scores_kernel(Ge
                 acc[i] = key <= limit ? acc[i] : NO_SCORE;
             }
         }
-        float tmax = fmaxf(acc[0], acc[1]);
+        // (v_max3 by hand: fmaxf first quiets each operand with a v_max of its own)
+        float tmax;
+        asm("v_max3_f32 %0, %1, %2, %3" : "=v"(tmax) : "v"(acc[0]), "v"(acc[1]), "v"(acc[2]));
 #pragma unroll
-        for (int i = 2; i < 16; i += 2) tmax = fmaxf(tmax, fmaxf(acc[i], acc[i + 1]));
+        for (int i = 3; i < 15; i += 2) asm("v_max3_f32 %0, %1, %2, %3" : "=v"(tmax) : "v"(tmax), "v"(acc[i]), "v"(acc[i + 1]));
+        asm("v_max_f32 %0, %1, %2" : "=v"(tmax) : "v"(tmax), "v"(acc[15]));
         tmax = across_rows<32, 64>(tmax, MaxOp{});
         // scores in the log2 domain: s = acc * c, the tile's maximum t = tmax * c (c > 0).  A masked score is
-        // NO_SCORE * c - t: far below any exponent, 0; with the whole tile masked t is that too, and the
-        // probabilities are set to 0 outright.
+        // NO_SCORE * c - t: far below any exponent, 0.  With the whole tile masked t would be NO_SCORE * c itself
+        // and the difference the product's rounding error: 0 is subtracted then, and every probability is 0.
         const float t_log2 = tmax * a.c;
         const bool none = tmax <= 0.5f * NO_SCORE;
+        const float t_sub = none ? 0.0f : t_log2;
         half2_ ph[8];
         float sum = 0.0f;
 #pragma unroll
         for (int i = 0; i < 16; i += 2) {
-            const float e0 = none ? 0.0f : __builtin_amdgcn_exp2f(fmaf(acc[i], a.c, -t_log2));
-            const float e1 = none ? 0.0f : __builtin_amdgcn_exp2f(fmaf(acc[i + 1], a.c, -t_log2));
-            ph[i / 2] = half2_{(_Float16)e0, (_Float16)e1};
+            const float2_ e = {__builtin_amdgcn_exp2f(fmaf(acc[i], a.c, -t_sub)), __builtin_amdgcn_exp2f(fmaf(acc[i + 1], a.c, -t_sub))};
+            ph[i / 2] = __builtin_convertvector(e, half2_);
             // the sum of what the second product multiplies: the rounded halves, added in f32
             sum = __builtin_amdgcn_fdot2(ph[i / 2], half2_{(_Float16)1.0f, (_Float16)1.0f}, sum, false);
         }
