@@ -59,6 +59,8 @@ class TokenParams:
 
 
 def _stream(stream=None):
+    if isinstance(stream, ctypes.c_void_p):  # what a plan op is handed
+        return stream
     s = stream if stream is not None else torch.cuda.current_stream()
     return ctypes.c_void_p(s.cuda_stream)
 

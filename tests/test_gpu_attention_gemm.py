@@ -182,3 +182,28 @@ def test_sweep(seed, monkeypatch):
         want = oracle.prefill(q16.astype(np.float32), kf, vf, pos, tokens, q_and_gate=qg, threads=8)
         assert np.isfinite(got).all(), (seed, done, kind, pos, tokens, slices)
         assert np.abs(got - want).max() < MAX_ABS and oracle.rel_rms(got, want) < REL_RMS, (seed, done, kind, pos, tokens, slices)
+
+
+def test_replayed_from_a_graph_equals_the_eager_call():
+    # The call only enqueues kernels once its buffers exist (made by a first eager call), so a plan can
+    # capture it: three replays with other work and synchronizations between them, each against the eager
+    # result, bit for bit (the same kernels in the same order on the same inputs).
+    pos, tokens = 1500, 300
+    q16, k, v, qg = spread_case(pos, tokens)
+    kc, vc, _, _ = make_cache(saetta.KvBits.Eight, k, v, 1856)
+    q, g = dev(q16), dev(qg)
+    p = saetta.FlashParams(H, KV, pos, tokens, 1.0 / math.sqrt(D))
+    gemm = saetta.attention_gemm.AttGemm(tokens, KV)
+    eager = torch.empty(tokens, H, D, device="cuda")
+    gemm.encode(q, None, None, (kc, vc), g, eager, p)
+    out = torch.full((tokens, H, D), float("nan"), device="cuda")
+    plan = saetta.Plan()
+    plan.op("attention_gemm", lambda s: gemm.encode(q, None, None, (kc, vc), g, out, p, stream=s))
+    built = plan.build(graph=True)
+    for replay in range(3):
+        out.fill_(float("nan"))
+        built.run()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), replay
+        junk = torch.randn(1 << 20, device="cuda").sum().item()  # eager work between the replays
+        assert junk == junk
