@@ -2,8 +2,10 @@
  * saetta_hip.h -- C ABI of the MI355X (gfx950) attention hot path.
  *
  * The library replaces, for this one path, what the reference's Rust modules
- * src/kv_quant.rs, src/attention.rs, src/rows.rs (verify attention) and
- * src/attention_prefill.rs dispatch to Metal.  Every entry point is
+ * src/kv_quant.rs, src/attention.rs, src/rows.rs (verify attention),
+ * src/attention_prefill.rs and src/attention_gemm.rs dispatch to Metal (and,
+ * next to the path, the store step and the Gated DeltaNet kernels of
+ * src/gpu_layers.rs and src/prefill.rs).  Every entry point is
  * extern "C", takes plain device pointers, POD parameter blocks that are
  * field-for-field the reference's #[repr(C)] structs, and an explicit HIP
  * stream; it enqueues work on that stream and returns without synchronising.

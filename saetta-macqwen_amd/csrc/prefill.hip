@@ -11,7 +11,8 @@
 // cache is seen "through half": every value is f16(f32(s)*code + f32(z)),
 // exactly what round_trip_as_half (src/kv_quant.rs:119-125) gives the CPU path.
 //
-// Two kernels.
+// Two kernels (and, further down, the reference's other route to the same output, AttGemm of
+// src/attention_gemm.rs: two more kernels on the same images, block by block of 1024 keys).
 //
 // prefill_prepare_kernel<16|8|4> turns the keys and values the chunk can see into
 // f16 tile images in a workspace, one image per (kv head, block of 32 keys): the K tile
