@@ -358,6 +358,24 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8, gemm=False):
         ts.append(e0.elapsed_time(e1) * 1e3)
     kern_us = median(ts)
     achieved = flops / (kern_us * 1e-6) / 1e12
+    roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4),
+                "traffic": MEASURED_TRAFFIC.get("prefill") if (tokens, pos, bits, gemm) == (4096, 4096, 8, False) else None,
+                "kernel": "attention_prefill_kernel", "avg_us": round(kern_us, 2)}
+    if gemm:
+        # What bounds this route is the scratch it writes and reads back.  Algorithmic bytes per query row: 2 B out
+        # and 2 B in per key its 32-token tile sees (in whole tiles of 32 keys); per block of 1024 keys it
+        # touches, 1 KB of output sums in and 1 KB out and its q twice (one read per half of the block's tiles).
+        nbytes = 0
+        for t0 in range(0, tokens, 32):
+            last_key = pos + min(t0 + 32, tokens) - 1
+            rows = (min(t0 + 32, tokens) - t0) * H
+            nbytes += rows * ((last_key // 32 + 1) * 32 * 4 + (last_key // 1024 + 1) * 3072)
+        gbs = nbytes / (kern_us * 1e-6) / 1e9
+        roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                    "kernel": "attention_gemm_scores_kernel + attention_gemm_pv_kernel", "avg_us": round(kern_us, 2),
+                    "bytes": nbytes, "mfma_TFLOPs": round(achieved, 2), "mfma_frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4)}
     # CPU baseline on a bounded sample: the last `sample` tokens of the chunk (the longest rows).
     sample = max(16, 512 * 8192 // (pos + tokens))  # 512 tokens at the headline shape: about 7 s on one core
     groups = (pos + tokens) * 8
@@ -390,11 +408,7 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8, gemm=False):
                              "roofline: median of event-timed prepare + attention calls"
                              + (f" ({2 * -(-(pos + tokens) // 1024)} launches: scores and pv per block of 1024 keys)" if gemm else ""),
                    "inputs": "q (through bf16), K, V, gate ~ N(0,1) from torch's device generator (Philox, seed 99)"},
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC.get("prefill") if (tokens, pos, bits, gemm) == (4096, 4096, 8, False) else None,
-                     "kernel": "attention_gemm_scores_kernel + attention_gemm_pv_kernel" if gemm else "attention_prefill_kernel",
-                     "avg_us": round(kern_us, 2)},
+        "roofline": roofline,
         "cpu_baseline": {"value": round(cpu_flops / cpu_s / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
                          "sample": f"the last {sample} tokens of the chunk ({cpu_s:.2f} s)"},
         "parity_rel_rms_vs_oracle": float(f"{rel_rms:.3e}"),
