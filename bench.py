@@ -364,12 +364,12 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8, gemm=False):
                 "kernel": "attention_prefill_kernel", "avg_us": round(kern_us, 2)}
     if gemm:
         # What bounds this route is the scratch it writes and reads back.  Algorithmic bytes per query row: 2 B out
-        # and 2 B in per key its 32-token tile sees (in whole tiles of 32 keys); per block of 1024 keys it
+        # and 2 B in per key its 16-token tile sees (in whole tiles of 32 keys); per block of 1024 keys it
         # touches, 1 KB of output sums in and 1 KB out and its q twice (one read per half of the block's tiles).
         nbytes = 0
-        for t0 in range(0, tokens, 32):
-            last_key = pos + min(t0 + 32, tokens) - 1
-            rows = (min(t0 + 32, tokens) - t0) * H
+        for t0 in range(0, tokens, 16):
+            last_key = pos + min(t0 + 16, tokens) - 1
+            rows = (min(t0 + 16, tokens) - t0) * H
             nbytes += rows * ((last_key // 32 + 1) * 32 * 4 + (last_key // 1024 + 1) * 3072)
         gbs = nbytes / (kern_us * 1e-6) / 1e9
         roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
