@@ -949,8 +949,7 @@ __global__ __launch_bounds__(AG_THREADS, 3) void attention_gemm_scores_kernel(Ge
     const uint32_t tok = tok0 + 4 * wave + (col >> 3), head = kv * SAETTA_GQA_GROUP + (col & 7);
 
     // A tile's K part goes global -> registers (two register sets, four and three tiles ahead) -> LDS (three
-    // buffers, two and one tile ahead) -> MFMA operands; the products of tile t + 1 are issued before the
-    // softmax of tile t, so that they run under it.  One barrier a tile.
+    // buffers, two and one tile ahead) -> MFMA operands.  One barrier a tile.
     const unsigned char *img = a.images + (size_t(kv) * a.nblocks + a.j0 / BK + first) * IMG_BYTES;
     u32x4 pre[2][4];
     // (Fetches and LDS writes past the last tile are made all the same, of the last tile again and into a
@@ -1053,16 +1052,13 @@ __global__ __launch_bounds__(AG_THREADS, 3) void attention_gemm_scores_kernel(Ge
     put(pre[1], 1);
     fetch(pre[1], 3);
     __syncthreads();
-    floatx16 cur = products(0);
-    // iteration t: the set holds tile t + 2 and goes to the buffer tile t - 1 was read from (every wave has
-    // passed the barrier of iteration t - 1 after those reads); tile t + 1 is in LDS since iteration t - 1.
+    // iteration t: behind its barrier tile t is in LDS (written two iterations ago) and every wave is done with
+    // tile t - 1, whose buffer takes tile t + 2 from the register set, which is then sent for tile t + 4.
     auto step = [&](u32x4 *set, uint32_t t) {
+        if (t) __syncthreads();
         put(set, t + 2);
         fetch(set, t + 4);
-        __syncthreads();
-        const floatx16 next = products(t + 1);  // (past the last tile: of a buffer's leftovers, never used)
-        softmax(cur, t);
-        cur = next;
+        softmax(products(t), t);
     };
     // (The first pair stands in front of the loop: the loads and stores in flight where the loop is entered
     // are then the ones in flight where it repeats, and the waits inside it are exact.)
