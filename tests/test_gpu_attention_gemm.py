@@ -161,6 +161,13 @@ def test_rejections(monkeypatch):
     assert lib.saetta_attn_gemm(*args, 0, 4, ws.data_ptr(), need) != 0
     assert "stages" in lib.saetta_last_error().decode()
     assert lib.saetta_attn_gemm(*args, 0, 0, ws.data_ptr(), need) == 0
+    want = host(out).copy()
+    # no workspace: the library's own, grown on demand (not under capture)
+    out.zero_()
+    assert lib.saetta_attn_gemm(*args, 0, 0, None, 0) == 0
+    assert np.array_equal(host(out), want)
+    assert lib.saetta_attn_gemm(*args, 7, 0, None, 0) == 0  # three slices of 7, 7 and 6 tokens
+    assert np.abs(host(out) - want).max() < 1e-6
 
 
 @pytest.mark.parametrize("seed", [31, 32])
