@@ -214,3 +214,27 @@ def test_replayed_from_a_graph_equals_the_eager_call():
         assert torch.equal(out, eager), replay
         junk = torch.randn(1 << 20, device="cuda").sum().item()  # eager work between the replays
         assert junk == junk
+
+
+@pytest.mark.parametrize("kv_heads", [1, 4])
+def test_other_head_counts_both_routes(kv_heads):
+    # 8 and 32 q heads (1 and 4 kv heads) over a half cache, 1100 keys: the flash kernel and AttGemm against the
+    # oracle.  (The model has 16 / 2; the entry points take any kv head count with 8 q heads each.)
+    rng = np.random.default_rng(70 + kv_heads)
+    heads, pos, tokens = 8 * kv_heads, 1000, 100
+    n = pos + tokens
+    q16 = rng.standard_normal((tokens, heads, D)).astype(np.float16)
+    k16 = rng.standard_normal((n, kv_heads * D)).astype(np.float16)
+    v16 = rng.standard_normal((n, kv_heads * D)).astype(np.float16)
+    qg = rng.standard_normal((tokens, heads, 2 * D)).astype(np.float32)
+    want = oracle.prefill(q16.astype(np.float32), k16.astype(np.float32), v16.astype(np.float32), pos, tokens,
+                          heads=heads, kv_heads=kv_heads, q_and_gate=qg, threads=8)
+    p = saetta.FlashParams(heads, kv_heads, pos, tokens, 1.0 / math.sqrt(D))
+    q, kc, vc, g = dev(q16), dev(k16), dev(v16), dev(qg)
+    flash = torch.full((tokens, heads, D), float("nan"), device="cuda")
+    saetta.attention_prefill.encode(saetta.attention_prefill.DEFAULT, q, kc, vc, g, flash, p)
+    gemm = torch.full((tokens, heads, D), float("nan"), device="cuda")
+    saetta.attention_gemm.AttGemm(tokens, kv_heads).encode(q, kc, vc, None, g, gemm, p)
+    for got in (host(flash), host(gemm)):
+        assert np.isfinite(got).all()
+        assert np.abs(got - want).max() < MAX_ABS and oracle.rel_rms(got, want) < REL_RMS
