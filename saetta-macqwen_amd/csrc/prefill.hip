@@ -903,7 +903,8 @@ constexpr int AG_TILES = AG_KEYS / BK;
 constexpr int AG_WAVES = 4;
 constexpr int AG_THREADS = 64 * AG_WAVES;
 constexpr int AG_TOKENS = 4 * AG_WAVES;   // tokens of a workgroup
-constexpr int AG_SPLIT = 2;               // scores: workgroups that share a block's tiles for one token tile
+constexpr int AG_SPLIT = 2;
+constexpr int AG_RG = 2;                  // scores: row groups per wave, which share every fragment of keys it reads               // scores: workgroups that share a block's tiles for one token tile
 constexpr int AG_P_TILE_BYTES = BK * 32 * 2;  // the P^T operands of one row group and tile of keys
 
 struct GemmArgs {
@@ -925,28 +926,29 @@ struct GemmArgs {
 
 // Key of the last token of the workgroup's token tile, and how many of the block's tiles hold keys that
 // some token of the tile can see.
-__device__ __forceinline__ uint32_t ag_last_key(const GemmArgs &a, uint32_t tok0) {
-    const uint32_t end = tok0 + AG_TOKENS < a.tokens ? tok0 + AG_TOKENS : a.tokens;
+__device__ __forceinline__ uint32_t ag_last_key(const GemmArgs &a, uint32_t tok0, uint32_t span = AG_TOKENS) {
+    const uint32_t end = tok0 + span < a.tokens ? tok0 + span : a.tokens;
     return a.pos + end - 1;
 }
-__device__ __forceinline__ uint32_t ag_tiles(const GemmArgs &a, uint32_t tok0) {
-    const uint32_t last_key = ag_last_key(a, tok0);
+__device__ __forceinline__ uint32_t ag_tiles(const GemmArgs &a, uint32_t tok0, uint32_t span = AG_TOKENS) {
+    const uint32_t last_key = ag_last_key(a, tok0, span);
     if (last_key < a.j0) return 0;
     const uint32_t n = (last_key - a.j0) / BK + 1;
     return n < uint32_t(AG_TILES) ? n : uint32_t(AG_TILES);
 }
 
-__global__ __launch_bounds__(AG_THREADS, 3) void attention_gemm_scores_kernel(GemmArgs a) {
+__global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_scores_kernel(GemmArgs a) {
     __shared__ __attribute__((aligned(1024))) unsigned char k_lds[3][PART_BYTES];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 31, hf = lane >> 5;
-    const uint32_t tok0 = blockIdx.y * AG_TOKENS, kv = blockIdx.z;
-    const uint32_t need = ag_tiles(a, tok0);
+    // a workgroup takes AG_RG token tiles of the pv kernel: a wave AG_RG row groups in a row (8 tokens)
+    const uint32_t tok0 = blockIdx.y * (AG_TOKENS * AG_RG), kv = blockIdx.z;
+    const uint32_t need = ag_tiles(a, tok0, AG_TOKENS * AG_RG);
     constexpr uint32_t PER = AG_TILES / AG_SPLIT;
     const uint32_t first = blockIdx.x * PER;
     if (first >= need) return;  // (the whole workgroup)
     const uint32_t count = need - first < PER ? need - first : PER;
-    const uint32_t rg = blockIdx.y * AG_WAVES + wave;
-    const uint32_t tok = tok0 + 4 * wave + (col >> 3), head = kv * SAETTA_GQA_GROUP + (col & 7);
+    const uint32_t rg0 = (blockIdx.y * AG_WAVES + wave) * AG_RG;                    // the wave's first row group
+    const uint32_t wtok0 = tok0 + 4 * AG_RG * wave, head = kv * SAETTA_GQA_GROUP + (col & 7);  // and its first token
 
     // A tile's K part goes global -> registers (two register sets, four and three tiles ahead) -> LDS (three
     // buffers, two and one tile ahead) -> MFMA operands.  One barrier a tile.
@@ -969,43 +971,49 @@ __global__ __launch_bounds__(AG_THREADS, 3) void attention_gemm_scores_kernel(Ge
     fetch(pre[1], 1);
 
     // Q^T operands: lane (col, hf) holds dims 16 f + 8 hf .. + 7 of query row col
-    half8 qf[16];
-    if (tok < a.tokens) {
-        const half8 *qp = reinterpret_cast<const half8 *>(a.q + (size_t(tok) * a.heads + head) * DIM) + hf;
+    half8 qf[AG_RG][16];
 #pragma unroll
-        for (int f = 0; f < 16; f++) qf[f] = qp[2 * f];
-    } else {
+    for (int r = 0; r < AG_RG; r++) {
+        const uint32_t tok = wtok0 + 4 * r + (col >> 3);
+        if (tok < a.tokens) {
+            const half8 *qp = reinterpret_cast<const half8 *>(a.q + (size_t(tok) * a.heads + head) * DIM) + hf;
 #pragma unroll
-        for (int f = 0; f < 16; f++) qf[f] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+            for (int f = 0; f < 16; f++) qf[r][f] = qp[2 * f];
+        } else {
+#pragma unroll
+            for (int f = 0; f < 16; f++) qf[r][f] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+        }
     }
 
     typedef __attribute__((address_space(3))) half8 lds_half8;
     const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(&k_lds[0][0]));
-    auto products = [&](uint32_t t) {
+    auto products = [&](uint32_t t, floatx16 (&acc)[AG_RG]) {
         // One address per tile, the fragments by the instruction's offset field (the address is hidden from
         // the loop optimizer, which otherwise keeps sixteen running addresses and two additions a read).
         uint32_t frag = lds0 + (t % 3) * PART_BYTES + lane * 16;
         asm volatile("" : "+v"(frag));
-        floatx16 acc;
 #pragma unroll
-        for (int i = 0; i < 16; i++) acc[i] = 0.0f;
+        for (int r = 0; r < AG_RG; r++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[r][i] = 0.0f;
 #pragma unroll
         for (int f = 0; f < 16; f++) {
             const half8 kf = *reinterpret_cast<const lds_half8 *>(uintptr_t(frag + f * 1024));
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[f], acc, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < AG_RG; r++) acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[r][f], acc[r], 0, 0, 0);
         }
-        return acc;
     };
 
-    const uint32_t limit = a.pos + tok;  // the last key the row sees
-    // slot of (row group, tile) in the scratch: the four row groups of a workgroup side by side, tile after
-    // tile, so that what a workgroup writes at a step (8 KB of P) and over its tiles is one run of memory
-    const size_t slot0 = ((size_t(kv) * a.row_groups + rg) / AG_WAVES * AG_TILES + first) * AG_WAVES + wave;
-    auto softmax = [&](floatx16 acc, uint32_t t) {
+    auto softmax = [&](floatx16 acc, uint32_t t, int r) {
+        const uint32_t rg = rg0 + r;
+        const uint32_t limit = a.pos + wtok0 + 4 * r + (col >> 3);  // the last key the row sees
+        // slot of (row group, tile) in the scratch: the four row groups of a token tile side by side, tile after
+        // tile, so that what a workgroup writes at a step and over its tiles are long runs of memory
+        const size_t slot0 = ((size_t(kv) * a.row_groups + rg) / AG_WAVES * AG_TILES + first) * AG_WAVES + rg % AG_WAVES;
         // register i is key 8 (i / 4) + 4 hf + i % 4 of the tile.  Only a tile that reaches past the first
-        // token of the wave's row group has anything to mask (wave-uniform).
+        // token of the row group has anything to mask (wave-uniform).
         const uint32_t key0 = a.j0 + (first + t) * BK;
-        if (key0 + BK - 1 > a.pos + tok0 + 4 * wave) {
+        if (key0 + BK - 1 > a.pos + wtok0 + 4 * r) {
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const uint32_t key = key0 + 4 * hf + 8 * (i >> 2) + (i & 3);
@@ -1058,7 +1066,10 @@ __global__ __launch_bounds__(AG_THREADS, 3) void attention_gemm_scores_kernel(Ge
         if (t) __syncthreads();
         put(set, t + 2);
         fetch(set, t + 4);
-        softmax(products(t), t);
+        floatx16 acc[AG_RG];
+        products(t, acc);
+#pragma unroll
+        for (int r = 0; r < AG_RG; r++) softmax(acc[r], t, r);
     };
     // (The first pair stands in front of the loop: the loads and stores in flight where the loop is entered
     // are then the ones in flight where it repeats, and the waits inside it are exact.)
@@ -1207,7 +1218,10 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_pv_kernel(GemmAr
 size_t align_up(size_t n, size_t a) { return (n + a - 1) / a * a; }
 
 // Row groups of the scratch per kv head for slices of up to `slice` tokens: whole workgroups.
-size_t gemm_row_groups(uint32_t slice) { return size_t((slice + AG_TOKENS - 1) / AG_TOKENS) * AG_WAVES; }
+size_t gemm_row_groups(uint32_t slice) {
+    constexpr uint32_t SPAN = AG_TOKENS * AG_RG;  // what a scores workgroup covers
+    return size_t((slice + SPAN - 1) / SPAN) * AG_WAVES * AG_RG;
+}
 
 size_t gemm_scratch_bytes(uint32_t slice, uint32_t kv_heads) {
     const size_t groups = gemm_row_groups(slice) * kv_heads;
@@ -1263,7 +1277,7 @@ int run_gemm(hipStream_t stream, int bits, const uint16_t *q, const void *kdata,
         const uint64_t end = uint64_t(a.pos) + a.tokens;
         for (uint64_t j0 = 0; j0 < end; j0 += AG_KEYS) {
             a.j0 = uint32_t(j0);
-            attention_gemm_scores_kernel<<<dim3(AG_SPLIT, tiles, p.kv_heads), AG_THREADS, 0, stream>>>(a);
+            attention_gemm_scores_kernel<<<dim3(AG_SPLIT, (tiles + AG_RG - 1) / AG_RG, p.kv_heads), AG_THREADS, 0, stream>>>(a);
             if (stages == 1 || stages == 2) continue;
             attention_gemm_pv_kernel<<<dim3(1, tiles, p.kv_heads), AG_THREADS, 0, stream>>>(a);
         }
