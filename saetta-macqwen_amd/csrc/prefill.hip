@@ -1101,8 +1101,13 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_pv_kernel(GemmAr
     // slot of (row group, tile): as the scores kernel wrote them
     const size_t slot0 = rows / AG_WAVES * AG_TILES * AG_WAVES + wave;
     const float *tm = a.tmax + slot0 * 32 + col, *ts = a.tsum + slot0 * 32 + col;
-    float mb = NO_SCORE;
-    for (uint32_t t = 0; t < need; t++) mb = fmaxf(mb, tm[t * AG_WAVES * 32]);
+    // (all of the block's tile maxima requested at once: a loop over `need` waits for each load in turn)
+    float tmaxes[AG_TILES];
+#pragma unroll
+    for (int t = 0; t < AG_TILES; t++) tmaxes[t] = tm[(uint32_t(t) < need ? t : need - 1) * AG_WAVES * 32];
+    float mb = tmaxes[0];
+#pragma unroll
+    for (int t = 1; t < AG_TILES; t++) mb = fmaxf(mb, tmaxes[t]);
     // (every row sees key 0, so m is a score from the first block on)
     const float m_old = first_block ? NO_SCORE : a.m[state], l_old = first_block ? 0.0f : a.l[state];
     const float m_new = fmaxf(m_old, mb);
