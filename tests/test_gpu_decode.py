@@ -391,3 +391,49 @@ def test_equal_keys_give_the_mean_of_the_values(kind, ctx, m):
         want = np.repeat(mean, H // KV, axis=0) * gate
         worst = np.abs(got[r] - want).max()
         assert worst < MAX_ABS_F64, (kind, ctx, m, r, worst)
+
+
+@pytest.mark.parametrize("kv_heads", [1, 4])
+@pytest.mark.parametrize("kind", KINDS)
+def test_other_head_counts(kind, kv_heads):
+    # 8 and 32 q heads (1 and 4 kv heads): one row and three verify rows at a short and at a long context (the
+    # register kernels, and for the codes at 32768 the loader kernels), against the f64 formula.  The model
+    # has 16 / 2; the entry points take any kv head count with 8 q heads each.
+    rng = np.random.default_rng(900 + kv_heads)
+    heads, values = 8 * kv_heads, kv_heads * D
+    for ctx in (300, 4000 if kind is saetta.KvBits.Half else 32768):
+        m = 3
+        capacity = -(-(ctx + m) // 128) * 128
+        tokens = ctx - 1 + m
+        k = rng.standard_normal((tokens, values)).astype(np.float32)
+        v = rng.standard_normal((tokens, values)).astype(np.float32)
+        q = rng.standard_normal((m, heads, D)).astype(np.float32)
+        qg = rng.standard_normal((m, heads, 2 * D)).astype(np.float32)
+        if kind is saetta.KvBits.Half:
+            kc = torch.full((capacity, values), float("nan"), dtype=torch.float16, device="cuda")
+            vc = torch.full((capacity, values), float("nan"), dtype=torch.float16, device="cuda")
+            kc[:tokens], vc[:tokens] = dev(k.astype(np.float16)), dev(v.astype(np.float16))
+            kf, vf = oracle.round_trip(k, 16), oracle.round_trip(v, 16)
+        else:
+            kc, vc = saetta.QuantRows(kind, values, capacity), saetta.QuantRows(kind, values, capacity)
+            for c, x in ((kc, k), (vc, v)):
+                c.scales[:], c.biases[:], c.data[:] = float("nan"), float("inf"), -1
+                c.encode(dev(x.reshape(-1)), 0, tokens)
+            bits = kind.value
+            kf, vf = oracle.round_trip(k, bits), oracle.round_trip(v, bits)
+        pos = ctx - 1
+        rows = saetta.AttentionRows(heads, kv_heads, capacity, saetta.MAX_ROWS)
+        out = torch.full((m, heads, D), float("nan"), device="cuda")
+        params = [saetta.TokenParams(0, pos + r).as_tensor("cuda") for r in range(m)]
+        plan = saetta.Plan()
+        (rows.record if kind is saetta.KvBits.Half else rows.record_quant)(plan, m, dev(q), kc, vc, dev(qg), out, params)
+        plan.build().run()
+        want = oracle.rows(q, kf, vf, pos, m, heads=heads, kv_heads=kv_heads, q_and_gate=qg, threads=8, f64=True)
+        assert np.abs(host(out) - want).max() < MAX_ABS_F64, (kind, kv_heads, ctx)
+        att = saetta.DecodeAttention(heads, kv_heads, D, capacity)
+        one = torch.full((heads, D), float("nan"), device="cuda")
+        plan = saetta.Plan()
+        (att.record if kind is saetta.KvBits.Half else att.record_quant)(plan, dev(q[0]), kc, vc, dev(qg[0]), one)
+        plan.set_params(saetta.TokenParams(0, pos))
+        plan.build().run()
+        assert np.abs(host(one) - want[0]).max() < MAX_ABS_F64, (kind, kv_heads, ctx)
