@@ -238,3 +238,16 @@ def test_other_head_counts_both_routes(kv_heads):
     for got in (host(flash), host(gemm)):
         assert np.isfinite(got).all()
         assert np.abs(got - want).max() < MAX_ABS and oracle.rel_rms(got, want) < REL_RMS
+
+
+def test_bench_mirrors_the_reference():
+    # bench (src/attention_gemm.rs:366-470) at a small shape: both kernels timed at the last and the middle
+    # chunk, the passes one by one, and the two outputs compared as the reference prints them.
+    assert saetta.attention_gemm.KEYS == 1024
+    (row,) = saetta.attention_gemm.bench([3000], 512, 10)
+    assert row["context"] == 3072 and row["chunk"] == 512
+    for name in ("rows2", "gemm"):
+        assert row[name]["last_ms"] > 0 and row[name]["last_TFLOP/s"] > 0 and row[name]["prefill_attention_s"] > 0
+    assert set(row["stages"]) == {"scores_ms", "scores_TFLOP/s", "softmax_ms", "pv_ms", "pv_TFLOP/s", "final_ms"}
+    assert row["stages"]["scores_ms"] > 0
+    assert row["rel_rms"] < 1e-3 and row["max_abs"] < MAX_ABS
