@@ -900,6 +900,8 @@ int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kda
 //            key writes out = O / l * sigmoid(gate) instead of O.
 constexpr int AG_KEYS = SAETTA_AG_KEYS;
 constexpr int AG_TILES = AG_KEYS / BK;
+constexpr int AG_SPAN = 4;                // blocks that one pv launch folds in: the output sums go to memory and back once per span
+constexpr int AG_SPAN_TILES = AG_SPAN * AG_TILES;
 constexpr int AG_WAVES = 4;
 constexpr int AG_THREADS = 64 * AG_WAVES;
 constexpr int AG_TOKENS = 4 * AG_WAVES;   // tokens of a workgroup
@@ -921,6 +923,7 @@ struct GemmArgs {
     uint32_t nblocks;    // images per kv head
     uint32_t row_groups; // per kv head in the scratch
     uint32_t j0;         // the block's first key
+    uint32_t g0;         // the first key of the span of blocks it belongs to
     uint32_t write_out;  // 0: the outputs are never written (timing the passes apart)
 };
 
@@ -1009,7 +1012,7 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_scores_kernel(Ge
         const uint32_t limit = a.pos + wtok0 + 4 * r + (col >> 3);  // the last key the row sees
         // slot of (row group, tile) in the scratch: the four row groups of a token tile side by side, tile after
         // tile, so that what a workgroup writes at a step and over its tiles are long runs of memory
-        const size_t slot0 = ((size_t(kv) * a.row_groups + rg) / AG_WAVES * AG_TILES + first) * AG_WAVES + rg % AG_WAVES;
+        const size_t slot0 = ((size_t(kv) * a.row_groups + rg) / AG_WAVES * AG_SPAN_TILES + (a.j0 - a.g0) / BK + first) * AG_WAVES + rg % AG_WAVES;
         // register i is key 8 (i / 4) + 4 hf + i % 4 of the tile.  Only a tile that reaches past the first
         // token of the row group has anything to mask (wave-uniform).
         const uint32_t key0 = a.j0 + (first + t) * BK;
@@ -1089,25 +1092,27 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_pv_kernel(GemmAr
     __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2][PART_BYTES];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 31, hf = lane >> 5;
     const uint32_t tok0 = blockIdx.y * AG_TOKENS, kv = blockIdx.z;
-    const uint32_t need = ag_tiles(a, tok0);
-    if (need == 0) return;  // the tile sees nothing of this block (its outputs were written at an earlier one)
-    const bool last_block = ag_last_key(a, tok0) < a.j0 + AG_KEYS;
+    // the tiles of the span's blocks that hold keys some token of the tile can see
+    if (ag_last_key(a, tok0) < a.g0) return;  // nothing of this span (the outputs were written at an earlier one)
+    const uint32_t seen = (ag_last_key(a, tok0) - a.g0) / BK + 1;
+    const uint32_t need = seen < uint32_t(AG_SPAN_TILES) ? seen : uint32_t(AG_SPAN_TILES);
+    const bool last_block = ag_last_key(a, tok0) < a.g0 + AG_SPAN * AG_KEYS;
     const uint32_t rg = blockIdx.y * AG_WAVES + wave;
     const uint32_t tok = tok0 + 4 * wave + (col >> 3), head = kv * SAETTA_GQA_GROUP + (col & 7);
     const size_t rows = size_t(kv) * a.row_groups + rg;
     const size_t state = rows * 32 + col;
-    const bool first_block = a.j0 == 0;
+    const bool first_block = a.g0 == 0;
 
     // slot of (row group, tile): as the scores kernel wrote them
-    const size_t slot0 = rows / AG_WAVES * AG_TILES * AG_WAVES + wave;
+    const size_t slot0 = rows / AG_WAVES * AG_SPAN_TILES * AG_WAVES + wave;
     const float *tm = a.tmax + slot0 * 32 + col, *ts = a.tsum + slot0 * 32 + col;
     // (all of the block's tile maxima requested at once: a loop over `need` waits for each load in turn)
-    float tmaxes[AG_TILES];
+    float tmaxes[AG_SPAN_TILES];
 #pragma unroll
-    for (int t = 0; t < AG_TILES; t++) tmaxes[t] = tm[(uint32_t(t) < need ? t : need - 1) * AG_WAVES * 32];
+    for (int t = 0; t < AG_SPAN_TILES; t++) tmaxes[t] = tm[(uint32_t(t) < need ? t : need - 1) * AG_WAVES * 32];
     float mb = tmaxes[0];
 #pragma unroll
-    for (int t = 1; t < AG_TILES; t++) mb = fmaxf(mb, tmaxes[t]);
+    for (int t = 1; t < AG_SPAN_TILES; t++) mb = fmaxf(mb, tmaxes[t]);
     // (every row sees key 0, so m is a score from the first block on)
     const float m_old = first_block ? NO_SCORE : a.m[state], l_old = first_block ? 0.0f : a.l[state];
     const float m_new = fmaxf(m_old, mb);
@@ -1132,7 +1137,7 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_pv_kernel(GemmAr
     }
 
     // the V^T part of an image
-    const unsigned char *img = a.images + (size_t(kv) * a.nblocks + a.j0 / BK) * IMG_BYTES + PART_BYTES;
+    const unsigned char *img = a.images + (size_t(kv) * a.nblocks + a.g0 / BK) * IMG_BYTES + PART_BYTES;
     // a tile's operands are fetched into registers two tiles ahead (two register sets, the loop in pairs)
     struct Ahead {
         u32x4 v[4];
@@ -1230,7 +1235,7 @@ size_t gemm_row_groups(uint32_t slice) {
 
 size_t gemm_scratch_bytes(uint32_t slice, uint32_t kv_heads) {
     const size_t groups = gemm_row_groups(slice) * kv_heads;
-    return groups * (size_t(AG_TILES) * AG_P_TILE_BYTES + 2 * size_t(AG_TILES) * 32 * 4 + 32 * size_t(DIM) * 4 + 2 * 32 * 4);
+    return groups * (size_t(AG_SPAN_TILES) * AG_P_TILE_BYTES + 2 * size_t(AG_SPAN_TILES) * 32 * 4 + 32 * size_t(DIM) * 4 + 2 * 32 * 4);
 }
 
 uint32_t gemm_slice(uint32_t tokens, uint32_t slice_tokens) {
@@ -1260,9 +1265,9 @@ int run_gemm(hipStream_t stream, int bits, const uint16_t *q, const void *kdata,
     unsigned char *at = static_cast<unsigned char *>(workspace) + align_up(workspace_bytes(p.pos, p.tokens, p.kv_heads), 256);
     GemmArgs a{};
     a.images = static_cast<const unsigned char *>(workspace);
-    a.p = at, at += groups * AG_TILES * AG_P_TILE_BYTES;
-    a.tmax = reinterpret_cast<float *>(at), at += groups * AG_TILES * 32 * 4;
-    a.tsum = reinterpret_cast<float *>(at), at += groups * AG_TILES * 32 * 4;
+    a.p = at, at += groups * AG_SPAN_TILES * AG_P_TILE_BYTES;
+    a.tmax = reinterpret_cast<float *>(at), at += groups * AG_SPAN_TILES * 32 * 4;
+    a.tsum = reinterpret_cast<float *>(at), at += groups * AG_SPAN_TILES * 32 * 4;
     a.o = reinterpret_cast<float *>(at), at += groups * 32 * DIM * 4;
     a.m = reinterpret_cast<float *>(at), at += groups * 32 * 4;
     a.l = reinterpret_cast<float *>(at);
@@ -1282,9 +1287,12 @@ int run_gemm(hipStream_t stream, int bits, const uint16_t *q, const void *kdata,
         const uint64_t end = uint64_t(a.pos) + a.tokens;
         for (uint64_t j0 = 0; j0 < end; j0 += AG_KEYS) {
             a.j0 = uint32_t(j0);
+            a.g0 = uint32_t(j0 / (AG_SPAN * AG_KEYS) * (AG_SPAN * AG_KEYS));
             attention_gemm_scores_kernel<<<dim3(AG_SPLIT, (tiles + AG_RG - 1) / AG_RG, p.kv_heads), AG_THREADS, 0, stream>>>(a);
             if (stages == 1 || stages == 2) continue;
-            attention_gemm_pv_kernel<<<dim3(1, tiles, p.kv_heads), AG_THREADS, 0, stream>>>(a);
+            // pv once per span of blocks: behind the span's last block, or the chunk's
+            if (j0 + AG_KEYS >= end || (j0 / AG_KEYS) % AG_SPAN == AG_SPAN - 1)
+                attention_gemm_pv_kernel<<<dim3(1, tiles, p.kv_heads), AG_THREADS, 0, stream>>>(a);
         }
     }
     return launch_status(what);
