@@ -922,22 +922,21 @@ struct GemmArgs {
     float c;             // scale * log2(e)
     uint32_t nblocks;    // images per kv head
     uint32_t row_groups; // per kv head in the scratch
-    uint32_t j0;         // the block's first key
-    uint32_t g0;         // the first key of the span of blocks it belongs to
+    uint32_t g0;         // the first key of the span of blocks the launch takes
     uint32_t write_out;  // 0: the outputs are never written (timing the passes apart)
 };
 
-// Key of the last token of the workgroup's token tile, and how many of the block's tiles hold keys that
-// some token of the tile can see.
+// Key of the last token of a token tile of `span` tokens at tok0, and how many of the tiles of the launch's span
+// of blocks hold keys that some token of the tile can see.
 __device__ __forceinline__ uint32_t ag_last_key(const GemmArgs &a, uint32_t tok0, uint32_t span = AG_TOKENS) {
     const uint32_t end = tok0 + span < a.tokens ? tok0 + span : a.tokens;
     return a.pos + end - 1;
 }
 __device__ __forceinline__ uint32_t ag_tiles(const GemmArgs &a, uint32_t tok0, uint32_t span = AG_TOKENS) {
     const uint32_t last_key = ag_last_key(a, tok0, span);
-    if (last_key < a.j0) return 0;
-    const uint32_t n = (last_key - a.j0) / BK + 1;
-    return n < uint32_t(AG_TILES) ? n : uint32_t(AG_TILES);
+    if (last_key < a.g0) return 0;
+    const uint32_t n = (last_key - a.g0) / BK + 1;
+    return n < uint32_t(AG_SPAN_TILES) ? n : uint32_t(AG_SPAN_TILES);
 }
 
 __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_scores_kernel(GemmArgs a) {
@@ -946,7 +945,7 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_scores_kernel(Ge
     // a workgroup takes AG_RG token tiles of the pv kernel: a wave AG_RG row groups in a row (8 tokens)
     const uint32_t tok0 = blockIdx.y * (AG_TOKENS * AG_RG), kv = blockIdx.z;
     const uint32_t need = ag_tiles(a, tok0, AG_TOKENS * AG_RG);
-    constexpr uint32_t PER = AG_TILES / AG_SPLIT;
+    constexpr uint32_t PER = AG_SPAN_TILES / AG_SPLIT;
     const uint32_t first = blockIdx.x * PER;
     if (first >= need) return;  // (the whole workgroup)
     const uint32_t count = need - first < PER ? need - first : PER;
@@ -955,7 +954,7 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_scores_kernel(Ge
 
     // A tile's K part goes global -> registers (two register sets, four and three tiles ahead) -> LDS (three
     // buffers, two and one tile ahead) -> MFMA operands.  One barrier a tile.
-    const unsigned char *img = a.images + (size_t(kv) * a.nblocks + a.j0 / BK + first) * IMG_BYTES;
+    const unsigned char *img = a.images + (size_t(kv) * a.nblocks + a.g0 / BK + first) * IMG_BYTES;
     u32x4 pre[2][4];
     // (Fetches and LDS writes past the last tile are made all the same, of the last tile again and into a
     // buffer nobody reads any more: with no branch around a load or a store the compiler knows how many are in
@@ -1012,10 +1011,10 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_scores_kernel(Ge
         const uint32_t limit = a.pos + wtok0 + 4 * r + (col >> 3);  // the last key the row sees
         // slot of (row group, tile) in the scratch: the four row groups of a token tile side by side, tile after
         // tile, so that what a workgroup writes at a step and over its tiles are long runs of memory
-        const size_t slot0 = ((size_t(kv) * a.row_groups + rg) / AG_WAVES * AG_SPAN_TILES + (a.j0 - a.g0) / BK + first) * AG_WAVES + rg % AG_WAVES;
+        const size_t slot0 = ((size_t(kv) * a.row_groups + rg) / AG_WAVES * AG_SPAN_TILES + first) * AG_WAVES + rg % AG_WAVES;
         // register i is key 8 (i / 4) + 4 hf + i % 4 of the tile.  Only a tile that reaches past the first
         // token of the row group has anything to mask (wave-uniform).
-        const uint32_t key0 = a.j0 + (first + t) * BK;
+        const uint32_t key0 = a.g0 + (first + t) * BK;
         if (key0 + BK - 1 > a.pos + wtok0 + 4 * r) {
 #pragma unroll
             for (int i = 0; i < 16; i++) {
@@ -1092,10 +1091,8 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_pv_kernel(GemmAr
     __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2][PART_BYTES];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 31, hf = lane >> 5;
     const uint32_t tok0 = blockIdx.y * AG_TOKENS, kv = blockIdx.z;
-    // the tiles of the span's blocks that hold keys some token of the tile can see
-    if (ag_last_key(a, tok0) < a.g0) return;  // nothing of this span (the outputs were written at an earlier one)
-    const uint32_t seen = (ag_last_key(a, tok0) - a.g0) / BK + 1;
-    const uint32_t need = seen < uint32_t(AG_SPAN_TILES) ? seen : uint32_t(AG_SPAN_TILES);
+    const uint32_t need = ag_tiles(a, tok0);
+    if (need == 0) return;  // nothing of this span (the outputs were written at an earlier one)
     const bool last_block = ag_last_key(a, tok0) < a.g0 + AG_SPAN * AG_KEYS;
     const uint32_t rg = blockIdx.y * AG_WAVES + wave;
     const uint32_t tok = tok0 + 4 * wave + (col >> 3), head = kv * SAETTA_GQA_GROUP + (col & 7);
@@ -1285,14 +1282,12 @@ int run_gemm(hipStream_t stream, int bits, const uint16_t *q, const void *kdata,
         a.q = q + t0 * width, a.q_and_gate = q_and_gate + t0 * width * 2, a.out = out + t0 * width;
         const uint32_t tiles = (a.tokens + AG_TOKENS - 1) / AG_TOKENS;
         const uint64_t end = uint64_t(a.pos) + a.tokens;
-        for (uint64_t j0 = 0; j0 < end; j0 += AG_KEYS) {
-            a.j0 = uint32_t(j0);
-            a.g0 = uint32_t(j0 / (AG_SPAN * AG_KEYS) * (AG_SPAN * AG_KEYS));
+        // a span of AG_SPAN blocks of AG_KEYS keys at a time: its scores, then its pv
+        for (uint64_t g0 = 0; g0 < end; g0 += uint64_t(AG_SPAN) * AG_KEYS) {
+            a.g0 = uint32_t(g0);
             attention_gemm_scores_kernel<<<dim3(AG_SPLIT, (tiles + AG_RG - 1) / AG_RG, p.kv_heads), AG_THREADS, 0, stream>>>(a);
             if (stages == 1 || stages == 2) continue;
-            // pv once per span of blocks: behind the span's last block, or the chunk's
-            if (j0 + AG_KEYS >= end || (j0 / AG_KEYS) % AG_SPAN == AG_SPAN - 1)
-                attention_gemm_pv_kernel<<<dim3(1, tiles, p.kv_heads), AG_THREADS, 0, stream>>>(a);
+            attention_gemm_pv_kernel<<<dim3(1, tiles, p.kv_heads), AG_THREADS, 0, stream>>>(a);
         }
     }
     return launch_status(what);
