@@ -51,7 +51,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # script, so the figures are carried here for the workloads they were measured on.
 MEASURED_TRAFFIC = {"decode8_32k": 38.2e6, "prefill": 294.3e6, "decode4_150k": 91.7e6, "verify4": 45.1e6,
                     "deltanet_prefill": 664.1e6,  # (the three kernels of the chunk together)
-                    "prefill_gemm": 2.66e9}       # (the 10 launches of a call together)
+                    "prefill_gemm": 2.18e9}       # (the 2 launches of a call together)
 
 
 def median(xs):
@@ -366,13 +366,13 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8, gemm=False):
     if gemm:
         # What bounds this route is the scratch it writes and reads back.  Algorithmic bytes per query row: 2 B out
         # and 2 B in per key its 16-token tile sees (in whole tiles of 32 keys), and a maximum and a sum (8 B)
-        # out and in per tile of 32 keys; per block of 1024 keys it touches its q twice (one read per half of
-        # the block's tiles), per span of four blocks 1 KB of output sums in and 1 KB out.
+        # out and in per tile of 32 keys; per span of eight blocks of 1024 keys it touches, its q twice (one read
+        # per half of the span's tiles) and 1 KB of output sums in and 1 KB out.
         nbytes = 0
         for t0 in range(0, tokens, 16):
             last_key = pos + min(t0 + 16, tokens) - 1
             rows = (min(t0 + 16, tokens) - t0) * H
-            nbytes += rows * ((last_key // 32 + 1) * (32 * 4 + 16) + (last_key // 1024 + 1) * 1024 + (last_key // 4096 + 1) * 2048)
+            nbytes += rows * ((last_key // 32 + 1) * (32 * 4 + 16) + (last_key // 8192 + 1) * 3072)
         gbs = nbytes / (kern_us * 1e-6) / 1e9
         roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(gbs / HBM_PEAK_GBS, 4),
@@ -409,7 +409,7 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8, gemm=False):
                    "heads": H, "kv_heads": KV, "head_dim": D, "flops": flops,
                    "timing": "value: wall time of steps (2 x kv_quantize of the chunk + prepare + attention); "
                              "roofline: median of event-timed prepare + attention calls"
-                             + (f" ({2 * -(-(pos + tokens) // 1024)} launches: scores and pv per block of 1024 keys)" if gemm else ""),
+                             + (f" ({2 * -(-(pos + tokens) // 8192)} launches: scores and pv per span of eight blocks of 1024 keys)" if gemm else ""),
                    "inputs": "q (through bf16), K, V, gate ~ N(0,1) from torch's device generator (Philox, seed 99)"},
         "roofline": roofline,
         "cpu_baseline": {"value": round(cpu_flops / cpu_s / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",

@@ -421,10 +421,10 @@ int saetta_attn_prefill_quant(saetta_stream_t stream, int bits, const uint16_t *
 /* Bytes of workspace AttGemm needs for a chunk at (pos, tokens) run in slices
  * of up to slice_tokens tokens (0: one slice): the key and value tile images
  * of saetta_prefill_workspace_bytes, then what AttGemm::new allocates for one
- * slice (src/attention_gemm.rs:118-142): the probabilities of four blocks of
- * keys (the output sums go to memory and back once per four blocks), the tile
- * maxima and sums, the output sums and the per-row softmax state; about 10 KB
- * per query row of a slice. */
+ * slice (src/attention_gemm.rs:118-142): the probabilities of eight blocks of
+ * keys (a pair of launches takes eight blocks, so that q and the output sums
+ * go through memory once per eight), the tile maxima and sums, the output sums
+ * and the per-row softmax state; about 19 KB per query row of a slice. */
 size_t saetta_attn_gemm_workspace_bytes(uint32_t pos, uint32_t tokens, uint32_t slice_tokens,
                                         uint32_t kv_heads);
 

@@ -888,19 +888,22 @@ int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kda
 // into the running (m, l, O) of every row: O = alpha O + sum over tiles of e^(t - m) (P_tile V_tile).
 // The scratch is for one slice of the chunk's tokens; the slices run one after the other.
 //
-// Here a tile is 32 keys (one key image), a row group is 4 tokens x 8 heads as above, and a workgroup is
-// 4 waves with a row group each (a 16-token tile).  Both kernels take the image parts through LDS (the
-// next tile's part is fetched into registers while the current one is used; one barrier a tile) and run
+// Here the pair of launches takes a span of AG_SPAN blocks (the scratch holds that many blocks'
+// probabilities: q and the output sums then go through memory once per span, and there are as many times
+// fewer launches).  A tile is 32 keys (one key image), a row group is 4 tokens x 8 heads as above, and a
+// workgroup is 4 waves: a row group each in pv (a 16-token tile), two each in scores.  Both kernels take the
+// image parts through LDS (the parts of the tiles ahead are fetched into registers while the current one
+// is used; one barrier a tile) and run
 // the same transposed products as the flash kernel, so a lane owns a query row in both:
 //   scores   S^T = K Q^T (Q^T in registers), mask, tile maximum and sum per row, P = 2^(s - t) as f16,
 //            stored as the P^T operands of the second product (the accumulator's registers 8 sp .. 8 sp + 7
 //            are the operand of k-step sp: 1 KB per wave and k-step, read back as it was written);
 //   pv       m' = max(m, max_t t), O^T = alpha O^T + sum_t V^T_t (f_t P^T_t) with f_t = 2^(t - m') rounded
-//            to f16 (the row sum takes the same rounded f_t); the block that holds a tile's last visible
+//            to f16 (the row sum takes the same rounded f_t); the span that holds a tile's last visible
 //            key writes out = O / l * sigmoid(gate) instead of O.
 constexpr int AG_KEYS = SAETTA_AG_KEYS;
 constexpr int AG_TILES = AG_KEYS / BK;
-constexpr int AG_SPAN = 4;                // blocks that one pv launch folds in: the output sums go to memory and back once per span
+constexpr int AG_SPAN = 8;                // blocks that one pair of launches takes: q and the output sums go through memory once per span
 constexpr int AG_SPAN_TILES = AG_SPAN * AG_TILES;
 constexpr int AG_WAVES = 4;
 constexpr int AG_THREADS = 64 * AG_WAVES;
@@ -1104,12 +1107,14 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_pv_kernel(GemmAr
     const size_t slot0 = rows / AG_WAVES * AG_SPAN_TILES * AG_WAVES + wave;
     const float *tm = a.tmax + slot0 * 32 + col, *ts = a.tsum + slot0 * 32 + col;
     // (all of the block's tile maxima requested at once: a loop over `need` waits for each load in turn)
-    float tmaxes[AG_SPAN_TILES];
+    float mb = NO_SCORE;
+    for (uint32_t c = 0; c < need; c += 64) {  // (64 at a time: so many registers are free here)
+        float tmaxes[64];
 #pragma unroll
-    for (int t = 0; t < AG_SPAN_TILES; t++) tmaxes[t] = tm[(uint32_t(t) < need ? t : need - 1) * AG_WAVES * 32];
-    float mb = tmaxes[0];
+        for (int t = 0; t < 64; t++) tmaxes[t] = tm[(c + t < need ? c + t : need - 1) * AG_WAVES * 32];
 #pragma unroll
-    for (int t = 1; t < AG_SPAN_TILES; t++) mb = fmaxf(mb, tmaxes[t]);
+        for (int t = 0; t < 64; t++) mb = fmaxf(mb, tmaxes[t]);
+    }
     // (every row sees key 0, so m is a score from the first block on)
     const float m_old = first_block ? NO_SCORE : a.m[state], l_old = first_block ? 0.0f : a.l[state];
     const float m_new = fmaxf(m_old, mb);

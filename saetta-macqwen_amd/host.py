@@ -828,7 +828,7 @@ class attention_gemm:
     KEYS = 1024    # src/attention_gemm.rs:28
     # Query slices a chunk runs in unless SAETTA_AG_SLICES says otherwise.  The reference takes 2
     # (src/attention_gemm.rs:59-63) to halve a scratch that shares the machine's one memory with the model;
-    # here one: 670 MB of scratch for a 4096-token chunk, and twice the workgroups per launch.
+    # here one: 1.2 GB of scratch for a 4096-token chunk, and twice the workgroups per launch.
     SLICES = 1
 
     @staticmethod
