@@ -3,7 +3,7 @@ the oracle's token-by-token f32 CPU attention, to the bar of the flash kernel's 
 diff < 2e-3 as tests/attention_prefill.rs:56-59, rel-RMS <= 1e-3), and against the flash kernel on the
 same buffers, which is what the reference's own check of this path prints (src/attention_gemm.rs:451-467).
 The reference holds no other test of it.  Shapes: the flash tests' and ones whose keys cross blocks of
-1024 and whose tokens cross slices.
+1024, spans of eight blocks and whose tokens cross slices.
 """
 import math
 
@@ -15,8 +15,9 @@ from gpu_common import D, H, KV, VALUES, dev, host, oracle, saetta
 from test_gpu_prefill import KINDS, MAX_ABS, REL_RMS, make_cache, run as run_flash
 
 pytestmark = pytest.mark.gpu
+# (the last three cross spans of eight blocks, 8192 keys, which is what a pair of launches takes)
 SHAPES = [(0, 1), (0, 7), (5, 8), (70, 100), (1000, 64), (0, 300), (4093, 37), (1020, 40), (2047, 2), (1024, 33),
-          (990, 1100)]
+          (990, 1100), (8100, 200), (8191, 2), (16380, 40)]
 
 
 def run(kind, q16, kc, vc, qg, pos, tokens, chunk=None, stages=0, fill=float("nan")):
