@@ -367,7 +367,7 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8, gemm=False):
         # What bounds this route is the scratch it writes and reads back.  Algorithmic bytes per query row: 2 B out
         # and 2 B in per key its 16-token tile sees (in whole tiles of 32 keys), and a maximum and a sum (8 B)
         # out and in per tile of 32 keys; per span of eight blocks of 1024 keys it touches, its q twice (one read
-        # per half of the span's tiles) and 1 KB of output sums in and 1 KB out.
+        # per part of the span's tiles: two at this chunk length) and 1 KB of output sums in and 1 KB out.
         nbytes = 0
         for t0 in range(0, tokens, 16):
             last_key = pos + min(t0 + 16, tokens) - 1

@@ -908,7 +908,7 @@ constexpr int AG_SPAN_TILES = AG_SPAN * AG_TILES;
 constexpr int AG_WAVES = 4;
 constexpr int AG_THREADS = 64 * AG_WAVES;
 constexpr int AG_TOKENS = 4 * AG_WAVES;   // tokens of a workgroup
-constexpr int AG_SPLIT = 2;
+constexpr int AG_WGS = 512;                // scores: workgroups a launch should have at least (two to a CU)
 constexpr int AG_RG = 2;                  // scores: row groups per wave, which share every fragment of keys it reads               // scores: workgroups that share a block's tiles for one token tile
 constexpr int AG_P_TILE_BYTES = BK * 32 * 2;  // the P^T operands of one row group and tile of keys
 
@@ -926,6 +926,7 @@ struct GemmArgs {
     uint32_t nblocks;    // images per kv head
     uint32_t row_groups; // per kv head in the scratch
     uint32_t g0;         // the first key of the span of blocks the launch takes
+    uint32_t split;      // scores: workgroups that share a span's tiles for one token tile (a power of two)
     uint32_t write_out;  // 0: the outputs are never written (timing the passes apart)
 };
 
@@ -948,10 +949,10 @@ __global__ __launch_bounds__(AG_THREADS, 2) void attention_gemm_scores_kernel(Ge
     // a workgroup takes AG_RG token tiles of the pv kernel: a wave AG_RG row groups in a row (8 tokens)
     const uint32_t tok0 = blockIdx.y * (AG_TOKENS * AG_RG), kv = blockIdx.z;
     const uint32_t need = ag_tiles(a, tok0, AG_TOKENS * AG_RG);
-    constexpr uint32_t PER = AG_SPAN_TILES / AG_SPLIT;
-    const uint32_t first = blockIdx.x * PER;
+    const uint32_t per = AG_SPAN_TILES / a.split;
+    const uint32_t first = blockIdx.x * per;
     if (first >= need) return;  // (the whole workgroup)
-    const uint32_t count = need - first < PER ? need - first : PER;
+    const uint32_t count = need - first < per ? need - first : per;
     const uint32_t rg0 = (blockIdx.y * AG_WAVES + wave) * AG_RG;                    // the wave's first row group
     const uint32_t wtok0 = tok0 + 4 * AG_RG * wave, head = kv * SAETTA_GQA_GROUP + (col & 7);  // and its first token
 
@@ -1287,10 +1288,14 @@ int run_gemm(hipStream_t stream, int bits, const uint16_t *q, const void *kdata,
         a.q = q + t0 * width, a.q_and_gate = q_and_gate + t0 * width * 2, a.out = out + t0 * width;
         const uint32_t tiles = (a.tokens + AG_TOKENS - 1) / AG_TOKENS;
         const uint64_t end = uint64_t(a.pos) + a.tokens;
+        // scores: as many workgroups per token tile as make AG_WGS in all (2 for chunks of 4096 tokens, 4 for 2048)
+        const uint32_t wide = (tiles + AG_RG - 1) / AG_RG;
+        a.split = 2;
+        while (a.split < 16 && a.split * wide * p.kv_heads < uint32_t(AG_WGS)) a.split *= 2;
         // a span of AG_SPAN blocks of AG_KEYS keys at a time: its scores, then its pv
         for (uint64_t g0 = 0; g0 < end; g0 += uint64_t(AG_SPAN) * AG_KEYS) {
             a.g0 = uint32_t(g0);
-            attention_gemm_scores_kernel<<<dim3(AG_SPLIT, (tiles + AG_RG - 1) / AG_RG, p.kv_heads), AG_THREADS, 0, stream>>>(a);
+            attention_gemm_scores_kernel<<<dim3(a.split, wide, p.kv_heads), AG_THREADS, 0, stream>>>(a);
             if (stages == 1 || stages == 2) continue;
             attention_gemm_pv_kernel<<<dim3(1, tiles, p.kv_heads), AG_THREADS, 0, stream>>>(a);
         }
