@@ -903,13 +903,13 @@ int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kda
 //            key writes out = O / l * sigmoid(gate) instead of O.
 constexpr int AG_KEYS = SAETTA_AG_KEYS;
 constexpr int AG_TILES = AG_KEYS / BK;
-constexpr int AG_SPAN = 8;                // blocks that one pair of launches takes: q and the output sums go through memory once per span
+constexpr int AG_SPAN = 8;                // blocks that one pair of launches takes
 constexpr int AG_SPAN_TILES = AG_SPAN * AG_TILES;
 constexpr int AG_WAVES = 4;
 constexpr int AG_THREADS = 64 * AG_WAVES;
 constexpr int AG_TOKENS = 4 * AG_WAVES;   // tokens of a workgroup
-constexpr int AG_WGS = 512;                // scores: workgroups a launch should have at least (two to a CU)
-constexpr int AG_RG = 2;                  // scores: row groups per wave, which share every fragment of keys it reads               // scores: workgroups that share a block's tiles for one token tile
+constexpr int AG_WGS = 512;               // scores: workgroups a launch should have at least (two to a CU)
+constexpr int AG_RG = 2;                  // scores: row groups per wave, which share every fragment of keys it reads
 constexpr int AG_P_TILE_BYTES = BK * 32 * 2;  // the P^T operands of one row group and tile of keys
 
 struct GemmArgs {
