@@ -327,12 +327,14 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8, gemm=False):
     p = s.FlashParams(H, KV, pos, tokens, 1.0 / math.sqrt(D))
     kx, vx = knew[pos:].reshape(-1).contiguous(), vnew[pos:].reshape(-1).contiguous()
     att_gemm = s.attention_gemm.AttGemm(tokens, KV) if gemm else None
+    # the key and value tile images of the flash kernel: allocated once, outside every timed region
+    ws = None if gemm else torch.empty(s.attention_prefill.workspace_bytes(p), dtype=torch.uint8, device="cuda")
 
     def attention():
         if gemm:
             att_gemm.encode(q, None, None, (keys, values), qg, out, p)
         else:
-            s.attention_prefill.encode_quant(q, keys, values, qg, out, p)
+            s.attention_prefill.encode_quant(q, keys, values, qg, out, p, workspace=ws)
 
     def step():
         # quantize-on-append of the chunk's K and V, then the attention over codes in place

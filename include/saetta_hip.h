@@ -49,7 +49,9 @@ enum {
     SAETTA_E_NULL = -3,     /* a required pointer is NULL */
     SAETTA_E_ALIGN = -4,    /* a pointer is not aligned as documented */
     SAETTA_E_DEVICE = -5,   /* no gfx950 device / code object not loadable */
-    SAETTA_E_SCRATCH = -6   /* scratch too small for the request */
+    SAETTA_E_SCRATCH = -6,  /* scratch too small for the request */
+    SAETTA_E_WAIT = -7      /* a kernel launched earlier on this device gave up a bounded wait: see
+                               saetta_device_status */
 };
 
 /* TokenParams (src/plan.rs:16-35; kernels/params.metal:7-15). */
@@ -167,6 +169,18 @@ int saetta_init(void);
 
 /* Text of the last error on this thread ("" if none). */
 const char *saetta_last_error(void);
+
+/* The sticky status word of the current device; 0 as long as nothing went wrong.  The waves of the
+ * decode / verify kernel that keeps a whole share of the cache in LDS meet through counters that
+ * they poll a bounded number of times, so that every wave ends whatever happens.  A wave whose
+ * wait runs out stores a code here (0x100 + the counter's index), marks the partial result of its
+ * workgroup with l = NaN, so that the reduce stage gives NaN for the (row, head) and never a
+ * plausible number, and goes on to its end.  The word lives in pinned host memory and is read
+ * without synchronising: it shows what the kernels that have run so far have left.  Once it is
+ * non-zero every entry point returns SAETTA_E_WAIT until a call with clear != 0 has reset it.
+ * Returns the word as it was before clearing.  The reference has no counterpart: its kernels wait
+ * at threadgroup barriers only. */
+uint32_t saetta_device_status(int clear);
 
 /* ---- kv_quant (src/kv_quant.rs) -------------------------------------------- */
 
@@ -349,7 +363,9 @@ int saetta_deltanet_conv_rows(saetta_stream_t stream, const float *x, const floa
  * [tokens][v_heads][v_dim]; state f32 [v_heads][v_dim][128] updated in place.
  * With snapshots, snaps f32 [tokens][v_heads][v_dim][128] gets the state after
  * each token (GpuDeltaNetSnaps.recurrent); else it may be NULL.  Key dim 128,
- * v_dim a multiple of 4 up to 256. */
+ * v_dim a multiple of 4 up to 256.  The call holds no buffer of the library's:
+ * it runs token by token at every length and only enqueues kernels, so calls on
+ * different streams share nothing.  A prefill chunk wants saetta_deltanet_rows_ws. */
 int saetta_deltanet_rows(saetta_stream_t stream, const float *mixed, const float *a, const float *b,
                          const float *a_log, const float *dt_bias, float *state, const float *z,
                          const float *norm_w, float *y, float *snaps, saetta_rows_step_params p);
@@ -357,11 +373,16 @@ int saetta_deltanet_rows(saetta_stream_t stream, const float *mixed, const float
 /* The same call with a workspace of the caller's (the reference's encode_deltanet
  * works in buffers of the prefill's own, src/prefill.rs:1433-1578): from 128 tokens
  * on, without snapshots and with v_dim a multiple of 16, the delta rule runs in
- * blocks of 64 tokens on the matrix cores and keeps per-block matrices in
- * `workspace` (saetta_deltanet_rows_workspace_bytes(p) bytes, 16-byte aligned; 0
- * bytes: the call runs token by token and takes no workspace).  With workspace
- * NULL this is saetta_deltanet_rows, which uses a workspace the library owns and
- * grows with hipMalloc (under stream capture it falls back to token by token). */
+ * blocks of 64 tokens on the matrix cores (231 against 700 us for 4096 tokens of the
+ * model's layer) and keeps per-block matrices in `workspace`
+ * (saetta_deltanet_rows_workspace_bytes(p) bytes, 16-byte aligned; 0 bytes: the call
+ * runs token by token and takes no workspace).  The workspace belongs to the call
+ * until its kernels have run: calls that may overlap (different streams) bring
+ * different workspaces.  With workspace NULL this is saetta_deltanet_rows.
+ * Range of the blocked form: its operands (state, values and the products between
+ * them) go to the matrix cores as pairs of halves, so magnitudes must stay below
+ * 65504, and parts below 2^-25 of a value are dropped; the token-by-token form is
+ * plain f32. */
 size_t saetta_deltanet_rows_workspace_bytes(saetta_rows_step_params p);
 int saetta_deltanet_rows_ws(saetta_stream_t stream, const float *mixed, const float *a, const float *b,
                             const float *a_log, const float *dt_bias, float *state, const float *z,
@@ -396,8 +417,8 @@ size_t saetta_prefill_workspace_bytes(uint32_t pos, uint32_t tokens, uint32_t kv
  * out f32 [tokens][heads][256].  workspace: device memory of at least
  * saetta_prefill_workspace_bytes(pos, tokens, kv_heads) bytes, 16-byte
  * aligned, overwritten by the call; NULL makes the library use one of its own
- * per device, which it grows with hipMalloc when needed (so not under stream
- * capture, and not from two streams at once).  Kernel replaced:
+ * per device and stream, which it grows with hipMalloc when needed (so not
+ * under stream capture) and keeps until the process ends.  Kernel replaced:
  * attention_fa{4,8} (kernels/attention_prefill.metal:38-169). */
 int saetta_attn_prefill(saetta_stream_t stream, const uint16_t *q_f16, const uint16_t *keys,
                         const uint16_t *values, const float *q_and_gate, float *out,

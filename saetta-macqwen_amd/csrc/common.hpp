@@ -17,8 +17,12 @@ char *error_buffer();
 int fail(int code, const char *fmt, ...);
 // Checks the device once per process; 0 or SAETTA_E_DEVICE.
 int ensure_device();
-// Turns the status of the launches since the last call into a return code.
+// Turns the status of the launches since the last call into a return code; SAETTA_E_WAIT once a
+// kernel on this device has left a code in the device's status word.
 int launch_status(const char *what);
+// Device address of the current device's sticky status word (pinned host memory): a kernel whose
+// bounded wait runs out stores a non-zero code there.  nullptr before the device's set-up.
+uint32_t *device_status_word();
 
 // One-time set-up of a source file's kernels on the current device: loads their code object and
 // raises their dynamic LDS limits, so that a first launch under stream capture has nothing left to
@@ -31,13 +35,11 @@ int setup_decode();
 int setup_prefill();
 // The chunked delta rule (deltanet_chunk.hip): the workspace a call needs (0: the call keeps to the
 // token-by-token kernels), and the call itself (the delta rule only; the gated norm follows as for the
-// token-by-token kernels) with a workspace of the caller's or the library's own (which may allocate).
+// token-by-token kernels) with a workspace of the caller's.
 size_t deltanet_chunk_workspace_bytes(const saetta_rows_step_params &p);
 int run_deltanet_chunk(hipStream_t stream, const float *mixed, const float *a, const float *b, const float *a_log,
                        const float *dt_bias, float *state, float *o, const saetta_rows_step_params &p, uint32_t channels,
                        void *workspace);
-int run_deltanet_chunk_owned(hipStream_t stream, const float *mixed, const float *a, const float *b, const float *a_log,
-                             const float *dt_bias, float *state, float *o, const saetta_rows_step_params &p, uint32_t channels);
 // Loads the code object `kernel` lives in.
 inline int load_kernel(const void *kernel) {
     hipFuncAttributes attr;

@@ -116,6 +116,7 @@ struct PartialArgs {
     uint32_t rows, nsplits;
     const saetta_token_params *tp;
     uint32_t decode_len;  // 1: every row sees min(kv_len, capacity); 0: row r sees position + r + 1
+    uint32_t *status;     // the device's sticky status word (pinned host memory)
 };
 
 __device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) {
@@ -1103,6 +1104,7 @@ struct KeysFirst {
     static constexpr int C_BUILT = 3;   // ... built their probability operands (8 per round)
     static constexpr int C_DONE = 4;    // ... are through with the round's values (8 per round)
     static constexpr int C_LENGTH = 5;  // (not a counter: the context length or the position, for every wave)
+    static constexpr int C_GAVE_UP = 6; // (not a counter: non-zero once a wave's wait has run out)
     static constexpr int C_QREAD = 7;   // computing waves that have a row's query operands in registers (several rows)
     static constexpr int C_KPART = 8;   // [3]: key loaders whose blocks 0-7 and scales | blocks 8-15 | block 16 have landed (2 per round)
     static constexpr int C_SLOT = 12;   // [5]: value loaders whose values of slot s have landed (2 per round)
@@ -1203,15 +1205,33 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
         asm volatile("" ::: "memory");
         return uint32_t(__builtin_amdgcn_readfirstlane(v));
     };
+    // A wait that runs out must not pass for a result: the wave leaves a code in the device's status word (a
+    // plain store by one lane; the host reads the word at its next call), marks the workgroup (the wave that
+    // writes the maxima and sums writes l = NaN then) and writes l = NaN itself in case that wave is through
+    // already, so that the reduce stage gives NaN for these heads; then it goes on to its end like any wave.
+    auto gave_up = [&](int c) {
+        if (lane == 0) {
+            __hip_atomic_store(a.status, 0x100u + uint32_t(c), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            __hip_atomic_store(sync_lds + W::C_GAVE_UP, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+        if (lane < 8 * M) {
+            const size_t slot = (size_t(lane >> 3) * a.nsplits + split) * a.heads + kv * 8 + (lane & 7);
+            a.part_ml[2 * slot + 1] = __builtin_nanf("");
+        }
+    };
     auto await = [&](int c, uint32_t want) {
         asm volatile("" ::: "memory");
-        for (uint32_t i = 0; i < W::SPIN_LIMIT; i++) {
+        uint32_t i = 0;
+        for (; i < W::SPIN_LIMIT; i++) {
             const uint32_t v = __hip_atomic_load(sync_lds + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             if (__builtin_amdgcn_readfirstlane(v) >= want) break;
             __builtin_amdgcn_s_sleep(1);
         }
+        if (__builtin_expect(i == W::SPIN_LIMIT, 0)) gave_up(c);
         asm volatile("" ::: "memory");
     };
+    // l of a partial as the writer of the maxima and sums stores it
+    auto marked = [&](float l) { return peek(W::C_GAVE_UP) ? __builtin_nanf("") : l; };
 
     if (loader && wave_all < W::K_LOADERS) {
         // ---- a key-loader wave: scales and biases of tokens 128 L .. 128 L + 127, keys of blocks L, L + 2, ...;
@@ -1665,7 +1685,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
                 const float l = round_sum(row_of(p, col_row), nm[p]);
                 if (j == 0 && r < M) {
                     const size_t slot = (size_t(r) * a.nsplits + split) * a.heads + kv * 8 + (n & 7);
-                    *reinterpret_cast<floatx2 *>(a.part_ml + 2 * slot) = floatx2{nm[p], l};
+                    *reinterpret_cast<floatx2 *>(a.part_ml + 2 * slot) = floatx2{nm[p], marked(l)};
                 }
             }
         }
@@ -1744,7 +1764,10 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
                 for (int part = 0; part < parts; part++) {
                     const int blk = wave + 8 * part;
                     if (uint32_t(blk) >= live_blocks) {
-                        // (a short round: no scores to take, and no operands will be made of this block)
+                        // (a short round: no scores to take, and no operands will be made of this block; the
+                        // table still holds the round before's entries until every wave has built its operands
+                        // from them, which is also what the key loader waits for before it overwrites the keys)
+                        if (round > 0) await(W::C_BUILT, W::WAVES * round);
                         if (j == 0 && n < 8) bmax_lds[n * W::BSTRIDE + blk] = NO_SCORE, bsum_lds[n * W::BSTRIDE + blk] = 0.0f;
                         continue;
                     }
@@ -1813,7 +1836,11 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
                     if (n < 8) *reinterpret_cast<floatx4 *>(s_block(blk, 0) + n * BLOCK + 4 * j) = s;
                     if (j == 0 && n < 8) bmax_lds[n * W::BSTRIDE + blk] = cm, bsum_lds[n * W::BSTRIDE + blk] = sum;
                 }
-                if (wave == 0 && !extra && j == 0 && n < 8) bmax_lds[n * W::BSTRIDE + 16] = NO_SCORE, bsum_lds[n * W::BSTRIDE + 16] = 0.0f;
+                if (wave == 0 && !extra) {
+                    // (block 16 of the round before, if it had one, is read until every wave has built its operands)
+                    if (round > 0) await(W::C_BUILT, W::WAVES * round);
+                    if (j == 0 && n < 8) bmax_lds[n * W::BSTRIDE + 16] = NO_SCORE, bsum_lds[n * W::BSTRIDE + 16] = 0.0f;
+                }
             }
             raise(W::C_SCORES);
             await(W::C_SCORES, W::WAVES * (round + 1));
@@ -1984,7 +2011,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
         await(W::C_MERGE + g, 1);
         if (wave == 0 && j == 0 && n < 8) {
             const size_t slot = size_t(split) * a.heads + kv * 8 + n;
-            *reinterpret_cast<floatx2 *>(a.part_ml + 2 * slot) = floatx2{m_run, l_run};
+            *reinterpret_cast<floatx2 *>(a.part_ml + 2 * slot) = floatx2{m_run, marked(l_run)};
         }
         if (j < 2) {
 #pragma unroll
@@ -2229,7 +2256,7 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
     if (one_per_cu && nsplits > MAX_SPLITS / 2) nsplits = MAX_SPLITS / 2;
     if (stages & SAETTA_STAGE_PARTIAL) {
         PartialArgs a{q,     kdata,    vdata,    ks,    kz,   vs,      vz,   part_o, part_ml,
-                      heads, kv_heads, capacity, scale, rows, nsplits, d_tp, decode_len ? 1u : 0u};
+                      heads, kv_heads, capacity, scale, rows, nsplits, d_tp, decode_len ? 1u : 0u, device_status_word()};
         if (bits == 8) {
             launch_partial_rows<8>(stream, a, one_per_cu, loaders, keys_first);
         } else if (bits == 4) {

@@ -819,23 +819,15 @@ extern "C" int saetta_deltanet_rows_ws(saetta_stream_t stream, const float *mixe
     if (int rc = ensure_device()) return rc;
     if (p.tokens == 0) return SAETTA_OK;
     const uint32_t channels = 2 * p.k_heads * K_DIM + p.v_heads * p.v_dim;
-    // A prefill chunk (128 tokens and more, no snapshots): the delta rule in blocks of 64 tokens on the
-    // matrix cores, with a workspace of the caller's or, outside stream capture, the library's own.
+    // A prefill chunk (128 tokens and more, no snapshots) whose caller brings a workspace: the delta rule in
+    // blocks of 64 tokens on the matrix cores.  Without a workspace the call keeps to the token-by-token
+    // kernels: the library holds no buffer of its own here, so calls on different streams share nothing.
     const size_t need = deltanet_chunk_workspace_bytes(p);
-    bool blocks = need > 0;
-    if (blocks && workspace) {
+    const bool blocks = need > 0 && workspace != nullptr;
+    if (blocks) {
         SAETTA_REQUIRE(workspace_size >= need && aligned(workspace, 16), SAETTA_E_SCRATCH,
                        "deltanet_rows: workspace of %zu bytes, %zu needed (16-byte aligned)", workspace_size, need);
-    } else if (blocks) {
-        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(as_stream(stream), &capturing) != hipSuccess) (void)hipGetLastError();
-        blocks = capturing == hipStreamCaptureStatusNone;  // (the library's own workspace may have to grow)
-    }
-    if (blocks) {
-        if (int rc = workspace ? run_deltanet_chunk(as_stream(stream), mixed, a, b, a_log, dt_bias, state, y, p, channels, workspace)
-                               : run_deltanet_chunk_owned(as_stream(stream), mixed, a, b, a_log, dt_bias, state, y, p, channels)) {
-            return rc;
-        }
+        if (int rc = run_deltanet_chunk(as_stream(stream), mixed, a, b, a_log, dt_bias, state, y, p, channels, workspace)) return rc;
     } else {
         RowsArgs args{mixed, a, b, a_log, dt_bias, state, y, snaps, p, channels};
         constexpr int LANES = ROWS_LANES_PER_ROW, ROWS_PER_WG = 256 / LANES;

@@ -29,7 +29,6 @@
 #include "deltanet_gates.hpp"
 #include "lanes.hpp"
 
-#include <mutex>
 #include <type_traits>
 
 namespace saetta {
@@ -725,15 +724,6 @@ __global__ __launch_bounds__(512) void deltanet_chunk_chain_kernel(ChunkArgs a) 
     }
 }
 
-// The workspace is the library's own, per device, grown on demand.
-struct OwnedWorkspace {
-    void *ptr = nullptr;
-    size_t bytes = 0;
-};
-constexpr int OWNED_DEVICES = 64;
-OwnedWorkspace g_owned[OWNED_DEVICES];
-std::mutex g_owned_mutex;
-
 }  // namespace
 
 int setup_deltanet_chunk() {
@@ -766,29 +756,6 @@ int run_deltanet_chunk(hipStream_t stream, const float *mixed, const float *a, c
     }
     deltanet_chunk_chain_kernel<<<dim3(p.v_dim / DV * p.v_heads), 512, ChainLds::BYTES, stream>>>(args);
     return SAETTA_OK;
-}
-
-int run_deltanet_chunk_owned(hipStream_t stream, const float *mixed, const float *a, const float *b, const float *a_log,
-                             const float *dt_bias, float *state, float *o, const saetta_rows_step_params &p, uint32_t channels) {
-    const size_t need = deltanet_chunk_workspace_bytes(p);
-    int dev = 0;
-    if (hipError_t e = hipGetDevice(&dev)) return fail(int(e), "deltanet_rows: %s", hipGetErrorString(e));
-    SAETTA_REQUIRE(dev >= 0 && dev < OWNED_DEVICES, SAETTA_E_DEVICE, "deltanet_rows: device index %d (up to %d)", dev, OWNED_DEVICES - 1);
-    // held until the launches that use the workspace are queued (as for the prefill workspace)
-    std::lock_guard<std::mutex> lock(g_owned_mutex);
-    OwnedWorkspace &w = g_owned[dev];
-    if (w.bytes < need) {
-        if (w.ptr) {
-            (void)hipDeviceSynchronize();
-            (void)hipFree(w.ptr);
-        }
-        w.ptr = nullptr;
-        w.bytes = 0;
-        hipError_t e = hipMalloc(&w.ptr, need);
-        if (e != hipSuccess) return fail(int(e), "deltanet_rows: workspace of %zu bytes: %s", need, hipGetErrorString(e));
-        w.bytes = need;
-    }
-    return run_deltanet_chunk(stream, mixed, a, b, a_log, dt_bias, state, o, p, channels, w.ptr);
 }
 
 }  // namespace saetta

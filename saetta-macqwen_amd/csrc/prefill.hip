@@ -42,7 +42,9 @@
 #include "common.hpp"
 #include "lanes.hpp"
 
+#include <map>
 #include <mutex>
+#include <utility>
 
 namespace saetta {
 namespace {
@@ -767,13 +769,15 @@ __global__ __launch_bounds__(THREADS, 2) void attention_prefill_kernel(PrefillAr
     }
 }
 
-// Workspace the library owns when the caller passes none: grown on demand, one per device.
+// Workspaces the library owns when the caller passes none: one per (device, stream), grown on demand,
+// so that calls on different streams never share one (work on one stream runs in order).  They are
+// kept until the process ends: a caller with many short-lived streams passes its own.
 struct OwnedWorkspace {
     void *ptr = nullptr;
     size_t bytes = 0;
 };
 constexpr int OWNED_DEVICES = 64;  // as many devices as the library's set-up admits
-OwnedWorkspace g_owned[OWNED_DEVICES];
+std::map<std::pair<int, hipStream_t>, OwnedWorkspace> g_owned;
 std::mutex g_owned_mutex;
 
 size_t workspace_bytes(uint32_t pos, uint32_t tokens, uint32_t kv_heads) {
@@ -799,10 +803,10 @@ int check_prefill(int bits, const uint16_t *q, const void *kdata, const void *vd
     return SAETTA_OK;
 }
 
-// The caller's workspace if it gave one of at least `need` bytes, else the library's own, grown to `need`.
-// The library's own is held under its lock until the launches that use it are queued (the caller keeps
-// `owned_lock` until then): a second host thread that has to grow it waits for them (hipDeviceSynchronize)
-// before it frees.
+// The caller's workspace if it gave one of at least `need` bytes, else the library's own for this device
+// and stream, grown to `need`.  The library's own is held under the lock until the launches that use it
+// are queued (the caller keeps `owned_lock` until then): a second host thread on the same stream that has
+// to grow it waits for them (hipStreamSynchronize) before it frees.
 int acquire_workspace(hipStream_t stream, void *&workspace, size_t workspace_size, size_t need,
                       std::unique_lock<std::mutex> &owned_lock, const char *what, const char *sizer) {
     if (workspace) {
@@ -810,8 +814,8 @@ int acquire_workspace(hipStream_t stream, void *&workspace, size_t workspace_siz
                        workspace_size, need);
         return SAETTA_OK;
     }
-    // No workspace given: use (and grow) the library's own.  This may allocate, which a stream
-    // under capture cannot do; work queued on other streams must not share it.
+    // No workspace given: use (and grow) the library's own for this stream.  This may allocate, which a
+    // stream under capture cannot do.
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) (void)hipGetLastError();
     SAETTA_REQUIRE(capturing == hipStreamCaptureStatusNone, SAETTA_E_SCRATCH,
@@ -820,10 +824,10 @@ int acquire_workspace(hipStream_t stream, void *&workspace, size_t workspace_siz
     if (hipError_t e = hipGetDevice(&dev)) return fail(int(e), "%s: %s", what, hipGetErrorString(e));
     SAETTA_REQUIRE(dev >= 0 && dev < OWNED_DEVICES, SAETTA_E_DEVICE, "%s: device index %d (up to %d)", what, dev, OWNED_DEVICES - 1);
     owned_lock.lock();
-    OwnedWorkspace &w = g_owned[dev];
+    OwnedWorkspace &w = g_owned[std::make_pair(dev, stream)];
     if (w.bytes < need) {
         if (w.ptr) {
-            (void)hipDeviceSynchronize();
+            (void)hipStreamSynchronize(stream);
             (void)hipFree(w.ptr);
         }
         w.ptr = nullptr;

@@ -7,7 +7,7 @@ LIB_PATH = os.environ.get("SAETTA_HIP_LIB") or os.path.join(_HERE, "lib", "libsa
 
 # Every symbol include/saetta_hip.h declares; tests check the library exports each.
 SYMBOLS = [
-    "saetta_init", "saetta_last_error", "saetta_kv_quantize", "saetta_kv_dequantize", "saetta_kv_dequantize_f32", "saetta_to_half", "saetta_attn_prep_store", "saetta_deltanet_conv", "saetta_deltanet_step", "saetta_deltanet_conv_rows", "saetta_deltanet_rows", "saetta_deltanet_rows_ws", "saetta_deltanet_rows_workspace_bytes", "saetta_deltanet_token", "saetta_deltanet_rows_fused",
+    "saetta_init", "saetta_last_error", "saetta_device_status", "saetta_kv_quantize", "saetta_kv_dequantize", "saetta_kv_dequantize_f32", "saetta_to_half", "saetta_attn_prep_store", "saetta_deltanet_conv", "saetta_deltanet_step", "saetta_deltanet_conv_rows", "saetta_deltanet_rows", "saetta_deltanet_rows_ws", "saetta_deltanet_rows_workspace_bytes", "saetta_deltanet_token", "saetta_deltanet_rows_fused",
     "saetta_part_o_bytes", "saetta_part_ml_bytes", "saetta_attn_decode", "saetta_attn_decode_quant",
     "saetta_attn_rows", "saetta_attn_rows_quant", "saetta_static_scratch_bytes", "saetta_attn_decode_quant_static", "saetta_prefill_workspace_bytes", "saetta_attn_prefill", "saetta_attn_prefill_quant",
     "saetta_attn_gemm_workspace_bytes", "saetta_attn_gemm",
@@ -61,6 +61,7 @@ def lib():
         vp, u32, i32, sz = ctypes.c_void_p, ctypes.c_uint32, ctypes.c_int, ctypes.c_size_t
         l.saetta_init.restype, l.saetta_init.argtypes = i32, []
         l.saetta_last_error.restype, l.saetta_last_error.argtypes = ctypes.c_char_p, []
+        l.saetta_device_status.restype, l.saetta_device_status.argtypes = u32, [i32]
         l.saetta_kv_quantize.restype = i32
         l.saetta_kv_quantize.argtypes = [vp, i32, vp, QuantRowsC, KvQuantParamsC, vp, u32]
         l.saetta_kv_dequantize.restype = i32

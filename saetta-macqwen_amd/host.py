@@ -714,6 +714,18 @@ def _workspace(t):
     return _ptr(t), t.numel()
 
 
+def _workspace_or_own(t, nbytes, like, stream):
+    """The caller's workspace, or a tensor of this call's own from torch's allocator (which hands a
+    block out again only behind the work queued on its stream): the library's own workspace, which a
+    NULL pointer would select, is one per device and stream that stays for the life of the process."""
+    if t is not None:
+        return t
+    t = torch.empty(nbytes, dtype=torch.uint8, device=like.device)
+    if isinstance(stream, torch.cuda.Stream):
+        t.record_stream(stream)
+    return t
+
+
 class FlashParams:
     """src/attention_prefill.rs:4-14."""
 
@@ -740,14 +752,15 @@ class attention_prefill:
     def encode(kernel, q, keys, values, q_and_gate, out, p, stream=None, workspace=None):
         """encode (src/attention_prefill.rs:39-72).  `kernel` picks a tile size in
         the reference; the one gfx950 kernel serves both names.  `workspace` is a
-        uint8 tensor of at least workspace_bytes(p) bytes, or None to let the
-        library use its own."""
+        uint8 tensor of at least workspace_bytes(p) bytes, or None for one of this
+        call's own (a caller that times the call, or records it, brings its own)."""
         if kernel not in attention_prefill.KERNELS:
             raise ValueError(f"no prefill attention kernel {kernel}")
         if p.heads != p.kv_heads * 8:
             raise ValueError(f"{kernel} needs 8 q heads per kv head")
         _need(q, torch.float16, "q"), _need(keys, torch.float16, "keys"), _need(values, torch.float16, "values")
         _need(q_and_gate, torch.float32, "q_and_gate"), _need(out, torch.float32, "out")
+        workspace = _workspace_or_own(workspace, attention_prefill.workspace_bytes(p), q, stream)
         ffi.check(ffi.lib().saetta_attn_prefill(_stream(stream), _ptr(q), _ptr(keys), _ptr(values),
                                                 _ptr(q_and_gate), _ptr(out), p.c(), *_workspace(workspace)),
                   "attn_prefill")
@@ -818,6 +831,7 @@ class attention_prefill:
         if p.heads != p.kv_heads * 8:
             raise ValueError("prefill attention needs 8 q heads per kv head")
         _need(q, torch.float16, "q"), _need(q_and_gate, torch.float32, "q_and_gate"), _need(out, torch.float32, "out")
+        workspace = _workspace_or_own(workspace, attention_prefill.workspace_bytes(p), q, stream)
         ffi.check(ffi.lib().saetta_attn_prefill_quant(_stream(stream), keys.bits.value, _ptr(q), keys.c(), values.c(),
                                                       _ptr(q_and_gate), _ptr(out), p.c(), *_workspace(workspace)),
                   "attn_prefill_quant")

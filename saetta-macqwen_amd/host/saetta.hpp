@@ -679,7 +679,8 @@ inline const char *const KERNELS[2] = {"attention_fa8", "attention_fa4"};
 inline const char *const DEFAULT = "attention_fa8";
 constexpr size_t KEY_BLOCK = 16;
 
-// Device memory the chunk's f16 tile images go to; the default lets the library use its own.
+// Device memory the chunk's f16 tile images go to; the default lets the library use its own (one per
+// device and stream, kept until the process ends).
 struct Workspace {
     void *ptr = nullptr;
     size_t bytes = 0;

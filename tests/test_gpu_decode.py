@@ -347,6 +347,27 @@ def test_large_cache_of_codes_one_row(kind, capacity):
         del kc, vc
 
 
+def test_four_bit_one_row_in_a_cache_of_131072_tokens():
+    # 4-bit codes in caches of 102401 to 139264 tokens go to the ring of four 64-token slots with shares of
+    # up to 64 blocks: sixteen iterations, eight rounds of the two teams, every slot refilled several times.
+    # Lengths: a single token; shares of 35 blocks (odd numbers of iterations per team); 120000 tokens; the
+    # whole capacity.  The rows past each length are poisoned.
+    rng = np.random.default_rng(131)
+    capacity, kind = 131072, saetta.KvBits.Four
+    k = (rng.standard_normal((capacity, VALUES)) * 2.0).astype(np.float32)
+    v = rng.standard_normal((capacity, VALUES)).astype(np.float32)
+    q = rng.standard_normal(H * D).astype(np.float32)
+    qg = rng.standard_normal(H * 2 * D).astype(np.float32)
+    att = saetta.DecodeAttention(H, KV, D, capacity)
+    for length in [1, 70001, 120000, capacity]:
+        kc, vc, kf, vf = cache_pair(k[:length], v[:length], kind, capacity, poison=True)
+        got = run_decode(att, kind, dev(q), kc, vc, dev(qg), length)
+        assert np.isfinite(got).all(), length
+        worst = np.abs(got - oracle.attention_f64(q, kf, vf, qg, length, threads=8)).max()
+        assert worst < MAX_ABS_F64, (length, worst)
+        del kc, vc
+
+
 @pytest.mark.parametrize("kind,ctx,m", [(saetta.KvBits.Eight, 32768, 1), (saetta.KvBits.Eight, 32768, 4),
                                         (saetta.KvBits.Eight, 131072, 1), (saetta.KvBits.Four, 150000, 1),
                                         (saetta.KvBits.Four, 32768, 3), (saetta.KvBits.Half, 4096, 2)])

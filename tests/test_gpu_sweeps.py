@@ -15,7 +15,7 @@ from test_gpu_prefill import make_cache, run as run_prefill
 
 pytestmark = pytest.mark.gpu
 KINDS = [saetta.KvBits.Half, saetta.KvBits.Eight, saetta.KvBits.Four]
-CAPACITIES = [128, 256, 1024, 4096, 8192, 16384, 24576, 24704, 32768, 34816, 34944, 40960, 61440, 65536, 81920]
+CAPACITIES = [128, 256, 1024, 4096, 8192, 16384, 24576, 24704, 32768, 34816, 34944, 40960, 61440, 65536, 81920, 106496, 131072]
 
 
 @pytest.mark.parametrize("seed", [1, 2, 3])

@@ -72,3 +72,61 @@ def test_more_heads_than_the_static_scratch_holds_are_rejected():
     p = ffi.DecodeParamsC(32, 4, 1024, 1.0 / 16)
     rc = ffi.lib().saetta_attn_decode_quant_static(None, 8, ptr(z), rows, rows, ptr(z), ptr(z), p, ptr(z), ffi.STAGE_ALL)
     assert rc == -6 and b"static scratch" in ffi.lib().saetta_last_error()
+
+
+def test_static_entry_allocates_nothing_replays_from_a_graph_and_splits_into_stages():
+    # What the entry point is for: a call under stream capture (nothing may allocate there), replayed at
+    # two positions against eager calls with scratch of the caller's; no device memory taken across the
+    # calls; and the partial and the reduce stage as two calls, the partials waiting in the static buffer.
+    lib = ffi.lib()
+    ffi.check(lib.saetta_init(), "init")
+    bits, capacity = 8, 32896
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    keys, values = saetta.QuantRows(saetta.KvBits.Eight, VALUES, capacity), saetta.QuantRows(saetta.KvBits.Eight, VALUES, capacity)
+    keys.encode(torch.randn(capacity * VALUES, generator=gen, device="cuda"), 0, capacity)
+    values.encode(torch.randn(capacity * VALUES, generator=gen, device="cuda"), 0, capacity)
+    q = torch.randn(H, D, generator=gen, device="cuda")
+    qg = torch.randn(H, 2 * D, generator=gen, device="cuda")
+    p = ffi.DecodeParamsC(H, KV, capacity, 1.0 / math.sqrt(D))
+    part_o = torch.empty(lib.saetta_part_o_bytes(H, capacity, 1) // 4, device="cuda")
+    part_ml = torch.empty(lib.saetta_part_ml_bytes(H, capacity, 1) // 4, device="cuda")
+    got, want = torch.empty(H, D, device="cuda"), torch.empty(H, D, device="cuda")
+    plan = saetta.Plan()
+    plan.op("attention_static", lambda st: ffi.check(lib.saetta_attn_decode_quant_static(
+        st, bits, ptr(q), keys.c(), values.c(), ptr(qg), ptr(got), p, ptr(plan.params), ffi.STAGE_ALL), "attn_decode_quant_static"))
+    built = plan.build(graph=True)  # captured: a hipMalloc here would fail the capture
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # (a first replay and a first eager call: what the runtime itself sets up on a first launch is not the call's)
+    plan.set_params(saetta.TokenParams(0, 5))
+    built.run()
+    ffi.check(lib.saetta_attn_decode_quant(stream, bits, ptr(q), keys.c(), values.c(), ptr(part_o), ptr(part_ml), ptr(qg),
+                                           ptr(want), p, ptr(plan.params), ffi.STAGE_ALL), "attn_decode_quant")
+    host(got), host(want)
+    free_before = torch.cuda.mem_get_info()[0]
+    for position in (32768, 700, 20000):
+        plan.set_params(saetta.TokenParams(0, position))
+        got.fill_(float("nan"))
+        built.run()
+        ffi.check(lib.saetta_attn_decode_quant(stream, bits, ptr(q), keys.c(), values.c(), ptr(part_o), ptr(part_ml), ptr(qg),
+                                               ptr(want), p, ptr(plan.params), ffi.STAGE_ALL), "attn_decode_quant")
+        g, w = host(got), host(want)
+        assert np.isfinite(g).all() and np.array_equal(g, w), position
+    # the two stages as two calls (eager, on the stream)
+    plan.set_params(saetta.TokenParams(0, 12345))
+    got.fill_(float("nan"))
+    for stage in (ffi.STAGE_PARTIAL, ffi.STAGE_REDUCE):
+        ffi.check(lib.saetta_attn_decode_quant_static(stream, bits, ptr(q), keys.c(), values.c(), ptr(qg), ptr(got), p,
+                                                      ptr(plan.params), stage), "attn_decode_quant_static")
+    ffi.check(lib.saetta_attn_decode_quant(stream, bits, ptr(q), keys.c(), values.c(), ptr(part_o), ptr(part_ml), ptr(qg),
+                                           ptr(want), p, ptr(plan.params), ffi.STAGE_ALL), "attn_decode_quant")
+    assert np.array_equal(host(got), host(want))
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "the calls took device memory"
+
+
+def test_no_bounded_wait_gave_up_in_this_process():
+    # Collected last: the sticky status word of the device is still 0 after every kernel the tests of
+    # this process have run (a wave whose bounded wait runs out leaves a code there).
+    ffi.check(ffi.lib().saetta_init(), "init")
+    torch.cuda.synchronize()
+    assert ffi.lib().saetta_device_status(0) == 0
