@@ -1025,6 +1025,21 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel_p(PartialArg
     attention_partial_body<BITS, 1, true, ITB_ONE_PER_CU, true>(a);
 }
 
+// What a wave of attention_partial_kernel_s does when a bounded wait on an LDS counter has run out (it never
+// should): one lane stores a code in the device's sticky status word, which the host reads at its next call
+// (a plain vector store to pinned host memory), and the workgroup's partials get l = NaN, so that the
+// reduce stage gives NaN for these (row, head) pairs and never a plausible number.  (If the wave that stores
+// the maxima and sums is still to come and has not given up itself, its store wins; the status word stands.)
+__device__ __noinline__ void wait_gave_up(uint32_t *status, float *part_ml, uint32_t code, uint32_t rows, uint32_t nsplits,
+                                          uint32_t split, uint32_t heads, uint32_t kv) {
+    const uint32_t lane = threadIdx.x & 63;
+    if (lane == 0) __hip_atomic_store(status, code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (lane < 8 * rows) {
+        const size_t slot = (size_t(lane >> 3) * nsplits + split) * heads + kv * 8 + (lane & 7);
+        part_ml[2 * slot + 1] = __builtin_nanf("");
+    }
+}
+
 // ---- one to four query rows over codes, keys first ------------------------------------------------
 // attention_partial_kernel_s: the workgroup's share is taken in rounds of up to 17 blocks of 16
 // tokens whose codes all lie in LDS at once (17: a context of 128 x 256 tokens and a few more still
@@ -1090,7 +1105,17 @@ struct KeysFirst {
     static constexpr int SYNC_OFF = ZS_OFF + WAVES * PAIRS * 16 * 4;  // 32 counters, u32
     static constexpr int K_OFF = (SYNC_OFF + 32 * 4 + 255) / 256 * 256;
     static constexpr int V_OFF = K_OFF + ROUND_BLOCKS * K_BLOCK_BYTES;
-    static constexpr int LDS_BYTES = V_OFF + ROUND_BLOCKS * K_BLOCK_BYTES;
+    // Several rows over a share of more than one round: rounds of SHORT_BLOCKS blocks, which leave room in
+    // LDS for every pair's query operands to stay ([pair][hi, lo][k-step][lane] half8, then [pair][hi, lo][lane][k-step]
+    // f16 of the key bias term), so that they need no registers between one round's scores and the next's.
+    // 8-bit codes: over the keys' blocks that short rounds never fill; 4-bit: behind the values.
+    static constexpr int SHORT_BLOCKS = 8;
+    static constexpr int QP_PAIR_BYTES = 2 * 8 * 64 * 16, QPZ_PAIR_BYTES = 2 * 64 * 16;
+    static constexpr int QP_BYTES = M > 1 ? PAIRS * (QP_PAIR_BYTES + QPZ_PAIR_BYTES) : 0;
+    static constexpr int QP_OFF = BITS == 8 ? K_OFF + SHORT_BLOCKS * K_BLOCK_BYTES : V_OFF + ROUND_BLOCKS * K_BLOCK_BYTES;
+    static constexpr int QPZ_OFF = QP_OFF + PAIRS * QP_PAIR_BYTES;
+    static_assert(BITS != 8 || QP_OFF + QP_BYTES <= V_OFF, "the query operands fit behind the short rounds' keys");
+    static constexpr int LDS_BYTES = (BITS == 8 || M == 1) ? V_OFF + ROUND_BLOCKS * K_BLOCK_BYTES : QP_OFF + QP_BYTES;
     // one row: the merge of two waves, [group][lane < 32][4 rows] of 16 bytes, lies over the query operands,
     // which nobody reads after the last scores
     static constexpr int X_OFF = Q_OFF;
@@ -1104,7 +1129,6 @@ struct KeysFirst {
     static constexpr int C_BUILT = 3;   // ... built their probability operands (8 per round)
     static constexpr int C_DONE = 4;    // ... are through with the round's values (8 per round)
     static constexpr int C_LENGTH = 5;  // (not a counter: the context length or the position, for every wave)
-    static constexpr int C_GAVE_UP = 6; // (not a counter: non-zero once a wave's wait has run out)
     static constexpr int C_QREAD = 7;   // computing waves that have a row's query operands in registers (several rows)
     static constexpr int C_KPART = 8;   // [3]: key loaders whose blocks 0-7 and scales | blocks 8-15 | block 16 have landed (2 per round)
     static constexpr int C_SLOT = 12;   // [5]: value loaders whose values of slot s have landed (2 per round)
@@ -1171,8 +1195,8 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
     const uint32_t last_tok = limit - 1;                   // rows past it are never read: loads are clamped to it
     const uint32_t range = blk_end - blk_begin;
     // rounds of equal size (to within a block), none longer than 17 blocks
-    // (several rows: the launch has made sure that no share is longer)
-    const uint32_t n_rounds = M > 1 ? 1 : (range + RBK - 1) / RBK;
+    // (several rows: one round of up to 17 blocks, or rounds of up to 8)
+    const uint32_t n_rounds = (M > 1 && range > uint32_t(RBK)) ? (range + W::SHORT_BLOCKS - 1) / W::SHORT_BLOCKS : (range + RBK - 1) / RBK;
     const uint32_t per_round = (range + n_rounds - 1) / n_rounds;
     auto blocks_of = [&](uint32_t round) { return min(range - round * per_round, per_round); };
 
@@ -1205,33 +1229,29 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
         asm volatile("" ::: "memory");
         return uint32_t(__builtin_amdgcn_readfirstlane(v));
     };
-    // A wait that runs out must not pass for a result: the wave leaves a code in the device's status word (a
-    // plain store by one lane; the host reads the word at its next call), marks the workgroup (the wave that
-    // writes the maxima and sums writes l = NaN then) and writes l = NaN itself in case that wave is through
-    // already, so that the reduce stage gives NaN for these heads; then it goes on to its end like any wave.
-    auto gave_up = [&](int c) {
-        if (lane == 0) {
-            __hip_atomic_store(a.status, 0x100u + uint32_t(c), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-            __hip_atomic_store(sync_lds + W::C_GAVE_UP, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        }
-        if (lane < 8 * M) {
-            const size_t slot = (size_t(lane >> 3) * a.nsplits + split) * a.heads + kv * 8 + (lane & 7);
-            a.part_ml[2 * slot + 1] = __builtin_nanf("");
-        }
-    };
+    // A wait that runs out must not pass for a result: the wave notes which counter it was, goes on to its
+    // end like any wave, and there (`leave`) leaves a code in the device's status word and l = NaN in the
+    // workgroup's partials (wait_gave_up, out of line: it never runs); the wave that stores the maxima and
+    // sums writes l = NaN itself if it has given up.  (The polling loop is kept rolled up: there are some
+    // twenty waits in the kernel, and its code has to come through the instruction cache at every launch.)
+    uint32_t lost = 0;
     auto await = [&](int c, uint32_t want) {
         asm volatile("" ::: "memory");
-        uint32_t i = 0;
-        for (; i < W::SPIN_LIMIT; i++) {
+        uint32_t left = W::SPIN_LIMIT;
+#pragma nounroll
+        do {
             const uint32_t v = __hip_atomic_load(sync_lds + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             if (__builtin_amdgcn_readfirstlane(v) >= want) break;
             __builtin_amdgcn_s_sleep(1);
-        }
-        if (__builtin_expect(i == W::SPIN_LIMIT, 0)) gave_up(c);
+        } while (--left);
+        if (__builtin_expect(left == 0, 0)) lost = 0x100u + uint32_t(c);
         asm volatile("" ::: "memory");
     };
+    auto leave = [&]() {
+        if (__builtin_expect(lost != 0, 0)) wait_gave_up(a.status, a.part_ml, lost, M, a.nsplits, split, a.heads, kv);
+    };
     // l of a partial as the writer of the maxima and sums stores it
-    auto marked = [&](float l) { return peek(W::C_GAVE_UP) ? __builtin_nanf("") : l; };
+    auto marked = [&](float l) { return lost ? __builtin_nanf("") : l; };
 
     if (loader && wave_all < W::K_LOADERS) {
         // ---- a key-loader wave: scales and biases of tokens 128 L .. 128 L + 127, keys of blocks L, L + 2, ...;
@@ -1296,6 +1316,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
             __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
             raise(W::C_KPART + 2);
         }
+        leave();
         return;
     }
     if (loader) {
@@ -1355,6 +1376,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
             __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
             raise(W::C_SLOT + 4);
         }
+        leave();
         return;
     }
 
@@ -1430,6 +1452,298 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
         const int at = wave / WT, wt = wave % WT;
         const int col_row = n >> 3;  // the row of the pair that this lane's column belongs to
         auto row_of = [&](int pair, int half) { return min(2 * pair + half, M - 1); };
+        if (range > uint32_t(RBK)) {
+            // ---- a share of more than one round (a context of more than 17 blocks per split) ----------
+            // Rounds of up to SHORT_BLOCKS blocks, in the blocks 0-7 of the keys' and the values' places.  What
+            // a round leaves behind, per column: the maximum so far, the sums so far relative to it (O in
+            // registers, l with wave 0), both brought to the new maximum before the next round's values are
+            // added.  The query operands of every pair wait in LDS (the blocks that short rounds never fill) and
+            // are read again for every round's scores, so that they hold no registers while the values are taken.
+            constexpr int SB = W::SHORT_BLOCKS, A_SHORT = SB / WT, S_SLOTS = SB / 4;
+            half8 *qp_lds = reinterpret_cast<half8 *>(lds_raw + W::QP_OFF);
+            _Float16 *qpz_lds = reinterpret_cast<_Float16 *>(lds_raw + W::QPZ_OFF);
+            {
+                const float qmul = a.scale * 1.4426950408889634f * Q_UP;
+#pragma unroll
+                for (int pair = 0; pair < PAIRS; pair++) {
+                    // this thread's item: k-step `wave`, lane `lane`: column n = (row n / 8 of the pair, head n % 8)
+                    half8 hi, lo;
+                    float sum = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        _Float16 h, lw;
+                        split_hi_lo(qv[pair][key_slot_dim<BITS>(e)] * qmul, h, lw);
+                        hi[e] = h, lo[e] = lw;
+                        sum += (float)h + (float)lw;
+                    }
+                    qp_lds[((pair * 2 + 0) * 8 + wave) * 64 + lane] = hi;
+                    qp_lds[((pair * 2 + 1) * 8 + wave) * 64 + lane] = lo;
+                    _Float16 h, lw;
+                    split_hi_lo(sum * (1.0f / Q_UP), h, lw);
+                    qpz_lds[((pair * 2 + 0) * 64 + lane) * 8 + wave] = h;
+                    qpz_lds[((pair * 2 + 1) * 64 + lane) * 8 + wave] = lw;
+                }
+                // blocks that a short round never has: maximum "none", sum 0 (the table of this wave's pair, by its first wave)
+                if (wt == 0 && j == 0) {
+                    const int my_row = row_of(at, col_row);
+#pragma unroll
+                    for (int b = SB; b < RBK; b++) bmax_lds[my_row * W::BROW + (n & 7) * W::BSTRIDE + b] = NO_SCORE, bsum_lds[my_row * W::BROW + (n & 7) * W::BSTRIDE + b] = 0.0f;
+                }
+            }
+            raise(W::C_QUERY);
+
+            float m_run[PAIRS], l_run[PAIRS], zacc[PAIRS];
+            floatx4 acc[PAIRS][4];  // [pair][tile of 16 dims 4n' + e]: rows 4j .. 4j+3 (columns of the pair), column n'
+#pragma unroll
+            for (int p = 0; p < PAIRS; p++) {
+                m_run[p] = NO_SCORE, l_run[p] = 0.0f, zacc[p] = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[p][e] = floatx4{0, 0, 0, 0};
+            }
+            uint32_t taken = 0;  // blocks whose scores this wave has written (two pairs: the handshake over a block's keys counts them)
+            await(W::C_QUERY, W::WAVES);
+#pragma unroll 1
+            for (uint32_t round = 0; round < n_rounds; round++) {
+                const uint32_t base = (blk_begin + round * per_round) * BLOCK, nb = blocks_of(round);
+                const uint32_t round_limit = min(limit, base + nb * BLOCK);  // tokens of this round end here
+                const uint32_t live_blocks = (nb + 1) & ~1u;  // k-steps are two blocks: the blocks of the k-steps that have tokens
+
+                // ---- phase A: the scores of this wave's blocks for its pair of rows ----
+                {
+                    const int my_row = row_of(at, col_row);
+                    const uint32_t my_limit = min<uint32_t>(round_limit, len_of(my_row));
+#pragma unroll 1
+                    for (int i = 0; i < A_SHORT; i++) {
+                        const int blk = wt + WT * i;
+                        if (uint32_t(blk) >= live_blocks) {
+                            // (no scores to take, and no operands will be made of this block; the table still holds the
+                            // round before's entries until every wave has built its operands from them)
+                            if (round > 0) await(W::C_BUILT, W::WAVES * round);
+                            if (j == 0) bmax_lds[my_row * W::BROW + (n & 7) * W::BSTRIDE + blk] = NO_SCORE, bsum_lds[my_row * W::BROW + (n & 7) * W::BSTRIDE + blk] = 0.0f;
+                            continue;
+                        }
+                        await(W::C_KPART + 0, W::K_LOADERS * (round + 1));  // the round's keys and scales are in LDS
+                        const unsigned char *kb = lds_raw + W::K_OFF + blk * W::K_BLOCK_BYTES;
+                        KeyRegs<BITS> kreg[4];
+#pragma unroll
+                        for (int gg = 0; gg < 4; gg++) {
+                            if constexpr (BITS == 8) {
+                                const u32x4 v = *reinterpret_cast<const u32x4 *>(kb + gg * 1024 + n * 64 + j * 16);
+                                kreg[gg].w[0] = v.x, kreg[gg].w[1] = v.y, kreg[gg].w[2] = v.z, kreg[gg].w[3] = v.w;
+                            } else {
+                                const u32x2 v = *reinterpret_cast<const u32x2 *>(kb + (gg >> 1) * 1024 + n * 64 + (gg & 1) * 32 + j * 8);
+                                kreg[gg].w[0] = v.x, kreg[gg].w[1] = v.y;
+                            }
+                        }
+                        const int tok0 = BLOCK * blk + 4 * j;  // this lane's 4 tokens of the round in C layout
+                        const uint32_t *sb_w = sb_lds + BLOCK * blk;
+                        const u32x2 zr = {sb_w[W::SB_ARRAY / 4 + n], sb_w[W::SB_ARRAY / 4 + RT + n]};
+                        const half8 zop = as_half8(perm(0, zr.x, 0x01000100u), perm(0, zr.x, 0x03020302u), perm(0, zr.y, 0x01000100u), perm(0, zr.y, 0x03020302u));
+                        const u32x4 s01 = *reinterpret_cast<const u32x4 *>(sb_w + 4 * j);
+                        const u32x4 s23 = *reinterpret_cast<const u32x4 *>(sb_w + RT + 4 * j);
+                        const uint32_t sw[8] = {s01.x, s23.x, s01.y, s23.y, s01.z, s23.z, s01.w, s23.w};
+                        floatx4 sc = {0, 0, 0, 0}, rr[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+                        sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, *reinterpret_cast<const half8 *>(qpz_lds + ((at * 2 + 0) * 64 + lane) * 8), sc, 0, 0, 0);
+                        sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, *reinterpret_cast<const half8 *>(qpz_lds + ((at * 2 + 1) * 64 + lane) * 8), sc, 0, 0, 0);
+                        // the hi parts of the pair's query operands, then the lo parts: one set in registers at a time
+                        // (the accumulators of the rounds so far are held as well), the key operands made once for each
+#pragma unroll
+                        for (int part = 0; part < 2; part++) {
+                            half8 q_part[8];
+#pragma unroll
+                            for (int k = 0; k < 8; k++) q_part[k] = qp_lds[((at * 2 + part) * 8 + k) * 64 + lane];
+#pragma unroll
+                            for (int gg = 0; gg < 4; gg++) {
+#pragma unroll
+                                for (int ab = 0; ab < 2; ab++) {
+                                    rr[gg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(key_operand<BITS>(kreg[gg], ab), q_part[gg * 2 + ab], rr[gg], 0, 0, 0);
+                                }
+                            }
+                            asm volatile("" ::: "memory");  // (the lo parts are not to be fetched while the hi parts are held)
+                        }
+                        constexpr float C1 = code_up<BITS>() / Q_UP;
+#pragma unroll
+                        for (int tk = 0; tk < 4; tk++) {
+                            float d = 0.0f;
+#pragma unroll
+                            for (int gg = 0; gg < 4; gg++) d += half_bits_to_float(sw[2 * tk + (gg >> 1)] >> (16 * (gg & 1))) * rr[gg][tk];
+                            const float v = sc[tk] + d * C1;
+                            sc[tk] = base + tok0 + tk < my_limit ? v : NO_SCORE;  // (also whatever a block past the round left in LDS)
+                        }
+                        // the block's softmax relative to its own maximum, per column
+                        float cm = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+                        cm = across_rows<16, 64>(cm, MaxOp());
+                        float sum = 0.0f;
+#pragma unroll
+                        for (int tk = 0; tk < 4; tk++) {
+                            sc[tk] = sc[tk] > 0.5f * NO_SCORE ? __builtin_amdgcn_exp2f(sc[tk] - cm) : 0.0f;
+                            sum += sc[tk];
+                        }
+                        sum = across_rows<16, 64>(sum, SumOp());
+                        if (j == 0) bmax_lds[my_row * W::BROW + (n & 7) * W::BSTRIDE + blk] = cm, bsum_lds[my_row * W::BROW + (n & 7) * W::BSTRIDE + blk] = sum;
+                        // the scores go over the block's own keys: when this wave has them in registers, and with
+                        // two pairs the other pair's wave of the same blocks, which takes them in the same order
+                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                        taken++;
+                        if constexpr (PAIRS > 1) {
+                            raise(W::C_MERGE + wt);
+                            await(W::C_MERGE + wt, PAIRS * taken);
+                        }
+                        *reinterpret_cast<floatx4 *>(s_block(blk, my_row) + (n & 7) * BLOCK + 4 * j) = sc;
+                    }
+                }
+                raise(W::C_SCORES);
+                await(W::C_SCORES, W::WAVES * (round + 1));
+
+                // ---- the columns' maxima; what was summed so far brought to them; the probability operands ----
+                float al[PAIRS];
+#pragma unroll
+                for (int p = 0; p < PAIRS; p++) {
+                    const float nm = round_max(row_of(p, col_row), m_run[p]);
+                    al[p] = __builtin_amdgcn_exp2f(m_run[p] - nm);  // (nothing summed so far: whatever it is, it scales zeros)
+                    m_run[p] = nm;
+                    zacc[p] *= al[p];
+                    if (wave == 0) l_run[p] = l_run[p] * al[p] + round_sum(row_of(p, col_row), nm);
+                }
+                half8 p_hi[PAIRS][S_SLOTS], p_lo[PAIRS][S_SLOTS];
+#pragma unroll
+                for (int sl = 0; sl < S_SLOTS; sl++) {
+                    if (uint32_t(2 * (2 * sl + b2)) >= nb) {  // the k-step has no tokens
+#pragma unroll
+                        for (int p = 0; p < PAIRS; p++) p_hi[p][sl] = p_lo[p][sl] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+                        continue;
+                    }
+                    const int ks = 2 * sl + b2;  // tokens 32 ks ..: blocks 2 ks and 2 ks + 1
+                    const int blk = 2 * ks + (j >> 1);
+                    const int sh = 16 * (g & 1);
+                    const uint32_t *vsp = sb_lds + 2 * (W::SB_ARRAY / 4) + (g >> 1) * RT + 32 * ks + 8 * j;
+                    const u32x4 sv0 = *reinterpret_cast<const u32x4 *>(vsp), sv1 = *reinterpret_cast<const u32x4 *>(vsp + 4);
+                    const u32x4 zv0 = *reinterpret_cast<const u32x4 *>(vsp + W::SB_ARRAY / 4), zv1 = *reinterpret_cast<const u32x4 *>(vsp + W::SB_ARRAY / 4 + 4);
+                    const uint32_t sw[8] = {sv0.x, sv0.y, sv0.z, sv0.w, sv1.x, sv1.y, sv1.z, sv1.w};
+                    const uint32_t zw[8] = {zv0.x, zv0.y, zv0.z, zv0.w, zv1.x, zv1.y, zv1.z, zv1.w};
+                    float vscale[8], vbias[8];
+#pragma unroll
+                    for (int e = 0; e < 8; e++) vscale[e] = half_bits_to_float(sw[e] >> sh), vbias[e] = half_bits_to_float(zw[e] >> sh);
+#pragma unroll
+                    for (int p = 0; p < PAIRS; p++) {
+                        const int r = row_of(p, col_row);
+                        const float *sp = s_block(blk, r) + (n & 7) * BLOCK + 8 * (j & 1);
+                        const floatx4 pt0 = *reinterpret_cast<const floatx4 *>(sp), pt1 = *reinterpret_cast<const floatx4 *>(sp + 4);
+                        const float pt[8] = {pt0[0], pt0[1], pt0[2], pt0[3], pt1[0], pt1[1], pt1[2], pt1[3]};
+                        // 2^(block maximum - maximum so far) * P_UP (2^8, so that the lo part stays a normal f16)
+                        const float f = __builtin_amdgcn_exp2f(bmax_lds[r * W::BROW + (n & 7) * W::BSTRIDE + blk] - m_run[p] + 8.0f);
+                        float x[8], lo[8], zb = 0.0f;
+#pragma unroll
+                        for (int e = 0; e < 8; e++) {
+                            zb += pt[e] * vbias[e];
+                            x[e] = pt[e] * f * vscale[e];
+                            lo[e] = x[e] - __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x[e]) & 0xffffe000u);
+                        }
+                        zacc[p] += zb * f;
+                        uint32_t o[8];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            // round toward zero: exact truncation to the hi part
+                            o[e] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x[2 * e], x[2 * e + 1]));
+                            o[4 + e] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo[2 * e], lo[2 * e + 1]));
+                        }
+                        asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]), "+v"(o[4]), "+v"(o[5]), "+v"(o[6]), "+v"(o[7]));
+                        p_hi[p][sl] = as_half8(o[0], o[1], o[2], o[3]);
+                        p_lo[p][sl] = as_half8(o[4], o[5], o[6], o[7]);
+                    }
+                }
+                raise(W::C_BUILT);  // this wave is through with the round's scores, scales and biases
+
+                // ---- phase C: O = O * 2^(old maximum - new) + P V ----
+                if (round > 0) {
+#pragma unroll
+                    for (int p = 0; p < PAIRS; p++) {
+                        // accumulator rows 4j + i are the pair's columns 4j + i: lane c (j = 0, n = c) holds column c's factor
+                        floatx4 al4;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) al4[i] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(4 * (4 * j + i), __builtin_bit_cast(int, al[p])));
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[p][e] *= al4;
+                    }
+                }
+#pragma unroll
+                for (int sl = 0; sl < S_SLOTS; sl++) {
+                    if (uint32_t(2 * (2 * sl + b2)) >= nb) continue;
+                    await(W::C_SLOT + sl, W::V_LOADERS * (round + 1));  // value slot sl is in LDS
+                    ValRegs<BITS> vreg;
+                    read_values(2 * sl + b2, g, vreg);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const half8 vop = val_operand<BITS>(vreg, e, n);
+#pragma unroll
+                        for (int p = 0; p < PAIRS; p++) {
+                            acc[p][e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p_hi[p][sl], vop, acc[p][e], 0, 0, 0);
+                            acc[p][e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p_lo[p][sl], vop, acc[p][e], 0, 0, 0);
+                        }
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the value codes are in registers
+                raise(W::C_DONE);
+            }
+
+            // ---- epilogue: the two waves of a group add up, wave 2g writes the partials ----
+#pragma unroll
+            for (int p = 0; p < PAIRS; p++) {
+                const float z = across_rows<16, 64>(zacc[p], SumOp());
+                if (j == 0) zs_lds[(wave * PAIRS + p) * 16 + n] = z;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            floatx4 mine[PAIRS][4];  // column 4j + i of the pair, dims 64 g + 4n .. + 3
+#pragma unroll
+            for (int p = 0; p < PAIRS; p++) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float zb = zs_lds[(wave * PAIRS + p) * 16 + 4 * j + i] * (1.0f / P_UP);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) mine[p][i][e] = acc[p][e][i] * unscale + zb;
+                }
+            }
+            // (the merge lies over the keys, which hold the last round's scores until every wave has built its operands;
+            // the key loaders request nothing after the last round)
+            floatx4 *x_o = reinterpret_cast<floatx4 *>(lds_raw + W::K_OFF);  // [pair][group][lane][4 columns]
+            static_assert(PAIRS * 4 * 64 * 4 * 16 <= W::SHORT_BLOCKS * W::K_BLOCK_BYTES || BITS == 4, "the merge stays clear of the query operands");
+            await(W::C_BUILT, W::WAVES * n_rounds);
+            if (b2 == 1) {
+#pragma unroll
+                for (int p = 0; p < PAIRS; p++) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) x_o[((p * 4 + g) * 64 + lane) * 4 + i] = mine[p][i];
+                }
+                raise(W::C_MERGE + 4 + g);
+                leave();
+                return;
+            }
+            if (wave == 0) {
+#pragma unroll
+                for (int p = 0; p < PAIRS; p++) {
+                    const int r = 2 * p + col_row;
+                    if (j == 0 && r < M) {
+                        const size_t slot = (size_t(r) * a.nsplits + split) * a.heads + kv * 8 + (n & 7);
+                        *reinterpret_cast<floatx2 *>(a.part_ml + 2 * slot) = floatx2{m_run[p], marked(l_run[p])};
+                    }
+                }
+            }
+            await(W::C_MERGE + 4 + g, 1);
+#pragma unroll
+            for (int p = 0; p < PAIRS; p++) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int c = 4 * j + i, r = 2 * p + (c >> 3);
+                    if (r < M) {
+                        const size_t slot = (size_t(r) * a.nsplits + split) * a.heads + kv * 8 + (c & 7);
+                        __builtin_nontemporal_store(mine[p][i] + x_o[((p * 4 + g) * 64 + lane) * 4 + i], reinterpret_cast<floatx4 *>(a.part_o + slot * DIM + 64 * g + 4 * n));
+                    }
+                }
+            }
+            leave();
+            return;
+        }
         const uint32_t base = blk_begin * BLOCK;
         const bool extra = range >= uint32_t(RBK);  // the round has block 16
         const uint32_t live_blocks = (range + 1) & ~1u;  // k-steps are two blocks: the blocks of the k-steps that have tokens
@@ -1676,6 +1990,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
                 for (int i = 0; i < 4; i++) x_o[((p * 4 + g) * 64 + lane) * 4 + i] = mine[p][i];
             }
             raise(W::C_MERGE + 4 + g);
+            leave();
             return;
         }
         if (wave == 0) {
@@ -2006,6 +2321,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
                 for (int i = 0; i < 4; i++) x_o[(g * 32 + lane) * 4 + i] = mine[i];
             }
             raise(W::C_MERGE + g);
+            leave();
             return;
         }
         await(W::C_MERGE + g, 1);
@@ -2021,6 +2337,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
             }
         }
     }
+    leave();
 }
 
 // Merges the splits of one (q head, row): weights 2^(m_c - M), then the gate
@@ -2246,11 +2563,10 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
     // against 31.1 at 131k, 8-bit); with two or three short rounds the ring of slots is ahead (14.1
     // against 15.6 us at 40k), and so it is for 4-bit codes above 100k tokens (28.0 against 29.3 at 131k).
     // Two to four rows over codes (a verify step) run the same kernel, the codes in LDS serving every
-    // row, where no share can be longer than the one round that kernel takes with several rows.
-    const uint32_t splits_one_per_cu = nsplits > MAX_SPLITS / 2 ? MAX_SPLITS / 2 : nsplits;
-    const uint32_t longest_share = (capacity / BLOCK + splits_one_per_cu - 1) / splits_one_per_cu;  // in blocks
-    const bool rows_keys_first = rows >= 2 && rows <= 4 && bits != 16 && capacity >= LOADERS_FROM && longest_share <= 17 &&
-                                 !(stages & SAETTA_STAGE_NO_LOADERS);
+    // row: one round where the context in use gives shares of up to 17 blocks (the kernel sees the
+    // length when it runs; a verify step at 32k tokens is one round in a cache of any size), rounds
+    // of 8 blocks beyond.
+    const bool rows_keys_first = rows >= 2 && rows <= 4 && bits != 16 && capacity >= LOADERS_FROM && !(stages & SAETTA_STAGE_NO_LOADERS);
     const bool keys_first = rows_keys_first || (loaders && (capacity <= KEYS_FIRST_ONE_ROUND || (capacity >= KEYS_FIRST_AGAIN_FROM &&
                                                                                (bits == 8 || capacity <= KEYS_FIRST_4BIT_UP_TO))));
     if (one_per_cu && nsplits > MAX_SPLITS / 2) nsplits = MAX_SPLITS / 2;

@@ -260,9 +260,9 @@ def test_capacity_must_be_whole_blocks():
 @pytest.mark.parametrize("kind", [saetta.KvBits.Eight, saetta.KvBits.Four])
 def test_large_cache_of_codes_several_rows(kind, m):
     # Two to four rows over codes in a cache of 24k tokens and more whose longest share is one round of
-    # 17 blocks (capacities up to 34816) run the keys-first kernel with two rows to a tile; three
-    # rows: the second tile's upper half repeats row 2.  Capacity 35072: a share can be 18 blocks, and
-    # the register kernels take over.  Positions: the first tokens of a cache (row r sees r + 1
+    # 17 blocks (capacities up to 34816) run the keys-first kernel in one round, two rows to a tile; three
+    # rows: the second tile's upper half repeats row 2.  Capacity 35072: a share can be 18 blocks, which
+    # the same kernel takes in three rounds of 6.  Positions: the first tokens of a cache (row r sees r + 1
     # tokens: whole shares are empty for the earlier rows); one block per share; shares of a few
     # blocks; shares of 16 and of 17 blocks side by side; the whole capacity.  The rows past the last
     # token are poisoned.
@@ -291,11 +291,44 @@ def test_large_cache_of_codes_several_rows(kind, m):
             del kc, vc
 
 
+@pytest.mark.parametrize("m", [2, 3, 4])
+@pytest.mark.parametrize("kind", [saetta.KvBits.Eight, saetta.KvBits.Four])
+def test_several_rows_in_caches_of_65536_and_131072_tokens(kind, m):
+    # The reference's caches are 8192 * 2^k tokens (src/gpu_model.rs:390,406-416): a verify step at 32k
+    # tokens runs in a cache of 65536.  The keys-first kernel sees the length when it runs: shares of up to
+    # 17 blocks are one round whatever the capacity is, longer ones rounds of up to 8 blocks with the
+    # maxima and sums carried from round to round.  Positions: the first tokens of a cache; a block per
+    # share; shares of 16 and 17 blocks side by side (one round); 18 to 20 blocks (three rounds of 6 and
+    # 7); 25 blocks (rounds of 7 and 4); the whole capacity (4 and 8 rounds of 8).  The rows past the last
+    # token are poisoned.
+    rng = np.random.default_rng(6500 + m)
+    q = rng.standard_normal((m, H, D)).astype(np.float32)
+    qg = rng.standard_normal((m, H, 2 * D)).astype(np.float32)
+    for capacity in (65536, 131072):
+        k = (rng.standard_normal((capacity, VALUES)) * 2.0).astype(np.float32)
+        v = rng.standard_normal((capacity, VALUES)).astype(np.float32)
+        rows = saetta.AttentionRows(H, KV, capacity, m)
+        for tokens in [m, 2049, 33000, 38000, 50001, capacity]:
+            pos = tokens - m
+            kc, vc, kf, vf = cache_pair(k[:tokens], v[:tokens], kind, capacity, poison=True)
+            out = torch.full((m, H, D), float("nan"), device="cuda")
+            params = [saetta.TokenParams(0, pos + r).as_tensor("cuda") for r in range(m)]
+            plan = saetta.Plan()
+            rows.record_quant(plan, m, dev(q), kc, vc, dev(qg), out, params)
+            plan.build().run()
+            got = host(out)
+            assert np.isfinite(got).all(), (capacity, tokens)
+            want64 = oracle.rows(q, kf, vf, pos, m, q_and_gate=qg, threads=8, f64=True)
+            worst = np.abs(got - want64).max()
+            assert worst < MAX_ABS_F64, (capacity, tokens, worst)
+            del kc, vc
+
+
 @pytest.mark.parametrize("splits", [100, 64, 7])
 def test_several_rows_with_fewer_splits(splits):
     # RowsAttentionParams.splits is an upper bound the caller may lower (src/rows.rs:344-367).  In a
     # cache of 24576 tokens: 100 splits are shares of 15 and 16 blocks, still one round of the
-    # keys-first kernel; 64 splits are shares of 24 blocks and 7 of 220, which the register kernels take.
+    # keys-first kernel; 64 splits are shares of 24 blocks (three rounds of 8) and 7 of 220 (28 rounds).
     rng = np.random.default_rng(4100 + splits)
     capacity, m, kind = 24576, 3, saetta.KvBits.Eight
     k = rng.standard_normal((capacity, VALUES)).astype(np.float32)
