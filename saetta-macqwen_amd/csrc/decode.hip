@@ -49,12 +49,10 @@
 //   attention_partial_kernel_p   one query row, one workgroup per CU (all registers)
 //   attention_partial_kernel_1   one query row over codes, two workgroups per CU (long 4-bit caches)
 //   attention_partial_kernel_n   2 rows (1 tile), 3-4 rows (2 tiles), 5-8 rows (4 tiles)
-//   attention_partial_kernel_d   one query row over codes in large caches: four more waves
-//                                move the codes into LDS (global_load_lds), two teams of four
-//                                computing waves take alternate 64-token iterations
-//   attention_partial_kernel_s   one to four query rows over codes in large caches: loader waves
-//                                again, a whole share in LDS with the keys requested first, the
-//                                waves meeting through counters in LDS
+//   attention_partial_kernel_s   one to four query rows over codes in large caches: four more waves
+//                                move the codes into LDS (global_load_lds), a whole share at once
+//                                with the keys requested first (longer shares: rounds in alternate
+//                                halves of LDS), the waves meeting through counters in LDS
 //   attention_reduce_kernel      the merge of the splits and the gate
 // Which one runs is decided in run_attention from the launch arguments alone, so that the partial
 // and the reduce stage of a step agree on the number of splits.
@@ -278,39 +276,10 @@ struct Shape {
     static constexpr int QZ_OFF = ALPHA_OFF + S_ROWS * 4;                   // [tile][hi, lo][lane] half8
     static constexpr int ZSUM_OFF = QZ_OFF + TILES * 2 * 64 * 16;           // [wave][S_ROWS] f32
     static constexpr int LDS_BYTES = ZSUM_OFF + 4 * S_ROWS * 4;
-    // With loader waves (codes only): four slots of one iteration's key and value codes each.  A
-    // load instruction brings 64 pieces of 16 bytes; a (token, kv head) row is PIECES of them.
-    // Keys: per block [piece][16 tokens]; values: whole token rows, as many as one instruction
-    // brings (four of 256 bytes, eight of 128), these groups 32 bytes apart so that the four lane
-    // groups of a value read hit different banks.
-    static constexpr int PIECES = row_bytes<BITS>() / 16;
-    static constexpr int DMA_PER_BLOCK = PIECES / 4;   // load instructions per block of keys, and of values
-    static constexpr int V_GROUP_TOKENS = 64 / PIECES;
-    static constexpr int DMA_SLOTS = 16 / ITB;  // 256 tokens of codes in LDS
-    static constexpr int K_BLOCK_BYTES = BLOCK * row_bytes<BITS>();
-    static constexpr int K_SLOT_BYTES = ITB * K_BLOCK_BYTES;
-    static constexpr int V_GROUP_BYTES = 1024 + 32;
-    static constexpr int V_SLOT_BYTES = ITB * DMA_PER_BLOCK * V_GROUP_BYTES;
-    // The teams share the query operands (the first array and qz); a further team's other arrays
-    // start where the first team's end, its own (unused) query area lying over them.
-    static constexpr int TEAM_SHIFT = LDS_BYTES - Q_BYTES;
-    static constexpr int dma_k_off(int teams) { return (LDS_BYTES + (teams - 1) * TEAM_SHIFT + 1023) / 1024 * 1024; }
-    static constexpr int dma_lds_bytes(int teams) {
-        return dma_k_off(teams) + DMA_SLOTS * (K_SLOT_BYTES + V_SLOT_BYTES);
-    }
 };
 
-// DMA: the workgroup has four more waves that do nothing but move key and value codes from global
-// memory into LDS (global_load_lds, no registers), slot by slot, as far ahead as the slots allow; a
-// wave that requests loads stands still while the request queues are full, and these waves have
-// nothing else to do.  The four computing waves take their operands from LDS instead.
-// TEAMS (with DMA): groups of four computing waves; in every round team t takes iteration
-// TEAMS * round + t, all in step (the barriers are the workgroup's), and team 0 merges the teams'
-// results at the end.
-template <int BITS, int TILES, bool PACKED, int ITB, bool UNCOND, bool DMA = false, int TEAMS = 1>
+template <int BITS, int TILES, bool PACKED, int ITB, bool UNCOND>
 __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
-    static_assert(TEAMS == 1 || (DMA && TEAMS == 2), "teams need the loader waves");
-    static_assert(!DMA || (BITS != 16 && PACKED && (ITB == 4 || ITB == 8)), "loader waves: one row over codes, 64- or 128-token iterations");
     using Sh = Shape<BITS, TILES, PACKED, ITB>;
     constexpr int IT_BLOCKS = ITB, IT_TOKENS = Sh::IT_TOKENS, SC_STRIDE = Sh::SC_STRIDE;
     constexpr int KROUNDS = ITB / 4, KSTEPS = ITB / 2;
@@ -318,20 +287,16 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     constexpr int PARTS = Sh::PARTS;
     constexpr int RB = row_bytes<BITS>();
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    // team: 0 .. TEAMS - 1 compute, TEAMS = the loader waves; tid and wave are the team's own
-    const int team = DMA ? int(threadIdx.x) / THREADS : 0;
-    const int tid = DMA ? int(threadIdx.x) % THREADS : int(threadIdx.x), lane = tid & 63, wave = tid >> 6;
-    unsigned char *lds_team = lds_raw + (DMA && team < TEAMS ? team * Sh::TEAM_SHIFT : 0);
-    constexpr int K_OFF = Sh::dma_k_off(TEAMS), V_OFF = K_OFF + Sh::DMA_SLOTS * Sh::K_SLOT_BYTES;
+    const int tid = int(threadIdx.x), lane = tid & 63, wave = tid >> 6;
     half8 *q_lds = reinterpret_cast<half8 *>(lds_raw + Sh::Q_OFF);
-    float *s_lds = reinterpret_cast<float *>(lds_team + Sh::S_OFF);
-    uint16_t *ks_lds = reinterpret_cast<uint16_t *>(lds_team + Sh::KS_OFF);
-    uint16_t *kz_lds = reinterpret_cast<uint16_t *>(lds_team + Sh::KZ_OFF);
-    uint16_t *vs_lds = reinterpret_cast<uint16_t *>(lds_team + Sh::VS_OFF);
-    uint16_t *vz_lds = reinterpret_cast<uint16_t *>(lds_team + Sh::VZ_OFF);
-    float *alpha_lds = reinterpret_cast<float *>(lds_team + Sh::ALPHA_OFF);
+    float *s_lds = reinterpret_cast<float *>(lds_raw + Sh::S_OFF);
+    uint16_t *ks_lds = reinterpret_cast<uint16_t *>(lds_raw + Sh::KS_OFF);
+    uint16_t *kz_lds = reinterpret_cast<uint16_t *>(lds_raw + Sh::KZ_OFF);
+    uint16_t *vs_lds = reinterpret_cast<uint16_t *>(lds_raw + Sh::VS_OFF);
+    uint16_t *vz_lds = reinterpret_cast<uint16_t *>(lds_raw + Sh::VZ_OFF);
+    float *alpha_lds = reinterpret_cast<float *>(lds_raw + Sh::ALPHA_OFF);
     _Float16 *qz_lds = reinterpret_cast<_Float16 *>(lds_raw + Sh::QZ_OFF);
-    float *zsum_lds = reinterpret_cast<float *>(lds_team + Sh::ZSUM_OFF);
+    float *zsum_lds = reinterpret_cast<float *>(lds_raw + Sh::ZSUM_OFF);
 
     const int n = lane & 15, j = lane >> 4;
     const uint32_t split = blockIdx.x, kv = blockIdx.y;
@@ -361,10 +326,8 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     };
     float q_early[TILES == 1 ? 2 : 1][8];
     if constexpr (TILES == 1) {
-        if (team < TEAMS) {
-            load_q_item(tid, q_early[0]);
-            load_q_item(tid + THREADS, q_early[1]);
-        }
+        load_q_item(tid, q_early[0]);
+        load_q_item(tid + THREADS, q_early[1]);
     }
 
     // ---- the context and this workgroup's share of it -----------------------------
@@ -386,7 +349,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     const uint32_t range = blk_end - blk_begin;
     const uint32_t n_it = (range + IT_BLOCKS - 1) / IT_BLOCKS;
     const uint32_t per_it = (range + n_it - 1) / n_it;
-    const uint32_t n_rounds = (n_it + TEAMS - 1) / TEAMS;
+    const uint32_t n_rounds = n_it;
 
     const uint32_t cap_rows = a.capacity * kvh;
     const __amdgpu_buffer_rsrc_t k_rsrc = make_rsrc(a.kdata, cap_rows * RB);
@@ -397,81 +360,6 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     const __amdgpu_buffer_rsrc_t vz_rsrc = make_rsrc(a.vbiases, QUANT ? cap_rows * 8 : 0);
     const int tok_stride = int(kvh) * RB;  // bytes between tokens of one kv head
 
-    if constexpr (DMA) {
-        if (team == TEAMS) {
-            // ---- a loader wave: block L of every iteration, keys then values ----------------
-            const uint32_t L = __builtin_amdgcn_readfirstlane(wave);
-            const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(lds_raw));
-            auto dma = [&](uint32_t lds_addr, uint32_t voff, const void *src) {
-                asm volatile("s_mov_b32 m0, %0\n"
-                             "s_nop 0\n"
-                             "global_load_lds_dwordx4 %1, %2\n"
-                             :
-                             : "s"(lds_addr), "v"(voff), "s"(src)
-                             : "memory", "m0");
-            };
-            const uint32_t last_row = a.capacity - 1;  // (global loads are not bounds checked)
-            constexpr int PER_BLOCK = Sh::DMA_PER_BLOCK;
-            constexpr int PER_REQUEST = 2 * PER_BLOCK * KROUNDS;  // loads of one iteration, per loader wave
-            auto request = [&](uint32_t it) {
-                const uint32_t slot = it % Sh::DMA_SLOTS;
-                // keys of every round first: phase A needs them first
-#pragma unroll
-                for (int r = 0; r < KROUNDS; r++) {
-                    const uint32_t blk = L + 4 * r, base = (blk_begin + it * per_it + blk) * BLOCK;
-                    // lane -> (piece lane / 16 of the instruction's four, token lane % 16)
-                    const uint32_t ktok = min(base + (lane & 15), last_row);
-                    const uint32_t kvoff = (ktok * kvh + kv) * RB + (lane >> 4) * 16;
-#pragma unroll
-                    for (int i = 0; i < PER_BLOCK; i++) {
-                        dma(lds0 + K_OFF + slot * Sh::K_SLOT_BYTES + blk * Sh::K_BLOCK_BYTES + i * 1024, kvoff + 64 * i, a.kdata);
-                    }
-                }
-#pragma unroll
-                for (int r = 0; r < KROUNDS; r++) {
-                    const uint32_t blk = L + 4 * r, base = (blk_begin + it * per_it + blk) * BLOCK;
-                    // lane -> (token lane / PIECES of the instruction's group, piece lane % PIECES)
-#pragma unroll
-                    for (int i = 0; i < PER_BLOCK; i++) {
-                        const uint32_t vtok = min(base + Sh::V_GROUP_TOKENS * i + lane / Sh::PIECES, last_row);
-                        dma(lds0 + V_OFF + slot * Sh::V_SLOT_BYTES + (PER_BLOCK * blk + i) * Sh::V_GROUP_BYTES,
-                            (vtok * kvh + kv) * RB + (lane % Sh::PIECES) * 16, a.vdata);
-                    }
-                }
-            };
-            uint32_t requested = min(n_it, uint32_t(Sh::DMA_SLOTS));
-            for (uint32_t it = 0; it < requested; it++) request(it);
-            __builtin_amdgcn_s_barrier();  // the computing waves' barrier after the query prologue
-            for (uint32_t round = 0; round < n_rounds; round++) {
-                // the round's iterations are in LDS when at most the later ones' loads are in flight
-                const uint32_t last = min(round * TEAMS + TEAMS - 1, n_it - 1);
-                const uint32_t later = requested - 1 - last;
-                static_assert(PER_REQUEST * (Sh::DMA_SLOTS - 1) < 64, "vmcnt is 6 bits");
-                if (Sh::DMA_SLOTS > 3 && later >= 3) {
-                    __builtin_amdgcn_s_waitcnt(vmcnt_only(PER_REQUEST * 3 < 64 ? PER_REQUEST * 3 : 63));
-                } else if (Sh::DMA_SLOTS > 2 && later == 2) {
-                    __builtin_amdgcn_s_waitcnt(vmcnt_only(PER_REQUEST * 2 < 64 ? PER_REQUEST * 2 : 63));
-                } else if (later == 1) {
-                    __builtin_amdgcn_s_waitcnt(vmcnt_only(PER_REQUEST));
-                } else {
-                    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
-                }
-                __builtin_amdgcn_s_barrier();  // "scales visible": the round may start
-                // every computing wave is past phase C of the round before: its slots take the next
-                if (round >= 1) {
-#pragma unroll
-                    for (int t = 0; t < TEAMS; t++) {
-                        if (requested < n_it) request(requested++);
-                    }
-                }
-                __builtin_amdgcn_s_barrier();  // scores done
-                __builtin_amdgcn_s_barrier();  // probabilities done
-            }
-            if constexpr (TEAMS > 1) __builtin_amdgcn_s_barrier();  // the teams' merge
-            return;
-        }
-    }
-
     // ---- the loads of one iteration ------------------------------------------------
     // Everything an iteration reads is requested before anything is computed: keys first
     // (phase A needs them first), then the small scale/bias rows, then the values.
@@ -480,7 +368,6 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     u32x2 ksr = {0, 0}, kzr = {0, 0}, vsr = {0, 0}, vzr = {0, 0};
     auto blocks_of = [&](uint32_t it) { return it < n_it ? min(per_it, blk_end - (blk_begin + it * per_it)) : 0u; };
     auto load_keys = [&](uint32_t it) {
-        if constexpr (DMA) return;
         const uint32_t base = (blk_begin + it * per_it) * BLOCK, nb = blocks_of(it);
         const int voff = int((base + BLOCK * wave + n) * kvh + kv) * RB + j * key_piece<BITS>();
 #pragma unroll
@@ -507,7 +394,6 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
         }
     };
     auto load_values = [&](uint32_t it) {
-        if constexpr (DMA) return;
         const uint32_t base = (blk_begin + it * per_it) * BLOCK, ksteps = (blocks_of(it) + 1) / 2;
         const int voff = int((base + 8 * j) * kvh + kv) * RB + val_lane_offset<BITS>(wave, n);
 #pragma unroll
@@ -526,9 +412,9 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
             }
         }
     };
-    load_scales(team);  // first: loads return in order, and the barrier that publishes the scales must not wait for the keys
-    load_keys(team);
-    load_values(team);
+    load_scales(0);  // first: loads return in order, and the barrier that publishes the scales must not wait for the keys
+    load_keys(0);
+    load_values(0);
 
     // ---- prologue: query rows to f16 hi/lo operands in LDS ------------------------
     // (while the first iteration's keys are in flight; the values are requested after it)
@@ -614,7 +500,7 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
     }
 
     for (uint32_t round = 0; round < n_rounds; round++) {
-        const uint32_t it = round * TEAMS + team;  // (a team without an iteration in the last round idles through it)
+        const uint32_t it = round;
         const uint32_t blk0 = blk_begin + it * per_it;
         const uint32_t nb = blocks_of(it);  // blocks of this iteration, 0..ITB
         const uint32_t base = blk0 * BLOCK;
@@ -642,26 +528,6 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
                 vz_lds[2 * IT_TOKENS + tid] = uint16_t(vzr.y), vz_lds[3 * IT_TOKENS + tid] = uint16_t(vzr.y >> 16);
             }
         }
-        if constexpr (DMA) {
-            // this wave's block: the lane's piece j of each group, its token n
-            const unsigned char *kb = lds_raw + K_OFF + (it % Sh::DMA_SLOTS) * Sh::K_SLOT_BYTES + wave * Sh::K_BLOCK_BYTES;
-#pragma unroll
-            for (int i = 0; i < KROUNDS; i++) {
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    if constexpr (BITS == 8) {
-                        const u32x4 v = *reinterpret_cast<const u32x4 *>(kb + i * 4 * Sh::K_BLOCK_BYTES + (4 * g + j) * 256 + n * 16);
-                        kreg[i][g].w[0] = v.x, kreg[i][g].w[1] = v.y, kreg[i][g].w[2] = v.z, kreg[i][g].w[3] = v.w;
-                    } else {
-                        // 8 bytes: half (j % 2) of piece 2 g + j / 2
-                        const u32x2 v = *reinterpret_cast<const u32x2 *>(kb + i * 4 * Sh::K_BLOCK_BYTES + (2 * g + (j >> 1)) * 256 +
-                                                                         n * 16 + (j & 1) * 8);
-                        kreg[i][g].w[0] = v.x, kreg[i][g].w[1] = v.y;
-                    }
-                }
-            }
-        }
-
         // ---- phase A: scores -------------------------------------------------------
 #pragma unroll
         for (int t = 0; t < TILES; t++) {
@@ -729,9 +595,9 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
             }
         }
         // The key registers and the scale registers are free: request the next iteration's.
-        if (it + TEAMS < n_it) {
-            load_scales(it + TEAMS);
-            load_keys(it + TEAMS);
+        if (it + 1 < n_it) {
+            load_scales(it + 1);
+            load_keys(it + 1);
         }
         __syncthreads();
 
@@ -833,18 +699,6 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
                 for (int ks = 0; ks < KSTEPS; ks++) {
                     if (uint32_t(ks) < ksteps) build_p(t, ks, phi[ks], plo[ks]);
                 }
-                if constexpr (DMA) {
-                    const unsigned char *vb = lds_raw + V_OFF + (it % Sh::DMA_SLOTS) * Sh::V_SLOT_BYTES + val_lane_offset<BITS>(wave, n);
-#pragma unroll
-                    for (int ks = 0; ks < KSTEPS; ks++) {
-#pragma unroll
-                        for (int e = 0; e < 8; e++) {
-                            const int tk = 32 * ks + 8 * j + e;  // token of the iteration
-                            vreg[ks].w[e] = *reinterpret_cast<const uint32_t *>(vb + (tk / Sh::V_GROUP_TOKENS) * Sh::V_GROUP_BYTES +
-                                                                                (tk % Sh::V_GROUP_TOKENS) * RB);
-                        }
-                    }
-                }
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ks++) {
                     if (uint32_t(ks) >= ksteps) break;
@@ -887,56 +741,9 @@ __device__ __forceinline__ void attention_partial_body(const PartialArgs &a) {
                 }
             }
         }
-        if (it + TEAMS < n_it) load_values(it + TEAMS);
+        if (it + 1 < n_it) load_values(it + 1);
     }
 
-    if constexpr (TEAMS > 1) {
-        // ---- epilogue with teams: every team finishes its own (m, l, O), team 1 hands its to team 0
-        // through LDS (the key slots are free by now), team 0 merges and writes the partial.
-        static_assert(TEAMS == 1 || (TILES == 1 && PACKED && QUANT), "teams: one row over codes");
-        l_part = group_reduce<Sh::TPR>(l_part, SumOp());
-        float *x_ml = reinterpret_cast<float *>(lds_raw + K_OFF);             // [team][m of 8 heads, l of 8 heads]
-        floatx4 *x_o = reinterpret_cast<floatx4 *>(lds_raw + K_OFF + 1024);  // [thread][4 rows]
-        if (b_part == 0) x_ml[team * 16 + b_row] = m_run, x_ml[team * 16 + 8 + b_row] = l_part;
-        {
-            const float z = across_rows<16, 64>(zacc[0], SumOp());
-            if (j == 0 && n < 8) zsum_lds[wave * Sh::S_ROWS + n] = z;
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-        }
-        constexpr float unscale = code_up<BITS>() / P_UP;
-        floatx4 mine[4];  // head 4j + i (j < 2), dims 64 wave + 4n .. + 3
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const float zb = zsum_lds[wave * Sh::S_ROWS + ((4 * j + i) & 7)] * (1.0f / P_UP);
-#pragma unroll
-            for (int e = 0; e < 4; e++) mine[i][e] = across_rows<32, 64>(acc[0][e][i], SumOp()) * unscale + zb;
-        }
-        if (team == 1 && j < 2) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) x_o[tid * 4 + i] = mine[i];
-        }
-        __syncthreads();
-        if (team != 0) return;
-        if (b_part == 0) {
-            const float m0 = x_ml[b_row], m1 = x_ml[16 + b_row], mm = fmaxf(m0, m1);
-            const float l = x_ml[8 + b_row] * __builtin_amdgcn_exp2f(m0 - mm) + x_ml[24 + b_row] * __builtin_amdgcn_exp2f(m1 - mm);
-            const size_t slot = size_t(split) * a.heads + kv * 8 + b_row;
-            *reinterpret_cast<floatx2 *>(a.part_ml + 2 * slot) = floatx2{mm, l};
-        }
-        if (j < 2) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int head = 4 * j + i;
-                const float m0 = x_ml[head], m1 = x_ml[16 + head], mm = fmaxf(m0, m1);
-                const float f0 = __builtin_amdgcn_exp2f(m0 - mm), f1 = __builtin_amdgcn_exp2f(m1 - mm);
-                const floatx4 other = x_o[tid * 4 + i];
-                const size_t slot = size_t(split) * a.heads + kv * 8 + head;
-                *reinterpret_cast<floatx4 *>(a.part_o + slot * DIM + 64 * wave + 4 * n) = mine[i] * f0 + other * f1;
-            }
-        }
-        return;
-    }
     // ---- epilogue: one partial per (row, head) ------------------------------------
     // m and l from the phase B threads.
     l_part = group_reduce<Sh::TPR>(l_part, SumOp());
@@ -1013,13 +820,6 @@ __global__ __launch_bounds__(THREADS) void attention_partial_kernel_n(PartialArg
     attention_partial_body<BITS, TILES, false, itb_rows<TILES>(), TILES == 1>(a);
 }
 
-// One query row over codes with loader waves: two teams of 4 computing waves + 4 loading waves.
-constexpr int ITB_DMA = 4, TEAMS_DMA = 2;
-template <int BITS>
-__global__ __launch_bounds__((TEAMS_DMA + 1) * THREADS) void attention_partial_kernel_d(PartialArgs a) {
-    attention_partial_body<BITS, 1, true, ITB_DMA, true, true, TEAMS_DMA>(a);
-}
-
 template <int BITS>
 __global__ __launch_bounds__(THREADS) void attention_partial_kernel_p(PartialArgs a) {
     attention_partial_body<BITS, 1, true, ITB_ONE_PER_CU, true>(a);
@@ -1073,6 +873,15 @@ struct KeysFirst {
     static constexpr int K_LOADERS = 2, V_LOADERS = 2;
     static constexpr int RB_ = BITS * 32;                   // bytes of a (token, kv head) row of codes
     static constexpr int ROUND_BLOCKS = 17, ROUND_TOKENS = ROUND_BLOCKS * BLOCK;
+    // One row, a share of more than one round: rounds of ALT_BLOCKS blocks that ALTERNATE between two halves of the
+    // keys' and the values' places (and of the scales and the block table), so that the loaders are a round ahead of
+    // the computing waves and the stream from memory never waits for them.  The halves are the blocks 0-7 and 8-15 of
+    // the single round's places.  (Rounds of 16 blocks for 4-bit codes, which are half the bytes, in places of 32
+    // blocks: measured slower, 30.0 against 28.3 us at 150k tokens; the code below takes either.)
+    static constexpr bool ALTERNATE = M == 1;
+    static constexpr int ALT_BLOCKS = 8;
+    static constexpr int AREA_BLOCKS = (ALTERNATE && 2 * ALT_BLOCKS > ROUND_BLOCKS) ? 2 * ALT_BLOCKS : ROUND_BLOCKS;  // blocks of codes LDS has room for, keys and values each
+    static constexpr int SB_TOKENS = AREA_BLOCKS * BLOCK;
     static constexpr int KSTEPS = (ROUND_BLOCKS + 1) / 2;   // of 32 tokens; the last one is half there
     static constexpr int SLOTS = (KSTEPS + 1) / 2;          // value slots of 64 tokens: 5, the last one block 16 alone
     static constexpr int PIECES = RB_ / 16;
@@ -1094,17 +903,18 @@ struct KeysFirst {
     static constexpr int QZ_OFF = Q_OFF + 8 * 64 * 16;             // [hi, lo][lane][k-step] f16
     // scales and biases: per array two planes of one dword per token, the f16 of groups (0, 1) and of (2, 3)
     static constexpr int SB_OFF = QZ_OFF + 2 * 64 * 16;            // [ks | kz | vs | vz][plane][token] u32
-    static constexpr int SB_ARRAY = 2 * ROUND_TOKENS * 4;
+    static constexpr int SB_ARRAY = 2 * SB_TOKENS * 4;
     // the blocks' maxima and sums, [row][head][block]: one row has room for a stride of 20 (16-byte reads; blocks 17-19
     // never exist: maximum "none", sum 0), several rows have not
-    static constexpr int BSTRIDE = M == 1 ? 20 : ROUND_BLOCKS;
+    static constexpr int BSTRIDE = M == 1 ? (AREA_BLOCKS + 3) / 4 * 4 : ROUND_BLOCKS;
+    static constexpr int BSINGLE = (ROUND_BLOCKS + 3) / 4 * 4;      // entries of a row that a single round looks at (one row)
     static constexpr int BROW = 8 * BSTRIDE;                       // floats of a row's table
     static constexpr int BMAX_OFF = SB_OFF + 4 * SB_ARRAY;         // [row][head][block] f32: the block's maximum score
     static constexpr int BSUM_OFF = BMAX_OFF + M * BROW * 4;       // [row][head][block] f32: sum of 2^(score - maximum)
     static constexpr int ZS_OFF = BSUM_OFF + M * BROW * 4;         // [wave][pair][column] f32 (one row: [wave][head])
     static constexpr int SYNC_OFF = ZS_OFF + WAVES * PAIRS * 16 * 4;  // 32 counters, u32
     static constexpr int K_OFF = (SYNC_OFF + 32 * 4 + 255) / 256 * 256;
-    static constexpr int V_OFF = K_OFF + ROUND_BLOCKS * K_BLOCK_BYTES;
+    static constexpr int V_OFF = K_OFF + AREA_BLOCKS * K_BLOCK_BYTES;
     // Several rows over a share of more than one round: rounds of SHORT_BLOCKS blocks, which leave room in
     // LDS for every pair's query operands to stay ([pair][hi, lo][k-step][lane] half8, then [pair][hi, lo][lane][k-step]
     // f16 of the key bias term), so that they need no registers between one round's scores and the next's.
@@ -1112,10 +922,10 @@ struct KeysFirst {
     static constexpr int SHORT_BLOCKS = 8;
     static constexpr int QP_PAIR_BYTES = 2 * 8 * 64 * 16, QPZ_PAIR_BYTES = 2 * 64 * 16;
     static constexpr int QP_BYTES = M > 1 ? PAIRS * (QP_PAIR_BYTES + QPZ_PAIR_BYTES) : 0;
-    static constexpr int QP_OFF = BITS == 8 ? K_OFF + SHORT_BLOCKS * K_BLOCK_BYTES : V_OFF + ROUND_BLOCKS * K_BLOCK_BYTES;
+    static constexpr int QP_OFF = BITS == 8 ? K_OFF + SHORT_BLOCKS * K_BLOCK_BYTES : V_OFF + AREA_BLOCKS * K_BLOCK_BYTES;
     static constexpr int QPZ_OFF = QP_OFF + PAIRS * QP_PAIR_BYTES;
     static_assert(BITS != 8 || QP_OFF + QP_BYTES <= V_OFF, "the query operands fit behind the short rounds' keys");
-    static constexpr int LDS_BYTES = (BITS == 8 || M == 1) ? V_OFF + ROUND_BLOCKS * K_BLOCK_BYTES : QP_OFF + QP_BYTES;
+    static constexpr int LDS_BYTES = (BITS == 8 || M == 1) ? V_OFF + AREA_BLOCKS * K_BLOCK_BYTES : QP_OFF + QP_BYTES;
     // one row: the merge of two waves, [group][lane < 32][4 rows] of 16 bytes, lies over the query operands,
     // which nobody reads after the last scores
     static constexpr int X_OFF = Q_OFF;
@@ -1129,6 +939,7 @@ struct KeysFirst {
     static constexpr int C_BUILT = 3;   // ... built their probability operands (8 per round)
     static constexpr int C_DONE = 4;    // ... are through with the round's values (8 per round)
     static constexpr int C_LENGTH = 5;  // (not a counter: the context length or the position, for every wave)
+    static constexpr int C_VREQ = 6;    // alternating rounds: value loaders that have requested a round's values (2 per round)
     static constexpr int C_QREAD = 7;   // computing waves that have a row's query operands in registers (several rows)
     static constexpr int C_KPART = 8;   // [3]: key loaders whose blocks 0-7 and scales | blocks 8-15 | block 16 have landed (2 per round)
     static constexpr int C_SLOT = 12;   // [5]: value loaders whose values of slot s have landed (2 per round)
@@ -1140,7 +951,7 @@ struct KeysFirst {
 template <int BITS, int M>
 __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::WAVES) * 64) void attention_partial_kernel_s(PartialArgs a) {
     using W = KeysFirst<BITS, M>;
-    constexpr int RB = W::RB_, RT = W::ROUND_TOKENS, RBK = W::ROUND_BLOCKS;
+    constexpr int RB = W::RB_, RT = W::SB_TOKENS, RBK = W::ROUND_BLOCKS;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const int lane = threadIdx.x & 63;
     const int wave_all = __builtin_amdgcn_readfirstlane(int(threadIdx.x) >> 6);
@@ -1196,7 +1007,9 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
     const uint32_t range = blk_end - blk_begin;
     // rounds of equal size (to within a block), none longer than 17 blocks
     // (several rows: one round of up to 17 blocks, or rounds of up to 8)
-    const uint32_t n_rounds = (M > 1 && range > uint32_t(RBK)) ? (range + W::SHORT_BLOCKS - 1) / W::SHORT_BLOCKS : (range + RBK - 1) / RBK;
+    constexpr uint32_t LONG_ROUND = W::ALTERNATE ? W::ALT_BLOCKS : W::SHORT_BLOCKS;
+    const uint32_t n_rounds = range > uint32_t(RBK) ? (range + LONG_ROUND - 1) / LONG_ROUND : 1;
+    const bool alt = W::ALTERNATE && n_rounds > 1;  // rounds in alternate halves of LDS
     const uint32_t per_round = (range + n_rounds - 1) / n_rounds;
     auto blocks_of = [&](uint32_t round) { return min(range - round * per_round, per_round); };
 
@@ -1258,7 +1071,44 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
         // loader 0 then block 16 with its scales and biases ----
         const uint32_t L = uint32_t(wave_all);
         const void *sb_src[4] = {a.kscales, a.kbiases, a.vscales, a.vbiases};
-        for (uint32_t round = 0; round < n_rounds; round++) {
+        if constexpr (W::ALTERNATE) if (alt) {
+            // ---- rounds of up to 8 blocks in alternate halves of LDS: loader L takes the rounds L, L + 2, ... whole, so
+            // that two rounds' keys can be on their way at once.  A round goes out when the values of the round before
+            // have been requested (the stream keeps the order keys, values, keys, ...) and when the round before last,
+            // which lay in the same half, has been used up: its scales are read until every wave has built its operands,
+            // its keys until every wave has its scores. ----
+            for (uint32_t round = L; round < n_rounds; round += 2) {
+                const uint32_t base = (blk_begin + round * per_round) * BLOCK, nb = blocks_of(round);
+                const uint32_t half = L * W::ALT_BLOCKS;  // the blocks of LDS this round goes to start here
+                if (round > 1) await(W::C_BUILT, W::WAVES * (round - 1));
+                if (round > 0) await(W::C_VREQ, round);
+#pragma unroll
+                for (int h = 0; h < W::ALT_BLOCKS / 4; h++) {
+                    const uint32_t voff = (min(base + 64 * h + lane, last_tok) * kvh + kv) * 8;
+#pragma unroll
+                    for (int arr = 0; arr < 4; arr++) {
+#pragma unroll
+                        for (int pl = 0; pl < 2; pl++) dma4(lds0 + W::SB_OFF + arr * W::SB_ARRAY + (pl * RT + BLOCK * half + 64 * h) * 4, voff + 4 * pl, sb_src[arr]);
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < W::ALT_BLOCKS; r++) {
+                    if (uint32_t(r) < nb) {
+                        const uint32_t tok = min(base + BLOCK * r + (lane >> 2), last_tok);
+                        const uint32_t voff = (tok * kvh + kv) * RB + (lane & 3) * 16;
+#pragma unroll
+                        for (int i = 0; i < W::PER_BLOCK; i++) dma(lds0 + W::K_OFF + (half + r) * W::K_BLOCK_BYTES + i * 1024, voff + 64 * i, a.kdata);
+                    }
+                }
+                raise(W::C_KEYS);
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+                raise(W::C_KPART + 0);
+            }
+            leave();
+            return;
+        }
+        // (one row: more than one round is taken above)
+        for (uint32_t round = 0; round < (M == 1 ? 1u : n_rounds); round++) {
             const uint32_t base = (blk_begin + round * per_round) * BLOCK, nb = blocks_of(round);
             // the round before: its scales are read until every wave has built its operands, its keys until every wave has its scores
             if (round > 0) await(W::C_BUILT, W::WAVES * round);
@@ -1323,7 +1173,33 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
         // ---- a value-loader wave: blocks L, L + 2, ... of every round, two of them in each 64-token slot;
         // loader 0 then block 16 (slot 4) ----
         const uint32_t L = uint32_t(wave_all) - W::K_LOADERS;
-        for (uint32_t round = 0; round < n_rounds; round++) {
+        if constexpr (W::ALTERNATE) if (alt) {
+            // ---- alternate halves: loader L takes the values of the rounds L, L + 2, ... whole, each behind its round's
+            // keys in the stream, into the half that the round before last has left (every wave through with its values) ----
+            for (uint32_t round = L; round < n_rounds; round += 2) {
+                const uint32_t base = (blk_begin + round * per_round) * BLOCK, nb = blocks_of(round);
+                const uint32_t half = L * W::ALT_BLOCKS;
+                await(W::C_KEYS, round + 1);
+                if (round > 1) await(W::C_DONE, W::WAVES * (round - 1));
+#pragma unroll
+                for (int r = 0; r < W::ALT_BLOCKS; r++) {
+                    if (uint32_t(r) < nb) {
+#pragma unroll
+                        for (int i = 0; i < W::PER_BLOCK; i++) {
+                            const uint32_t t = BLOCK * r + W::V_GROUP_TOKENS * i + lane / W::PIECES;  // token of the round
+                            const uint32_t piece = (lane % W::PIECES + W::PIECES - ((t >> 3) & 3) * (W::PIECES / 4)) % W::PIECES;
+                            dma(lds0 + W::V_OFF + (W::PER_BLOCK * (half + r) + i) * 1024, (min(base + t, last_tok) * kvh + kv) * RB + piece * 16, a.vdata);
+                        }
+                    }
+                }
+                raise(W::C_VREQ);
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+                raise(W::C_SLOT + 4);
+            }
+            leave();
+            return;
+        }
+        for (uint32_t round = 0; round < (M == 1 ? 1u : n_rounds); round++) {
             const uint32_t base = (blk_begin + round * per_round) * BLOCK, nb = blocks_of(round);
             // the keys of the first round have been requested | every wave is through with the values before
             if (round == 0) {
@@ -1402,9 +1278,9 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
     auto round_max = [&](int r, float start) {
         const float *bmx = bmax_lds + r * W::BROW + (n & 7) * W::BSTRIDE;
         float v = start;
-        if constexpr (W::BSTRIDE % 4 == 0) {
+        if constexpr (M == 1) {
 #pragma unroll
-            for (int i = 0; i < W::BSTRIDE / 4; i++) {
+            for (int i = 0; i < W::BSINGLE / 4; i++) {
                 const floatx4 w = reinterpret_cast<const floatx4 *>(bmx)[i];
                 v = fmaxf(v, fmaxf(fmaxf(w[0], w[1]), fmaxf(w[2], w[3])));
             }
@@ -1417,11 +1293,11 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
     // a row's sum of P of head n & 7 over the round's blocks, relative to the maximum nm: lane group j adds blocks j, j + 4, ...
     auto round_sum = [&](int r, float nm) {
         float sum = 0.0f;
-        if constexpr (W::BSTRIDE % 4 == 0) {
+        if constexpr (M == 1) {
             // lane group j adds blocks 5j .. 5j + 4
 #pragma unroll
-            for (int i = 0; i < W::BSTRIDE / 4; i++) {
-                const int b = (W::BSTRIDE / 4) * j + i;
+            for (int i = 0; i < W::BSINGLE / 4; i++) {
+                const int b = (W::BSINGLE / 4) * j + i;
                 sum += bsum_lds[r * W::BROW + (n & 7) * W::BSTRIDE + b] * __builtin_amdgcn_exp2f(bmax_lds[r * W::BROW + (n & 7) * W::BSTRIDE + b] - nm);
             }
             return across_rows<16, 64>(sum, SumOp());
@@ -2042,8 +1918,8 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
             qz_lds[(0 * 64 + lane) * 8 + wave] = h;
             qz_lds[(1 * 64 + lane) * 8 + wave] = lw;
             // blocks that never exist
-            if (wave == 0 && lane < 8 * (W::BSTRIDE - RBK)) {
-                const int idx = (lane / (W::BSTRIDE - RBK)) * W::BSTRIDE + RBK + lane % (W::BSTRIDE - RBK);
+            if (wave == 0 && lane < 8 * (W::BSINGLE - RBK)) {
+                const int idx = (lane / (W::BSINGLE - RBK)) * W::BSTRIDE + RBK + lane % (W::BSINGLE - RBK);
                 bmax_lds[idx] = NO_SCORE, bsum_lds[idx] = 0.0f;
             }
         }
@@ -2058,9 +1934,206 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
         for (int e = 0; e < 4; e++) acc[e] = floatx4{0, 0, 0, 0};
         await(W::C_QUERY, W::WAVES);
 
-        for (uint32_t round = 0; round < n_rounds; round++) {
+        if constexpr (W::ALTERNATE) if (alt) {
+            // ---- a share of more than one round: rounds of up to ALT_BLOCKS blocks in alternate halves of LDS ----
+            // Round r lies in the blocks ALT_BLOCKS (r % 2) .. of the keys' and the values' places, of the scales and of
+            // the block table: every computing wave takes the scores of one block (4-bit codes: two) and two k-steps (four)
+            // of O += P V per round, and the loaders fill the other half meanwhile.  A half is free for round r + 2 when
+            // every wave has built its operands (keys, scales, scores) and is through with the values of round r.
+            constexpr int AB = W::ALT_BLOCKS, WAVE_BLOCKS = AB / W::WAVES, WAVE_STEPS = AB / 4;
+#pragma unroll 1
+            for (uint32_t round = 0; round < n_rounds; round++) {
+                const uint32_t base = (blk_begin + round * per_round) * BLOCK, nb = blocks_of(round);
+                const int half = int(round & 1) * AB;  // the round's first block in LDS
+                const uint32_t round_limit = min(limit, base + nb * BLOCK);  // tokens of this round end here
+                const uint32_t live_blocks = (nb + 1) & ~1u;  // k-steps are two blocks: the blocks of the k-steps that have tokens
+                // ---- phase A: the scores of the blocks wave (, wave + 8) of the round ----
+#pragma unroll 1
+                for (int part = 0; part < WAVE_BLOCKS; part++) {
+                    const int rblk = wave + W::WAVES * part;  // of the round
+                    const int blk = half + rblk;              // in LDS
+                    if (uint32_t(rblk) >= live_blocks) {
+                        // (no scores to take, and no operands will be made of this block; the table still holds the entries of
+                        // the round before last until every wave has built its operands from them)
+                        if (round > 1) await(W::C_BUILT, W::WAVES * (round - 1));
+                        if (j == 0 && n < 8) bmax_lds[n * W::BSTRIDE + blk] = NO_SCORE, bsum_lds[n * W::BSTRIDE + blk] = 0.0f;
+                    } else {
+                        half8 q_reg[8], qz_reg[2];
+#pragma unroll
+                        for (int i = 0; i < 8; i++) q_reg[i] = q_lds[i * 64 + lane];
+                        qz_reg[0] = *reinterpret_cast<const half8 *>(qz_lds + lane * 8);
+                        qz_reg[1] = *reinterpret_cast<const half8 *>(qz_lds + (64 + lane) * 8);
+                        await(W::C_KPART + 0, round + 1);  // the round's keys and scales are in LDS (one loader per round)
+                        const unsigned char *kb = lds_raw + W::K_OFF + blk * W::K_BLOCK_BYTES;
+                        KeyRegs<BITS> kreg[4];
+#pragma unroll
+                        for (int gg = 0; gg < 4; gg++) {
+                            if constexpr (BITS == 8) {
+                                const u32x4 v = *reinterpret_cast<const u32x4 *>(kb + gg * 1024 + n * 64 + j * 16);
+                                kreg[gg].w[0] = v.x, kreg[gg].w[1] = v.y, kreg[gg].w[2] = v.z, kreg[gg].w[3] = v.w;
+                            } else {
+                                const u32x2 v = *reinterpret_cast<const u32x2 *>(kb + (gg >> 1) * 1024 + n * 64 + (gg & 1) * 32 + j * 8);
+                                kreg[gg].w[0] = v.x, kreg[gg].w[1] = v.y;
+                            }
+                        }
+                        const int tok0 = BLOCK * rblk + 4 * j;  // this lane's 4 tokens of the round in C layout
+                        const uint32_t *sb_w = sb_lds + BLOCK * blk;  // the block's dwords of groups (0, 1); + RT: groups (2, 3)
+                        floatx4 sc;
+                        {
+                            const u32x2 zr = {sb_w[W::SB_ARRAY / 4 + n], sb_w[W::SB_ARRAY / 4 + RT + n]};
+                            const half8 zop = as_half8(perm(0, zr.x, 0x01000100u), perm(0, zr.x, 0x03020302u), perm(0, zr.y, 0x01000100u),
+                                                       perm(0, zr.y, 0x03020302u));
+                            sc = floatx4{0, 0, 0, 0};
+                            sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz_reg[0], sc, 0, 0, 0);
+                            sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(zop, qz_reg[1], sc, 0, 0, 0);
+                        }
+                        floatx4 r[4];
+#pragma unroll
+                        for (int gg = 0; gg < 4; gg++) {
+                            r[gg] = floatx4{0, 0, 0, 0};
+#pragma unroll
+                            for (int ab = 0; ab < 2; ab++) {
+                                r[gg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(key_operand<BITS>(kreg[gg], ab), q_reg[gg * 2 + ab], r[gg], 0, 0, 0);
+                            }
+                        }
+                        const u32x4 s01 = *reinterpret_cast<const u32x4 *>(sb_w + 4 * j);
+                        const u32x4 s23 = *reinterpret_cast<const u32x4 *>(sb_w + RT + 4 * j);
+                        const uint32_t sw[8] = {s01.x, s23.x, s01.y, s23.y, s01.z, s23.z, s01.w, s23.w};
+                        constexpr float C1 = code_up<BITS>() / Q_UP;
+#pragma unroll
+                        for (int tk = 0; tk < 4; tk++) {
+                            float d = 0.0f;
+#pragma unroll
+                            for (int gg = 0; gg < 4; gg++) d += half_bits_to_float(sw[2 * tk + (gg >> 1)] >> (16 * (gg & 1))) * r[gg][tk];
+                            float v = sc[tk] + d * C1;
+                            v += dpp<0x128>(v);  // row_ror 8: the other part (hi | lo) of the same head
+                            sc[tk] = base + tok0 + tk < round_limit ? v : NO_SCORE;  // (also whatever a block past the round left in LDS)
+                        }
+                        float cm = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+                        cm = across_rows<16, 64>(cm, MaxOp());
+                        float sum = 0.0f;
+#pragma unroll
+                        for (int tk = 0; tk < 4; tk++) {
+                            sc[tk] = sc[tk] > 0.5f * NO_SCORE ? __builtin_amdgcn_exp2f(sc[tk] - cm) : 0.0f;
+                            sum += sc[tk];
+                        }
+                        sum = across_rows<16, 64>(sum, SumOp());
+                        // over the block's own keys (every lane of the wave has its key registers by now)
+                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                        if (n < 8) *reinterpret_cast<floatx4 *>(s_block(blk, 0) + n * BLOCK + 4 * j) = sc;
+                        if (j == 0 && n < 8) bmax_lds[n * W::BSTRIDE + blk] = cm, bsum_lds[n * W::BSTRIDE + blk] = sum;
+                    }
+                }
+                raise(W::C_SCORES);
+                await(W::C_SCORES, W::WAVES * (round + 1));
+
+                // ---- the round's maximum per head, and what was summed so far brought to it ----
+                float nm = m_run;
+                {
+                    const floatx4 *bmx = reinterpret_cast<const floatx4 *>(bmax_lds + (n & 7) * W::BSTRIDE + half);
+#pragma unroll
+                    for (int i = 0; i < AB / 4; i++) {
+                        const floatx4 w = bmx[i];
+                        nm = fmaxf(nm, fmaxf(fmaxf(w[0], w[1]), fmaxf(w[2], w[3])));
+                    }
+                }
+                const float al = __builtin_amdgcn_exp2f(m_run - nm);  // (first round: 2^(-1e30 - nm) = 0, and nothing to scale)
+                if (round > 0) {
+                    zacc *= al;
+                    floatx4 al4;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        al4[i] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(4 * ((4 * j + i) & 7), __builtin_bit_cast(int, al)));
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[e] *= al4;
+                }
+                m_run = nm;
+                if (wave == 0) {
+                    // the round's sum of P of head n & 7: lane group j adds the blocks (AB / 4) j ..
+                    float sum = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < AB / 4; i++) {
+                        const int b = half + (AB / 4) * j + i;
+                        sum += bsum_lds[(n & 7) * W::BSTRIDE + b] * __builtin_amdgcn_exp2f(bmax_lds[(n & 7) * W::BSTRIDE + b] - nm);  // (a block that is not there: sum 0)
+                    }
+                    l_run = l_run * al + across_rows<16, 64>(sum, SumOp());
+                }
+
+                // ---- probability operands of this wave's k-steps (as in a single round) ----
+                half8 p_alt[WAVE_STEPS];
+                {
+                    const int hh = n >> 3;  // this lane makes tokens 8j + 4 hh .. + 3 of a k-step
+                    const int sh = 16 * (g & 1);
+#pragma unroll
+                    for (int i = 0; i < WAVE_STEPS; i++) {
+                        if (uint32_t(2 * (2 * i + b2)) >= nb) {  // the k-step has no tokens
+                            p_alt[i] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+                            continue;
+                        }
+                        const int ks = half / 2 + 2 * i + b2;  // in LDS: tokens 32 ks ..: blocks 2 ks and 2 ks + 1
+                        const int blk = 2 * ks + (j >> 1);
+                        const floatx4 pt = *reinterpret_cast<const floatx4 *>(s_block(blk, 0) + (n & 7) * BLOCK + 8 * (j & 1) + 4 * hh);
+                        const uint32_t *vsp = sb_lds + 2 * (W::SB_ARRAY / 4) + (g >> 1) * RT + 32 * ks + 8 * j + 4 * hh;
+                        const u32x4 sv = *reinterpret_cast<const u32x4 *>(vsp);
+                        const u32x4 zv = *reinterpret_cast<const u32x4 *>(vsp + W::SB_ARRAY / 4);
+                        // 2^(block maximum - maximum so far) * P_UP (2^8, so that the lo part stays a normal f16)
+                        const float f = __builtin_amdgcn_exp2f(bmax_lds[(n & 7) * W::BSTRIDE + blk] - nm + 8.0f);
+                        const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w}, zw[4] = {zv.x, zv.y, zv.z, zv.w};
+                        float x[4], lo[4];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const float p = pt[e] * f;
+                            zacc += p * half_bits_to_float(zw[e] >> sh);
+                            x[e] = p * half_bits_to_float(sw[e] >> sh);
+                            lo[e] = x[e] - __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x[e]) & 0xffffe000u);
+                        }
+                        // round toward zero: exact truncation to the hi part
+                        const uint32_t hi0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x[0], x[1]));
+                        const uint32_t hi1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x[2], x[3]));
+                        const uint32_t lo0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo[0], lo[1]));
+                        const uint32_t lo1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo[2], lo[3]));
+                        const uint32_t send0 = hh ? hi0 : lo0, send1 = hh ? hi1 : lo1;
+                        const uint32_t recv0 = uint32_t(__builtin_amdgcn_update_dpp(0, int(send0), 0x128, 0xf, 0xf, false));  // row_ror 8
+                        const uint32_t recv1 = uint32_t(__builtin_amdgcn_update_dpp(0, int(send1), 0x128, 0xf, 0xf, false));
+                        uint32_t o[4] = {hh ? recv0 : hi0, hh ? recv1 : hi1, hh ? lo0 : recv0, hh ? lo1 : recv1};
+                        asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]));
+                        p_alt[i] = as_half8(o[0], o[1], o[2], o[3]);
+                    }
+                }
+                raise(W::C_BUILT);  // this wave is through with the round's keys, scores, scales and biases
+
+                // ---- phase C: O += P V of the wave's k-steps ----
+                await(W::C_SLOT + 4, round + 1);  // the round's values are in LDS (one loader per round)
+                {
+                    ValRegs<BITS> vreg[WAVE_STEPS];
+#pragma unroll
+                    for (int i = 0; i < WAVE_STEPS; i++) {
+                        if (uint32_t(2 * (2 * i + b2)) >= nb) continue;
+#pragma unroll
+                        for (int e = 0; e < 8; e++) {
+                            const int tk = BLOCK * half + 32 * (2 * i + b2) + 8 * j + e;
+                            vreg[i].w[e] = *reinterpret_cast<const uint32_t *>(lds_raw + W::V_OFF + tk * RB + ((val_lane_offset<BITS>(g, n) + j * (RB / 4)) & (RB - 1)));
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < WAVE_STEPS; i++) {
+                        if (uint32_t(2 * (2 * i + b2)) >= nb) continue;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p_alt[i], val_operand<BITS>(vreg[i], e, n), acc[e], 0, 0, 0);
+                        }
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the value codes are in registers
+                raise(W::C_DONE);
+            }
+        }
+        if (!alt) {
+            // ---- a share of up to 17 blocks: one round ----
+            constexpr uint32_t round = 0;  // (written as the first of several rounds)
+            constexpr bool more = false;
             const uint32_t base = (blk_begin + round * per_round) * BLOCK, nb = blocks_of(round);
-            const bool more = round + 1 < n_rounds;
             const bool extra = nb == uint32_t(RBK);  // the round has block 16
             const uint32_t round_limit = min(limit, base + nb * BLOCK);  // tokens of this round end here
             const uint32_t live_blocks = (nb + 1) & ~1u;  // k-steps are two blocks: the blocks of the k-steps that have tokens
@@ -2165,7 +2238,7 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
             {
                 const floatx4 *bmx = reinterpret_cast<const floatx4 *>(bmax_lds + (n & 7) * W::BSTRIDE);
 #pragma unroll
-                for (int i = 0; i < W::BSTRIDE / 4; i++) {
+                for (int i = 0; i < W::BSINGLE / 4; i++) {
                     const floatx4 w = bmx[i];
                     nm = fmaxf(nm, fmaxf(fmaxf(w[0], w[1]), fmaxf(w[2], w[3])));
                 }
@@ -2187,8 +2260,8 @@ __global__ __launch_bounds__((KeysFirst<BITS, M>::LOADERS + KeysFirst<BITS, M>::
                 // the round's sum of P of head n & 7: lane group j adds blocks 5j .. 5j + 4
                 float sum = 0.0f;
 #pragma unroll
-                for (int i = 0; i < W::BSTRIDE / 4; i++) {
-                    const int b = (W::BSTRIDE / 4) * j + i;
+                for (int i = 0; i < W::BSINGLE / 4; i++) {
+                    const int b = (W::BSINGLE / 4) * j + i;
                     sum += bsum_lds[(n & 7) * W::BSTRIDE + b] * __builtin_amdgcn_exp2f(bmax_lds[(n & 7) * W::BSTRIDE + b] - nm);  // (a block that is not there: sum 0)
                 }
                 l_run = l_run * al + across_rows<16, 64>(sum, SumOp());
@@ -2452,19 +2525,15 @@ uint32_t splits_for(uint32_t capacity, uint32_t wanted) {
     return s ? s : 1;
 }
 
-// One row over 8-bit codes: from this capacity on the kernel with loader waves is the faster one
-// (measured, per layer with the merge: 10.0 against 11.0 us at 4k tokens, equal at 32k, 20.9
-// against 22.3 at 50k, 35.5 against 36.5 at 131k).
-constexpr uint32_t LOADERS_FROM = 24 * 1024;
-// 4-bit codes: the same kernel from the same capacity (15.0 against 16.8 us at 32k, 29.5 against 31.6
-// at 131k), up to where the two-workgroups-per-CU kernel streams faster than the loader kernel's
-// two teams get through their iterations (29.1 against 28.5 us at 150k, 40.9 against 39.3 at 200k).
-constexpr uint32_t LOADERS_4BIT_UP_TO = 136 * 1024;
-// Which of the two: see run_attention.
-constexpr uint32_t KEYS_FIRST_ONE_ROUND = 17 * BLOCK * (MAX_SPLITS / 2), KEYS_FIRST_AGAIN_FROM = 60000, KEYS_FIRST_4BIT_UP_TO = 100 * 1024;
+// One to four rows over codes: from this capacity on the kernel whose loader waves keep a workgroup's share in
+// LDS, the keys first, is the faster one at every length (one row, 8-bit, against the register kernels: 10.0
+// against 11.0 us per layer at 4k tokens, 10.1 against 12.5 at 32k, 29.7 against 31.1 at 131k; shares of more
+// than one round in alternate halves of LDS: 13.4 against 14.1 us at 40k for the ring of four 64-token slots
+// that served there before, 28.3 against 29.7 at 150k, 4-bit, for the two-workgroups-per-CU kernel).
+constexpr uint32_t KEYS_FIRST_FROM = 24 * 1024;
 
 template <int BITS, int TILES, bool PACKED>
-void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu, bool loaders, bool keys_first) {
+void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu, bool keys_first) {
     void (*kernel)(PartialArgs);
     int lds_bytes;
     if constexpr (BITS != 16) {
@@ -2478,13 +2547,6 @@ void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu, b
             else if (a.rows == 2) launch(std::integral_constant<int, 2>());
             else if (a.rows == 3) launch(std::integral_constant<int, 3>());
             else launch(std::integral_constant<int, 4>());
-            return;
-        }
-    }
-    if constexpr (TILES == 1 && BITS != 16 && PACKED) {
-        if (loaders) {
-            attention_partial_kernel_d<BITS><<<dim3(a.nsplits, a.kv_heads), (TEAMS_DMA + 1) * THREADS,
-                                               Shape<BITS, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA), stream>>>(a);
             return;
         }
     }
@@ -2508,15 +2570,15 @@ void launch_partial(hipStream_t stream, const PartialArgs &a, bool one_per_cu, b
 }
 
 template <int BITS>
-void launch_partial_rows(hipStream_t stream, const PartialArgs &a, bool one_per_cu, bool loaders, bool keys_first) {
+void launch_partial_rows(hipStream_t stream, const PartialArgs &a, bool one_per_cu, bool keys_first) {
     if (a.rows == 1) {
-        launch_partial<BITS, 1, true>(stream, a, one_per_cu, loaders, keys_first);
+        launch_partial<BITS, 1, true>(stream, a, one_per_cu, keys_first);
     } else if (a.rows == 2) {
-        launch_partial<BITS, 1, false>(stream, a, one_per_cu, loaders, keys_first);
+        launch_partial<BITS, 1, false>(stream, a, one_per_cu, keys_first);
     } else if (a.rows <= 4) {
-        launch_partial<BITS, 2, false>(stream, a, one_per_cu, loaders, keys_first);
+        launch_partial<BITS, 2, false>(stream, a, one_per_cu, keys_first);
     } else {
-        launch_partial<BITS, 4, false>(stream, a, one_per_cu, loaders, keys_first);
+        launch_partial<BITS, 4, false>(stream, a, one_per_cu, keys_first);
     }
 }
 
@@ -2545,40 +2607,28 @@ int run_attention(hipStream_t stream, int bits, const float *q, const void *kdat
                    SAETTA_E_ALIGN, "%s: scales and biases must be 8-byte aligned", what);
     if (int rc = ensure_device()) return rc;
     uint32_t nsplits = splits_for(capacity, wanted_splits);
-    // One workgroup per CU (half as many splits, each twice as long) or two.  Two rows and more and a
-    // half cache need the whole register file anyway; one row over codes fits two workgroups per CU,
-    // which pays only for long contexts: up to 64k tokens the shorter merge of half as many partials
-    // is worth more (measured: 19.4 against 20.6 us per layer at 32k, 28.3 against 29.7 at 64k,
-    // but 44 against 35 at 146k, 4-bit).  Both stages derive the same number from the same arguments.
-    // One row over codes in a cache of 24k tokens and more (4-bit: up to 136k) goes to the kernel with
-    // loader waves, which is a one-workgroup-per-CU kernel at every length.
-    // SAETTA_STAGE_NO_LOADERS keeps to the register kernels (the caller's choice of kernel family,
-    // as DecodeAttention.kernel is in the reference, src/attention.rs:36-38).
-    const bool loaders = rows == 1 && bits != 16 && capacity >= LOADERS_FROM && (bits == 8 || capacity <= LOADERS_4BIT_UP_TO) &&
-                         !(stages & SAETTA_STAGE_NO_LOADERS);
-    const bool one_per_cu = rows >= 2 || bits == 16 || capacity <= 80 * 1024 || loaders;
-    // Of the two kernels with loader waves, the one that takes the keys first wins wherever a share
-    // is one round (up to 17 blocks of 16 tokens per split: 10.1 against 12.5 us at 32k tokens, 8-bit;
-    // 10.2 against 11.7, 4-bit) and again from about four rounds on (17.1 against 18.6 us at 64k, 29.7
-    // against 31.1 at 131k, 8-bit); with two or three short rounds the ring of slots is ahead (14.1
-    // against 15.6 us at 40k), and so it is for 4-bit codes above 100k tokens (28.0 against 29.3 at 131k).
-    // Two to four rows over codes (a verify step) run the same kernel, the codes in LDS serving every
-    // row: one round where the context in use gives shares of up to 17 blocks (the kernel sees the
-    // length when it runs; a verify step at 32k tokens is one round in a cache of any size), rounds
-    // of 8 blocks beyond.
-    const bool rows_keys_first = rows >= 2 && rows <= 4 && bits != 16 && capacity >= LOADERS_FROM && !(stages & SAETTA_STAGE_NO_LOADERS);
-    const bool keys_first = rows_keys_first || (loaders && (capacity <= KEYS_FIRST_ONE_ROUND || (capacity >= KEYS_FIRST_AGAIN_FROM &&
-                                                                               (bits == 8 || capacity <= KEYS_FIRST_4BIT_UP_TO))));
+    // One to four rows over codes in a cache of 24k tokens and more go to the kernel with loader waves, a
+    // one-workgroup-per-CU kernel at every length: a share of up to 17 blocks (the kernel sees the length
+    // when it runs: a step at 32k tokens is one round in a cache of any size) is one round, a longer one
+    // rounds of 8 blocks.  SAETTA_STAGE_NO_LOADERS keeps to the register kernels (the caller's choice of
+    // kernel family, as DecodeAttention.kernel is in the reference, src/attention.rs:36-38).
+    // The register kernels: one workgroup per CU (half as many splits, each twice as long) or two.  Two
+    // rows and more and a half cache need the whole register file anyway; one row over codes fits two
+    // workgroups per CU, which pays only for long contexts: up to 64k tokens the shorter merge of half as
+    // many partials is worth more (measured: 19.4 against 20.6 us per layer at 32k, 28.3 against 29.7 at
+    // 64k, but 44 against 35 at 146k, 4-bit).  Both stages derive the same number from the same arguments.
+    const bool keys_first = rows <= 4 && bits != 16 && capacity >= KEYS_FIRST_FROM && !(stages & SAETTA_STAGE_NO_LOADERS);
+    const bool one_per_cu = rows >= 2 || bits == 16 || capacity <= 80 * 1024 || keys_first;
     if (one_per_cu && nsplits > MAX_SPLITS / 2) nsplits = MAX_SPLITS / 2;
     if (stages & SAETTA_STAGE_PARTIAL) {
         PartialArgs a{q,     kdata,    vdata,    ks,    kz,   vs,      vz,   part_o, part_ml,
                       heads, kv_heads, capacity, scale, rows, nsplits, d_tp, decode_len ? 1u : 0u, device_status_word()};
         if (bits == 8) {
-            launch_partial_rows<8>(stream, a, one_per_cu, loaders, keys_first);
+            launch_partial_rows<8>(stream, a, one_per_cu, keys_first);
         } else if (bits == 4) {
-            launch_partial_rows<4>(stream, a, one_per_cu, loaders, keys_first);
+            launch_partial_rows<4>(stream, a, one_per_cu, keys_first);
         } else {
-            launch_partial_rows<16>(stream, a, one_per_cu, loaders, keys_first);
+            launch_partial_rows<16>(stream, a, one_per_cu, keys_first);
         }
     }
     if (stages & SAETTA_STAGE_REDUCE) {
@@ -2622,17 +2672,6 @@ int setup_decode() {
         float *ptr = nullptr;
         if (hipError_t e = hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch))) return int(e);
         g_static_scratch[dev] = ptr;
-    }
-    static_assert(Shape<8, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA) <= 160 * 1024, "LDS of a CU");
-    if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_partial_kernel_d<8>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         Shape<8, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA)))) {
-        return rc;
-    }
-    if (int rc = int(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_partial_kernel_d<4>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         Shape<4, 1, true, ITB_DMA>::dma_lds_bytes(TEAMS_DMA)))) {
-        return rc;
     }
     if (int rc = raise_lds_keys_first<8, 1>()) return rc;
     if (int rc = raise_lds_keys_first<8, 2>()) return rc;
