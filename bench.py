@@ -91,10 +91,14 @@ def make_decode_workload(s, torch, ctx, bits, rows, layers, seed=1234):
     return kind, capacity, caches, q, qg, out
 
 
-def bench_decode(s, torch, args, ctx, bits, rows, layers):
+def bench_decode(s, torch, args, ctx, bits, rows, layers, compact=False, workload=None):
+    """compact: a short record for the default line's "other_workloads": no CPU timing loops (one oracle
+    run on all cores for the parity figure), no reader floor.  workload: caches made before (with room for
+    `rows` rows), for the records that share them."""
     import oracle  # only for the CPU-baseline leg below
 
-    kind, capacity, caches, q, qg, out = make_decode_workload(s, torch, ctx, bits, rows, layers)
+    kind, capacity, caches, q, qg, out = workload or make_decode_workload(s, torch, ctx, bits, rows, layers)
+    q, qg, out = q[:rows], qg[:rows], out[:rows]
     plan = s.Plan()
     half = bits == 16
     if rows == 1:
@@ -170,8 +174,12 @@ def bench_decode(s, torch, args, ctx, bits, rows, layers):
             spent += ts[-1]
         return median(ts), ref
 
-    cpu1, ref = cpu_time(1, 8.0)
-    cpun, _ = cpu_time(threads_all, 4.0)
+    if compact:
+        cpu1 = cpun = None
+        ref = oracle.attend(qh, kf, vf, n_tok, q_and_gate=qgh, threads=threads_all)
+    else:
+        cpu1, ref = cpu_time(1, 8.0)
+        cpun, _ = cpu_time(threads_all, 4.0)
     # The GPU's answer for the same layer, checked against the oracle while we are here.
     check = s.Plan()
     if rows == 1:
@@ -198,13 +206,18 @@ def bench_decode(s, torch, args, ctx, bits, rows, layers):
                 s.ffi.lib().saetta_kv_quantize(st, bits, ctypes.c_void_p(x_new.data_ptr()), c, p, None, ctx), "kv_quantize"))
     append_us = kernel_us(append.build(graph))[0] if not half else 0.0
 
+    name = f"decode attention, {bits}-bit KV, ctx {ctx}, {rows} query row(s), {layers} layer caches per step"
+    if compact:
+        return {"metric": f"decode attn HBM GB/s @{ctx // 1024}k ctx {bits}-bit KV, {rows} row(s)", "value": round(value, 1),
+                "unit": "GB/s", "ms_per_step": round(ms_per_step, 4), "config": {"workload": name},
+                "append_4_tokens_k_and_v_us_per_layer": None if half else round(append_us, 3),
+                "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": round(achieved / HBM_PEAK_GBS, 4), "kernel": "attention_partial_kernel",
+                             "avg_us": round(part_us, 3), "reduce_kernel_us": round(red_us, 3)},
+                "parity_rel_rms_vs_oracle": float(f"{rel_rms:.3e}")}
     # The floor of a launch of this size: a plain read of the same bytes by 256 workgroups.
-    del caches, k0, v0
-    torch.cuda.empty_cache()
     reader, empty_us = reader_floor(s, torch, args, layer_bytes, layers) if not args.no_reader_floor else ({}, None)
     reader_us = min(reader.values()) if reader else None
-
-    name = f"decode attention, {bits}-bit KV, ctx {ctx}, {rows} query row(s), {layers} layer caches per step"
     res = {
         "metric": f"decode attn HBM GB/s @{ctx // 1024}k ctx {bits}-bit KV",
         "value": round(value, 1),
@@ -736,14 +749,32 @@ def main():
 
     if args.workload in ("default", "all"):
         # Both halves of the metric in one line: the decode record at the top level, the
-        # prefill-chunk record (same keys) under "prefill".
-        res = one("decode8_32k")
+        # prefill-chunk record (same keys) under "prefill"; then short records of the other
+        # configurations: the verify step of 2, 3 and 4 rows over the same caches, 4-bit decode at
+        # 150000 tokens with the 4-token append, the half cache at 4096 tokens, the Gated DeltaNet
+        # decode step and prefill chunk.
+        layers = args.layers or 32
+        shared = make_decode_workload(s, torch, args.ctx or 32768, 8, 4, layers)
+        res = bench_decode(s, torch, args, args.ctx or 32768, 8, 1, layers, workload=shared)
         res["metric"] = "decode attn HBM GB/s @32k ctx 8-bit KV; prefill-chunk attn TFLOP/s"
+        other = {}
+        for m in (2, 3, 4):
+            other[f"verify{m}"] = bench_decode(s, torch, args, args.ctx or 32768, 8, m, layers, compact=True, workload=shared)
+        del shared
         torch.cuda.empty_cache()
         res["prefill"] = one("prefill")
+        torch.cuda.empty_cache()
+        other["decode4_150k"] = bench_decode(s, torch, args, 150000, 4, 1, 12, compact=True)
+        torch.cuda.empty_cache()
+        other["decode16_4k"] = bench_decode(s, torch, args, 4096, 16, 1, 32, compact=True)
+        for w in ["deltanet", "deltanet_prefill"]:
+            torch.cuda.empty_cache()
+            r = one(w)
+            other[w] = {k: r[k] for k in ("metric", "value", "unit", "ms_per_step", "roofline", "parity_rel_rms_vs_oracle")}
+            other[w]["config"] = {"workload": r["config"]["workload"]}
+        res["other_workloads"] = other
     if args.workload == "all":
-        res["other_workloads"] = {}
-        for w in ["verify2", "verify3", "verify4", "decode4_150k", "decode16_4k", "prefill_131k", "prefill_gemm", "prefill_gemm_131k", "deltanet", "deltanet_prefill", "prep_store"]:
+        for w in ["prefill_131k", "prefill_gemm", "prefill_gemm_131k", "prep_store"]:
             torch.cuda.empty_cache()
             r = one(w)
             res["other_workloads"][w] = {k: r[k] for k in ("metric", "value", "unit", "ms_per_step", "roofline",

@@ -354,22 +354,20 @@ def test_several_rows_with_fewer_splits(splits):
 @pytest.mark.parametrize("capacity", [81920, 49152, 34816])
 @pytest.mark.parametrize("kind", [saetta.KvBits.Eight, saetta.KvBits.Four])
 def test_large_cache_of_codes_one_row(kind, capacity):
-    # One row over codes in a cache of 24k tokens and more runs one of the two kernels whose extra
-    # waves move the codes into LDS.  Capacity 49152: the ring of four 64-token slots with two teams
-    # of computing waves on alternate iterations.  Lengths: less than one block; one team idle; both
-    # teams, even and odd numbers of iterations; more iterations than slots (the slots are refilled);
-    # the whole capacity.  Capacities 81920 and 34816: the kernel that takes a share in rounds of up to
-    # 17 blocks with the keys requested first.  Lengths: a single block; rounds of fewer than 16
-    # blocks; shares of 16 and of 17 blocks side by side (33000 tokens, and the whole of 34816: every
-    # share has block 16); two and three rounds, the last one short.  The rows past each length are
-    # poisoned.
+    # One row over codes in a cache of 24k tokens and more runs the kernel whose extra waves move the
+    # codes into LDS, the keys first: a share of up to 17 blocks in one round, a longer one in rounds of up
+    # to 8 blocks in alternate halves of LDS.  Lengths: less than one block; a single block per share;
+    # shares of a few blocks; shares of 16 and of 17 blocks side by side (33000 tokens, and the whole of
+    # 34816: every share has block 16); 18 blocks and more: three rounds of 6 (34817 tokens and up), odd
+    # and even numbers of rounds, last rounds shorter than the others, up to five rounds at 81920.  The
+    # rows past each length are poisoned.
     rng = np.random.default_rng(77)
     k = (rng.standard_normal((capacity, VALUES)) * 2.0).astype(np.float32)
     v = rng.standard_normal((capacity, VALUES)).astype(np.float32)
     q = rng.standard_normal(H * D).astype(np.float32)
     qg = rng.standard_normal(H * 2 * D).astype(np.float32)
     att = saetta.DecodeAttention(H, KV, D, capacity)
-    for length in [1, 100, 2049, 8200, 16400, 33000, 34816, 50001, 81920]:
+    for length in [1, 100, 2049, 8200, 16400, 33000, 34816, 34817, 50001, 81920]:
         if length > capacity:
             continue
         kc, vc, kf, vf = cache_pair(k[:length], v[:length], kind, capacity, poison=True)
@@ -381,10 +379,10 @@ def test_large_cache_of_codes_one_row(kind, capacity):
 
 
 def test_four_bit_one_row_in_a_cache_of_131072_tokens():
-    # 4-bit codes in caches of 102401 to 139264 tokens go to the ring of four 64-token slots with shares of
-    # up to 64 blocks: sixteen iterations, eight rounds of the two teams, every slot refilled several times.
-    # Lengths: a single token; shares of 35 blocks (odd numbers of iterations per team); 120000 tokens; the
-    # whole capacity.  The rows past each length are poisoned.
+    # One row over 4-bit codes in a cache of 131072 tokens: shares of up to 64 blocks, eight rounds in alternate
+    # halves of LDS, each half refilled several times.  Lengths: a single token; shares of 35 blocks (an odd
+    # number of rounds, the last one short); 120000 tokens; the whole capacity.  The rows past each length
+    # are poisoned.
     rng = np.random.default_rng(131)
     capacity, kind = 131072, saetta.KvBits.Four
     k = (rng.standard_normal((capacity, VALUES)) * 2.0).astype(np.float32)
