@@ -123,8 +123,15 @@ template <int BITS>
 struct Stage {
     uint32_t k[BITS == 16 ? 16 : BITS];     // 32 dims: 64 B (f16), 32 B (8-bit), 16 B (4-bit)
     uint32_t v[8][BITS == 16 ? 2 : 1];      // per key 4 dims: 8 B (f16), 4 B (8-bit), 2 B (4-bit)
-    uint32_t ks, kz;                        // f16 scale and bias of (key, group of the piece)
-    uint32_t vs[8], vz[8];                  // per key, group of dq
+};
+
+// Scales and biases of a block's 32 keys, staged in LDS by the first 128 threads (8 bytes each: the four f16
+// of a key's groups) and read from there: per array [key][groups (0, 1) | groups (2, 3)] as pairs of f16.
+struct BlockScales {
+    uint32_t w[4][BK][2];  // [k scales | k biases | v scales | v biases]
+    __device__ __forceinline__ float get(int arr, int key, int group) const {
+        return (float)__builtin_bit_cast(_Float16, uint16_t(w[arr][key][group >> 1] >> (16 * (group & 1))));
+    }
 };
 
 struct Rsrc {
@@ -154,11 +161,6 @@ __device__ __forceinline__ void stage_load(Stage<BITS> &st, const Rsrc &r, uint3
                 st.k[4 * i] = x.x, st.k[4 * i + 1] = x.y, st.k[4 * i + 2] = x.z, st.k[4 * i + 3] = x.w;
             }
         }
-        if constexpr (BITS != 16) {
-            const int soff = (row * 4 + (piece >> 1)) * 2;
-            st.ks = __builtin_amdgcn_raw_buffer_load_b16(r.ks, soff, 0, 0);
-            st.kz = __builtin_amdgcn_raw_buffer_load_b16(r.kz, soff, 0, 0);
-        }
     }
     {
         const int dq = tid & 63, kq = tid >> 6;
@@ -173,11 +175,6 @@ __device__ __forceinline__ void stage_load(Stage<BITS> &st, const Rsrc &r, uint3
             } else {
                 const u32x2 x = __builtin_amdgcn_raw_buffer_load_b64(r.v, off, 0, 0);
                 st.v[i][0] = x.x, st.v[i][1] = x.y;
-            }
-            if constexpr (BITS != 16) {
-                const int soff = (row * 4 + (dq >> 4)) * 2;
-                st.vs[i] = __builtin_amdgcn_raw_buffer_load_b16(r.vs, soff, 0, 0);
-                st.vz[i] = __builtin_amdgcn_raw_buffer_load_b16(r.vz, soff, 0, 0);
             }
         }
     }
@@ -198,7 +195,7 @@ __device__ __forceinline__ constexpr int vt_pos(int key) {
 // (the end of the chunk) are written as zeros: their probabilities are 0, and 0 * 0
 // stays 0 whatever the cache rows hold.
 template <int BITS>
-__device__ __forceinline__ void stage_store(const Stage<BITS> &st, unsigned char *k_img, unsigned char *v_img,
+__device__ __forceinline__ void stage_store(const Stage<BITS> &st, const BlockScales &sb, unsigned char *k_img, unsigned char *v_img,
                                             uint32_t key0, uint32_t key_limit, int tid) {
     {
         const int key = tid >> 3, piece = tid & 7;
@@ -207,7 +204,7 @@ __device__ __forceinline__ void stage_store(const Stage<BITS> &st, unsigned char
 #pragma unroll
             for (int i = 0; i < 16; i++) o[i] = st.k[i];
         } else {
-            const float s = h2f(st.ks), z = h2f(st.kz);
+            const float s = sb.get(0, key, piece >> 1), z = sb.get(1, key, piece >> 1);
             constexpr int PER = 32 / BITS;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
@@ -242,7 +239,7 @@ __device__ __forceinline__ void stage_store(const Stage<BITS> &st, unsigned char
 #pragma unroll
                     for (int d = 0; d < 4; d++) x[u][d] = live ? h2f(st.v[i + u][d >> 1] >> (16 * (d & 1))) : 0.0f;
                 } else {
-                    const float s = h2f(st.vs[i + u]), z = h2f(st.vz[i + u]);
+                    const float s = sb.get(2, 8 * kq + i + u, dq >> 4), z = sb.get(3, 8 * kq + i + u, dq >> 4);
 #pragma unroll
                     for (int d = 0; d < 4; d++) x[u][d] = live ? dequant(s, z, code_of<BITS>(st.v[i + u][0], d)) : 0.0f;
                 }
@@ -260,10 +257,16 @@ __device__ __forceinline__ void stage_store(const Stage<BITS> &st, unsigned char
     }
 }
 
+// One workgroup per (block of 32 keys, kv head).  The K tile goes out as it is made (a wave's store is eight runs
+// of 128 bytes); the V^T tile is a transposition (a thread holds 4 dims of 8 keys, the image wants 8 keys of a dim
+// side by side), so it is put together in LDS and copied out as whole lines.
 template <int BITS>
 __global__ __launch_bounds__(PREP_THREADS) void prefill_prepare_kernel(PrepareArgs a) {
     constexpr int RB = row_bytes<BITS>();
+    __shared__ __attribute__((aligned(16))) unsigned char vt_lds[PART_BYTES];
+    __shared__ BlockScales sb;
     const uint32_t block = blockIdx.x, kv = blockIdx.y, kvh = a.kv_heads;
+    const int tid = threadIdx.x;
     const uint32_t cap_rows = a.key_limit * kvh;
     Rsrc rs;
     rs.k = make_rsrc(a.kdata, cap_rows * RB);
@@ -272,10 +275,27 @@ __global__ __launch_bounds__(PREP_THREADS) void prefill_prepare_kernel(PrepareAr
     rs.kz = make_rsrc(a.kbiases, BITS == 16 ? 0 : cap_rows * 8);
     rs.vs = make_rsrc(a.vscales, BITS == 16 ? 0 : cap_rows * 8);
     rs.vz = make_rsrc(a.vbiases, BITS == 16 ? 0 : cap_rows * 8);
+    if constexpr (BITS != 16) {
+        if (tid < 4 * BK) {
+            // (a key past the cache's end reads as zeros: its values are written as zeros whatever the scales are)
+            const int arr = tid / BK, key = tid % BK;
+            const int off = int((block * BK + key) * kvh + kv) * 8;
+            const __amdgpu_buffer_rsrc_t r = arr == 0 ? rs.ks : arr == 1 ? rs.kz : arr == 2 ? rs.vs : rs.vz;
+            const u32x2 x = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+            sb.w[arr][key][0] = x.x, sb.w[arr][key][1] = x.y;
+        }
+    }
     Stage<BITS> st;
-    stage_load<BITS>(st, rs, kvh, block * BK, kv, threadIdx.x);
+    stage_load<BITS>(st, rs, kvh, block * BK, kv, tid);
+    __syncthreads();  // the scales are in LDS
     unsigned char *img = a.images + (size_t(kv) * a.nblocks + block) * IMG_BYTES;
-    stage_store<BITS>(st, img, img + PART_BYTES, block * BK, a.key_limit, threadIdx.x);
+    stage_store<BITS>(st, sb, img, vt_lds, block * BK, a.key_limit, tid);
+    __syncthreads();  // the V^T tile is in LDS
+#pragma unroll
+    for (int i = 0; i < PART_BYTES / 16 / PREP_THREADS; i++) {
+        const int at = (i * PREP_THREADS + tid) * 16;
+        *reinterpret_cast<u32x4 *>(img + PART_BYTES + at) = *reinterpret_cast<const u32x4 *>(vt_lds + at);
+    }
 }
 
 // What a wave copies global -> LDS per step: 8 KB as eight global_load_lds_dwordx4 (64 lanes x
@@ -488,6 +508,11 @@ __device__ __forceinline__ float max_across_halves(float x) {
     asm volatile("s_nop 1\nv_permlane32_swap_b32 %0, %1\n" : "+v"(u), "+v"(v));
     return fmaxf(__builtin_bit_cast(float, u), __builtin_bit_cast(float, v));
 }
+
+// A workgroup barrier for data that went through LDS only: waits for this wave's LDS accesses, not for its
+// loads and stores to memory (__syncthreads waits for those too: behind the gate loads of a tile's end, or
+// the output stores, that is microseconds with nothing else to run).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // LDS: four K slots, then four V^T slots; block b uses slot b % 4 of each.
 constexpr int MERGE_WAVE_BYTES = (4 * 16 + 2) * 64 * 4;  // half of a wave's O, its m and l, on their way to its partner
@@ -722,7 +747,7 @@ __device__ __forceinline__ void prefill_tile(const PrefillArgs &a, unsigned char
     }
     mine_out[64 * 64] = m_ref;
     mine_out[65 * 64] = l_sum;
-    __syncthreads();
+    lds_barrier();  // (the gate values stay on their way)
     const float m_other = theirs_in[64 * 64], l_other = theirs_in[65 * 64];
     const float m_new = fmaxf(m_ref, m_other);
     const float mine = __builtin_amdgcn_exp2f(m_ref - m_new), theirs = __builtin_amdgcn_exp2f(m_other - m_new);
@@ -764,7 +789,7 @@ __global__ __launch_bounds__(THREADS, 2) void attention_prefill_kernel(PrefillAr
     const uint32_t ntiles = (a.tokens + TQ - 1) / TQ, total = ntiles * a.kv_heads, G = gridDim.x;
     for (uint32_t first = 0, round = 0; first < total; first += G, round++) {
         const uint32_t idx = first + ((round & 1) ? G - 1 - blockIdx.x : blockIdx.x);
-        if (round) __syncthreads();  // the last tile's merge has been read: the next tile's keys may land on it
+        if (round) lds_barrier();  // the last tile's merge has been read: the next tile's keys may land on it (its stores go on meanwhile)
         if (idx < total) prefill_tile(a, tiles, ntiles - 1 - idx / a.kv_heads, idx % a.kv_heads);
     }
 }
