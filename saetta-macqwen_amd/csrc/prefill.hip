@@ -80,6 +80,7 @@ struct PrepareArgs {
     unsigned char *images;  // [kv head][block][IMG_BYTES]
     uint32_t kv_heads, nblocks;
     uint32_t key_limit;  // pos + tokens: rows the cache holds; keys from here on are zeros
+    uint32_t *tiles_taken;  // behind the images (or nullptr): the attention kernel's count of tiles handed out, set to 0 here
 };
 
 struct PrefillArgs {
@@ -90,6 +91,7 @@ struct PrefillArgs {
     uint32_t heads, kv_heads, pos, tokens;
     float scale;
     uint32_t nblocks;  // images per kv head
+    uint32_t *tiles_taken;  // tiles handed out past every workgroup's first (zero at the start: the prepare kernel's doing)
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
@@ -267,6 +269,7 @@ __global__ __launch_bounds__(PREP_THREADS) void prefill_prepare_kernel(PrepareAr
     __shared__ BlockScales sb;
     const uint32_t block = blockIdx.x, kv = blockIdx.y, kvh = a.kv_heads;
     const int tid = threadIdx.x;
+    if (a.tiles_taken && block == 0 && kv == 0 && tid == 0) *a.tiles_taken = 0;
     const uint32_t cap_rows = a.key_limit * kvh;
     Rsrc rs;
     rs.k = make_rsrc(a.kdata, cap_rows * RB);
@@ -521,7 +524,7 @@ __device__ __forceinline__ uint32_t k_slot(uint32_t b) { return (b & 3) * PART_B
 __device__ __forceinline__ uint32_t v_slot(uint32_t b) { return (4 + (b & 3)) * PART_BYTES; }
 
 // One tile of TQ tokens x 8 heads of kv head `kv` against the keys it sees.
-__device__ __forceinline__ void prefill_tile(const PrefillArgs &a, unsigned char *tiles, uint32_t tile, uint32_t kv) {
+__device__ __forceinline__ void prefill_tile(const PrefillArgs &a, unsigned char *tiles, uint32_t tile, uint32_t kv, bool ask, uint32_t *next_tile) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, hf = lane >> 5;
@@ -712,6 +715,12 @@ __device__ __forceinline__ void prefill_tile(const PrefillArgs &a, unsigned char
     }
 
     settle(acc);
+    // Which tile this workgroup takes next: asked for here, where the workgroups are apart in time (their tiles differ in
+    // length; at the kernel's start every one of them would ask at once, and the adds on one word come one after the
+    // other), and looked at when the tile has ended.  (Before the gate loads: behind them the one more register that is
+    // live with them costs 150 bytes of spills.)
+    uint32_t got = ask ? 0u : 0xffffffffu;
+    if (ask && tid == 0) got = gridDim.x + atomicAdd(a.tiles_taken, 1u);
 
     // The gate values of this wave's half of the dims, asked for before the merge below so that they travel while
     // it runs (scattered 16-byte pieces, one round trip for the lot; a token past the end: the last token's, unused).
@@ -722,7 +731,6 @@ __device__ __forceinline__ void prefill_tile(const PrefillArgs &a, unsigned char
 #pragma unroll
         for (int i = 0; i < 16; i++) g[i] = *reinterpret_cast<const float4 *>(gate + 32 * (i >> 2) + 8 * (i & 3) + 4 * hf);
     }
-
     // ---- the two waves of a row group merge their halves of the keys ----------------------
     // Each wave finishes half of the dims: parity 0 the accumulators 0..3 (dims 0..127), parity 1
     // the rest.  It hands the other half, m and l to its partner through LDS (the tiles are done
@@ -777,20 +785,26 @@ __device__ __forceinline__ void prefill_tile(const PrefillArgs &a, unsigned char
             *reinterpret_cast<float4 *>(out + 32 * mt + 8 * q4 + 4 * hf) = w;
         }
     }
+    if (tid == 0) *next_tile = got;
 }
 
-// A workgroup takes tiles until there are none left: with more tiles than workgroups (one per CU:
-// the LDS ring fills a CU), the next tile starts without a new workgroup having to be dispatched.
-// Tiles are numbered from the one with the most keys down, the kv heads side by side, and handed
-// out boustrophedon: round 0 gives workgroup w tile w, round 1 tile 2 G - 1 - w, ... so that every
-// workgroup gets the same amount of keys to within a tile.
+// A workgroup takes tiles until there are none left: with more tiles than workgroups (one per CU: the LDS ring
+// fills a CU), the next tile starts without a new workgroup having to be dispatched.  Tiles are numbered from the
+// one with the most keys down, the kv heads side by side.  Workgroup w starts with tile w; the others are handed
+// out in that order to whoever asks next (one atomic add per tile on a counter behind the images, asked for
+// before the tile's epilogue so that the answer is there when it ends): a workgroup that took a long tile, or runs
+// on a slower CU, asks later and gets a shorter one, so that all of them end together (tiles dealt beforehand, the
+// longest with the shortest, ended 40 us apart: the workgroups' rates differ by a tenth).
 __global__ __launch_bounds__(THREADS, 2) void attention_prefill_kernel(PrefillArgs a) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char tiles[];
+    __shared__ uint32_t next_tile;
     const uint32_t ntiles = (a.tokens + TQ - 1) / TQ, total = ntiles * a.kv_heads, G = gridDim.x;
-    for (uint32_t first = 0, round = 0; first < total; first += G, round++) {
-        const uint32_t idx = first + ((round & 1) ? G - 1 - blockIdx.x : blockIdx.x);
-        if (round) lds_barrier();  // the last tile's merge has been read: the next tile's keys may land on it (its stores go on meanwhile)
-        if (idx < total) prefill_tile(a, tiles, ntiles - 1 - idx / a.kv_heads, idx % a.kv_heads);
+    for (uint32_t idx = blockIdx.x; idx < total;) {
+        // (the tiles from G on are handed out by one question each: the tiles before the last G ask one, when they end,
+        // and the last G none: nothing is left by then, and the kernel's last epilogues do not wait for an answer)
+        prefill_tile(a, tiles, ntiles - 1 - idx / a.kv_heads, idx % a.kv_heads, idx + G < total, &next_tile);
+        lds_barrier();  // the next tile is known; this tile's merge has been read: the next tile's keys may land on it (its stores go on meanwhile)
+        idx = next_tile;
     }
 }
 
@@ -805,10 +819,12 @@ constexpr int OWNED_DEVICES = 64;  // as many devices as the library's set-up ad
 std::map<std::pair<int, hipStream_t>, OwnedWorkspace> g_owned;
 std::mutex g_owned_mutex;
 
-size_t workspace_bytes(uint32_t pos, uint32_t tokens, uint32_t kv_heads) {
+// The images, then a line for the attention kernel's count of tiles handed out.
+size_t images_bytes(uint32_t pos, uint32_t tokens, uint32_t kv_heads) {
     const size_t blocks = (size_t(pos) + tokens + BK - 1) / BK;
     return blocks * kv_heads * IMG_BYTES;
 }
+size_t workspace_bytes(uint32_t pos, uint32_t tokens, uint32_t kv_heads) { return images_bytes(pos, tokens, kv_heads) + 256; }
 
 // The checks both prefill paths share.
 int check_prefill(int bits, const uint16_t *q, const void *kdata, const void *vdata, const uint16_t *ks,
@@ -868,10 +884,10 @@ int acquire_workspace(hipStream_t stream, void *&workspace, size_t workspace_siz
 // The images of rows 0 .. rows - 1 of the cache, at the start of the workspace.
 uint32_t launch_prepare(hipStream_t stream, int bits, const void *kdata, const void *vdata, const uint16_t *ks,
                         const uint16_t *kz, const uint16_t *vs, const uint16_t *vz, void *workspace, uint32_t kv_heads,
-                        uint64_t rows) {
+                        uint64_t rows, uint32_t *tiles_taken = nullptr) {
     const uint32_t nblocks = uint32_t((rows + BK - 1) / BK);
     PrepareArgs pa{kdata, vdata, ks, kz, vs, vz, static_cast<unsigned char *>(workspace), kv_heads, nblocks,
-                   uint32_t(rows)};
+                   uint32_t(rows), tiles_taken};
     const dim3 pgrid(nblocks, kv_heads);
     if (bits == 8) {
         prefill_prepare_kernel<8><<<pgrid, PREP_THREADS, 0, stream>>>(pa);
@@ -894,9 +910,10 @@ int run_prefill(hipStream_t stream, int bits, const uint16_t *q, const void *kda
     const size_t need = workspace_bytes(p.pos, p.tokens, p.kv_heads);
     std::unique_lock<std::mutex> owned_lock(g_owned_mutex, std::defer_lock);
     if (int rc = acquire_workspace(stream, workspace, workspace_size, need, owned_lock, what, "saetta_prefill_workspace_bytes")) return rc;
-    const uint32_t nblocks = launch_prepare(stream, bits, kdata, vdata, ks, kz, vs, vz, workspace, p.kv_heads, rows);
+    uint32_t *tiles_taken = reinterpret_cast<uint32_t *>(static_cast<unsigned char *>(workspace) + images_bytes(p.pos, p.tokens, p.kv_heads));
+    const uint32_t nblocks = launch_prepare(stream, bits, kdata, vdata, ks, kz, vs, vz, workspace, p.kv_heads, rows, tiles_taken);
     PrefillArgs a{q, static_cast<const unsigned char *>(workspace), q_and_gate, out, p.heads, p.kv_heads, p.pos,
-                  p.tokens, p.scale, nblocks};
+                  p.tokens, p.scale, nblocks, tiles_taken};
     // one workgroup per CU at most: a workgroup's LDS ring fills a CU, and further tiles are taken in the kernel
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
