@@ -252,7 +252,8 @@ _calib = None
 
 
 def calib_lib(s):
-    """The calibration kernels (a plain streaming read): a library of their own beside the product's."""
+    """The calibration kernels (a plain streaming read; the prefill kernel's MFMA streams alone): a library of
+    their own beside the product's."""
     global _calib
     if _calib is None:
         import ctypes
@@ -261,6 +262,9 @@ def calib_lib(s):
         _calib.saetta_calib_read.restype = ctypes.c_int
         _calib.saetta_calib_read.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint32,
                                              ctypes.c_uint32, ctypes.c_void_p]
+        _calib.saetta_calib_mfma.restype = ctypes.c_int
+        _calib.saetta_calib_mfma.argtypes = [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32,
+                                             ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p]
     return _calib
 
 
@@ -301,6 +305,62 @@ def reader_floor(s, torch, args, nbytes, layers, workgroups=256):
     empty = round(timed(0, 16 * workgroups), 3)
     assert int(sink.sum().item()) == 0
     return out, empty
+
+
+def mfma_floor(s, torch, args, steps=192, workgroups=256, nbytes=16 * 1024 * 1024 + 768 * 1024):
+    """What rate of f16 MFMAs ONE launch shaped like the prefill attention kernel (a workgroup of 8 waves per CU,
+    `steps` x 32 MFMAs per wave: 192 steps are the two tiles a workgroup takes at 4096 tokens behind 4096) sustains
+    with nothing else to do, and at what shader clock: on operands that never change, on operands that change with
+    every MFMA, and as the prefill kernel's own instruction streams (fragment reads from LDS, global -> LDS copies
+    out of a buffer of the key and value images' size, a barrier per step) without the softmax.  The operands are
+    N(0, 1) values in f16, like the keys and queries of the prefill workload.  Launches back to back, timed with
+    events like the prefill kernel.  Returns {variant: {"TFLOP/s", "GHz", "us"}}."""
+    import ctypes
+    lib = calib_lib(s)
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    operands = torch.randn(nbytes // 2, generator=gen, device="cuda").to(torch.float16)
+    out = torch.zeros(2 * workgroups, dtype=torch.int64, device="cuda")
+    sink = torch.zeros(workgroups, dtype=torch.float32, device="cuda")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    names = {0: "operands that never change", 1: "operands that change with every MFMA",
+             2: "the prefill kernel's streams (LDS fragment reads, copies, barrier), no softmax"}
+    flops = workgroups * 8 * steps * 32 * 32768.0
+    res = {}
+    for v, name in names.items():
+        def run():
+            s.ffi.check(lib.saetta_calib_mfma(stream, v, steps, workgroups, ctypes.c_void_p(operands.data_ptr()), nbytes,
+                                              ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(sink.data_ptr())), "calib_mfma")
+        for _ in range(max(3, args.warmup)):
+            run()
+        ts, ghz = [], []
+        for _ in range(max(5, args.steps)):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            run()
+            e1.record()
+            e1.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e3)
+            c = out.view(workgroups, 2).double()
+            ghz.append(float((c[:, 0] / (c[:, 1] * 10.0)).mean().item()))
+        us = median(ts)
+        res[name] = {"TFLOP/s": round(flops / (us * 1e-6) / 1e12, 1), "GHz": round(median(ghz), 3), "us": round(us, 1)}
+    return res
+
+
+def bench_mfma_floor(s, torch, args):
+    variants = mfma_floor(s, torch, args)
+    best = variants["the prefill kernel's streams (LDS fragment reads, copies, barrier), no softmax"]
+    return {
+        "metric": "f16 MFMA rate of the prefill kernel's streams alone, TFLOP/s",
+        "value": best["TFLOP/s"], "unit": "TFLOP/s", "ms_per_step": round(best["us"] / 1e3, 4),
+        "dtype": "f16 MFMA",
+        "config": {"workload": "calibration: one launch of 256 workgroups of 8 waves, 192 steps of 32 "
+                               "v_mfma_f32_32x32x16_f16 per wave, N(0,1) operands", "variants": variants},
+        "roofline": {"bound": "mfma", "achieved": best["TFLOP/s"], "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(best["TFLOP/s"] / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "calib_mfma_stream_kernel", "avg_us": best["us"]},
+        "cpu_baseline": None,
+    }
 
 
 def bench_reader_floor(s, torch, args, ctx=32768, layers=32):
@@ -378,6 +438,12 @@ def bench_prefill(s, torch, args, tokens=4096, pos=4096, bits=8, gemm=False):
                 "unit": "TFLOP/s", "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4),
                 "traffic": MEASURED_TRAFFIC.get("prefill") if (tokens, pos, bits, gemm) == (4096, 4096, 8, False) else None,
                 "kernel": "attention_prefill_kernel", "avg_us": round(kern_us, 2)}
+    if not gemm and not args.no_reader_floor:
+        # what the kernel's own MFMA streams reach with no softmax, prologue or epilogue around them
+        floor = mfma_floor(s, torch, args)
+        stream_only = floor["the prefill kernel's streams (LDS fragment reads, copies, barrier), no softmax"]["TFLOP/s"]
+        roofline["mfma_streams_alone"] = floor
+        roofline["frac_of_streams_alone"] = round(achieved / stream_only, 4)
     if gemm:
         # What bounds this route is the scratch it writes and reads back.  Algorithmic bytes per query row: 2 B out
         # and 2 B in per key its 16-token tile sees (in whole tiles of 32 keys), and a maximum and a sum (8 B)
@@ -692,7 +758,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="default",
                     choices=["decode8_32k", "decode4_150k", "decode16_4k", "verify2", "verify3", "verify4", "prefill", "prefill_131k", "prefill_gemm", "prefill_gemm_131k", "deltanet",
-                             "deltanet_prefill", "prep_store", "reader_floor", "default", "all"])
+                             "deltanet_prefill", "prep_store", "reader_floor", "mfma_floor", "default", "all"])
     ap.add_argument("--no-graph", action="store_true", help="launch from Python instead of replaying a HIP graph")
     ap.add_argument("--layers", type=int, default=0, help="layer caches per step (default 32; 12 at 150k)")
     ap.add_argument("--ctx", type=int, default=0, help="context length of the decode and verify workloads (default: the workload's own)")
@@ -737,6 +803,8 @@ def main():
             return bench_prep_store(s, torch, args)
         if workload == "reader_floor":
             return bench_reader_floor(s, torch, args)
+        if workload == "mfma_floor":
+            return bench_mfma_floor(s, torch, args)
         if workload == "prefill_131k":
             # the last 4096-token chunk of a 131072-token context: whether the one flash kernel holds up where
             # the reference switches to its multi-pass form (src/attention_gemm.rs)
