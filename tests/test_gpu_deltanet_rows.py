@@ -132,6 +132,41 @@ def test_real_shape_longer_chunk_against_oracle():
     check_against_oracle(layer, 250, [100, 150], snapshots=False)
 
 
+@pytest.mark.parametrize("scale", [1e-3, 1.0, 1e3])
+def test_blocks_of_tokens_hold_values_and_states_far_from_one(scale):
+    # The blocks' products take every operand as an f16 hi part and an f16 lo part: a value v (or a state entry) keeps
+    # 22 bits while its lo part is a normal f16 (|v| above 2^-3), fewer below (the lo part of 1e-3 is 5e-7, a subnormal
+    # with a step of 6e-8: 14 bits left), and nothing above 65504.  The delta rule is linear in (state, values) together,
+    # so the state after the same tokens with both scaled by 1e-3 and by 1e3 is held to the oracle's f32 chain at that
+    # scale, relative to the largest entry: 2e-5 at 1 and 1e3, 3e-4 at 1e-3 (measured 1e-4; a real layer's values are O(1)).
+    # The output is normalised per head with eps = 1e-6 under the root: at scale 1 that eps mutes the heads whose output
+    # nearly cancels, at 1e3 it does not, and what is left of such a head's output is its rounding (measured 3e-4 of the
+    # largest output against 2e-5 at scale 1): held to 1e-3 there.
+    layer = Layer(16, 32, 128, 4, seed=21)
+    tokens = 200
+    x, z, a, b = layer.inputs(tokens)
+    mixed = np.tanh(x).astype(np.float32)  # what a convolution would hand over: q, k and v of every token
+    mixed[:, 2 * layer.key:] *= scale
+    state0 = (scale * 0.5 * layer.rng.standard_normal(layer.v_heads * layer.v_dim * K_DIM)).astype(np.float32)
+    state_cpu = state0.copy()
+    want_y = np.stack([oracle.deltanet_step(m[:layer.key], m[layer.key:2 * layer.key], m[2 * layer.key:], a[t], b[t],
+                                            layer.a_log, layer.dt_bias, state_cpu, z[t], layer.norm, layer.k_heads,
+                                            layer.v_heads, K_DIM, layer.v_dim, EPS).reshape(-1) for t, m in enumerate(mixed)])
+    state = dev(state0)
+    y = torch.empty(tokens, layer.val, device="cuda")
+    plan = saetta.Plan()
+    saetta.deltanet_rows(plan, dev(mixed), dev(a), dev(b), dev(layer.a_log), dev(layer.dt_bias), state, dev(z),
+                         dev(layer.norm), y, layer.k_heads, layer.v_heads, layer.v_dim, tokens, EPS, None)
+    plan.build().run()
+    torch.cuda.synchronize()
+    tol = 3e-4 if scale < 1 else 2e-5
+    got = host(state).reshape(-1)
+    assert np.isfinite(got).all()
+    err = float(np.abs(got - state_cpu).max() / np.abs(state_cpu).max())
+    assert err <= tol, (scale, err)
+    assert close(host(y), want_y, 2e-5 if scale == 1.0 else 1e-3), scale
+
+
 def test_blocks_of_tokens_other_value_dims():
     # value dims that are multiples of 16 take the blocks too; 24 keeps to the token-by-token kernels
     for v_dim, tokens in ((16, 130), (64, 192), (256, 129), (24, 140)):
