@@ -122,11 +122,12 @@ def test_bad_arguments_are_rejected_before_any_launch():
     fp = ffi.FlashParamsC(16, 2, 0, 1, 0.0625)
     assert lib.saetta_attn_prefill_quant(None, 16, 16, rows, rows, 16, 16, fp, None, 0) == -1
     assert lib.saetta_attn_prefill_quant(None, 8, 16, rows, rows, 16, 16, fp, 8, 1 << 30) == -4  # workspace alignment
-    # 32 keys per image, one image per kv head and block, whole kilobytes each
-    one = lib.saetta_prefill_workspace_bytes(0, 32, 1)
+    # 32 keys per image, one image per kv head and block, whole kilobytes each; behind them a 256-byte line
+    # (the attention kernel's count of tiles handed out)
+    one = lib.saetta_prefill_workspace_bytes(0, 32, 1) - 256
     assert one % 1024 == 0 and one >= 2 * 32 * 256 * 2
-    assert lib.saetta_prefill_workspace_bytes(4096, 4096, 2) == one * 2 * 256
-    assert lib.saetta_prefill_workspace_bytes(0, 33, 1) == 2 * one
+    assert lib.saetta_prefill_workspace_bytes(4096, 4096, 2) == one * 2 * 256 + 256
+    assert lib.saetta_prefill_workspace_bytes(0, 33, 1) == 2 * one + 256
     with pytest.raises(ffi.SaettaError):
         ffi.check(-1, "demo")
 
