@@ -49,7 +49,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # rocprofv3 --pmc, each scaled by what the same counter reads for a 256 MiB copy in the same run;
 # the runs are summarised in profiles/*_hbm_traffic.txt).  Counters cannot be read inside this
 # script, so the figures are carried here for the workloads they were measured on.
-MEASURED_TRAFFIC = {"decode8_32k": 38.2e6, "prefill": 294.3e6, "decode4_150k": 91.7e6, "verify4": 45.1e6,
+MEASURED_TRAFFIC = {"decode8_32k": 38.2e6, "prefill": 421.5e6, "decode4_150k": 88.9e6, "verify4": 45.0e6,
                     "deltanet_prefill": 664.1e6,  # (the three kernels of the chunk together)
                     "prefill_gemm": 2.18e9}       # (the 2 launches of a call together)
 
