@@ -12,11 +12,11 @@ from . import ffi
 from .host import (GROUP, KV_ALIGN, MAX_ROWS, AttentionRows, Built, DecodeAttention, FlashParams, GpuKvCache, KvBits,
                    Plan, RowBackup,
                    PrepParams, QuantRows, TokenParams, attention_gemm, attention_prefill, bench, deltanet_conv, deltanet_conv_rows, deltanet_rows, deltanet_rows_fused, deltanet_token,
-                   deltanet_step, dequantize, quantize, round_trip,
+                   deltanet_step, dequantize, device_status, quantize, round_trip,
                    record_store, round_trip_as_half, test_slack, to_half)
 
 __all__ = ["ffi", "GROUP", "KV_ALIGN", "MAX_ROWS", "AttentionRows", "Built", "DecodeAttention", "FlashParams",
            "GpuKvCache", "KvBits", "RowBackup",
            "Plan", "PrepParams", "QuantRows", "TokenParams", "attention_gemm", "attention_prefill", "bench", "deltanet_conv", "deltanet_conv_rows",
-           "deltanet_rows", "deltanet_rows_fused", "deltanet_token", "deltanet_step", "dequantize", "quantize",
+           "deltanet_rows", "deltanet_rows_fused", "deltanet_token", "deltanet_step", "dequantize", "device_status", "quantize",
            "record_store", "round_trip", "round_trip_as_half", "test_slack", "to_half"]

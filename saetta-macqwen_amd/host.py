@@ -69,6 +69,12 @@ def _ptr(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
+def device_status(clear=False):
+    """The current device's sticky status word: 0 unless a kernel's bounded wait gave up, after which
+    every call on the device raises (SAETTA_E_WAIT) until the word is cleared."""
+    return int(ffi.lib().saetta_device_status(1 if clear else 0))
+
+
 def _need(t, dtype, what):
     if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == dtype and t.is_contiguous()):
         raise TypeError(f"{what}: expected a contiguous {dtype} tensor on the GPU")

@@ -43,6 +43,9 @@ inline void check(int rc, const char *what) {
 inline void hip_check(hipError_t e, const char *what) {
     if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
 }
+// The current device's sticky status word: 0 unless a kernel's bounded wait gave up, after which every call on the
+// device fails (check() throws) until the word is cleared.  The reference asserts on its command buffers' status.
+inline uint32_t device_status(bool clear = false) { return saetta_device_status(clear ? 1 : 0); }
 
 namespace gpu {
 

@@ -129,4 +129,4 @@ def test_no_bounded_wait_gave_up_in_this_process():
     # this process have run (a wave whose bounded wait runs out leaves a code there).
     ffi.check(ffi.lib().saetta_init(), "init")
     torch.cuda.synchronize()
-    assert ffi.lib().saetta_device_status(0) == 0
+    assert saetta.device_status() == 0
