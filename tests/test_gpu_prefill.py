@@ -183,12 +183,15 @@ def test_spread_rows2_and_bench_mirror_the_reference():
         assert [r["tokens"] for r in rows] == [256, 1000] and all(r["GB/s"] > 0 and r["reduce_ms"] > 0 for r in rows)
 
 
-def test_equal_keys_give_running_means_at_full_size():
+@pytest.mark.parametrize("pos,tokens", [(4096, 4096), (0, 1000), (37, 3001), (100, 9000)])
+def test_equal_keys_give_running_means_at_full_size(pos, tokens):
     # A closed form for every one of the 4096 x 16 rows of the headline shape: with the same key in every cache
     # row all scores of a token are equal, so token i's output is the mean of the first pos + i + 1 value rows
     # (as the half values the cache is read through) times sigmoid(gate), whatever q is.  A key block skipped,
     # taken twice or masked at the wrong place, or a wrong merge of the two waves of a row group, moves it.
-    pos = tokens = 4096
+    # The other shapes are the other ways the tiles reach the workgroups (one workgroup per CU takes tiles until
+    # none are left, the ones past its first by asking a counter): 126 tiles, fewer than workgroups; 376, between
+    # one and two each; 1126, more than four each, the chunk and its position ragged against tiles and key blocks.
     n = pos + tokens
     kind = saetta.KvBits.Eight
     gen = torch.Generator(device="cuda").manual_seed(17)
@@ -207,6 +210,7 @@ def test_equal_keys_give_running_means_at_full_size():
     vf = oracle.dequantize(host(vc.data).view(np.uint32), host(vc.scales).view(np.uint16), host(vc.biases).view(np.uint16), 8)
     vf = vf.reshape(n, VALUES).astype(np.float16).astype(np.float64)
     sums = np.cumsum(vf[pos:], axis=0) + vf[:pos].sum(axis=0)          # [tokens, 512]
+    assert np.isfinite(got).all()
     means = (sums / (pos + 1 + np.arange(tokens))[:, None]).reshape(tokens, KV, D)
     gate = 1.0 / (1.0 + np.exp(-host(qg).reshape(tokens, H, 2 * D)[:, :, D:].astype(np.float64)))
     want = np.repeat(means, H // KV, axis=1) * gate
